@@ -1,0 +1,140 @@
+// Shared device helpers for the gfx950 GGUF kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/cut_hip.h"
+
+namespace cuthip {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+
+// Block geometry (interface/loader/gguf/gguf_types.hpp:109-142).
+template <int FMT> struct Fmt;
+template <> struct Fmt<CUTHIP_Q8_0> { static constexpr int elems = 32, bytes = 34; };
+template <> struct Fmt<CUTHIP_Q4_0> { static constexpr int elems = 32, bytes = 18; };
+template <> struct Fmt<CUTHIP_Q4_K> { static constexpr int elems = 256, bytes = 144; };
+template <> struct Fmt<CUTHIP_Q6_K> { static constexpr int elems = 256, bytes = 210; };
+
+__host__ __device__ inline int fmt_elems(int fmt) { return (fmt == CUTHIP_Q8_0 || fmt == CUTHIP_Q4_0) ? 32 : 256; }
+__host__ __device__ inline int fmt_bytes(int fmt) {
+  return fmt == CUTHIP_Q8_0 ? 34 : fmt == CUTHIP_Q4_0 ? 18 : fmt == CUTHIP_Q4_K ? 144 : 210;
+}
+
+// GGUF blocks are only 2-byte aligned (34, 18 and 210 byte strides); gfx950
+// serves unaligned vector loads from global memory, so wide loads go through
+// packed views and the compiler still emits global_load_dwordx2/x4.
+struct __attribute__((packed, aligned(2))) U16x1 { uint16_t v; };
+struct __attribute__((packed, aligned(2))) U32x2p { uint32_t v[2]; };
+struct __attribute__((packed, aligned(2))) U32x4p { uint32_t v[4]; };
+
+__device__ inline uint32_t ld_u16(const uint8_t *p) { return reinterpret_cast<const U16x1 *>(p)->v; }
+__device__ inline u32x2 ld_u32x2(const uint8_t *p) {
+  U32x2p t = *reinterpret_cast<const U32x2p *>(p);
+  return u32x2{t.v[0], t.v[1]};
+}
+__device__ inline u32x4 ld_u32x4(const uint8_t *p) {
+  U32x4p t = *reinterpret_cast<const U32x4p *>(p);
+  return u32x4{t.v[0], t.v[1], t.v[2], t.v[3]};
+}
+
+__device__ inline float f16bits_to_f32(uint32_t h) {
+  uint16_t b = (uint16_t)h;
+  return (float)__builtin_bit_cast(half_t, b);  // exact, subnormals included
+}
+__device__ inline bool f16bits_finite(uint32_t h) { return (h & 0x7C00u) != 0x7C00u; }
+
+// fp32 -> fp16 bits with the reference's host narrowing (llama.cpp:445-482):
+// round half away from zero, subnormals kept, overflow and NaN -> +-Inf.
+// Setting the lowest fp32 mantissa bit turns every exact tie into "just above
+// the tie" and moves no other value across a rounding boundary, so the
+// hardware's round-to-nearest-even conversion then gives the same bits.
+// Valid for finite inputs only (an Inf would become a NaN).
+__device__ inline uint32_t f32_to_f16bits_finite(float v) {
+  uint32_t u = __builtin_bit_cast(uint32_t, v) | 1u;
+  half_t h = (half_t)__builtin_bit_cast(float, u);
+  return (uint32_t)__builtin_bit_cast(uint16_t, h);
+}
+// Any input, bit for bit the reference's algorithm.
+__device__ inline uint32_t f32_to_f16bits_any(float v) {
+  uint32_t u = __builtin_bit_cast(uint32_t, v);
+  uint32_t sign = (u >> 16) & 0x8000u;
+  if ((u & 0x7F800000u) == 0x7F800000u) return sign | 0x7C00u;
+  return f32_to_f16bits_finite(v);
+}
+
+__device__ inline float cvt_ubyte0(uint32_t v) { return (float)(v & 0xFFu); }
+__device__ inline float cvt_ubyte1(uint32_t v) { return (float)((v >> 8) & 0xFFu); }
+__device__ inline float cvt_ubyte2(uint32_t v) { return (float)((v >> 16) & 0xFFu); }
+__device__ inline float cvt_ubyte3(uint32_t v) { return (float)(v >> 24); }
+
+// Q4_K: the eight 6-bit (scale, min) pairs of a super-block from its 12 packed
+// bytes s0|s1|s2, four per dword (get_scale_min_k4, gguf_reader.cpp:668-676).
+__device__ inline void q4k_scales(uint32_t s0, uint32_t s1, uint32_t s2, uint32_t &sc_lo, uint32_t &sc_hi,
+                                  uint32_t &m_lo, uint32_t &m_hi) {
+  sc_lo = s0 & 0x3F3F3F3Fu;                                    // j = 0..3
+  m_lo = s1 & 0x3F3F3F3Fu;
+  sc_hi = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);      // j = 4..7
+  m_hi = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
+}
+
+// Unary / binary epilogues of the matmul (MatMulQ8Common.cuh:58-109).
+__device__ inline float apply_unary(int op, float v) {
+  switch (op) {
+  case CUTHIP_UNARY_SILU: return v / (1.0f + __expf(-v));
+  case CUTHIP_UNARY_RELU: return v > 0.0f ? v : 0.0f;
+  case CUTHIP_UNARY_GELU_TANH: {
+    float t = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+    return 0.5f * v * (1.0f + tanhf(t));
+  }
+  case CUTHIP_UNARY_SIGMOID: return 1.0f / (1.0f + __expf(-v));
+  case CUTHIP_UNARY_TANH: return tanhf(v);
+  case CUTHIP_UNARY_NEG: return -v;
+  }
+  return v;
+}
+__device__ inline float apply_binary(int op, float v, float d) {
+  switch (op) {
+  case CUTHIP_BINARY_ADD: return v + d;
+  case CUTHIP_BINARY_SUB: return v - d;
+  case CUTHIP_BINARY_MUL: return v * d;
+  case CUTHIP_BINARY_DIV: return v / d;
+  case CUTHIP_BINARY_MIN: return fminf(v, d);
+  case CUTHIP_BINARY_MAX: return fmaxf(v, d);
+  }
+  return v;
+}
+
+struct Epilogue {
+  int kind;  // cuthip_epilogue
+  int op;
+  const void *D;
+};
+
+// Stores one output element with the fused epilogue applied.
+__device__ inline void store_out(void *C, const Epilogue &e, int c_f16, size_t idx, float v) {
+  if (e.kind == CUTHIP_EPI_UNARY) {
+    v = apply_unary(e.op, v);
+  } else if (e.kind == CUTHIP_EPI_BINARY) {
+    float d = c_f16 ? (float)reinterpret_cast<const half_t *>(e.D)[idx] : reinterpret_cast<const float *>(e.D)[idx];
+    v = apply_binary(e.op, v, d);
+  }
+  if (c_f16)
+    reinterpret_cast<half_t *>(C)[idx] = (half_t)v;
+  else
+    reinterpret_cast<float *>(C)[idx] = v;
+}
+
+void set_error(const char *fmt, ...);
+int check_hip(hipError_t e, const char *what);
+
+}  // namespace cuthip

@@ -1,0 +1,114 @@
+"""ctypes binding of libcut_hip.so (the C ABI declared in include/cut_hip.h).
+
+The library is built in-tree by ``__graft_entry__.build()`` / ``make -C
+cut_amd/csrc``.  There is no CPU fallback: if the shared object is missing or a
+call fails, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libcut_hip.so")
+
+Q8_0, Q4_0, Q4_K, Q6_K = 0, 1, 2, 3
+F32, F16 = 0, 1
+OP_DEQUANT, OP_MATMUL_GGUF, OP_MATMUL_Q8, OP_MATMUL_Q4 = 0, 1, 2, 3
+EPI_NONE, EPI_UNARY, EPI_BINARY = 0, 1, 2
+UNARY = {"silu": 0, "relu": 1, "gelu_tanh": 2, "sigmoid": 3, "tanh": 4, "neg": 5}
+BINARY = {"add": 0, "sub": 1, "mul": 2, "div": 3, "min": 4, "max": 5}
+FORMATS = {"Q8_0": Q8_0, "Q4_0": Q4_0, "Q4_K": Q4_K, "Q6_K": Q6_K}
+BLOCK_ELEMS = {Q8_0: 32, Q4_0: 32, Q4_K: 256, Q6_K: 256}
+BLOCK_BYTES = {Q8_0: 34, Q4_0: 18, Q4_K: 144, Q6_K: 210}
+
+# every symbol include/cut_hip.h declares
+EXPORTS = [
+    "cuthip_init", "cuthip_last_error", "cuthip_device_info",
+    "cuthip_malloc", "cuthip_free", "cuthip_memcpy_h2d", "cuthip_memcpy_d2h", "cuthip_memcpy_d2d", "cuthip_memset",
+    "cuthip_stream_create", "cuthip_stream_destroy", "cuthip_stream_sync",
+    "cuthip_event_create", "cuthip_event_destroy", "cuthip_event_record", "cuthip_event_sync", "cuthip_event_elapsed_ms",
+    "cuthip_variant_count", "cuthip_variant_default", "cuthip_variant_info", "cuthip_variant_lookup",
+    "cuthip_dequant", "cuthip_matmul_gguf",
+]
+
+
+class CutHipError(RuntimeError):
+    """A C-ABI call returned non-zero (the reference throws std::runtime_error)."""
+
+
+class DeviceInfo(C.Structure):
+    _fields_ = [("name", C.c_char * 64), ("arch", C.c_char * 32), ("compute_units", C.c_int),
+                ("wave_size", C.c_int), ("lds_bytes_per_workgroup", C.c_int), ("clock_khz", C.c_int),
+                ("memory_clock_khz", C.c_int), ("memory_bus_bits", C.c_int), ("hbm_bytes", C.c_size_t),
+                ("l2_bytes", C.c_size_t)]
+
+
+class VariantInfo(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("wgX", C.c_uint32), ("wgY", C.c_uint32), ("effTileM", C.c_uint32),
+                ("effTileN", C.c_uint32), ("description", C.c_char_p)]
+
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Loads the shared object; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise CutHipError(f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                          "or `make -C cut_amd/csrc` (there is no CPU fallback)")
+    lib = C.CDLL(LIB_PATH)
+    vp, u32, i = C.c_void_p, C.c_uint32, C.c_int
+    lib.cuthip_last_error.restype = C.c_char_p
+    lib.cuthip_last_error.argtypes = []
+    lib.cuthip_init.argtypes = [i]
+    lib.cuthip_device_info.argtypes = [C.POINTER(DeviceInfo)]
+    lib.cuthip_malloc.argtypes = [C.POINTER(vp), C.c_size_t]
+    lib.cuthip_free.argtypes = [vp]
+    for n in ("cuthip_memcpy_h2d", "cuthip_memcpy_d2h", "cuthip_memcpy_d2d"):
+        getattr(lib, n).argtypes = [vp, vp, C.c_size_t, vp]
+    lib.cuthip_memset.argtypes = [vp, i, C.c_size_t, vp]
+    lib.cuthip_stream_create.argtypes = [C.POINTER(vp)]
+    lib.cuthip_stream_destroy.argtypes = [vp]
+    lib.cuthip_stream_sync.argtypes = [vp]
+    lib.cuthip_event_create.argtypes = [C.POINTER(vp)]
+    lib.cuthip_event_destroy.argtypes = [vp]
+    lib.cuthip_event_record.argtypes = [vp, vp]
+    lib.cuthip_event_sync.argtypes = [vp]
+    lib.cuthip_event_elapsed_ms.argtypes = [vp, vp, C.POINTER(C.c_float)]
+    lib.cuthip_variant_count.argtypes = [i]
+    lib.cuthip_variant_default.argtypes = [i]
+    lib.cuthip_variant_info.argtypes = [i, i, C.POINTER(VariantInfo)]
+    lib.cuthip_variant_lookup.argtypes = [i, C.c_char_p]
+    lib.cuthip_dequant.argtypes = [i, vp, vp, i, u32, u32, u32, vp]
+    lib.cuthip_matmul_gguf.argtypes = [i, vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, i, vp]
+    for n in EXPORTS:
+        if n != "cuthip_last_error":
+            getattr(lib, n).restype = i
+    _lib = lib
+    return lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        raise CutHipError(f"cut_hip error {rc}: {load().cuthip_last_error().decode()}")
+
+
+def variants(op: int) -> list[dict]:
+    lib = load()
+    out = []
+    for idx in range(lib.cuthip_variant_count(op)):
+        v = VariantInfo()
+        check(lib.cuthip_variant_info(op, idx, C.byref(v)))
+        out.append({"index": idx, "name": v.name.decode(), "wgX": v.wgX, "wgY": v.wgY, "effTileM": v.effTileM,
+                    "effTileN": v.effTileN, "description": v.description.decode()})
+    return out
+
+
+def device_info() -> dict:
+    d = DeviceInfo()
+    check(load().cuthip_device_info(C.byref(d)))
+    return {f: (getattr(d, f).decode() if isinstance(getattr(d, f), bytes) else getattr(d, f)) for f, _ in d._fields_}

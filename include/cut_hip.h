@@ -1,0 +1,152 @@
+/*
+ * cut_hip.h -- C ABI of the MI355X (gfx950) backend for CUT's GGUF
+ * quantized-matmul path: block dequantization, the batch-1..8 quantized GEMV
+ * of decode and the dequant-to-LDS MFMA GEMM of prefill.
+ *
+ * Plain pointers and sizes only; every pointer named "device" is a HIP device
+ * address owned by the caller.  No entry point below allocates device memory
+ * unless its comment says so.  All functions return 0 on success and a
+ * negative cuthip_status otherwise; cuthip_last_error() then holds a message
+ * (thread-local).  A C++ caller maps non-zero to std::runtime_error, which is
+ * how the reference reports failures (core/api/src/ComputeCommon.cpp:48-52).
+ *
+ * Precedent in the reference for "HIP behind a C ABI so host .cpp files need
+ * no HIP header": benchmarks/vendor/amd/rocblas_wrappers.hip:1-120.
+ */
+#ifndef CUT_HIP_H
+#define CUT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  CUTHIP_OK = 0,
+  CUTHIP_ERR_INVALID = -1,   /* bad argument / unsupported shape */
+  CUTHIP_ERR_HIP = -2,       /* a HIP runtime call failed */
+  CUTHIP_ERR_NO_DEVICE = -3, /* no gfx950 device */
+  CUTHIP_ERR_UNKNOWN_VARIANT = -4
+} cuthip_status;
+
+/* GGUF block formats (interface/loader/gguf/gguf_types.hpp:109-142):
+ * Q8_0 34 B / 32, Q4_0 18 B / 32, Q4_K 144 B / 256, Q6_K 210 B / 256. */
+typedef enum { CUTHIP_Q8_0 = 0, CUTHIP_Q4_0 = 1, CUTHIP_Q4_K = 2, CUTHIP_Q6_K = 3 } cuthip_format;
+typedef enum { CUTHIP_F32 = 0, CUTHIP_F16 = 1 } cuthip_dtype;
+
+/* Operator families with variant tables (the shape of
+ * operators/impl/matmul/MatMulQ4Variants.generated.h:11-29). */
+typedef enum { CUTHIP_OP_DEQUANT = 0, CUTHIP_OP_MATMUL_GGUF = 1, CUTHIP_OP_MATMUL_Q8 = 2, CUTHIP_OP_MATMUL_Q4 = 3 } cuthip_op;
+
+/* Fused epilogues of the matmul (operators/impl/matmul/MatMulQ8Common.cuh:58-109;
+ * MatMulOp.h:14 "MatMulFusion { None, Unary, Binary }"). */
+typedef enum { CUTHIP_EPI_NONE = 0, CUTHIP_EPI_UNARY = 1, CUTHIP_EPI_BINARY = 2 } cuthip_epilogue;
+typedef enum { CUTHIP_UNARY_SILU = 0, CUTHIP_UNARY_RELU = 1, CUTHIP_UNARY_GELU_TANH = 2, CUTHIP_UNARY_SIGMOID = 3, CUTHIP_UNARY_TANH = 4, CUTHIP_UNARY_NEG = 5 } cuthip_unary_op;
+typedef enum { CUTHIP_BINARY_ADD = 0, CUTHIP_BINARY_SUB = 1, CUTHIP_BINARY_MUL = 2, CUTHIP_BINARY_DIV = 3, CUTHIP_BINARY_MIN = 4, CUTHIP_BINARY_MAX = 5 } cuthip_binary_op;
+
+typedef struct {
+  char name[64];
+  char arch[32];
+  int compute_units;
+  int wave_size;
+  int lds_bytes_per_workgroup;
+  int clock_khz;
+  int memory_clock_khz;
+  int memory_bus_bits;
+  size_t hbm_bytes;
+  size_t l2_bytes;
+} cuthip_device_info_t;
+
+/* One row of a variant table: MatMulQ4VariantInfo{name,wgX,wgY,effTileM,
+ * effTileN,description} (MatMulQ4Variants.generated.h:11-18). Indices are ABI
+ * and never renumbered (MatMulOp.cpp:353-356). */
+typedef struct {
+  const char *name;
+  uint32_t wgX, wgY;
+  uint32_t effTileM, effTileN;
+  const char *description;
+} cuthip_variant_info_t;
+
+/* ---- library / device -------------------------------------------------- */
+
+/* Selects the device and checks that it is gfx950.  Replaces the backend
+ * constructor's device pick-up (core/backends/cuda/CudaCompute.cpp:60-100). */
+int cuthip_init(int device);
+const char *cuthip_last_error(void);
+/* DeviceCaps + DeviceInfo of the reference (core/api/include/ComputeCommon.h:92-97). */
+int cuthip_device_info(cuthip_device_info_t *info);
+
+/* ---- memory, streams, events (ComputeInterface::createBuffer /
+ * copyDataToBuffer / copyDataFromBuffer, core/api/include/ComputeInterface.h:45-120;
+ * stream and event use of core/backends/cuda/CudaCommandBuffer.cpp:128-360).
+ * cuthip_malloc is the ONLY call in this header that allocates device memory. */
+int cuthip_malloc(void **device_ptr, size_t bytes);
+int cuthip_free(void *device_ptr);
+int cuthip_memcpy_h2d(void *device_dst, const void *host_src, size_t bytes, void *stream);
+int cuthip_memcpy_d2h(void *host_dst, const void *device_src, size_t bytes, void *stream);
+int cuthip_memcpy_d2d(void *device_dst, const void *device_src, size_t bytes, void *stream);
+int cuthip_memset(void *device_dst, int value, size_t bytes, void *stream);
+int cuthip_stream_create(void **stream);
+int cuthip_stream_destroy(void *stream);
+int cuthip_stream_sync(void *stream); /* NULL = the default stream */
+int cuthip_event_create(void **event);
+int cuthip_event_destroy(void *event);
+int cuthip_event_record(void *event, void *stream);
+int cuthip_event_sync(void *event);
+int cuthip_event_elapsed_ms(void *start, void *stop, float *ms);
+
+/* ---- variant tables ---------------------------------------------------- */
+int cuthip_variant_count(int op);
+int cuthip_variant_default(int op);
+int cuthip_variant_info(int op, int index, cuthip_variant_info_t *info);
+/* Index of a variant by name, or CUTHIP_ERR_UNKNOWN_VARIANT: an unknown name is
+ * a hard error, never a silently skipped dispatch (the hazard described in
+ * core/backends/cuda/CudaCommandBuffer.cpp:146-162). */
+int cuthip_variant_lookup(int op, const char *name);
+
+/* ---- dequantization ----------------------------------------------------
+ * Replaces Operations::dequantize(raw, fmt, rows, cols) / DequantOpNode
+ * (runtime/Operations.cpp:1354-1361, operators/impl/dequant/DequantOp.cpp:7-67;
+ * kernels DequantQ4K.cu:6-50, DequantQ6K.cu:6-64) and the host loops
+ * GGUFReader::dequantize_* (interface/loader/gguf/gguf_reader.cpp:541-850).
+ *
+ * blocks : device, rows x (cols/blk) GGUF blocks, row-major, 2-byte aligned
+ * out    : device, [rows, out_stride] elements of out_dtype; the reference
+ *          uses out_stride = (cols+3)&~3 (DequantOp.cpp:15)
+ * fp32 output is bit-identical to the reference's CPU dequantizers; fp16
+ * output is bit-identical to that followed by the host narrowing f32ToF16
+ * (interface/runner/llama/llama.cpp:445-482, used at :805-811 and :922-928).
+ * cols must be a multiple of the block size (32 or 256). */
+int cuthip_dequant(int fmt, const void *blocks, void *out, int out_dtype, uint32_t rows, uint32_t cols,
+                   uint32_t out_stride, void *stream);
+
+/* ---- quantized matmul on native GGUF blocks ------------------------------
+ * C[m,n] (op)= sum_k A[m,k] * dequant(W)[n,k]   ("A . dequant_cpu(W)^T")
+ *
+ * The op-level call behind Operations::matmul(a, packedB, scales)
+ * (runtime/Operations.cpp:226-231 -> MatMulOpNode 3-input constructor,
+ * operators/impl/matmul/MatMulOp.cpp:271-383) for weights kept as GGUF blocks:
+ * it supersedes MatMulQ{4,8}GemvKPar8.cu (M == 1 decode default,
+ * MatMulOp.cpp:336-356) and MatMulQ{4,8}CoopMatTiled.cu (M > 1 default,
+ * MatMulOp.cpp:363-374).
+ *
+ * W      : device, N rows of K/blk GGUF blocks (the file layout: GGUF dims
+ *          [K, N], gguf_reader.cpp:404-406); the base must be 16-byte aligned
+ *          and every row must start 2-byte aligned (always true)
+ * A      : device, [M, strideA] of a_dtype (fp32 as in the reference, or fp16)
+ * C      : device, [M, strideC] of c_dtype
+ * D      : device, [M, strideC] of c_dtype, second operand of a BINARY
+ *          epilogue (residual add etc.), else NULL
+ * K must be a multiple of the block size; fp32 accumulation throughout.
+ * variant: index into the CUTHIP_OP_MATMUL_GGUF table, or -1 = choose by shape
+ *          (M <= 8 -> streaming GEMV, else the LDS-tiled MFMA GEMM). */
+int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M, uint32_t K,
+                       uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D,
+                       int variant, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUT_HIP_H */
