@@ -1,0 +1,217 @@
+#!/usr/bin/env python3
+"""Benchmark of the GGUF quantized-matmul hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+Workload (BASELINE.json configs[2], the configuration the metric is quoted on):
+Q4_K GEMV at the FFN shapes of an 8B dense transformer, batch 1, fp16
+activations in and out, fp32 accumulation.  One step = the three GEMVs of one
+FFN block (gate and up 14336 x 4096, down 4096 x 14336).  Weights are resident
+in HBM before the timed region and every step reads a different copy of them
+(COPIES sets, 595 MB in total), so they stream from HBM and not from the
+256 MB Infinity Cache.  The K timed steps are replayed as one HIP graph.
+
+Prints one JSON line: metric/value = algorithmic bytes per second over the
+whole timed region, plus "roofline" (the GEMV kernel against the 8 TB/s HBM
+peak) and "cpu_baseline" (the CPU restatement of the reference's path on the
+same workload, single thread).  "extras" carries the other configurations.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+N_FF, N_EMBD = 14336, 4096
+COPIES = 6
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_q_weights(fmt_name, n, k, seed):
+    import numpy as np
+    from cut_amd import quantize as Q
+    w = np.random.default_rng(seed).standard_normal(n * k, dtype=np.float32) * np.float32(0.02)
+    return Q.quantize(fmt_name, w)
+
+
+def timed_graph(torch, fn_step, steps, warmup):
+    """Runs `warmup` eager steps, captures `steps` steps into one HIP graph and
+    replays it once.  Returns (wall_seconds, event_ms, used_graph)."""
+    for s in range(warmup):
+        fn_step(s)
+    torch.cuda.synchronize()
+    used_graph = True
+    try:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for s in range(steps):
+                fn_step(s)
+        torch.cuda.synchronize()
+        run = g.replay
+    except Exception as e:  # noqa: BLE001
+        log(f"[bench] graph capture failed ({e}); timing eager launches")
+        used_graph = False
+
+        def run():
+            for s in range(steps):
+                fn_step(s)
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record()
+    run()
+    ev1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return t1 - t0, ev0.elapsed_time(ev1), used_graph
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--no-extras", action="store_true", help="skip the other configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it")
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from cut_amd import lib, ops
+
+    lib.check(lib.load().cuthip_init(0))
+    info = lib.device_info()
+    dev = torch.device("cuda:0")
+    log(f"[bench] {info['name']} {info['arch']} CUs={info['compute_units']}")
+
+    # ---- resident inputs ---------------------------------------------------
+    t_in = time.time()
+    w_up_h = make_q_weights("Q4_K", N_FF, N_EMBD, 0)
+    w_down_h = make_q_weights("Q4_K", N_EMBD, N_FF, 1)
+    gate = [torch.from_numpy(w_up_h).to(dev).clone() for _ in range(COPIES)]
+    up = [torch.from_numpy(w_up_h).to(dev).clone() for _ in range(COPIES)]
+    down = [torch.from_numpy(w_down_h).to(dev).clone() for _ in range(COPIES)]
+    rng = np.random.default_rng(1)
+    x_h = rng.standard_normal((8, N_EMBD), dtype=np.float32).astype(np.float16)
+    h_h = rng.standard_normal((8, N_FF), dtype=np.float32).astype(np.float16)
+    x, h = torch.from_numpy(x_h).to(dev), torch.from_numpy(h_h).to(dev)
+    y_gate = torch.empty((8, N_FF), dtype=torch.float16, device=dev)
+    y_up = torch.empty((8, N_FF), dtype=torch.float16, device=dev)
+    y_down = torch.empty((8, N_EMBD), dtype=torch.float16, device=dev)
+    torch.cuda.synchronize()
+    log(f"[bench] inputs ready in {time.time() - t_in:.1f}s")
+
+    w_bytes = ops.n_bytes("Q4_K", N_FF, N_EMBD)  # 33,030,144 for either shape
+
+    def ffn_step(b):
+        def step(s):
+            i = s % COPIES
+            ops.matmul_gguf(x[:b], gate[i], "Q4_K", N_FF, N_EMBD, out=y_gate[:b])
+            ops.matmul_gguf(x[:b], up[i], "Q4_K", N_FF, N_EMBD, out=y_up[:b])
+            ops.matmul_gguf(h[:b], down[i], "Q4_K", N_EMBD, N_FF, out=y_down[:b])
+        return step
+
+    def ffn_bytes(b):
+        return 3 * w_bytes + b * 2 * (2 * (N_EMBD + N_FF) + (N_FF + N_EMBD))
+
+    # ---- headline: batch 1 --------------------------------------------------
+    wall, ev_ms, used_graph = timed_graph(torch, ffn_step(1), args.steps, args.warmup)
+    step_bytes = ffn_bytes(1)
+    value = step_bytes * args.steps / wall / 1e9
+    launches = 3 * args.steps
+    avg_launch_us = ev_ms * 1e3 / launches
+    launch_bytes = step_bytes / 3.0
+    achieved = launch_bytes / (avg_launch_us * 1e-6) / 1e9
+    log(f"[bench] b=1: {value:.0f} GB/s wall, {achieved:.0f} GB/s by events ({avg_launch_us:.2f} us per launch)")
+
+    result = {
+        "metric": "Q4_K GEMV achieved HBM GB/s",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall / args.steps * 1e3, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE configs[2]: Q4_K GEMV, FFN shapes 14336x4096 (gate, up) + 4096x14336 (down), "
+                               "batch 1, fp16 in/out, fp32 accumulate; one step = the three GEMVs of one FFN block",
+                   "weight_copies_rotated": COPIES, "hip_graph": used_graph, "pct_of_hbm_peak": round(value / HBM_PEAK_GBS * 100, 1)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "cuthip::gemv_kernel<Q4_K, MT=1>", "algorithmic_bytes_per_launch": int(launch_bytes),
+                     "avg_launch_us": round(avg_launch_us, 3)},
+    }
+
+    # ---- other configurations ---------------------------------------------------
+    extras = {}
+    if not args.no_extras:
+        for b in (2, 4, 8):
+            wall_b, ev_b, _ = timed_graph(torch, ffn_step(b), 120, 12)
+            extras[f"q4k_ffn_gemv_batch{b}_GBps"] = round(ffn_bytes(b) * 120 / wall_b / 1e9, 1)
+        del gate, up, down
+        torch.cuda.empty_cache()
+        # config 2: dequant of 256 Mi elements to fp16 (a 4 Mi-element tile repeated 64 times)
+        n_el = 256 * 1024 * 1024
+        out = torch.empty((n_el // 4096, 4096), dtype=torch.float16, device=dev)
+        for name in ("Q8_0", "Q4_0", "Q4_K", "Q6_K"):
+            tile = make_q_weights(name, 1024, 4096, 2)
+            raw = torch.from_numpy(tile).to(dev).repeat(64)
+            in_bytes = raw.numel()
+
+            def dq(_s, raw=raw, name=name):
+                ops.dequantize(raw, name, n_el // 4096, 4096, torch.float16, out=out)
+            wall_d, ev_d, _ = timed_graph(torch, dq, 20, 3)
+            extras[f"dequant_{name}_to_f16_256Mi_GBps"] = round((in_bytes + n_el * 2) * 20 / (ev_d * 1e-3) / 1e9, 1)
+            del raw
+        del out
+        torch.cuda.empty_cache()
+        # LM head: Q6_K 128256 x 4096, batch 1 (431 MB per launch: streams from HBM by itself)
+        head = torch.from_numpy(make_q_weights("Q6_K", 4008, 4096, 3)).to(dev).repeat(32)
+        logits = torch.empty((1, 128256), dtype=torch.float16, device=dev)
+
+        def lm_head(_s):
+            ops.matmul_gguf(x[:1], head, "Q6_K", 128256, N_EMBD, out=logits)
+        wall_h, ev_h, _ = timed_graph(torch, lm_head, 20, 3)
+        extras["q6k_lm_head_128256x4096_gemv_GBps"] = round((head.numel() + 2 * (4096 + 128256)) * 20 / (ev_h * 1e-3) / 1e9, 1)
+        del head
+    result["extras"] = extras
+
+    # ---- CPU baseline: the oracle's restatement of the reference path -------------
+    if not args.no_cpu:
+        import oracle
+        a1 = x_h[:1].astype(np.float32)
+        h1 = h_h[:1].astype(np.float32)
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            oracle.matmul_gguf(oracle.Q4_K, w_up_h, a1, N_FF)
+            oracle.matmul_gguf(oracle.Q4_K, w_up_h, a1, N_FF)
+            oracle.matmul_gguf(oracle.Q4_K, w_down_h, h1, N_EMBD)
+            reps += 1
+            if time.perf_counter() - t0 > 10.0 or reps >= 40:
+                break
+        cpu_s = (time.perf_counter() - t0) / reps
+        result["cpu_baseline"] = {
+            "value": round(step_bytes / cpu_s / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} full FFN steps (gate, up, down GEMV at batch 1) through oracle/cut_oracle.c "
+                      f"(dequantize one row, fp32 sequential dot), {cpu_s * 1e3:.0f} ms per step, "
+                      f"host has {os.cpu_count()} logical cores"}
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

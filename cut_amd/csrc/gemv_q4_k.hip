@@ -1,0 +1,6 @@
+// Instantiates the streaming GEMV / skinny GEMM kernels for one block format.
+#include "gemv_kernel.hpp"
+
+namespace cuthip {
+template int launch_fmt<CUTHIP_Q4_K>(GemvParams, hipStream_t);
+}

@@ -75,10 +75,12 @@ def test_q4k_ffn_shapes_fp16_io(ops, N, K, M):
     want = oracle.matmul_gguf(fmt, Ws, A.astype(np.float32), len(rows), f64=True)
     err = normwise_rel_err(got[:, rows], want)
     assert err < 6e-4, err  # fp16 output rounding: 2^-11 / sqrt(3) ~ 2.8e-4 rms
-    # batch rows are independent: row 0 of the batched call == the M=1 call
+    # batch rows are independent: row 0 of the batched call agrees with the M=1 call
+    # (the two launches may split K differently, so fp32 sums can round to
+    # neighbouring fp16 values)
     if M > 1:
         one = gpu_matmul(ops, fmt, W, A[:1], N, K)
-        assert np.array_equal(one[0], got[0])
+        assert np.all(np.abs(one[0] - got[0]) <= np.abs(got[0]) * 2.0 ** -10 + 1e-6)
 
 
 def test_linearity_and_row_permutation(ops):
