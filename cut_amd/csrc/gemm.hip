@@ -1,0 +1,329 @@
+// Prefill GEMM on native GGUF blocks for gfx950:
+//   C[m,n] = sum_k A[m,k] * dequant(W)[n,k],  M > 32.
+//
+// Supersedes MatMulQ{4,8}CoopMatTiled.cu (operators/impl/matmul): 32x32x16
+// tiles with one 16x16x16 MMA per warp between two barriers.  Here a workgroup
+// of four waves owns a BM x 128 tile of C (BM = 256 or 128), each wave a
+// (BM/2) x 64 sub-tile held in fp32 accumulators, and walks K in slices of 64.
+// Per slice the workgroup
+//   * copies the A slice to LDS as fp16 (fp32 activations are rounded once),
+//   * decodes the W slice straight from the GGUF blocks: every thread takes one
+//     32-element quantization sub-block of one weight row, evaluates the
+//     reference's fp32 expression (d*sc)*q - dmin*m for it and stores the 32
+//     values to LDS as fp16 (round to nearest even), so each weight is decoded
+//     once per BM rows of activations,
+//   * feeds both tiles to v_mfma_f32_32x32x16_f16 (fp32 accumulate).
+// Both LDS tiles are K-contiguous with a 16-byte row pad, which is the operand
+// layout of the MFMA (lane l: row l & 31, k = 8*(l >> 5) .. +7) and keeps the
+// 16-byte fragment reads off each other's banks.
+//
+// The global loads of slice t+1 are issued before the MFMAs of slice t and
+// land in registers; two workgroups fit on a CU, so one computes while the
+// other waits at its barrier.  Workgroup ids are remapped so that all M-tiles
+// of one 128-column weight panel run on the same XCD and share its L2.
+//
+// Error budget against the fp32 CPU path: weights rounded to fp16 (2^-11
+// relative), fp16 activations exact, fp32 accumulation: ~3e-4 normwise.
+#include "common.hpp"
+
+namespace cuthip {
+
+struct GemmParams {
+  const uint8_t *W;
+  const void *A;
+  void *C;
+  Epilogue epi;
+  uint32_t M, K, N, strideA, strideC;
+  uint32_t row_bytes;
+  uint32_t mtiles, ntiles;
+  int a_f16, c_f16;
+};
+
+constexpr int kBN = 128, kBK = 64, kLdsRow = kBK + 8;  // halfs per LDS row
+
+// ---- decode of one 32-element sub-block -------------------------------------
+// sub: index of the 32-element sub-block inside its row (k = 32*sub .. +31).
+// Raw holds what one thread loads for it; decode() writes 32 fp16 values.
+template <int FMT> struct Sub;
+
+template <> struct Sub<CUTHIP_Q4_K> {
+  struct Raw { u32x4 hdr; u32x4 q[2]; };
+  __device__ static void load(Raw &r, const uint8_t *row, uint32_t sub) {
+    const uint8_t *blk = row + (size_t)(sub >> 3) * 144;
+    r.hdr = ld_u32x4(blk);
+    const uint8_t *qs = blk + 16 + 32 * ((sub & 7) >> 1);
+    r.q[0] = ld_u32x4(qs);
+    r.q[1] = ld_u32x4(qs + 16);
+  }
+  __device__ static void decode(const Raw &r, uint32_t sub, half_t (&w)[32]) {
+    uint32_t j = sub & 7;
+    float d = f16bits_to_f32(r.hdr.x & 0xFFFF), dmin = f16bits_to_f32(r.hdr.x >> 16);
+    uint32_t sc_lo, sc_hi, m_lo, m_hi;
+    q4k_scales(r.hdr.y, r.hdr.z, r.hdr.w, sc_lo, sc_hi, m_lo, m_hi);
+    uint32_t bsh = 8 * (j & 3);
+    float d1 = d * (float)(((j < 4 ? sc_lo : sc_hi) >> bsh) & 0xFF);
+    float dm1 = dmin * (float)(((j < 4 ? m_lo : m_hi) >> bsh) & 0xFF);
+    uint32_t sh = (j & 1) * 4;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      uint32_t word = i < 4 ? r.q[0][i] : r.q[1][i - 4];
+      word = (word >> sh) & 0x0F0F0F0Fu;
+      w[4 * i + 0] = (half_t)(d1 * cvt_ubyte0(word) - dm1);
+      w[4 * i + 1] = (half_t)(d1 * cvt_ubyte1(word) - dm1);
+      w[4 * i + 2] = (half_t)(d1 * cvt_ubyte2(word) - dm1);
+      w[4 * i + 3] = (half_t)(d1 * cvt_ubyte3(word) - dm1);
+    }
+  }
+};
+
+template <> struct Sub<CUTHIP_Q6_K> {
+  struct Raw { u32x4 ql[2]; u32x4 qh[2]; uint32_t sc, d; };
+  __device__ static void load(Raw &r, const uint8_t *row, uint32_t sub) {
+    const uint8_t *blk = row + (size_t)(sub >> 3) * 210;
+    uint32_t H = (sub >> 2) & 1, s = sub & 3;
+    const uint8_t *ql = blk + 64 * H + 32 * (s & 1), *qh = blk + 128 + 32 * H;
+    r.ql[0] = ld_u32x4(ql); r.ql[1] = ld_u32x4(ql + 16);
+    r.qh[0] = ld_u32x4(qh); r.qh[1] = ld_u32x4(qh + 16);
+    r.sc = ld_u16(blk + 192 + 8 * H + 2 * s);
+    r.d = ld_u16(blk + 208);
+  }
+  __device__ static void decode(const Raw &r, uint32_t sub, half_t (&w)[32]) {
+    uint32_t s = sub & 3;
+    float d = f16bits_to_f32(r.d);
+    float dsc0 = d * (float)(int)(int8_t)(r.sc & 0xFF), dsc1 = d * (float)(int)(int8_t)(r.sc >> 8);
+    uint32_t lsh = (s >> 1) * 4, hsh = 2 * s;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      uint32_t wl = i < 4 ? r.ql[0][i] : r.ql[1][i - 4], wh = i < 4 ? r.qh[0][i] : r.qh[1][i - 4];
+      uint32_t q6 = ((wl >> lsh) & 0x0F0F0F0Fu) | (((wh >> hsh) & 0x03030303u) << 4);
+      float dsc = i < 4 ? dsc0 : dsc1;  // elements 0-15 / 16-31 of the 32
+      w[4 * i + 0] = (half_t)(dsc * (cvt_ubyte0(q6) - 32.0f));
+      w[4 * i + 1] = (half_t)(dsc * (cvt_ubyte1(q6) - 32.0f));
+      w[4 * i + 2] = (half_t)(dsc * (cvt_ubyte2(q6) - 32.0f));
+      w[4 * i + 3] = (half_t)(dsc * (cvt_ubyte3(q6) - 32.0f));
+    }
+  }
+};
+
+template <> struct Sub<CUTHIP_Q8_0> {
+  struct Raw { u32x4 q[2]; uint32_t d; };
+  __device__ static void load(Raw &r, const uint8_t *row, uint32_t sub) {
+    const uint8_t *blk = row + (size_t)sub * 34;
+    r.d = ld_u16(blk);
+    r.q[0] = ld_u32x4(blk + 2);
+    r.q[1] = ld_u32x4(blk + 18);
+  }
+  __device__ static void decode(const Raw &r, uint32_t, half_t (&w)[32]) {
+    float d = f16bits_to_f32(r.d);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      uint32_t word = (i < 4 ? r.q[0][i] : r.q[1][i - 4]) ^ 0x80808080u;  // q + 128 as unsigned bytes
+      w[4 * i + 0] = (half_t)(d * (cvt_ubyte0(word) - 128.0f));
+      w[4 * i + 1] = (half_t)(d * (cvt_ubyte1(word) - 128.0f));
+      w[4 * i + 2] = (half_t)(d * (cvt_ubyte2(word) - 128.0f));
+      w[4 * i + 3] = (half_t)(d * (cvt_ubyte3(word) - 128.0f));
+    }
+  }
+};
+
+template <> struct Sub<CUTHIP_Q4_0> {
+  struct Raw { u32x4 q; uint32_t d; };
+  __device__ static void load(Raw &r, const uint8_t *row, uint32_t sub) {
+    const uint8_t *blk = row + (size_t)sub * 18;
+    r.d = ld_u16(blk);
+    r.q = ld_u32x4(blk + 2);
+  }
+  __device__ static void decode(const Raw &r, uint32_t, half_t (&w)[32]) {
+    float d = f16bits_to_f32(r.d);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint32_t lo = r.q[i] & 0x0F0F0F0Fu, hi = (r.q[i] >> 4) & 0x0F0F0F0Fu;
+      w[4 * i + 0] = (half_t)(d * (cvt_ubyte0(lo) - 8.0f));
+      w[4 * i + 1] = (half_t)(d * (cvt_ubyte1(lo) - 8.0f));
+      w[4 * i + 2] = (half_t)(d * (cvt_ubyte2(lo) - 8.0f));
+      w[4 * i + 3] = (half_t)(d * (cvt_ubyte3(lo) - 8.0f));
+      w[16 + 4 * i + 0] = (half_t)(d * (cvt_ubyte0(hi) - 8.0f));
+      w[16 + 4 * i + 1] = (half_t)(d * (cvt_ubyte1(hi) - 8.0f));
+      w[16 + 4 * i + 2] = (half_t)(d * (cvt_ubyte2(hi) - 8.0f));
+      w[16 + 4 * i + 3] = (half_t)(d * (cvt_ubyte3(hi) - 8.0f));
+    }
+  }
+};
+
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+
+// ---- the kernel -----------------------------------------------------------------
+template <int FMT, int BM, bool AF16>
+__global__ void __launch_bounds__(256, 2) gemm_kernel(GemmParams p) {
+  using S = Sub<FMT>;
+  constexpr int MI = BM / 64;          // 32-row MFMA tiles per wave along M
+  constexpr int AV = BM * kBK / 8 / 256;  // 16-byte A vectors per thread per slice
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  half_t *As = reinterpret_cast<half_t *>(lds);             // [BM][kLdsRow]
+  half_t *Bs = As + BM * kLdsRow;                           // [kBN][kLdsRow]
+
+  // XCD-aware tile order: ids id, id+8, id+16, ... share an XCD; give them the
+  // M-tiles of the same weight panel.
+  uint32_t id = blockIdx.x, mt, nt;
+  if (p.ntiles % 8 == 0) {
+    uint32_t xcd = id & 7, slot = id >> 3;
+    nt = (slot / p.mtiles) * 8 + xcd;
+    mt = slot % p.mtiles;
+  } else {
+    nt = id / p.mtiles;
+    mt = id % p.mtiles;
+  }
+  const uint32_t m0 = mt * BM, n0 = nt * kBN;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // weight decode assignment: thread -> (row n0 + tid/2, sub-block tid&1 of the slice)
+  const uint32_t brow = min(n0 + (uint32_t)(tid >> 1), p.N - 1);
+  const uint8_t *wrow = p.W + (size_t)brow * p.row_bytes;
+  const uint32_t bsub = tid & 1;
+  const uint32_t nsub = p.K / 32;  // sub-blocks per row
+
+  f32x16 acc[MI][2];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+  typename S::Raw braw;
+  u32x4 araw[AV], araw2[AF16 ? 1 : AV];  // araw2: second half of an fp32 group of 8
+
+  auto load_slice = [&](uint32_t k0) {
+    uint32_t sub = min(k0 / 32 + bsub, nsub - 1);
+    S::load(braw, wrow, sub);
+#pragma unroll
+    for (int v = 0; v < AV; ++v) {
+      int idx = v * 256 + tid;              // vector index in the [BM][8] grid of the slice
+      uint32_t r = min(m0 + (uint32_t)(idx >> 3), p.M - 1), kc = k0 + (idx & 7) * 8;
+      kc = min(kc, p.K - 8);
+      size_t off = (size_t)r * p.strideA + kc;
+      if constexpr (AF16) {
+        araw[v] = ld_u32x4(reinterpret_cast<const uint8_t *>(p.A) + off * 2);
+      } else {
+        araw[v] = ld_u32x4(reinterpret_cast<const uint8_t *>(p.A) + off * 4);
+        araw2[v] = ld_u32x4(reinterpret_cast<const uint8_t *>(p.A) + off * 4 + 16);
+      }
+    }
+  };
+  auto store_slice = [&](uint32_t k0) {
+    half_t w[32];
+    S::decode(braw, k0 / 32 + bsub, w);
+    bool live = k0 + 32 * bsub < p.K;  // sub-blocks past K (ragged last slice) are zero
+    half_t *dst = Bs + (tid >> 1) * kLdsRow + 32 * bsub;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      half8v o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = live ? w[8 * c + e] : (half_t)0.0f;
+      *reinterpret_cast<half8v *>(dst + 8 * c) = o;
+    }
+#pragma unroll
+    for (int v = 0; v < AV; ++v) {
+      int idx = v * 256 + tid;
+      bool alive = k0 + (idx & 7) * 8 < p.K;
+      half8v o;
+      if constexpr (AF16) {
+        o = __builtin_bit_cast(half8v, araw[v]);
+      } else {
+        f32x4 lo = __builtin_bit_cast(f32x4, araw[v]), hi = __builtin_bit_cast(f32x4, araw2[v]);
+        o = half8v{(half_t)lo.x, (half_t)lo.y, (half_t)lo.z, (half_t)lo.w,
+                   (half_t)hi.x, (half_t)hi.y, (half_t)hi.z, (half_t)hi.w};
+      }
+      if (!alive) o = half8v{0, 0, 0, 0, 0, 0, 0, 0};
+      *reinterpret_cast<half8v *>(As + (idx >> 3) * kLdsRow + (idx & 7) * 8) = o;
+    }
+  };
+
+  const uint32_t nslices = (p.K + kBK - 1) / kBK;
+  load_slice(0);
+  for (uint32_t t = 0; t < nslices; ++t) {
+    __syncthreads();           // everyone is done reading the previous slice
+    store_slice(t * kBK);
+    __syncthreads();
+    if (t + 1 < nslices) load_slice((t + 1) * kBK);
+    const half_t *a_base = As + (wm * (BM / 2) + (lane & 31)) * kLdsRow + 8 * (lane >> 5);
+    const half_t *b_base = Bs + (wn * 64 + (lane & 31)) * kLdsRow + 8 * (lane >> 5);
+#pragma unroll
+    for (int s = 0; s < kBK / 16; ++s) {
+      half8v bf[2], af[MI];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bf[j] = *reinterpret_cast<const half8v *>(b_base + 32 * j * kLdsRow + 16 * s);
+#pragma unroll
+      for (int i = 0; i < MI; ++i) af[i] = *reinterpret_cast<const half8v *>(a_base + 32 * i * kLdsRow + 16 * s);
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    }
+  }
+
+  // C tile: register r of lane l holds row 8*(r/4) + 4*(l>>5) + r%4, column l & 31 of its 32x32 block
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      uint32_t col = n0 + wn * 64 + 32 * j + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        uint32_t row = m0 + wm * (BM / 2) + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (row < p.M && col < p.N) store_out(p.C, p.epi, p.c_f16, (size_t)row * p.strideC + col, acc[i][j][r]);
+      }
+    }
+}
+
+template <int FMT, int BM, bool AF16> static int launch_gemm_bm(GemmParams p, hipStream_t stream) {
+  p.mtiles = (p.M + BM - 1) / BM;
+  p.ntiles = (p.N + kBN - 1) / kBN;
+  size_t lds = (size_t)(BM + kBN) * kLdsRow * 2;
+  auto kern = gemm_kernel<FMT, BM, AF16>;
+  if (lds > 64 * 1024) {
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                           "hipFuncSetAttribute"))
+      return rc;
+  }
+  uint64_t grid = (uint64_t)p.mtiles * p.ntiles;
+  if (grid > 0x7FFFFFFFull) {
+    set_error("cuthip_matmul_gguf: problem too large for one launch");
+    return CUTHIP_ERR_INVALID;
+  }
+  hipLaunchKernelGGL(kern, dim3((uint32_t)grid), dim3(256), lds, stream, p);
+  return check_hip(hipGetLastError(), "gemm launch");
+}
+
+template <int FMT> static int launch_gemm_fmt(const GemmParams &p, hipStream_t stream) {
+  // 256-row tiles once they fill the chip (>= 2 workgroups per CU), else 128-row tiles.
+  // fp32 activations and Q6_K need more staging registers and always take 128 rows.
+  if (!p.a_f16) return launch_gemm_bm<FMT, 128, false>(p, stream);
+  uint64_t tiles256 = (uint64_t)((p.M + 255) / 256) * ((p.N + kBN - 1) / kBN);
+  if constexpr (FMT != CUTHIP_Q6_K) {
+    if (tiles256 >= 512) return launch_gemm_bm<FMT, 256, true>(p, stream);
+  }
+  return launch_gemm_bm<FMT, 128, true>(p, stream);
+}
+
+int launch_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K, uint32_t N,
+                uint32_t strideA, uint32_t strideC, Epilogue epi, hipStream_t stream) {
+  GemmParams p;
+  p.W = reinterpret_cast<const uint8_t *>(W);
+  p.A = A;
+  p.C = C;
+  p.epi = epi;
+  p.M = M; p.K = K; p.N = N; p.strideA = strideA; p.strideC = strideC;
+  p.row_bytes = (uint32_t)((uint64_t)(K / fmt_elems(fmt)) * fmt_bytes(fmt));
+  p.mtiles = p.ntiles = 0;
+  p.a_f16 = a_f16; p.c_f16 = c_f16;
+  switch (fmt) {
+  case CUTHIP_Q8_0: return launch_gemm_fmt<CUTHIP_Q8_0>(p, stream);
+  case CUTHIP_Q4_0: return launch_gemm_fmt<CUTHIP_Q4_0>(p, stream);
+  case CUTHIP_Q4_K: return launch_gemm_fmt<CUTHIP_Q4_K>(p, stream);
+  default: return launch_gemm_fmt<CUTHIP_Q6_K>(p, stream);
+  }
+}
+
+}  // namespace cuthip

@@ -17,24 +17,24 @@ GemvShape pick_gemv_shape(uint32_t N, uint32_t nsteps, int mt) {
   // CUT_HIP_GEMV_SHAPE="kp,waves" overrides the heuristic (tuning aid).
   if (const char *env = std::getenv("CUT_HIP_GEMV_SHAPE")) {
     int kp = 0, w = 0;
-    if (sscanf(env, "%d,%d", &kp, &w) == 2 && (kp == 1 || kp == 2 || kp == 4) && (w == 1 || w == 2 || w == 4 || w == 8)) {
-      if (mt > 2 && kp > 2) kp = 2;
+    if (sscanf(env, "%d,%d", &kp, &w) == 2 && (kp == 1 || kp == 2) && (w == 1 || w == 2 || w == 4 || w == 8)) {
       if (mt > 8) kp = 1;
       return GemvShape{kp, w};
     }
   }
-  const int kp_max = mt <= 2 ? 4 : (mt <= 8 ? 2 : 1);
-  int kp = 1;
-  while (kp < kp_max && (uint64_t)(N + 31) / 32 * kp < 512 && nsteps / (uint32_t)(2 * kp) >= 2) kp *= 2;
+  // Measured on MI355X at the projection shapes of an 8B model: two parts per
+  // wave (16 weight rows per workgroup) win for M <= 2 unless N is huge, and
+  // K is split over as many waves as keep >= 2 steps of 256 per part.
+  const uint32_t tiles32 = (N + 31) / 32;
+  int kp = (mt <= 2 && tiles32 < 1024 && nsteps >= 4) ? 2 : 1;
   const int w_max = mt * kp > 16 ? 4 : 8;
   int w = 1;
-  while (w < w_max) {
-    uint32_t per_part = nsteps / (uint32_t)(2 * w * kp);  // steps per part after doubling
-    uint64_t waves_now = (uint64_t)(N + 31) / 32 * kp * w;
-    if (per_part >= 4 || (waves_now < 2048 && per_part >= 2)) w *= 2; else break;
-  }
+  while (w < w_max && nsteps / (uint32_t)(2 * w * kp) >= 2) w *= 2;
   return GemvShape{kp, w};
 }
+
+int launch_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K, uint32_t N,
+                uint32_t strideA, uint32_t strideC, Epilogue epi, hipStream_t stream);
 
 static int launch_gemv(int fmt, const GemvParams &p, hipStream_t stream) {
   switch (fmt) {
@@ -94,11 +94,25 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
     set_error("cuthip_matmul_gguf: K too large");
     return CUTHIP_ERR_INVALID;
   }
+  // variant table: 0 streaming GEMV (M <= 8), 1 skinny passes of 32 rows, 2 LDS-tiled GEMM
+  Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
+  if (variant == 0 && M > 8) {
+    set_error("cuthip_matmul_gguf: variant 0 (GEMV) handles M <= 8, got M = %u", M);
+    return CUTHIP_ERR_INVALID;
+  }
+  if (variant == 2 || (variant == -1 && M > 32)) {
+    if ((uint64_t)N * row_bytes > 0xFFFFFFFFFFFFull) {
+      set_error("cuthip_matmul_gguf: weight matrix too large");
+      return CUTHIP_ERR_INVALID;
+    }
+    return launch_gemm(fmt, W, A, a_dtype == CUTHIP_F16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC, epi,
+                       reinterpret_cast<hipStream_t>(stream));
+  }
   GemvParams p;
   p.W = reinterpret_cast<const uint8_t *>(W);
   p.A = A;
   p.C = C;
-  p.epi = Epilogue{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
+  p.epi = epi;
   p.M = M; p.K = K; p.N = N; p.strideA = strideA; p.strideC = strideC;
   p.nsteps = (K + 255) / 256;
   p.row_bytes = (uint32_t)row_bytes;

@@ -103,7 +103,6 @@ template <> struct Step<CUTHIP_Q4_K> {
       q = mfma(xa[8 * g + 5], hi_b, q);
       fma_acc<R>(acc, p, ds[2 * g]);
       fma_acc<R>(acc, q, ds[2 * g + 1]);
-      __builtin_amdgcn_sched_barrier(0);  // keep two MFMA chains (32 accumulator registers) live, not eight
     }
 #pragma unroll
     for (int r_ = 0; r_ < R; ++r_) {

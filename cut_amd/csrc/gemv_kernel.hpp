@@ -326,9 +326,6 @@ template <int FMT, int MT, int KP> static int launch_waves(const GemvParams &p, 
 }
 
 template <int FMT, int MT> static int launch_kp(const GemvParams &p, int kp, int waves, hipStream_t stream) {
-  if constexpr (MT <= 2) {
-    if (kp == 4) return launch_waves<FMT, MT, 4>(p, waves, stream);
-  }
   if constexpr (MT <= 8) {
     if (kp >= 2) return launch_waves<FMT, MT, 2>(p, waves, stream);
   }

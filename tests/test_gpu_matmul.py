@@ -135,7 +135,7 @@ def test_skinny_gemm_passes(ops, M):
     N, K = 96, 1024
     W = quantized_weights(fmt, N, K, seed=8)
     A = gauss_acts((M, K), seed=3, dtype=np.float16)
-    got = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32)
+    got = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=1)  # 32-row passes of the streaming kernel
     want = oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)
     assert normwise_rel_err(got, want) < TOL_F16_ACT
 
