@@ -80,6 +80,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain 1 GiB device copy 5 times (reference traffic for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it")
@@ -92,6 +94,14 @@ def main():
     lib.check(lib.load().cuthip_init(0))
     info = lib.device_info()
     dev = torch.device("cuda:0")
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4, "launches": 5}))
+        return
     log(f"[bench] {info['name']} {info['arch']} CUs={info['compute_units']}")
 
     # ---- resident inputs ---------------------------------------------------
@@ -187,7 +197,22 @@ def main():
             ops.matmul_gguf(x[:1], head, "Q6_K", 128256, N_EMBD, out=logits)
         wall_h, ev_h, _ = timed_graph(torch, lm_head, 20, 3)
         extras["q6k_lm_head_128256x4096_gemv_GBps"] = round((head.numel() + 2 * (4096 + 128256)) * 20 / (ev_h * 1e-3) / 1e9, 1)
-        del head
+        del head, logits
+        torch.cuda.empty_cache()
+        # config 5: prefill GEMM, Q4_K weights, fp16 activations, fp16 MFMA with fp32 accumulate
+        for (M, N, K) in ((512, N_FF, N_EMBD), (2048, N_FF, N_EMBD), (512, N_EMBD, N_FF), (2048, N_EMBD, N_FF)):
+            w_h = w_up_h if N == N_FF else w_down_h
+            wq = torch.from_numpy(w_h).to(dev)
+            a = torch.randn((M, K), dtype=torch.float16, device=dev)
+            c = torch.empty((M, N), dtype=torch.float16, device=dev)
+
+            def gemm(_s, a=a, wq=wq, c=c, N=N, K=K):
+                ops.matmul_gguf(a, wq, "Q4_K", N, K, out=c)
+            wall_g, ev_g, _ = timed_graph(torch, gemm, 10, 2)
+            tflops = 2.0 * M * N * K * 10 / (ev_g * 1e-3) / 1e12
+            extras[f"q4k_prefill_gemm_M{M}_N{N}_K{K}_TFLOPs"] = round(tflops, 1)
+            extras[f"q4k_prefill_gemm_M{M}_N{N}_K{K}_pct_of_f16_mfma_peak"] = round(tflops / 2500.0 * 100, 1)
+            del wq, a, c
     result["extras"] = extras
 
     # ---- CPU baseline: the oracle's restatement of the reference path -------------
