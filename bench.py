@@ -162,7 +162,7 @@ def main():
                    "weight_copies_rotated": COPIES, "hip_graph": used_graph, "pct_of_hbm_peak": round(value / HBM_PEAK_GBS * 100, 1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "cuthip::gemv_kernel<Q4_K, MT=1>", "algorithmic_bytes_per_launch": int(launch_bytes),
+                     "kernel": "cuthip::gemv_rows8_kernel<Q4_K, MT=1>", "algorithmic_bytes_per_launch": int(launch_bytes),
                      "avg_launch_us": round(avg_launch_us, 3)},
     }
 

@@ -34,12 +34,15 @@ static const cuthip_variant_info_t kMatMulGgufVariants[] = {
     {"MatMulGgufSkinnyMfma", 64, 4, 32, 32, "same pipeline with a 32-row activation tile (8 < M <= 32 per pass)"},
     {"MatMulGgufGemmLds", 256, 1, 128, 128,
      "prefill GEMM: weights dequantized to fp16 tiles in LDS, 32x32x16 f16 MFMA, fp32 accumulate"},
+    {"MatMulGgufGemvRows8", 64, 4, 8, 8,
+     "decode GEMV (M <= 8): 8 weight rows x 128-byte runs per wave instruction, four 64-element pieces per row as "
+     "MFMA columns, register ring of loads, no cross-wave reduction unless K is split"},
 };
 
 static const cuthip_variant_info_t *table(int op, int *count) {
   switch (op) {
   case CUTHIP_OP_DEQUANT: *count = 1; return kDequantVariants;
-  case CUTHIP_OP_MATMUL_GGUF: *count = 3; return kMatMulGgufVariants;
+  case CUTHIP_OP_MATMUL_GGUF: *count = 4; return kMatMulGgufVariants;
   }
   *count = 0;
   return nullptr;

@@ -5,6 +5,7 @@
 #include <cstdlib>
 
 #include "gemv_kernel.hpp"
+#include "gemv_rows8.hpp"
 
 namespace cuthip {
 
@@ -12,6 +13,40 @@ extern template int launch_fmt<CUTHIP_Q8_0>(GemvParams, hipStream_t);
 extern template int launch_fmt<CUTHIP_Q4_0>(GemvParams, hipStream_t);
 extern template int launch_fmt<CUTHIP_Q4_K>(GemvParams, hipStream_t);
 extern template int launch_fmt<CUTHIP_Q6_K>(GemvParams, hipStream_t);
+
+#define CUTHIP_EXTERN_ROWS8(F) \
+  extern template int launch_rows8_fmt<F>(const GemvParams &, hipStream_t); \
+  extern template bool rows8_fits<F>(const GemvParams &);
+CUTHIP_EXTERN_ROWS8(CUTHIP_Q8_0)
+CUTHIP_EXTERN_ROWS8(CUTHIP_Q4_0)
+CUTHIP_EXTERN_ROWS8(CUTHIP_Q4_K)
+CUTHIP_EXTERN_ROWS8(CUTHIP_Q6_K)
+#undef CUTHIP_EXTERN_ROWS8
+
+// Workgroup shape of the rows8 GEMV: split K (kw step ranges per 8-row group)
+// while the grid has fewer than ~6 waves per CU and each wave keeps >= 2 steps.
+Rows8Shape pick_rows8_shape(uint32_t N, uint32_t nsteps) {
+  if (const char *env = std::getenv("CUT_HIP_ROWS8_SHAPE")) {   // "rwg,kw" tuning aid
+    int rwg = 0, kw = 0;
+    if (sscanf(env, "%d,%d", &rwg, &kw) == 2 && (kw == 1 || kw == 2 || kw == 4 || kw == 8)) return Rows8Shape{rwg, kw};
+  }
+  uint32_t groups = (N + 7) / 8;
+  int kw = 1;
+  while (kw < 8 && (uint64_t)groups * kw < 1536 && nsteps / (uint32_t)(2 * kw) >= 2) kw *= 2;
+  return Rows8Shape{groups >= 8192 ? 8 : 4, kw};
+}
+
+static int launch_rows8_any(int fmt, const GemvParams &p, hipStream_t stream, bool *taken) {
+  *taken = true;
+  switch (fmt) {
+  case CUTHIP_Q8_0: if (rows8_fits<CUTHIP_Q8_0>(p)) return launch_rows8_fmt<CUTHIP_Q8_0>(p, stream); break;
+  case CUTHIP_Q4_0: if (rows8_fits<CUTHIP_Q4_0>(p)) return launch_rows8_fmt<CUTHIP_Q4_0>(p, stream); break;
+  case CUTHIP_Q4_K: if (rows8_fits<CUTHIP_Q4_K>(p)) return launch_rows8_fmt<CUTHIP_Q4_K>(p, stream); break;
+  default: if (rows8_fits<CUTHIP_Q6_K>(p)) return launch_rows8_fmt<CUTHIP_Q6_K>(p, stream); break;
+  }
+  *taken = false;
+  return CUTHIP_OK;
+}
 
 GemvShape pick_gemv_shape(uint32_t N, uint32_t nsteps, int mt) {
   // CUT_HIP_GEMV_SHAPE="kp,waves" overrides the heuristic (tuning aid).
@@ -118,5 +153,15 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
   p.row_bytes = (uint32_t)row_bytes;
   p.a_f16 = a_dtype == CUTHIP_F16;
   p.c_f16 = c_dtype == CUTHIP_F16;
+  // variant 3 (and the automatic choice for M <= 8): 8 rows x 128-byte runs per wave instruction
+  if (variant == 3 || (variant == -1 && M <= 8)) {
+    bool taken = false;
+    int rc = launch_rows8_any(fmt, p, reinterpret_cast<hipStream_t>(stream), &taken);
+    if (taken) return rc;
+    if (variant == 3) {
+      set_error("cuthip_matmul_gguf: variant 3 needs M <= 8 and the activations to fit in LDS (M = %u, K = %u)", M, K);
+      return CUTHIP_ERR_INVALID;
+    }
+  }
   return launch_gemv(fmt, p, reinterpret_cast<hipStream_t>(stream));
 }

@@ -1,6 +1,9 @@
 // Instantiates the streaming GEMV / skinny GEMM kernels for one block format.
 #include "gemv_kernel.hpp"
+#include "gemv_rows8.hpp"
 
 namespace cuthip {
 template int launch_fmt<CUTHIP_Q8_0>(GemvParams, hipStream_t);
+template int launch_rows8_fmt<CUTHIP_Q8_0>(const GemvParams &, hipStream_t);
+template bool rows8_fits<CUTHIP_Q8_0>(const GemvParams &);
 }

@@ -1,0 +1,677 @@
+// Streaming quantized GEMV on native GGUF blocks for gfx950, batch 1..4:
+//   C[m,n] = sum_k A[m,k] * dequant(W)[n,k]
+//
+// Supersedes MatMulQ{4,8}GemvKPar8.cu (operators/impl/matmul), whose lanes
+// gather 4 bytes at a stride of N across k.  Here the weights stay in the GGUF
+// file layout (row n = K/blk consecutive blocks) and every wave instruction
+// reads 8 rows x 128 contiguous bytes (16 bytes per lane), which is what the
+// memory system streams best; nothing is read twice from HBM.
+//
+// Work decomposition.  K is cut in steps of 256 elements.  One wave owns 8
+// consecutive weight rows and a contiguous range of steps; a workgroup is RWG
+// row groups x KW step ranges.  Inside a wave the 32 B-columns of
+// v_mfma_f32_32x32x16_f16 are (row r, piece g) pairs, column j = 4r + g: the
+// four pieces of a row cover the four 64-element quarters of the step, so the
+// eight lanes (4 pieces x 2 k-halves) of a row load one contiguous run.  The
+// MFMA A-row j carries the activations of batch row j/4 for the same quarter
+// j%4, hence C[j][j'] is a valid partial sum when j%4 == j'%4; every lane
+// scales all its accumulator registers with its own column's scales and the
+// valid one is picked once at the end, followed by a 4-lane sum over pieces.
+//
+// Arithmetic.  Quants become fp16 subnormals with one AND per pair of weights
+// (a nibble in bits 0-3 of a 16-bit lane is q * 2^-24, in bits 4-7 q * 2^-20;
+// the matrix core multiplies subnormals exactly), so an MFMA chain gives the
+// exact integer dot product sum(q * x) of one quantization sub-block, which is
+// scaled in fp32 by d*sc; the "- min" / "- 8" / "- 32" / "+ 128" offsets become
+// -(offset scale) * sum(x) with per-sub-block sums of x kept next to the
+// staged activations.  Formats whose sub-block is spread over both k-halves of
+// a column (Q6_K, Q8_0, Q4_0) first exchange 8-byte halves between lane l and
+// lane l+32 (v_permlane32_swap), so that one MFMA always sees one sub-block.
+// Activations are consumed as fp16 (fp32 inputs are rounded to nearest even).
+//
+// Pipeline.  The workgroup stages the activations once: fp16, each group of 8
+// in the order (0,2,1,3,4,6,5,7) (the order AND/shift unpacking produces), 64
+// elements per 144-byte LDS group so the four pieces hit different banks.
+// Each lane then keeps D steps of weight loads in flight in a register ring;
+// the loop body is branch-free, so every step waits only for its own loads.
+#pragma once
+#include "gemv_formats.hpp"
+
+namespace cuthip {
+
+#ifndef CUTHIP_ROWS8_DOTMAX
+#define CUTHIP_ROWS8_DOTMAX 1
+#endif
+constexpr int kRows8DotMax = CUTHIP_ROWS8_DOTMAX;   // batch rows up to which the dot-product path is taken
+constexpr int kXGroup = 72;             // halfs per staged 64-element group (64 + 8 pad)
+constexpr int kXStep = 4 * kXGroup;     // halfs per 256-element step
+
+__device__ inline void swap_halves(uint32_t &lo, uint32_t &hi) {
+  // lanes 0-31: hi <- partner's lo ; lanes 32-63: lo <- partner's hi  (partner = lane ^ 32)
+  auto r = __builtin_amdgcn_permlane32_swap(lo, hi, false, false);
+  lo = r[0];
+  hi = r[1];
+}
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+__device__ inline float dot2(uint32_t a, uint32_t b, float c) {   // v_dot2_f32_f16; exact for subnormal a
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b), c, false);
+}
+// 8 products: the bytes of (u0, u1) masked to fp16 subnormals against 8 staged activations
+__device__ inline float dot_pairs(uint32_t u0, uint32_t u1, const u32x4 &x, uint32_t mask, float s) {
+  s = dot2(u0 & mask, x.x, s);
+  s = dot2((u0 >> 8) & mask, x.y, s);
+  s = dot2(u1 & mask, x.z, s);
+  return dot2((u1 >> 8) & mask, x.w, s);
+}
+
+struct LaneCtx {
+  int g, kg;            // piece (64-element quarter of the step) and k-half
+  uint32_t c0, c1, c2, c3;  // per-lane constants of the format
+};
+
+template <int FMT> struct Rows8;
+
+// ---- Q4_K -------------------------------------------------------------------
+// 144 B = [d][dmin][scales:12][qs:128]; piece g = qs[32g..32g+31]: low nibbles
+// are sub-block 2g, high nibbles sub-block 2g+1; lane kg takes bytes 16kg..+15.
+template <> struct Rows8<CUTHIP_Q4_K> {
+  static constexpr int NSUB = 8, SUBK = 32;
+  struct Raw { u32x4 hdr, q; };
+  __device__ static void init(LaneCtx &c) {
+    c.c0 = 16u * (c.g & 1);                 // bit offset of this piece's byte pair inside a scale dword
+    c.c1 = c.g < 2 ? 0x3F3Fu : 0u;          // 6-bit fields of sub-blocks 0-3
+    c.c2 = c.g < 2 ? 0u : 0x0F0Fu;          // low 4 bits of sub-blocks 4-7
+    c.c3 = c.g < 2 ? 0u : 0x3030u;          // their upper 2 bits, taken from bits 6-7 of dword 0 / 1
+  }
+  __device__ static void load(Raw &r, const uint8_t *row, uint32_t step, const LaneCtx &c, uint32_t) {
+    const uint8_t *p = row + (size_t)step * 144;
+    r.hdr = ld_u32x4(p);
+    r.q = ld_u32x4(p + 16 + 32 * c.g + 16 * c.kg);
+  }
+  // xa: staged x of this lane's A-row at (step, piece, kg); sx: sums of x for (batch row of acc quad q, step, piece)
+  template <int R>
+  __device__ static void compute(const Raw &r, const half_t *xa, const float *const *sx, const LaneCtx &c,
+                                 float (&acc)[R], float (&cacc)[(R + 3) / 4]) {
+    float d = f16bits_to_f32(r.hdr.x & 0xFFFF), dmin = f16bits_to_f32(r.hdr.x >> 16);
+    uint32_t a0 = r.hdr.y >> c.c0, a1 = r.hdr.z >> c.c0, a2 = r.hdr.w >> c.c0;
+    uint32_t scp = (a0 & c.c1) | (a2 & c.c2) | ((a0 >> 2) & c.c3);          // (sc[2g], sc[2g+1]) in bytes 0, 1
+    uint32_t mp = (a1 & c.c1) | ((a2 >> 4) & c.c2) | ((a1 >> 2) & c.c3);   // (m[2g], m[2g+1])
+    float ds0 = d * kTwo24 * cvt_ubyte0(scp), ds1 = d * kTwo20 * cvt_ubyte1(scp);
+    float dm0 = dmin * cvt_ubyte0(mp), dm1 = dmin * cvt_ubyte1(mp);
+    u32x4 w = r.q;
+    half8_t lo_a = as_half8(w.x & kNibLo, (w.x >> 8) & kNibLo, w.y & kNibLo, (w.y >> 8) & kNibLo);
+    half8_t lo_b = as_half8(w.z & kNibLo, (w.z >> 8) & kNibLo, w.w & kNibLo, (w.w >> 8) & kNibLo);
+    half8_t hi_a = as_half8(w.x & kNibHi, (w.x >> 8) & kNibHi, w.y & kNibHi, (w.y >> 8) & kNibHi);
+    half8_t hi_b = as_half8(w.z & kNibHi, (w.z >> 8) & kNibHi, w.w & kNibHi, (w.w >> 8) & kNibHi);
+    const half8_t *x8 = reinterpret_cast<const half8_t *>(xa);   // elements 64g + 16kg + {0, 8, 32, 40}
+    f32x16 p = mfma(x8[0], lo_a, zero16());
+    f32x16 q = mfma(x8[4], hi_a, zero16());
+    p = mfma(x8[1], lo_b, p);
+    q = mfma(x8[5], hi_b, q);
+    fma_acc<R>(acc, p, ds0);
+    fma_acc<R>(acc, q, ds1);
+#pragma unroll
+    for (int qd = 0; qd < (R + 3) / 4; ++qd) {
+      const float *s = sx[qd] + 2 * c.g;
+      cacc[qd] = fmaf(dm0, s[0], cacc[qd]);
+      cacc[qd] = fmaf(dm1, s[1], cacc[qd]);
+    }
+  }
+  __device__ static float finish(float acc, float cacc) { return acc - cacc; }
+
+  // Batch 1 without the matrix core: the lane's 16 low and 16 high nibbles against its own 32 activations.
+  // Both k-halves of a piece add half of the "- min" term, so that their sum carries it once.
+  __device__ static int x_offset(const LaneCtx &c) { return c.g * kXGroup + 16 * c.kg; }
+  __device__ static void init_dot(LaneCtx &c) { init(c); }
+  __device__ static int x_offset_dot(const LaneCtx &c) { return c.g * kXGroup + 16 * c.kg; }
+  template <int MT>
+  __device__ static void dot(const Raw &r, const half_t *xa, int xrow, const float *sx, int sxrow, const LaneCtx &c,
+                             float (&acc)[MT], float (&cacc)[MT]) {
+    float d = f16bits_to_f32(r.hdr.x & 0xFFFF), dmin = f16bits_to_f32(r.hdr.x >> 16);
+    uint32_t a0 = r.hdr.y >> c.c0, a1 = r.hdr.z >> c.c0, a2 = r.hdr.w >> c.c0;
+    uint32_t scp = (a0 & c.c1) | (a2 & c.c2) | ((a0 >> 2) & c.c3);
+    uint32_t mp = (a1 & c.c1) | ((a2 >> 4) & c.c2) | ((a1 >> 2) & c.c3);
+    float ds0 = d * kTwo24 * cvt_ubyte0(scp), ds1 = d * kTwo20 * cvt_ubyte1(scp);
+    float dm0 = dmin * cvt_ubyte0(mp), dm1 = dmin * cvt_ubyte1(mp);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const u32x4 *x4 = reinterpret_cast<const u32x4 *>(xa + m * xrow);   // elements 64g + 16kg + {0, 8, 32, 40}
+      u32x4 xl0 = x4[0], xl1 = x4[1], xh0 = x4[4], xh1 = x4[5];
+      float pl = dot_pairs(r.q.x, r.q.y, xl0, kNibLo, 0.0f), ph = dot_pairs(r.q.x, r.q.y, xh0, kNibHi, 0.0f);
+      pl = dot_pairs(r.q.z, r.q.w, xl1, kNibLo, pl);
+      ph = dot_pairs(r.q.z, r.q.w, xh1, kNibHi, ph);
+      acc[m] = fmaf(pl, ds0, acc[m]);
+      acc[m] = fmaf(ph, ds1, acc[m]);
+      cacc[m] = fmaf(dm0, sx[m * sxrow + 2 * c.g], cacc[m]);
+      cacc[m] = fmaf(dm1, sx[m * sxrow + 2 * c.g + 1], cacc[m]);
+    }
+  }
+  __device__ static float finish_dot(float acc, float cacc) { return fmaf(-0.5f, cacc, acc); }
+};
+
+// ---- Q6_K -------------------------------------------------------------------
+// 210 B = [ql:128][qh:64][sc:16 x i8][d].  Piece g = (H = g>>1, sigma = g&1)
+// owns ql[64H+32sigma .. +31]: low nibbles are quarter s = sigma, high nibbles
+// quarter s = sigma+2 of half H; qh[32H + l] holds bits 4-5 of all four
+// quarters.  Sub-blocks are 16 elements (lam = l>>4).  Lane kg loads the 16
+// bytes of lam = kg and swaps halves with its partner, after which both hold
+// bytes 8kg..8kg+7 of lam = 0 (registers 0-1) and lam = 1 (registers 2-3).
+template <> struct Rows8<CUTHIP_Q6_K> {
+  static constexpr int NSUB = 16, SUBK = 16;
+  struct Raw { u32x4 ql, qh, sc; uint32_t d; };
+  __device__ static void init(LaneCtx &c) {
+    c.c0 = 2u * (c.g & 1);        // qh bit offset of quarter sigma
+    c.c1 = 16u * (c.g & 1);       // bit offset of scale byte pair (2 sigma, 2 sigma + 1) inside its dword
+    c.c2 = (uint32_t)(c.g >> 1);  // H
+    c.c3 = 0;
+  }
+  __device__ static void load(Raw &r, const uint8_t *row, uint32_t step, const LaneCtx &c, uint32_t) {
+    const uint8_t *p = row + (size_t)step * 210;
+    r.ql = ld_u32x4(p + 32 * c.g + 16 * c.kg);
+    r.qh = ld_u32x4(p + 128 + 32 * (c.g >> 1) + 16 * c.kg);
+    r.sc = ld_u32x4(p + 192);
+    r.d = ld_u16(p + 208);
+  }
+  template <int R>
+  __device__ static void compute(const Raw &r, const half_t *xa, const float *const *sx, const LaneCtx &c,
+                                 float (&acc)[R], float (&cacc)[(R + 3) / 4]) {
+    constexpr uint32_t kH45 = 0x00300030u, kH89 = 0x03000300u;
+    uint32_t ql[4] = {r.ql.x, r.ql.y, r.ql.z, r.ql.w}, qh[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
+    swap_halves(ql[0], ql[2]); swap_halves(ql[1], ql[3]);
+    swap_halves(qh[0], qh[2]); swap_halves(qh[1], qh[3]);
+    float d = f16bits_to_f32(r.d);
+    uint32_t wlo = c.c2 ? r.sc.z : r.sc.x;   // scales of quarter s = sigma   live in dword 2H
+    uint32_t whi = c.c2 ? r.sc.w : r.sc.y;   // scales of quarter s = sigma+2 live in dword 2H+1
+    const half8_t *x8 = reinterpret_cast<const half8_t *>(xa);
+    // x8 offsets (in 8-half chunks): quarter sigma, lam: 2*lam ; quarter sigma+2, lam: 9 + 2*lam  (72 halfs = 9 chunks)
+#pragma unroll
+    for (int lam = 0; lam < 2; ++lam) {
+      uint32_t v_lo[4], v_hi[4];
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        uint32_t w = ql[2 * lam + k], hs = qh[2 * lam + k] >> c.c0;
+        uint32_t w8 = w >> 8, hl = hs << 4, hr = hs >> 4;
+        v_lo[2 * k + 0] = (w & kNibLo) | (hl & kH45);
+        v_lo[2 * k + 1] = (w8 & kNibLo) | (hr & kH45);
+        v_hi[2 * k + 0] = (w & kNibHi) | (hl & kH89);
+        v_hi[2 * k + 1] = (w8 & kNibHi) | (hr & kH89);
+      }
+      f32x16 p = mfma(x8[2 * lam], as_half8(v_lo[0], v_lo[1], v_lo[2], v_lo[3]), zero16());
+      f32x16 q = mfma(x8[9 + 2 * lam], as_half8(v_hi[0], v_hi[1], v_hi[2], v_hi[3]), zero16());
+      float s_lo = (float)(int)__builtin_amdgcn_sbfe((int)wlo, c.c1 + 8 * lam, 8);
+      float s_hi = (float)(int)__builtin_amdgcn_sbfe((int)whi, c.c1 + 8 * lam, 8);
+      float dlo = d * s_lo, dhi = d * s_hi;
+      fma_acc<R>(acc, p, dlo * kTwo24);
+      fma_acc<R>(acc, q, dhi * kTwo20);
+      int j_lo = 8 * (c.g >> 1) + 2 * (c.g & 1) + lam;   // sub-block of (H, s = sigma, lam); s = sigma+2 is 4 further
+#pragma unroll
+      for (int qd = 0; qd < (R + 3) / 4; ++qd) {
+        cacc[qd] = fmaf(dlo, sx[qd][j_lo], cacc[qd]);
+        cacc[qd] = fmaf(dhi, sx[qd][j_lo + 4], cacc[qd]);
+      }
+    }
+  }
+  __device__ static float finish(float acc, float cacc) { return fmaf(-32.0f, cacc, acc); }
+
+  // Batch 1 without the matrix core: lane kg owns the 16-element sub-blocks lam = kg of quarters sigma and sigma+2.
+  __device__ static void init_dot(LaneCtx &c) {
+    init(c);
+    c.c1 += 8u * c.kg;   // bit offset of scale byte 2 sigma + kg
+  }
+  __device__ static int x_offset(const LaneCtx &c) { return 2 * (c.g >> 1) * kXGroup + 32 * (c.g & 1) + 8 * c.kg; }
+  __device__ static int x_offset_dot(const LaneCtx &c) { return 2 * (c.g >> 1) * kXGroup + 32 * (c.g & 1) + 16 * c.kg; }
+  template <int MT>
+  __device__ static void dot(const Raw &r, const half_t *xa, int xrow, const float *sx, int sxrow, const LaneCtx &c,
+                             float (&acc)[MT], float (&cacc)[MT]) {
+    constexpr uint32_t kH45 = 0x00300030u, kH89 = 0x03000300u;
+    const uint32_t ql[4] = {r.ql.x, r.ql.y, r.ql.z, r.ql.w}, qh[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
+    uint32_t vl[8], vh[8];   // 6-bit quants as fp16 subnormals: q * 2^-24 (quarter sigma) and q * 2^-20 (quarter sigma+2)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      uint32_t w = ql[k], hs = qh[k] >> c.c0;
+      uint32_t w8 = w >> 8, hl = hs << 4, hr = hs >> 4;
+      vl[2 * k] = (w & kNibLo) | (hl & kH45);
+      vl[2 * k + 1] = (w8 & kNibLo) | (hr & kH45);
+      vh[2 * k] = (w & kNibHi) | (hl & kH89);
+      vh[2 * k + 1] = (w8 & kNibHi) | (hr & kH89);
+    }
+    float d = f16bits_to_f32(r.d);
+    uint32_t wlo = c.c2 ? r.sc.z : r.sc.x, whi = c.c2 ? r.sc.w : r.sc.y;
+    float dlo = d * (float)(int)__builtin_amdgcn_sbfe((int)wlo, c.c1, 8);
+    float dhi = d * (float)(int)__builtin_amdgcn_sbfe((int)whi, c.c1, 8);
+    const int j_lo = 8 * (c.g >> 1) + 2 * (c.g & 1) + c.kg;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const u32x4 *x4 = reinterpret_cast<const u32x4 *>(xa + m * xrow);   // quarter sigma: chunks 0, 1 ; sigma+2: 9, 10
+      const u32x4 xl0 = x4[0], xl1 = x4[1], xh0 = x4[9], xh1 = x4[10];
+      float pl = dot2(vl[0], xl0.x, 0.0f), ph = dot2(vh[0], xh0.x, 0.0f);
+      pl = dot2(vl[1], xl0.y, pl); ph = dot2(vh[1], xh0.y, ph);
+      pl = dot2(vl[2], xl0.z, pl); ph = dot2(vh[2], xh0.z, ph);
+      pl = dot2(vl[3], xl0.w, pl); ph = dot2(vh[3], xh0.w, ph);
+      pl = dot2(vl[4], xl1.x, pl); ph = dot2(vh[4], xh1.x, ph);
+      pl = dot2(vl[5], xl1.y, pl); ph = dot2(vh[5], xh1.y, ph);
+      pl = dot2(vl[6], xl1.z, pl); ph = dot2(vh[6], xh1.z, ph);
+      pl = dot2(vl[7], xl1.w, pl); ph = dot2(vh[7], xh1.w, ph);
+      acc[m] = fmaf(pl, dlo * kTwo24, acc[m]);
+      acc[m] = fmaf(ph, dhi * kTwo20, acc[m]);
+      cacc[m] = fmaf(dlo, sx[m * sxrow + j_lo], cacc[m]);
+      cacc[m] = fmaf(dhi, sx[m * sxrow + j_lo + 4], cacc[m]);
+    }
+  }
+  __device__ static float finish_dot(float acc, float cacc) { return fmaf(-32.0f, cacc, acc); }
+};
+
+// ---- Q8_0 -------------------------------------------------------------------
+// 34 B = [d][q:32 x i8]; a step is 8 blocks, piece g = blocks 2g and 2g+1.
+// Lane kg loads block 2g+kg; after the swap registers (0,1) / (4,5) hold bytes
+// 8kg..+7 / 16+8kg..+7 of block 2g and (2,3) / (6,7) those of block 2g+1.
+template <> struct Rows8<CUTHIP_Q8_0> {
+  static constexpr int NSUB = 8, SUBK = 32;
+  struct Raw { u32x4 q0, q1; uint32_t d; };
+  __device__ static void init(LaneCtx &c) { c.c0 = c.c1 = c.c2 = c.c3 = 0; }
+  __device__ static void load(Raw &r, const uint8_t *row, uint32_t step, const LaneCtx &c, uint32_t K) {
+    uint32_t nblk = K / 32, b = step * 8 + 2 * c.g + c.kg;
+    const uint8_t *p = row + (size_t)min(b, nblk - 1) * 34;
+    r.q0 = ld_u32x4(p + 2);
+    r.q1 = ld_u32x4(p + 18);
+    uint32_t d = ld_u16(p);
+    r.d = b < nblk ? d : 0u;   // blocks past K contribute zero
+  }
+  template <int R>
+  __device__ static void compute(const Raw &r, const half_t *xa, const float *const *sx, const LaneCtx &c,
+                                 float (&acc)[R], float (&cacc)[(R + 3) / 4]) {
+    constexpr uint32_t kByte = 0x00FF00FFu, kFlip = 0x80808080u;
+    uint32_t w[8] = {r.q0.x ^ kFlip, r.q0.y ^ kFlip, r.q0.z ^ kFlip, r.q0.w ^ kFlip,
+                     r.q1.x ^ kFlip, r.q1.y ^ kFlip, r.q1.z ^ kFlip, r.q1.w ^ kFlip};
+    swap_halves(w[0], w[2]); swap_halves(w[1], w[3]);
+    swap_halves(w[4], w[6]); swap_halves(w[5], w[7]);
+    uint32_t da = r.d, db = r.d;
+    swap_halves(da, db);   // lanes 0-31: (own, partner) ; lanes 32-63: (partner, own) = (block 2g, block 2g+1)
+    float d_a = f16bits_to_f32(da), d_b = f16bits_to_f32(db);
+    const half8_t *x8 = reinterpret_cast<const half8_t *>(xa);   // elements 64g + 8kg + {0, 16, 32, 48}
+    auto op = [&](uint32_t u0, uint32_t u1) { return as_half8(u0 & kByte, (u0 >> 8) & kByte, u1 & kByte, (u1 >> 8) & kByte); };
+    f32x16 p = mfma(x8[0], op(w[0], w[1]), zero16());
+    f32x16 q = mfma(x8[4], op(w[2], w[3]), zero16());
+    p = mfma(x8[2], op(w[4], w[5]), p);
+    q = mfma(x8[6], op(w[6], w[7]), q);
+    fma_acc<R>(acc, p, d_a * kTwo24);
+    fma_acc<R>(acc, q, d_b * kTwo24);
+#pragma unroll
+    for (int qd = 0; qd < (R + 3) / 4; ++qd) {
+      const float *s = sx[qd] + 2 * c.g;
+      cacc[qd] = fmaf(d_a, s[0], cacc[qd]);
+      cacc[qd] = fmaf(d_b, s[1], cacc[qd]);
+    }
+  }
+  __device__ static float finish(float acc, float cacc) { return fmaf(-128.0f, cacc, acc); }
+
+  // Batch 1 without the matrix core: lane kg owns block 2g+kg.
+  __device__ static void init_dot(LaneCtx &c) { init(c); }
+  __device__ static int x_offset(const LaneCtx &c) { return c.g * kXGroup + 8 * c.kg; }
+  __device__ static int x_offset_dot(const LaneCtx &c) { return c.g * kXGroup + 32 * c.kg; }
+  template <int MT>
+  __device__ static void dot(const Raw &r, const half_t *xa, int xrow, const float *sx, int sxrow, const LaneCtx &c,
+                             float (&acc)[MT], float (&cacc)[MT]) {
+    constexpr uint32_t kByte = 0x00FF00FFu, kFlip = 0x80808080u;
+    const uint32_t w[8] = {r.q0.x ^ kFlip, r.q0.y ^ kFlip, r.q0.z ^ kFlip, r.q0.w ^ kFlip,
+                           r.q1.x ^ kFlip, r.q1.y ^ kFlip, r.q1.z ^ kFlip, r.q1.w ^ kFlip};
+    float d = f16bits_to_f32(r.d);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const u32x4 *x4 = reinterpret_cast<const u32x4 *>(xa + m * xrow);
+      u32x4 x0 = x4[0], x1 = x4[1], x2 = x4[2], x3 = x4[3];
+      float p0 = dot_pairs(w[0], w[1], x0, kByte, 0.0f), p1 = dot_pairs(w[2], w[3], x1, kByte, 0.0f);
+      p0 = dot_pairs(w[4], w[5], x2, kByte, p0);
+      p1 = dot_pairs(w[6], w[7], x3, kByte, p1);
+      acc[m] = fmaf(p0 + p1, d * kTwo24, acc[m]);
+      cacc[m] = fmaf(d, sx[m * sxrow + 2 * c.g + c.kg], cacc[m]);
+    }
+  }
+  __device__ static float finish_dot(float acc, float cacc) { return fmaf(-128.0f, cacc, acc); }
+};
+
+// ---- Q4_0 -------------------------------------------------------------------
+// 18 B = [d][qs:16]: low nibble of qs[i] is element i, high nibble element i+16.
+// Lane kg loads block 2g+kg; after the swap registers (0,1) hold bytes 8kg..+7
+// of block 2g and (2,3) those of block 2g+1.
+template <> struct Rows8<CUTHIP_Q4_0> {
+  static constexpr int NSUB = 8, SUBK = 32;
+  struct Raw { u32x4 q; uint32_t d; };
+  __device__ static void init(LaneCtx &c) { c.c0 = c.c1 = c.c2 = c.c3 = 0; }
+  __device__ static void load(Raw &r, const uint8_t *row, uint32_t step, const LaneCtx &c, uint32_t K) {
+    uint32_t nblk = K / 32, b = step * 8 + 2 * c.g + c.kg;
+    const uint8_t *p = row + (size_t)min(b, nblk - 1) * 18;
+    r.q = ld_u32x4(p + 2);
+    uint32_t d = ld_u16(p);
+    r.d = b < nblk ? d : 0u;
+  }
+  template <int R>
+  __device__ static void compute(const Raw &r, const half_t *xa, const float *const *sx, const LaneCtx &c,
+                                 float (&acc)[R], float (&cacc)[(R + 3) / 4]) {
+    uint32_t w[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+    swap_halves(w[0], w[2]); swap_halves(w[1], w[3]);
+    uint32_t da = r.d, db = r.d;
+    swap_halves(da, db);
+    float d_a = f16bits_to_f32(da), d_b = f16bits_to_f32(db);
+    const half8_t *x8 = reinterpret_cast<const half8_t *>(xa);   // elements 64g + 8kg + {0, 16, 32, 48}
+    auto lo = [&](uint32_t u0, uint32_t u1) { return as_half8(u0 & kNibLo, (u0 >> 8) & kNibLo, u1 & kNibLo, (u1 >> 8) & kNibLo); };
+    auto hi = [&](uint32_t u0, uint32_t u1) { return as_half8(u0 & kNibHi, (u0 >> 8) & kNibHi, u1 & kNibHi, (u1 >> 8) & kNibHi); };
+    f32x16 p0 = mfma(x8[0], lo(w[0], w[1]), zero16());   // block 2g, elements 0-15
+    f32x16 p1 = mfma(x8[2], hi(w[0], w[1]), zero16());   // block 2g, elements 16-31 (x 2^-20)
+    f32x16 q0 = mfma(x8[4], lo(w[2], w[3]), zero16());
+    f32x16 q1 = mfma(x8[6], hi(w[2], w[3]), zero16());
+    fma_acc<R>(acc, p0, d_a * kTwo24);
+    fma_acc<R>(acc, p1, d_a * kTwo20);
+    fma_acc<R>(acc, q0, d_b * kTwo24);
+    fma_acc<R>(acc, q1, d_b * kTwo20);
+#pragma unroll
+    for (int qd = 0; qd < (R + 3) / 4; ++qd) {
+      const float *s = sx[qd] + 2 * c.g;
+      cacc[qd] = fmaf(d_a, s[0], cacc[qd]);
+      cacc[qd] = fmaf(d_b, s[1], cacc[qd]);
+    }
+  }
+  __device__ static float finish(float acc, float cacc) { return fmaf(-8.0f, cacc, acc); }
+
+  // Batch 1 without the matrix core: lane kg owns block 2g+kg.
+  __device__ static void init_dot(LaneCtx &c) { init(c); }
+  __device__ static int x_offset(const LaneCtx &c) { return c.g * kXGroup + 8 * c.kg; }
+  __device__ static int x_offset_dot(const LaneCtx &c) { return c.g * kXGroup + 32 * c.kg; }
+  template <int MT>
+  __device__ static void dot(const Raw &r, const half_t *xa, int xrow, const float *sx, int sxrow, const LaneCtx &c,
+                             float (&acc)[MT], float (&cacc)[MT]) {
+    float d = f16bits_to_f32(r.d);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const u32x4 *x4 = reinterpret_cast<const u32x4 *>(xa + m * xrow);
+      u32x4 x0 = x4[0], x1 = x4[1], x2 = x4[2], x3 = x4[3];
+      float pl = dot_pairs(r.q.x, r.q.y, x0, kNibLo, 0.0f), ph = dot_pairs(r.q.x, r.q.y, x2, kNibHi, 0.0f);
+      pl = dot_pairs(r.q.z, r.q.w, x1, kNibLo, pl);
+      ph = dot_pairs(r.q.z, r.q.w, x3, kNibHi, ph);
+      acc[m] = fmaf(pl, d * kTwo24, acc[m]);
+      acc[m] = fmaf(ph, d * kTwo20, acc[m]);
+      cacc[m] = fmaf(d, sx[m * sxrow + 2 * c.g + c.kg], cacc[m]);
+    }
+  }
+  __device__ static float finish_dot(float acc, float cacc) { return fmaf(-8.0f, cacc, acc); }
+};
+
+// ---- activations -> LDS ---------------------------------------------------------
+// xs[m][(K/64) groups of 72 halfs], sxs[m][K/SUBK]; elements past K are zero.
+// A thread handles XR groups of 8 elements of each of the MT batch rows per
+// batch; the loads of a batch are issued together (XStage::load) and converted
+// / stored later (XStage::store), so the caller can put the weight loads in
+// between: memory returns in issue order, hence the wait for the activations
+// leaves the weight loads in flight.
+template <int SUBK, int THREADS, int MT, int XR> struct XStage {
+  u32x4 ra[MT * XR], rb[MT * XR];
+  // base: first group (of a row) of this batch; gpr: groups per padded row
+  __device__ void load(const GemvParams &p, uint32_t base, int tid, uint32_t gpr) {
+    const uint32_t esz = p.a_f16 ? 2u : 4u;
+#pragma unroll
+    for (int u = 0; u < MT * XR; ++u) {
+      const uint32_t m = u / XR, gi = base + (u % XR) * THREADS + tid, k = gi * 8;
+      // lanes without a group issue nothing (the unused slots of a batch cost no traffic); store() masks them
+      if (m < p.M && k < p.K) {
+        const uint8_t *src = reinterpret_cast<const uint8_t *>(p.A) + ((size_t)m * p.strideA + k) * esz;
+        ra[u] = ld_u32x4(src);
+        if (!p.a_f16) rb[u] = ld_u32x4(src + 16);
+      }
+    }
+  }
+  __device__ void store(const GemvParams &p, uint32_t base, int tid, uint32_t gpr, half_t *xs, float *sxs, int xrow,
+                        int sxrow) const {
+#pragma unroll
+    for (int u = 0; u < MT * XR; ++u) {
+      const uint32_t m = u / XR, gi = base + (u % XR) * THREADS + tid, k = gi * 8;
+      const bool active = m < p.M && gi < gpr, ok = active && k < p.K;
+      half_t h[8];
+      if (p.a_f16) {
+        half8_t v = __builtin_bit_cast(half8_t, ra[u]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) h[i] = v[i];
+      } else {
+        f32x4 lo = __builtin_bit_cast(f32x4, ra[u]), hi = __builtin_bit_cast(f32x4, rb[u]);
+        h[0] = (half_t)lo.x; h[1] = (half_t)lo.y; h[2] = (half_t)lo.z; h[3] = (half_t)lo.w;
+        h[4] = (half_t)hi.x; h[5] = (half_t)hi.y; h[6] = (half_t)hi.z; h[7] = (half_t)hi.w;
+      }
+      float s = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        h[i] = ok ? h[i] : (half_t)0.0f;
+        s += (float)h[i];
+      }
+      s += __shfl_xor(s, 1);
+      if (SUBK == 32) s += __shfl_xor(s, 2);
+      if (active) {
+        half8_t o{h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
+        *reinterpret_cast<half8_t *>(xs + m * xrow + (gi >> 3) * kXGroup + (gi & 7) * 8) = o;
+        constexpr uint32_t per = SUBK / 8;
+        if ((gi & (per - 1)) == 0) sxs[m * sxrow + gi / per] = s;
+      }
+    }
+  }
+};
+
+// ---- the kernel -----------------------------------------------------------------
+// MT: batch rows held (1, 2 or 4); RWG x KW waves per workgroup; D ring depth.
+// MT == 1 takes the lane-local dot-product path (v_dot2_f32_f16 on the same
+// subnormal operands: a quarter of the issue cycles of the matrix-core path,
+// whose 32 A-rows would be 7/8 padding); MT > 1 goes through the matrix core.
+template <int FMT, int MT, int RWG, int KW, int D, int XWANT>
+__global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_kernel(GemvParams p) {
+  using S = Rows8<FMT>;
+  constexpr bool DOT = MT <= kRows8DotMax;
+  constexpr int WAVES = RWG * KW, THREADS = 64 * WAVES;
+  // accumulators: dot path one per batch row; matrix-core path rows 4m + g of C, RQ quads of four pieces
+  constexpr int R = DOT ? MT : 2 * MT, RQ = DOT ? MT : R / 4;
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rg = wave / KW, kw = wave - rg * KW;
+  LaneCtx c;
+  c.kg = lane >> 5;
+  const int j = lane & 31;
+  c.g = j & 3;
+  const int r8 = j >> 2;
+  if (DOT) S::init_dot(c);
+  else S::init(c);
+
+  const uint32_t kpad = p.nsteps * 256u;
+  const int xrow = (int)(p.nsteps * kXStep), sxrow = (int)(p.nsteps * S::NSUB);
+  half_t *xs = reinterpret_cast<half_t *>(lds);
+  float *sxs = reinterpret_cast<float *>(lds + (size_t)MT * xrow * 2);
+
+  const uint32_t n0 = (blockIdx.x * RWG + rg) * 8u;
+  const uint32_t n = min(n0 + (uint32_t)r8, p.N - 1);
+  const uint8_t *row = p.W + (size_t)n * p.row_bytes;
+  const uint32_t sb = (uint32_t)(((uint64_t)p.nsteps * kw) / KW);
+  const uint32_t se = (uint32_t)(((uint64_t)p.nsteps * (kw + 1)) / KW);
+  const uint32_t cnt = se - sb, last = min(se > sb ? se - 1 : sb, p.nsteps - 1);
+
+  // activation loads first (they must not queue behind the weight loads), then the weight ring, then the
+  // conversion of the activations; batches beyond the first (large M * K only) are staged behind the ring
+  // groups of 8 activations per thread and batch row in the first batch: sized so that typical shapes need no
+  // second batch (every further batch is one more memory round trip before the first step can start)
+  constexpr int XCAP = 8 / MT, XR = XWANT < XCAP ? XWANT : XCAP;
+  const uint32_t gpr = kpad / 8;   // 8-element groups per padded row
+  XStage<S::SUBK, THREADS, MT, XR> xst;
+  xst.load(p, 0, tid, gpr);
+  typename S::Raw buf[D];
+#pragma unroll
+  for (int i = 0; i < D; ++i) {
+    S::load(buf[i], row, min(sb + i, last), c, p.K);
+    __builtin_amdgcn_sched_barrier(0);   // keep issue order = ring order, so that step i waits for its own loads only
+  }
+  xst.store(p, 0, tid, gpr, xs, sxs, xrow, sxrow);
+  for (uint32_t base = THREADS * XR; base < gpr; base += THREADS * XR) {
+    xst.load(p, base, tid, gpr);
+    xst.store(p, base, tid, gpr, xs, sxs, xrow, sxrow);
+  }
+  __syncthreads();
+
+  // Matrix-core path: A-row j of this lane is batch row j>>2 (clamped), piece j&3, and accumulator quad q
+  // holds batch row 2q + kg.  Dot path: the lane's own slice of every batch row, accumulator q = batch row q.
+  const half_t *xbase = DOT ? xs + S::x_offset_dot(c) : xs + min(j >> 2, (int)p.M - 1) * xrow + S::x_offset(c);
+  const float *sxq[RQ];
+#pragma unroll
+  for (int q = 0; q < RQ; ++q) sxq[q] = sxs + (DOT ? 0 : min(2 * q + c.kg, (int)p.M - 1) * sxrow);
+
+  float acc[R], cacc[RQ];
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+#pragma unroll
+  for (int q = 0; q < RQ; ++q) cacc[q] = 0.0f;
+
+  auto do_step = [&](const typename S::Raw &raw, uint32_t step) {
+    if constexpr (DOT) {
+      S::template dot<MT>(raw, xbase + step * kXStep, xrow, sxq[0] + step * S::NSUB, sxrow, c, acc, cacc);
+    } else {
+      const float *sx[RQ];
+#pragma unroll
+      for (int q = 0; q < RQ; ++q) sx[q] = sxq[q] + step * S::NSUB;
+      S::template compute<R>(raw, xbase + step * kXStep, sx, c, acc, cacc);
+    }
+    // keep the scale FMAs of this step here: without the pin they are sunk behind the last step and spill
+#pragma unroll
+    for (int r = 0; r < R; ++r) asm volatile("" : "+v"(acc[r]));
+#pragma unroll
+    for (int q = 0; q < RQ; ++q) asm volatile("" : "+v"(cacc[q]));
+  };
+
+  uint32_t i0 = 0;
+  for (; i0 + 2 * D <= cnt; i0 += D) {   // steady state: every refill is in range, no branches around loads
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      do_step(buf[u], sb + i0 + u);
+      S::load(buf[u], row, sb + i0 + u + D, c, p.K);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < 2 * D; ++u) {      // tail: at most 2D - 1 steps
+    uint32_t i = i0 + u;
+    if (i < cnt) {
+      do_step(buf[u % D], sb + i);
+      if (i + D < cnt) S::load(buf[u % D], row, sb + i + D, c, p.K);
+    }
+  }
+
+  // One value per (weight row, batch row): dot path = sum over the 8 lanes of the row; matrix-core path =
+  // the valid accumulator (row 4m + g of C) summed over the four pieces.  Then fold the K ranges.
+  float out[RQ];
+  bool writer;
+  if constexpr (DOT) {
+#pragma unroll
+    for (int q = 0; q < RQ; ++q) {
+      float v = S::finish_dot(acc[q], cacc[q]);
+      v += __shfl_xor(v, 1);
+      v += __shfl_xor(v, 2);
+      v += __shfl_xor(v, 32);
+      out[q] = v;
+    }
+    writer = c.g == 0 && c.kg == 0;
+  } else {
+#pragma unroll
+    for (int q = 0; q < RQ; ++q) {
+      float v = c.g == 0 ? acc[4 * q] : c.g == 1 ? acc[4 * q + 1] : c.g == 2 ? acc[4 * q + 2] : acc[4 * q + 3];
+      v = S::finish(v, cacc[q]);
+      v += __shfl_xor(v, 1);
+      v += __shfl_xor(v, 2);
+      out[q] = v;   // batch row 2q + kg
+    }
+    writer = c.g == 0;
+  }
+  if (KW == 1) {
+    if (writer && n0 + r8 < p.N) {
+#pragma unroll
+      for (int q = 0; q < RQ; ++q) {
+        int m = DOT ? q : 2 * q + c.kg;
+        if (m < (int)p.M) store_out(p.C, p.epi, p.c_f16, (size_t)m * p.strideC + n0 + r8, out[q]);
+      }
+    }
+  } else {
+    __syncthreads();   // all waves are done with the staged activations
+    float *red = reinterpret_cast<float *>(lds);   // [RWG][KW][MT][8]
+    if (writer) {
+#pragma unroll
+      for (int q = 0; q < RQ; ++q) {
+        int m = DOT ? q : 2 * q + c.kg;
+        if (m < MT) red[((rg * KW + kw) * MT + m) * 8 + r8] = out[q];
+      }
+    }
+    __syncthreads();
+    if (tid < RWG * MT * 8) {
+      int rgi = tid / (MT * 8), m = (tid / 8) % MT, rr = tid & 7;
+      uint32_t nn = (blockIdx.x * RWG + rgi) * 8u + rr;
+      if (m < (int)p.M && nn < p.N) {
+        float v = 0.0f;
+#pragma unroll
+        for (int k = 0; k < KW; ++k) v += red[((rgi * KW + k) * MT + m) * 8 + rr];
+        store_out(p.C, p.epi, p.c_f16, (size_t)m * p.strideC + nn, v);
+      }
+    }
+  }
+}
+
+template <int FMT> static size_t rows8_lds_bytes(const GemvParams &p, int mt) {
+  return (size_t)mt * ((size_t)p.nsteps * kXStep * 2 + (size_t)p.nsteps * Rows8<FMT>::NSUB * 4);
+}
+
+template <int FMT, int MT, int RWG, int KW, int D, int XWANT>
+static int launch_rows8(const GemvParams &p, hipStream_t stream) {
+  size_t lds = rows8_lds_bytes<FMT>(p, MT);
+  size_t red = (size_t)RWG * KW * MT * 8 * 4;
+  if (red > lds) lds = red;
+  auto kern = gemv_rows8_kernel<FMT, MT, RWG, KW, D, XWANT>;
+  if (lds > 64 * 1024) {
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                           "hipFuncSetAttribute"))
+      return rc;
+  }
+  uint32_t groups = (p.N + 7) / 8;
+  dim3 grid((groups + RWG - 1) / RWG), block(64 * RWG * KW);
+  hipLaunchKernelGGL(kern, grid, block, lds, stream, p);
+  return check_hip(hipGetLastError(), "gemv launch");
+}
+
+// Workgroup shapes: (RWG row groups, KW step ranges).  K is split while the
+// grid would otherwise have fewer than ~6 waves per CU and every wave keeps at
+// least 4 steps.
+template <int FMT, int MT> static int launch_rows8_shape(const GemvParams &p, int rwg, int kw, hipStream_t stream) {
+  constexpr int D = 4;   // 4 steps in flight per wave cover the memory latency; deeper rings slow the stream down
+  // last argument: groups of 8 activations a thread stages per batch row in the first batch (K / 8 / threads,
+  // rounded up to what the shape class usually needs)
+  if (kw == 1) {
+    if (rwg >= 8 || MT == 8) return launch_rows8<FMT, MT, 8, 1, D, 1>(p, stream);
+    return launch_rows8<FMT, MT, 4, 1, D, 2>(p, stream);
+  }
+  if (kw == 2) return launch_rows8<FMT, MT, 2, 2, D, 4>(p, stream);
+  if (kw == 4) {
+    if (p.nsteps <= 16) return launch_rows8<FMT, MT, 1, 4, D, 2>(p, stream);
+    return launch_rows8<FMT, MT, 1, 4, D, 8>(p, stream);
+  }
+  return launch_rows8<FMT, MT, 1, 8, D, 4>(p, stream);
+}
+
+struct Rows8Shape { int rwg, kw; };
+Rows8Shape pick_rows8_shape(uint32_t N, uint32_t nsteps);
+
+// true if the rows8 kernel can take the problem (activations must fit in LDS)
+template <int FMT> bool rows8_fits(const GemvParams &p) {
+  if (p.M > 8) return false;
+  int mt = p.M <= 1 ? 1 : (p.M <= 2 ? 2 : (p.M <= 4 ? 4 : 8));
+  return rows8_lds_bytes<FMT>(p, mt) <= 96 * 1024;
+}
+
+template <int FMT> int launch_rows8_fmt(const GemvParams &p, hipStream_t stream) {
+  Rows8Shape s = pick_rows8_shape(p.N, p.nsteps);
+  if (p.M <= 1) return launch_rows8_shape<FMT, 1>(p, s.rwg, s.kw, stream);
+  if (p.M <= 2) return launch_rows8_shape<FMT, 2>(p, s.rwg, s.kw, stream);
+  if (p.M <= 4) return launch_rows8_shape<FMT, 4>(p, s.rwg, s.kw, stream);
+  return launch_rows8_shape<FMT, 8>(p, s.rwg, s.kw, stream);
+}
+
+}  // namespace cuthip

@@ -76,11 +76,13 @@ def test_q4k_ffn_shapes_fp16_io(ops, N, K, M):
     err = normwise_rel_err(got[:, rows], want)
     assert err < 6e-4, err  # fp16 output rounding: 2^-11 / sqrt(3) ~ 2.8e-4 rms
     # batch rows are independent: row 0 of the batched call agrees with the M=1 call
-    # (the two launches may split K differently, so fp32 sums can round to
-    # neighbouring fp16 values)
+    # (the two launches use different kernels and K orders, so fp32 sums can
+    # round to neighbouring fp16 values, and outputs that cancel to almost
+    # zero differ by the fp32 rounding of their terms)
     if M > 1:
         one = gpu_matmul(ops, fmt, W, A[:1], N, K)
-        assert np.all(np.abs(one[0] - got[0]) <= np.abs(got[0]) * 2.0 ** -10 + 1e-6)
+        rms = float(np.sqrt(np.mean(got[0].astype(np.float64) ** 2)))
+        assert np.all(np.abs(one[0] - got[0]) <= np.abs(got[0]) * 2.0 ** -10 + 1e-4 * rms)
 
 
 def test_linearity_and_row_permutation(ops):
