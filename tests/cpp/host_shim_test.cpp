@@ -1,0 +1,150 @@
+// Exercises include/cut_hip_ops.hpp the way the reference's operator tests do
+// (tests/harness/OpRegistry.h:1929-2086): construct nodes, dispatch, compare
+// with a CPU reference.  "--cpu": variant tables and constructor validation
+// only (no device call).  "--gpu": known-answer and seeded cases on device 0,
+// checked against the C oracle.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "cut_hip_ops.hpp"
+extern "C" {
+#include "cut_oracle.h"
+}
+
+using namespace cut::hip;
+
+static int g_fail = 0;
+#define EXPECT(cond)                                                     \
+  do {                                                                   \
+    if (!(cond)) {                                                       \
+      std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond);        \
+      ++g_fail;                                                          \
+    }                                                                    \
+  } while (0)
+
+template <class F> static bool throws(F f) {
+  try {
+    f();
+  } catch (const std::runtime_error &) {
+    return true;
+  }
+  return false;
+}
+
+static void test_tables() {
+  EXPECT(variantCount(CUTHIP_OP_DEQUANT) >= 1);
+  uint32_t n = variantCount(CUTHIP_OP_MATMUL_GGUF);
+  EXPECT(n >= 4);
+  // indices are ABI: these names must stay at these positions
+  EXPECT(getMatMulGgufVariantName(0) == "MatMulGgufGemvMfma");
+  EXPECT(getMatMulGgufVariantName(1) == "MatMulGgufSkinnyMfma");
+  EXPECT(getMatMulGgufVariantName(2) == "MatMulGgufGemmLds");
+  EXPECT(getMatMulGgufVariantName(3) == "MatMulGgufGemvRows8");
+  for (uint32_t i = 0; i < n; ++i) EXPECT(lookupVariant(CUTHIP_OP_MATMUL_GGUF, variantInfo(CUTHIP_OP_MATMUL_GGUF, i).name) == i);
+  EXPECT(throws([] { lookupVariant(CUTHIP_OP_MATMUL_GGUF, "NoSuchVariant"); }));
+  EXPECT(throws([&] { variantInfo(CUTHIP_OP_MATMUL_GGUF, n); }));
+}
+
+static void test_validation() {
+  DeviceBuffer none;   // empty: constructors must reject before touching the device
+  Tensor raw{&none, {0}, DataType::Float32, 0};
+  EXPECT(throws([&] { DequantOpNode n(raw, GgufFormat::Q4_K, 4, 100); }));    // cols not a multiple of 256
+  EXPECT(throws([&] { DequantOpNode n(raw, GgufFormat::Q4_K, 4, 256); }));    // raw too small
+  Tensor a{&none, {1, 2, 3}, DataType::Float16, 0};
+  EXPECT(throws([&] { MatMulGgufOpNode n(a, raw, GgufFormat::Q8_0, 8); }));   // rank 3
+  Tensor a2{&none, {2, 48}, DataType::Float16, 0};
+  EXPECT(throws([&] { MatMulGgufOpNode n(a2, raw, GgufFormat::Q8_0, 8); }));  // K not a multiple of 32
+  Tensor a3{&none, {2, 64}, DataType::Float16, 0};
+  EXPECT(throws([&] { MatMulGgufOpNode n(a3, raw, GgufFormat::Q8_0, 8); }));  // weights too small
+}
+
+static double normwise(const std::vector<float> &got, const std::vector<double> &want) {
+  double num = 0, den = 0;
+  for (size_t i = 0; i < got.size(); ++i) {
+    num += (got[i] - want[i]) * (got[i] - want[i]);
+    den += want[i] * want[i];
+  }
+  return std::sqrt(num / (den > 0 ? den : 1));
+}
+
+static void test_gpu() {
+  init(0);
+  std::mt19937 rng(7);
+  std::normal_distribution<float> gw(0.0f, 0.02f), ga(0.0f, 1.0f);
+  const GgufFormat fmts[4] = {GgufFormat::Q8_0, GgufFormat::Q4_0, GgufFormat::Q4_K, GgufFormat::Q6_K};
+  for (GgufFormat f : fmts) {
+    const uint32_t N = 72, K = 512;
+    std::vector<float> w((size_t)N * K);
+    for (auto &v : w) v = gw(rng);
+    std::vector<uint8_t> blocks(ggufBytes(f, (uint64_t)N * K));
+    EXPECT(orc_quantize((int)f, w.data(), (size_t)N * K, blocks.data()) == 0);
+    DeviceBuffer wdev(blocks.data(), blocks.size());
+    Tensor wt{&wdev, {(uint32_t)blocks.size()}, DataType::Float32, 0};
+
+    // dequant: bit-exact against the oracle, fp32 with the reference's padded stride
+    DequantOpNode dq(wt, f, N, K);
+    dq.dispatch();
+    std::vector<float> got((size_t)N * dq.outputStride()), want((size_t)N * K);
+    dq.output().buffer->download(got.data(), got.size() * 4);
+    EXPECT(orc_dequant((int)f, blocks.data(), want.data(), (size_t)N * K) == 0);
+    bool same = true;
+    for (uint32_t r = 0; r < N && same; ++r)
+      same = std::memcmp(&got[(size_t)r * dq.outputStride()], &want[(size_t)r * K], K * 4) == 0;
+    EXPECT(same);
+
+    // matmul at M = 1 (rank-1 A), 3 and 40 (GEMV, batched GEMV, tiled GEMM), fp32 in / fp32 out
+    for (uint32_t M : {1u, 3u, 40u}) {
+      std::vector<float> a((size_t)M * K);
+      for (auto &v : a) v = ga(rng);
+      DeviceBuffer adev(a.data(), a.size() * 4);
+      Tensor at{&adev, M == 1 ? std::vector<uint32_t>{K} : std::vector<uint32_t>{M, K}, DataType::Float32, 0};
+      MatMulGgufOpNode mm(at, wt, f, N);
+      mm.dispatch();
+      std::vector<float> c((size_t)M * N);
+      mm.output().buffer->download(c.data(), c.size() * 4);
+      std::vector<double> ref((size_t)M * N);
+      EXPECT(orc_matmul_gguf_f64((int)f, blocks.data(), a.data(), M, K, N, ref.data()) == 0);
+      double err = normwise(c, ref);
+      if (!(err < 1e-3)) std::printf("fmt %d M %u err %g\n", (int)f, M, err);
+      EXPECT(err < 1e-3);
+
+      // fused residual add: C = A.W^T + D
+      std::vector<float> d((size_t)M * N, 0.5f);
+      DeviceBuffer ddev(d.data(), d.size() * 4);
+      Tensor dt{&ddev, {M, N}, DataType::Float32, N};
+      MatMulGgufOpNode mf(at, wt, f, N);
+      mf.setFusion(MatMulFusion::Binary, CUTHIP_BINARY_ADD, dt);
+      mf.dispatch();
+      std::vector<float> cf((size_t)M * N);
+      mf.output().buffer->download(cf.data(), cf.size() * 4);
+      bool ok = true;
+      for (size_t i = 0; i < cf.size() && ok; ++i) ok = std::fabs(cf[i] - (c[i] + 0.5f)) <= 1e-5f * (1.0f + std::fabs(c[i]));
+      EXPECT(ok);
+    }
+  }
+  // an explicit variant that cannot take the shape is an error, not a silent fallback
+  {
+    std::vector<uint8_t> blocks(ggufBytes(GgufFormat::Q8_0, 64 * 64), 0);
+    DeviceBuffer wdev(blocks.data(), blocks.size());
+    Tensor wt{&wdev, {(uint32_t)blocks.size()}, DataType::Float32, 0};
+    std::vector<float> a(16 * 64, 1.0f);
+    DeviceBuffer adev(a.data(), a.size() * 4);
+    Tensor at{&adev, {16, 64}, DataType::Float32, 0};
+    MatMulGgufOpNode mm(at, wt, GgufFormat::Q8_0, 64, DataType::Float32, 0u);   // variant 0 handles M <= 8
+    EXPECT(throws([&] { mm.dispatch(); }));
+  }
+}
+
+int main(int argc, char **argv) {
+  std::string mode = argc > 1 ? argv[1] : "--cpu";
+  test_tables();
+  test_validation();
+  if (mode == "--gpu") test_gpu();
+  std::printf("%s: %d failure(s)\n", mode.c_str(), g_fail);
+  return g_fail ? 1 : 0;
+}
