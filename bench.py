@@ -73,6 +73,12 @@ def timed_graph(torch, fn_step, steps, warmup):
     return t1 - t0, ev0.elapsed_time(ev1), used_graph
 
 
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE (x 2.000, the factor a plain
+# 1 GiB copy gives on this part) + WRITE_SIZE (x 1.000), launch-weighted over gate, up, down
+# (profiles/gemv_q4k_ffn_batch1.md holds the counters and the commands)
+TRAFFIC_BYTES_PER_LAUNCH = 33690829
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -161,7 +167,7 @@ def main():
                                "batch 1, fp16 in/out, fp32 accumulate; one step = the three GEMVs of one FFN block",
                    "weight_copies_rotated": COPIES, "hip_graph": used_graph, "pct_of_hbm_peak": round(value / HBM_PEAK_GBS * 100, 1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
                      "kernel": "cuthip::gemv_rows8_kernel<Q4_K, MT=1>", "algorithmic_bytes_per_launch": int(launch_bytes),
                      "avg_launch_us": round(avg_launch_us, 3)},
     }
