@@ -88,6 +88,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (reference traffic for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--gemm-only", type=int, default=0, metavar="M",
+                    help="only run the Q4_K prefill GEMM (M x 4096) . (14336 x 4096)^T twelve times (target of rocprofv3 runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it")
@@ -107,6 +109,24 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4, "launches": 5}))
+        return
+    if args.gemm_only:
+        M = args.gemm_only
+        wq = torch.from_numpy(make_q_weights("Q4_K", N_FF, N_EMBD, 0)).to(dev)
+        a = torch.randn((M, N_EMBD), dtype=torch.float16, device=dev)
+        c = torch.empty((M, N_FF), dtype=torch.float16, device=dev)
+        for _ in range(2):
+            ops.matmul_gguf(a, wq, "Q4_K", N_FF, N_EMBD, out=c)
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(10):
+            ops.matmul_gguf(a, wq, "Q4_K", N_FF, N_EMBD, out=c)
+        ev1.record()
+        torch.cuda.synchronize()
+        us = ev0.elapsed_time(ev1) * 1e3 / 10
+        print(json.dumps({"gemm": f"Q4_K M={M} N={N_FF} K={N_EMBD}", "us_per_launch": round(us, 1),
+                          "TFLOPs": round(2.0 * M * N_FF * N_EMBD / us / 1e6, 1)}))
         return
     log(f"[bench] {info['name']} {info['arch']} CUs={info['compute_units']}")
 

@@ -24,6 +24,8 @@
 //
 // Error budget against the fp32 CPU path: weights rounded to fp16 (2^-11
 // relative), fp16 activations exact, fp32 accumulation: ~3e-4 normwise.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace cuthip {
@@ -68,6 +70,7 @@ template <> struct Sub<CUTHIP_Q4_K> {
     for (int i = 0; i < 8; ++i) {
       uint32_t word = i < 4 ? r.q[0][i] : r.q[1][i - 4];
       word = (word >> sh) & 0x0F0F0F0Fu;
+      asm volatile("" : "+v"(word));   // one shift + mask per four quants, then v_cvt_f32_ubyte0..3
       w[4 * i + 0] = (half_t)(d1 * cvt_ubyte0(word) - dm1);
       w[4 * i + 1] = (half_t)(d1 * cvt_ubyte1(word) - dm1);
       w[4 * i + 2] = (half_t)(d1 * cvt_ubyte2(word) - dm1);
@@ -96,6 +99,7 @@ template <> struct Sub<CUTHIP_Q6_K> {
     for (int i = 0; i < 8; ++i) {
       uint32_t wl = i < 4 ? r.ql[0][i] : r.ql[1][i - 4], wh = i < 4 ? r.qh[0][i] : r.qh[1][i - 4];
       uint32_t q6 = ((wl >> lsh) & 0x0F0F0F0Fu) | (((wh >> hsh) & 0x03030303u) << 4);
+      asm volatile("" : "+v"(q6));
       float dsc = i < 4 ? dsc0 : dsc1;  // elements 0-15 / 16-31 of the 32
       w[4 * i + 0] = (half_t)(dsc * (cvt_ubyte0(q6) - 32.0f));
       w[4 * i + 1] = (half_t)(dsc * (cvt_ubyte1(q6) - 32.0f));
@@ -209,22 +213,24 @@ __global__ void __launch_bounds__(256, 2) gemm_kernel(GemmParams p) {
       }
     }
   };
-  auto store_slice = [&](uint32_t k0) {
+  // TAIL: the last slice of a K that is not a multiple of 64 (Q8_0 / Q4_0 only); columns past K are zeroed
+  auto store_slice = [&](uint32_t k0, auto tail) {
+    constexpr bool TAIL = decltype(tail)::value;
     half_t w[32];
     S::decode(braw, k0 / 32 + bsub, w);
-    bool live = k0 + 32 * bsub < p.K;  // sub-blocks past K (ragged last slice) are zero
+    const bool live = !TAIL || k0 + 32 * bsub < p.K;
     half_t *dst = Bs + (tid >> 1) * kLdsRow + 32 * bsub;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       half8v o;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] = live ? w[8 * c + e] : (half_t)0.0f;
+      for (int e = 0; e < 8; ++e) o[e] = w[8 * c + e];
+      if (TAIL && !live) o = half8v{0, 0, 0, 0, 0, 0, 0, 0};
       *reinterpret_cast<half8v *>(dst + 8 * c) = o;
     }
 #pragma unroll
     for (int v = 0; v < AV; ++v) {
       int idx = v * 256 + tid;
-      bool alive = k0 + (idx & 7) * 8 < p.K;
       half8v o;
       if constexpr (AF16) {
         o = __builtin_bit_cast(half8v, araw[v]);
@@ -233,18 +239,11 @@ __global__ void __launch_bounds__(256, 2) gemm_kernel(GemmParams p) {
         o = half8v{(half_t)lo.x, (half_t)lo.y, (half_t)lo.z, (half_t)lo.w,
                    (half_t)hi.x, (half_t)hi.y, (half_t)hi.z, (half_t)hi.w};
       }
-      if (!alive) o = half8v{0, 0, 0, 0, 0, 0, 0, 0};
+      if (TAIL && !(k0 + (idx & 7) * 8 < p.K)) o = half8v{0, 0, 0, 0, 0, 0, 0, 0};
       *reinterpret_cast<half8v *>(As + (idx >> 3) * kLdsRow + (idx & 7) * 8) = o;
     }
   };
-
-  const uint32_t nslices = (p.K + kBK - 1) / kBK;
-  load_slice(0);
-  for (uint32_t t = 0; t < nslices; ++t) {
-    __syncthreads();           // everyone is done reading the previous slice
-    store_slice(t * kBK);
-    __syncthreads();
-    if (t + 1 < nslices) load_slice((t + 1) * kBK);
+  auto mma_slice = [&]() {
     const half_t *a_base = As + (wm * (BM / 2) + (lane & 31)) * kLdsRow + 8 * (lane >> 5);
     const half_t *b_base = Bs + (wn * 64 + (lane & 31)) * kLdsRow + 8 * (lane >> 5);
 #pragma unroll
@@ -260,6 +259,22 @@ __global__ void __launch_bounds__(256, 2) gemm_kernel(GemmParams p) {
         for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
     }
+  };
+
+  const uint32_t nfull = p.K / kBK, nslices = (p.K + kBK - 1) / kBK;
+  load_slice(0);
+  for (uint32_t t = 0; t < nfull; ++t) {
+    __syncthreads();           // everyone is done reading the previous slice
+    store_slice(t * kBK, std::false_type{});
+    __syncthreads();
+    if (t + 1 < nslices) load_slice((t + 1) * kBK);
+    mma_slice();
+  }
+  if (nfull < nslices) {
+    __syncthreads();
+    store_slice(nfull * kBK, std::true_type{});
+    __syncthreads();
+    mma_slice();
   }
 
   // C tile: register r of lane l holds row 8*(r/4) + 4*(l>>5) + r%4, column l & 31 of its 32x32 block
