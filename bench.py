@@ -198,7 +198,50 @@ def main():
         for b in (2, 4, 8):
             wall_b, ev_b, _ = timed_graph(torch, ffn_step(b), 120, 12)
             extras[f"q4k_ffn_gemv_batch{b}_GBps"] = round(ffn_bytes(b) * 120 / wall_b / 1e9, 1)
-        del gate, up, down
+        # gate and up as one launch (rows concatenated, the reference's fused w_gate_up: llama.cpp:1288-1330)
+        gate_up = [torch.cat([gate[i], up[i]]) for i in range(COPIES)]
+        y_gu = torch.empty((1, 2 * N_FF), dtype=torch.float16, device=dev)
+
+        def gu_step(s):
+            ops.matmul_gguf(x[:1], gate_up[s % COPIES], "Q4_K", 2 * N_FF, N_EMBD, out=y_gu)
+        wall_gu, ev_gu, _ = timed_graph(torch, gu_step, 120, 12)
+        gu_bytes = 2 * w_bytes + 2 * (N_EMBD + 2 * N_FF)
+        extras["q4k_gate_up_fused_28672x4096_gemv_GBps"] = round(gu_bytes * 120 / (ev_gu * 1e-3) / 1e9, 1)
+        del gate, up, down, gate_up
+        torch.cuda.empty_cache()
+        # config 4, weight-streaming part only: every quantized matmul of one decode step of the 8B shape
+        # (32 layers: fused q+k 5120x4096 Q4_K, v 1024x4096 Q6_K, o 4096x4096 Q4_K + residual, fused gate+up
+        # 28672x4096 Q4_K, down 4096x14336 Q4_K + residual; then the Q6_K head 128256x4096), distinct memory per
+        # layer, one HIP graph.  Norms, RoPE, attention over the KV cache and sampling are not part of it.
+        lw = {"qk": ("Q4_K", 5120, N_EMBD), "v": ("Q6_K", 1024, N_EMBD), "o": ("Q4_K", N_EMBD, N_EMBD),
+              "gu": ("Q4_K", 2 * N_FF, N_EMBD), "down": ("Q4_K", N_EMBD, N_FF)}
+        base = {k: torch.from_numpy(make_q_weights(f, min(n, 1024), kk, 7)).to(dev).repeat((n + 1023) // 1024)[:ops.n_bytes(f, n, kk)]
+                for k, (f, n, kk) in lw.items()}
+        layers = [{k: v.clone() for k, v in base.items()} for _ in range(32)]
+        head = torch.from_numpy(make_q_weights("Q6_K", 4008, 4096, 3)).to(dev).repeat(32)
+        hid = torch.from_numpy(x_h[:1]).to(dev)
+        res = torch.zeros((1, N_EMBD), dtype=torch.float16, device=dev)
+        t_qk = torch.empty((1, 5120), dtype=torch.float16, device=dev)
+        t_v = torch.empty((1, 1024), dtype=torch.float16, device=dev)
+        t_o = torch.empty((1, N_EMBD), dtype=torch.float16, device=dev)
+        t_gu = torch.empty((1, 2 * N_FF), dtype=torch.float16, device=dev)
+        t_dn = torch.empty((1, N_EMBD), dtype=torch.float16, device=dev)
+        logits = torch.empty((1, 128256), dtype=torch.float16, device=dev)
+
+        def decode_chain(_s):
+            for L in layers:
+                ops.matmul_gguf(hid, L["qk"], "Q4_K", 5120, N_EMBD, out=t_qk)
+                ops.matmul_gguf(hid, L["v"], "Q6_K", 1024, N_EMBD, out=t_v)
+                ops.matmul_gguf(t_qk[:, :N_EMBD], L["o"], "Q4_K", N_EMBD, N_EMBD, out=t_o, binary="add", d=res)
+                ops.matmul_gguf(t_o, L["gu"], "Q4_K", 2 * N_FF, N_EMBD, out=t_gu)
+                ops.matmul_gguf(t_gu[:, :N_FF], L["down"], "Q4_K", N_EMBD, N_FF, out=t_dn, binary="add", d=res)
+            ops.matmul_gguf(t_dn, head, "Q6_K", 128256, N_EMBD, out=logits)
+        wall_c, ev_c, _ = timed_graph(torch, decode_chain, 5, 1)
+        chain_bytes = 32 * sum(v.numel() for v in base.values()) + head.numel()
+        extras["decode_step_8b_quantized_matmuls_only_ms"] = round(ev_c / 5, 3)
+        extras["decode_step_8b_quantized_matmuls_only_GBps"] = round(chain_bytes * 5 / (ev_c * 1e-3) / 1e9, 1)
+        extras["decode_step_8b_quantized_matmuls_only_tok_per_s_upper_bound"] = round(5e3 / ev_c, 1)
+        del layers, base, head, logits
         torch.cuda.empty_cache()
         # config 2: dequant of 256 Mi elements to fp16 (a 4 Mi-element tile repeated 64 times)
         n_el = 256 * 1024 * 1024
