@@ -79,6 +79,40 @@ def timed_graph(torch, fn_step, steps, warmup):
 TRAFFIC_BYTES_PER_LAUNCH = 33690829
 
 
+def bench_decode_step(torch, np, ops, dev, x_h, steps=5):
+    """config 4: one full decode step of the 8B shape at KV context 2048 (32 layers: RMSNorm, fused q+k and v
+    matmuls, RoPE + KV write, GQA attention over the fp16 cache, wo + residual, RMSNorm, fused gate+up,
+    SiLU * up, w_down + residual; output norm, Q6_K head, arg-max), distinct weight memory per layer, random
+    init, captured once into a HIP graph.  Bytes per token: weights + KV cache read."""
+    from cut_amd.decode import DecodeConfig, DecodeStep
+    cfg = DecodeConfig()
+    lw = {"qk": (cfg.fmt_attn, cfg.q_dim + cfg.kv_dim, cfg.hidden), "v": (cfg.fmt_v, cfg.kv_dim, cfg.hidden),
+          "o": (cfg.fmt_attn, cfg.hidden, cfg.q_dim), "gate_up": (cfg.fmt_ffn, 2 * cfg.ffn, cfg.hidden),
+          "down": (cfg.fmt_ffn, cfg.hidden, cfg.ffn)}
+    base = {k: torch.from_numpy(make_q_weights(f, min(n, 1024), kk, 7)).to(dev).repeat((n + 1023) // 1024)[:ops.n_bytes(f, n, kk)]
+            for k, (f, n, kk) in lw.items()}
+    ones = torch.ones(cfg.hidden, dtype=torch.float32, device=dev)
+    layers = [dict({k: v.clone() for k, v in base.items()}, attn_norm=ones, ffn_norm=ones) for _ in range(cfg.n_layers)]
+    head = torch.from_numpy(make_q_weights(cfg.fmt_head, 4008, cfg.hidden, 3)).to(dev).repeat(32)
+    dstep = DecodeStep(cfg, layers, ones, head, dev)
+    for kc, vc in zip(dstep.k_cache, dstep.v_cache):
+        kc.normal_(0.0, 0.5)
+        vc.normal_(0.0, 1.0)
+    dstep.set_position(cfg.max_ctx - 1)
+    x0 = torch.from_numpy(x_h[0].astype(np.float32)).to(dev)
+
+    def decode_step(_s):
+        dstep.x.copy_(x0)      # the embedding of the current token
+        dstep.step()
+    wall_c, ev_c, _ = timed_graph(torch, decode_step, steps, 1)
+    w_bytes_tok = cfg.n_layers * sum(v.numel() for v in base.values()) + head.numel()
+    kv_bytes_tok = cfg.n_layers * 2 * cfg.max_ctx * cfg.kv_dim * 2
+    return {"decode_step_8b_ctx2048_ms_per_token": round(ev_c / steps, 3),
+            "decode_step_8b_ctx2048_tok_per_s": round(steps * 1e3 / ev_c, 1),
+            "decode_step_8b_ctx2048_GBps": round((w_bytes_tok + kv_bytes_tok) * steps / (ev_c * 1e-3) / 1e9, 1),
+            "decode_step_8b_bytes_per_token": int(w_bytes_tok + kv_bytes_tok)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -90,6 +124,8 @@ def main():
                     help="only run a plain 1 GiB device copy 5 times (reference traffic for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--gemm-only", type=int, default=0, metavar="M",
                     help="only run the Q4_K prefill GEMM (M x 4096) . (14336 x 4096)^T twelve times (target of rocprofv3 runs)")
+    ap.add_argument("--decode-only", action="store_true",
+                    help="only run the 8B-shape decode step (target of rocprofv3 runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it")
@@ -109,6 +145,10 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4, "launches": 5}))
+        return
+    if args.decode_only:
+        x_h = np.random.default_rng(1).standard_normal((8, N_EMBD), dtype=np.float32).astype(np.float16)
+        print(json.dumps(bench_decode_step(torch, np, ops, dev, x_h)))
         return
     if args.gemm_only:
         M = args.gemm_only
@@ -209,39 +249,7 @@ def main():
         extras["q4k_gate_up_fused_28672x4096_gemv_GBps"] = round(gu_bytes * 120 / (ev_gu * 1e-3) / 1e9, 1)
         del gate, up, down, gate_up
         torch.cuda.empty_cache()
-        # config 4, weight-streaming part only: every quantized matmul of one decode step of the 8B shape
-        # (32 layers: fused q+k 5120x4096 Q4_K, v 1024x4096 Q6_K, o 4096x4096 Q4_K + residual, fused gate+up
-        # 28672x4096 Q4_K, down 4096x14336 Q4_K + residual; then the Q6_K head 128256x4096), distinct memory per
-        # layer, one HIP graph.  Norms, RoPE, attention over the KV cache and sampling are not part of it.
-        lw = {"qk": ("Q4_K", 5120, N_EMBD), "v": ("Q6_K", 1024, N_EMBD), "o": ("Q4_K", N_EMBD, N_EMBD),
-              "gu": ("Q4_K", 2 * N_FF, N_EMBD), "down": ("Q4_K", N_EMBD, N_FF)}
-        base = {k: torch.from_numpy(make_q_weights(f, min(n, 1024), kk, 7)).to(dev).repeat((n + 1023) // 1024)[:ops.n_bytes(f, n, kk)]
-                for k, (f, n, kk) in lw.items()}
-        layers = [{k: v.clone() for k, v in base.items()} for _ in range(32)]
-        head = torch.from_numpy(make_q_weights("Q6_K", 4008, 4096, 3)).to(dev).repeat(32)
-        hid = torch.from_numpy(x_h[:1]).to(dev)
-        res = torch.zeros((1, N_EMBD), dtype=torch.float16, device=dev)
-        t_qk = torch.empty((1, 5120), dtype=torch.float16, device=dev)
-        t_v = torch.empty((1, 1024), dtype=torch.float16, device=dev)
-        t_o = torch.empty((1, N_EMBD), dtype=torch.float16, device=dev)
-        t_gu = torch.empty((1, 2 * N_FF), dtype=torch.float16, device=dev)
-        t_dn = torch.empty((1, N_EMBD), dtype=torch.float16, device=dev)
-        logits = torch.empty((1, 128256), dtype=torch.float16, device=dev)
-
-        def decode_chain(_s):
-            for L in layers:
-                ops.matmul_gguf(hid, L["qk"], "Q4_K", 5120, N_EMBD, out=t_qk)
-                ops.matmul_gguf(hid, L["v"], "Q6_K", 1024, N_EMBD, out=t_v)
-                ops.matmul_gguf(t_qk[:, :N_EMBD], L["o"], "Q4_K", N_EMBD, N_EMBD, out=t_o, binary="add", d=res)
-                ops.matmul_gguf(t_o, L["gu"], "Q4_K", 2 * N_FF, N_EMBD, out=t_gu)
-                ops.matmul_gguf(t_gu[:, :N_FF], L["down"], "Q4_K", N_EMBD, N_FF, out=t_dn, binary="add", d=res)
-            ops.matmul_gguf(t_dn, head, "Q6_K", 128256, N_EMBD, out=logits)
-        wall_c, ev_c, _ = timed_graph(torch, decode_chain, 5, 1)
-        chain_bytes = 32 * sum(v.numel() for v in base.values()) + head.numel()
-        extras["decode_step_8b_quantized_matmuls_only_ms"] = round(ev_c / 5, 3)
-        extras["decode_step_8b_quantized_matmuls_only_GBps"] = round(chain_bytes * 5 / (ev_c * 1e-3) / 1e9, 1)
-        extras["decode_step_8b_quantized_matmuls_only_tok_per_s_upper_bound"] = round(5e3 / ev_c, 1)
-        del layers, base, head, logits
+        extras.update(bench_decode_step(torch, np, ops, dev, x_h))
         torch.cuda.empty_cache()
         # config 2: dequant of 256 Mi elements to fp16 (a 4 Mi-element tile repeated 64 times)
         n_el = 256 * 1024 * 1024

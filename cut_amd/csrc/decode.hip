@@ -1,0 +1,404 @@
+// The small operators between the quantized matmuls of one decode step, for
+// gfx950: RMSNorm, RoPE + KV-cache write, GQA decode attention over an fp16
+// KV cache, SiLU(gate) * up, arg-max.  Semantics follow the reference
+// kernels (operators/impl/rmsnorm/RMSNorm.cu, attention/FusedRoPEKVWrite.cu,
+// attention/Attention.cu): fp32 arithmetic, half-split RoPE with cos / sin
+// tables [pos][headDim/2], cache rows [pos][alignedKvDim], position and
+// sequence length read from a device buffer so that a captured graph can be
+// replayed for the next token.
+//
+// The attention differs from the reference in structure, not in result: the
+// reference runs one workgroup per query head over the whole context (every
+// K/V row is read nRep times, scores staged in 8 KB of shared memory).  Here
+// a workgroup owns one KV head and a chunk of 64 positions; its four waves
+// are the (up to four at a time) query heads sharing that KV head, so K and V
+// are read from HBM once, staged in LDS, and the softmax is carried as
+// (max, sum, weighted V) partials that a second kernel merges (the usual
+// split-context decode attention).
+#include <cmath>
+#include <cstdint>
+
+#include "common.hpp"
+
+namespace cuthip {
+
+__device__ inline float ld_act(const void *p, int f16, size_t i) {
+  return f16 ? (float)reinterpret_cast<const half_t *>(p)[i] : reinterpret_cast<const float *>(p)[i];
+}
+__device__ inline void st_act(void *p, int f16, size_t i, float v) {
+  if (f16)
+    reinterpret_cast<half_t *>(p)[i] = (half_t)v;
+  else
+    reinterpret_cast<float *>(p)[i] = v;
+}
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+__device__ inline float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+  return v;
+}
+
+// ---- RMSNorm: out = x * rsqrt(mean(x^2) + eps) * weight; one workgroup per row ----
+// A thread owns groups of 8 consecutive elements; up to kNormGroups of them stay in registers between the two
+// passes and all their loads are issued before the first use (a decode row is a few KB: one memory round trip).
+constexpr int kNormGroups = 4;   // 256 threads x 8 elements x 4 = rows of up to 8192 elements without a re-read
+
+template <bool F16> __device__ inline void ld8(const void *p, size_t i, uint32_t n_left, float (&v)[8]) {
+  if (n_left >= 8) {
+    if (F16) {
+      half8_t h = *reinterpret_cast<const half8_t *>(reinterpret_cast<const half_t *>(p) + i);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = (float)h[e];
+    } else {
+      f32x4 a = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(p) + i);
+      f32x4 b = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(p) + i + 4);
+      v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (uint32_t)e < n_left ? ld_act(p, F16, i + e) : 0.0f;
+  }
+}
+
+template <bool XF16, bool OF16>
+__global__ void __launch_bounds__(256) rmsnorm_kernel(const void *x, const float *weight, void *out, uint32_t dim,
+                                                      uint32_t stride, float eps, int aligned) {
+  __shared__ float red[4];
+  const uint32_t row = blockIdx.x, tid = threadIdx.x;
+  const size_t off = (size_t)row * stride;
+  float v[kNormGroups][8];
+  float s = 0.0f;
+#pragma unroll
+  for (int g = 0; g < kNormGroups; ++g) {
+    uint32_t i = (g * 256 + tid) * 8;
+    if (i < dim) ld8<XF16>(x, off + i, aligned ? dim - i : min(dim - i, 7u), v[g]);   // unaligned rows: element loads
+  }
+#pragma unroll
+  for (int g = 0; g < kNormGroups; ++g) {
+    uint32_t i = (g * 256 + tid) * 8;
+    if (i < dim)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s = fmaf(v[g][e], v[g][e], s);
+  }
+  for (uint32_t i = kNormGroups * 2048 + tid; i < dim; i += 256) {   // rows longer than the register window
+    float t = ld_act(x, XF16, off + i);
+    s = fmaf(t, t, s);
+  }
+  s = wave_sum(s);
+  if ((tid & 63) == 0) red[tid >> 6] = s;
+  __syncthreads();
+  float total = red[0] + red[1] + red[2] + red[3];
+  float scale = 1.0f / sqrtf(total / (float)dim + eps);
+  const bool wide = aligned && reinterpret_cast<uintptr_t>(out) % 16 == 0 && reinterpret_cast<uintptr_t>(weight) % 16 == 0;
+#pragma unroll
+  for (int g = 0; g < kNormGroups; ++g) {
+    uint32_t i = (g * 256 + tid) * 8;
+    if (i < dim) {
+      uint32_t n = min(dim - i, 8u);
+      if (wide && n == 8) {   // 16-byte weight loads and output stores
+        f32x4 w0 = *reinterpret_cast<const f32x4 *>(weight + i), w1 = *reinterpret_cast<const f32x4 *>(weight + i + 4);
+        float r[8] = {v[g][0] * scale * w0.x, v[g][1] * scale * w0.y, v[g][2] * scale * w0.z, v[g][3] * scale * w0.w,
+                      v[g][4] * scale * w1.x, v[g][5] * scale * w1.y, v[g][6] * scale * w1.z, v[g][7] * scale * w1.w};
+        if (OF16) {
+          half8_t h;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) h[e] = (half_t)r[e];
+          *reinterpret_cast<half8_t *>(reinterpret_cast<half_t *>(out) + off + i) = h;
+        } else {
+          float *o = reinterpret_cast<float *>(out) + off + i;
+          *reinterpret_cast<f32x4 *>(o) = f32x4{r[0], r[1], r[2], r[3]};
+          *reinterpret_cast<f32x4 *>(o + 4) = f32x4{r[4], r[5], r[6], r[7]};
+        }
+      } else {
+        for (uint32_t e = 0; e < n; ++e) st_act(out, OF16, off + i + e, v[g][e] * scale * weight[i + e]);
+      }
+    }
+  }
+  for (uint32_t i = kNormGroups * 2048 + tid; i < dim; i += 256)
+    st_act(out, OF16, off + i, ld_act(x, XF16, off + i) * scale * weight[i]);
+}
+
+// ---- RoPE on q and k, k and v appended to the cache at position params[0] ----
+__global__ void __launch_bounds__(256) rope_kv_kernel(const void *q, const void *k, const void *v, int in_f16,
+                                                      const uint32_t *params, const float *cosT, const float *sinT,
+                                                      half_t *kCache, half_t *vCache, void *qOut, int qout_f16, uint32_t qDim,
+                                                      uint32_t kvDim, uint32_t headDim, uint32_t alignedKvDim) {
+  const uint32_t gid = blockIdx.x * 256 + threadIdx.x, halfDim = headDim / 2;
+  if (gid >= qDim + 2 * kvDim) return;
+  const uint32_t pos = params[0];
+  const float *c = cosT + (size_t)pos * halfDim, *s = sinT + (size_t)pos * halfDim;
+  auto rot = [&](const void *src, uint32_t i) {
+    uint32_t d = i % headDim;
+    if (d < halfDim) return ld_act(src, in_f16, i) * c[d] - ld_act(src, in_f16, i + halfDim) * s[d];
+    return ld_act(src, in_f16, i - halfDim) * s[d - halfDim] + ld_act(src, in_f16, i) * c[d - halfDim];
+  };
+  if (gid < qDim) {
+    st_act(qOut, qout_f16, gid, rot(q, gid));
+  } else if (gid < qDim + kvDim) {
+    uint32_t i = gid - qDim;
+    kCache[(size_t)pos * alignedKvDim + i] = (half_t)rot(k, i);
+  } else {
+    uint32_t i = gid - qDim - kvDim;
+    vCache[(size_t)pos * alignedKvDim + i] = (half_t)ld_act(v, in_f16, i);
+  }
+}
+
+// ---- decode attention, split over the context ----
+constexpr int kAttnChunk = 64;    // positions per workgroup (one per lane)
+constexpr int kAttnMaxHd = 128;   // head dimension limit (as the reference's sharedQ[128])
+constexpr int kAttnRow = kAttnMaxHd + 8;   // LDS row in halfs: +16 bytes keeps the 64 rows off each other's banks
+
+// partial layout per (query head h, split s): [m, l, o[headDim]] floats at ((h * nsplit + s) * (2 + headDim))
+__global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_f16, const half_t *kCache, const half_t *vCache,
+                                                           const uint32_t *params, float *partial, uint32_t nHeads,
+                                                           uint32_t nKvHeads, uint32_t headDim, uint32_t alignedKvDim,
+                                                           float scale, uint32_t nsplit) {
+  __shared__ __attribute__((aligned(16))) half_t Ks[kAttnChunk * kAttnRow];
+  __shared__ __attribute__((aligned(16))) half_t Vs[kAttnChunk * kAttnRow];
+  __shared__ float Qs[4 * kAttnMaxHd];
+  __shared__ float Ps[4 * kAttnChunk];
+  const uint32_t kvH = blockIdx.x, split = blockIdx.y, nRep = nHeads / nKvHeads;
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t seqLen = params[1];
+  const uint32_t t0 = split * kAttnChunk;
+  const uint32_t nvalid = t0 < seqLen ? min((uint32_t)kAttnChunk, seqLen - t0) : 0u;
+
+  // stage the chunk of K and V (16-byte pieces; rows past the sequence are zero)
+  const uint32_t pieces = headDim / 8;
+  for (uint32_t i = tid; i < kAttnChunk * pieces; i += 256) {
+    uint32_t r = i / pieces, c8 = i % pieces;
+    u32x4 kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
+    if (r < nvalid) {
+      size_t off = (size_t)(t0 + r) * alignedKvDim + kvH * headDim + c8 * 8;
+      kv = ld_u32x4(reinterpret_cast<const uint8_t *>(kCache + off));
+      vv = ld_u32x4(reinterpret_cast<const uint8_t *>(vCache + off));
+    }
+    *reinterpret_cast<u32x4 *>(Ks + r * kAttnRow + c8 * 8) = kv;
+    *reinterpret_cast<u32x4 *>(Vs + r * kAttnRow + c8 * 8) = vv;
+  }
+  // query heads of this KV head are handled four at a time, one per wave
+  for (uint32_t rep0 = 0; rep0 < nRep; rep0 += 4) {
+    const uint32_t rep = rep0 + wave;
+    const bool live = rep < nRep;
+    const uint32_t h = kvH * nRep + (live ? rep : 0);
+    __syncthreads();   // K, V staged (first pass) / Qs, Ps free again (later passes)
+    for (uint32_t d = lane; d < headDim; d += 64) Qs[wave * kAttnMaxHd + d] = ld_act(q, q_f16, (size_t)h * headDim + d);
+    __syncthreads();
+    // score of position t0 + lane
+    float sc = 0.0f;
+    const half_t *krow = Ks + lane * kAttnRow;
+    const float *qv = Qs + wave * kAttnMaxHd;
+    for (uint32_t d = 0; d < headDim; d += 8) {
+      half8_t k8 = *reinterpret_cast<const half8_t *>(krow + d);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sc = fmaf(qv[d + e], (float)k8[e], sc);
+    }
+    sc = lane < nvalid ? sc * scale : -INFINITY;
+    float m = wave_max(sc);
+    float p = lane < nvalid ? expf(sc - m) : 0.0f;
+    float l = wave_sum(p);
+    Ps[wave * kAttnChunk + lane] = p;
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // weighted V: lane owns dims lane and lane + 64
+    float o0 = 0.0f, o1 = 0.0f;
+    for (uint32_t t = 0; t < nvalid; ++t) {
+      float pt = Ps[wave * kAttnChunk + t];
+      o0 = fmaf(pt, (float)Vs[t * kAttnRow + lane], o0);
+      if (headDim > 64) o1 = fmaf(pt, (float)Vs[t * kAttnRow + 64 + lane], o1);
+    }
+    if (live) {
+      float *dst = partial + ((size_t)h * nsplit + split) * (2 + headDim);
+      if (lane == 0) {
+        dst[0] = nvalid ? m : -INFINITY;
+        dst[1] = l;
+      }
+      if (lane < headDim) dst[2 + lane] = o0;
+      if (64 + lane < headDim) dst[2 + 64 + lane] = o1;
+    }
+  }
+}
+
+// One workgroup of 128 threads per query head: the (max, sum) pairs of the splits are taken one per lane, so the
+// merge weights need two wave reductions instead of a serial walk over the splits; thread d then sums dimension d.
+constexpr int kAttnMaxSplit = 1024;   // splits per head the merge kernel holds weights for (context of 65,536)
+
+__global__ void __launch_bounds__(128) attn_merge_kernel(const float *partial, const uint32_t *params, void *out, int out_f16,
+                                                         uint32_t headDim, uint32_t nsplit) {
+  __shared__ float Ws[kAttnMaxSplit];
+  __shared__ float red[4];
+  const uint32_t h = blockIdx.x, tid = threadIdx.x;
+  const uint32_t seqLen = params[1];
+  const uint32_t used = min(nsplit, (seqLen + kAttnChunk - 1) / kAttnChunk);
+  const uint32_t rec = 2 + headDim;
+  const float *base = partial + (size_t)h * nsplit * rec;
+  float m = -INFINITY;
+  for (uint32_t s = tid; s < used; s += 128) m = fmaxf(m, base[(size_t)s * rec]);
+  m = wave_max(m);
+  if ((tid & 63) == 0) red[tid >> 6] = m;
+  __syncthreads();
+  const float M = fmaxf(red[0], red[1]);
+  float l = 0.0f;
+  for (uint32_t s = tid; s < used; s += 128) {
+    float w = expf(base[(size_t)s * rec] - M);
+    Ws[s] = w;
+    l = fmaf(base[(size_t)s * rec + 1], w, l);
+  }
+  l = wave_sum(l);
+  if ((tid & 63) == 0) red[2 + (tid >> 6)] = l;
+  __syncthreads();
+  const float L = red[2] + red[3];
+  if (tid < headDim) {
+    float o = 0.0f;
+#pragma unroll 8
+    for (uint32_t s = 0; s < used; ++s) o = fmaf(base[(size_t)s * rec + 2 + tid], Ws[s], o);
+    st_act(out, out_f16, (size_t)h * headDim + tid, used ? o / L : 0.0f);
+  }
+}
+
+// ---- SiLU(gate) * up on the output of a fused gate+up matmul: in = [gate(n) | up(n)] ----
+__global__ void __launch_bounds__(256) silu_mul_kernel(const void *in, int in_f16, void *out, int out_f16, uint32_t n) {
+  uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float g = ld_act(in, in_f16, i), u = ld_act(in, in_f16, (size_t)n + i);
+  st_act(out, out_f16, i, g / (1.0f + __expf(-g)) * u);
+}
+
+// ---- arg-max (first index of the maximum), one workgroup ----
+__global__ void __launch_bounds__(1024) argmax_kernel(const void *x, int x_f16, uint32_t n, uint32_t *out) {
+  __shared__ float bv[16];
+  __shared__ uint32_t bi[16];
+  const uint32_t tid = threadIdx.x;
+  float best = -INFINITY;
+  uint32_t idx = 0xFFFFFFFFu;
+  for (uint32_t i = tid; i < n; i += 1024) {
+    float v = ld_act(x, x_f16, i);
+    if (v > best || (v == best && i < idx)) {
+      best = v;
+      idx = i;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    float ov = __shfl_xor(best, o);
+    uint32_t oi = __shfl_xor(idx, o);
+    if (ov > best || (ov == best && oi < idx)) {
+      best = ov;
+      idx = oi;
+    }
+  }
+  if ((tid & 63) == 0) {
+    bv[tid >> 6] = best;
+    bi[tid >> 6] = idx;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < 16; ++w)
+      if (bv[w] > best || (bv[w] == best && bi[w] < idx)) {
+        best = bv[w];
+        idx = bi[w];
+      }
+    out[0] = idx;
+  }
+}
+
+static bool bad_dtype(int d) { return d != CUTHIP_F32 && d != CUTHIP_F16; }
+
+}  // namespace cuthip
+
+using namespace cuthip;
+
+extern "C" {
+
+int cuthip_rmsnorm(const void *x, int x_dtype, const float *weight, void *out, int out_dtype, uint32_t rows, uint32_t dim,
+                   uint32_t stride, float eps, void *stream) {
+  if (!x || !weight || !out || rows == 0 || dim == 0 || stride < dim || bad_dtype(x_dtype) || bad_dtype(out_dtype)) {
+    set_error("cuthip_rmsnorm: bad argument (rows %u, dim %u, stride %u)", rows, dim, stride);
+    return CUTHIP_ERR_INVALID;
+  }
+  const bool xf = x_dtype == CUTHIP_F16, of = out_dtype == CUTHIP_F16;
+  // 16-byte loads need rows that start on a 16-byte boundary
+  const int aligned = (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (stride % 8 == 0);
+  auto kern = xf ? (of ? rmsnorm_kernel<true, true> : rmsnorm_kernel<true, false>)
+                 : (of ? rmsnorm_kernel<false, true> : rmsnorm_kernel<false, false>);
+  hipLaunchKernelGGL(kern, dim3(rows), dim3(256), 0, (hipStream_t)stream, x, weight, out, dim, stride, eps, aligned);
+  return check_hip(hipGetLastError(), "rmsnorm launch");
+}
+
+int cuthip_rope_kv_write(const void *q, const void *k, const void *v, int in_dtype, const uint32_t *runtime_params,
+                         const float *cos_table, const float *sin_table, void *k_cache, void *v_cache, void *q_out,
+                         int q_out_dtype, uint32_t q_dim, uint32_t kv_dim, uint32_t head_dim, uint32_t aligned_kv_dim,
+                         void *stream) {
+  if (!q || !k || !v || !runtime_params || !cos_table || !sin_table || !k_cache || !v_cache || !q_out || head_dim == 0 ||
+      head_dim % 2 || q_dim % head_dim || kv_dim % head_dim || aligned_kv_dim < kv_dim || bad_dtype(in_dtype) ||
+      bad_dtype(q_out_dtype)) {
+    set_error("cuthip_rope_kv_write: bad argument (q_dim %u, kv_dim %u, head_dim %u)", q_dim, kv_dim, head_dim);
+    return CUTHIP_ERR_INVALID;
+  }
+  uint32_t total = q_dim + 2 * kv_dim;
+  hipLaunchKernelGGL(rope_kv_kernel, dim3((total + 255) / 256), dim3(256), 0, (hipStream_t)stream, q, k, v,
+                     in_dtype == CUTHIP_F16, runtime_params, cos_table, sin_table, (half_t *)k_cache, (half_t *)v_cache, q_out,
+                     q_out_dtype == CUTHIP_F16, q_dim, kv_dim, head_dim, aligned_kv_dim);
+  return check_hip(hipGetLastError(), "rope launch");
+}
+
+size_t cuthip_attn_decode_workspace_bytes(uint32_t n_heads, uint32_t head_dim, uint32_t max_seq_len) {
+  size_t nsplit = (max_seq_len + kAttnChunk - 1) / kAttnChunk;
+  return (size_t)n_heads * nsplit * (2 + head_dim) * sizeof(float);
+}
+
+int cuthip_attn_decode(const void *q, int q_dtype, const void *k_cache, const void *v_cache, const uint32_t *runtime_params,
+                       void *out, int out_dtype, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                       uint32_t aligned_kv_dim, float scale, uint32_t max_seq_len, void *workspace, size_t workspace_bytes,
+                       void *stream) {
+  if (!q || !k_cache || !v_cache || !runtime_params || !out || !workspace || n_heads == 0 || n_kv_heads == 0 ||
+      n_heads % n_kv_heads || head_dim == 0 || head_dim > kAttnMaxHd || head_dim % 8 || max_seq_len == 0 ||
+      aligned_kv_dim < n_kv_heads * head_dim || aligned_kv_dim % 8 || bad_dtype(q_dtype) || bad_dtype(out_dtype)) {
+    set_error("cuthip_attn_decode: bad argument (heads %u/%u, head_dim %u (<= %d, multiple of 8), aligned_kv_dim %u)", n_heads,
+              n_kv_heads, head_dim, kAttnMaxHd, aligned_kv_dim);
+    return CUTHIP_ERR_INVALID;
+  }
+  if ((max_seq_len + kAttnChunk - 1) / kAttnChunk > (uint32_t)kAttnMaxSplit) {
+    set_error("cuthip_attn_decode: max_seq_len %u exceeds %d", max_seq_len, kAttnMaxSplit * kAttnChunk);
+    return CUTHIP_ERR_INVALID;
+  }
+  if (workspace_bytes < cuthip_attn_decode_workspace_bytes(n_heads, head_dim, max_seq_len)) {
+    set_error("cuthip_attn_decode: workspace of %zu bytes, need %zu", workspace_bytes,
+              cuthip_attn_decode_workspace_bytes(n_heads, head_dim, max_seq_len));
+    return CUTHIP_ERR_INVALID;
+  }
+  uint32_t nsplit = (max_seq_len + kAttnChunk - 1) / kAttnChunk;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(attn_partial_kernel, dim3(n_kv_heads, nsplit), dim3(256), 0, s, q, q_dtype == CUTHIP_F16,
+                     (const half_t *)k_cache, (const half_t *)v_cache, runtime_params, (float *)workspace, n_heads, n_kv_heads,
+                     head_dim, aligned_kv_dim, scale, nsplit);
+  if (int rc = check_hip(hipGetLastError(), "attention launch")) return rc;
+  hipLaunchKernelGGL(attn_merge_kernel, dim3(n_heads), dim3(128), 0, s, (const float *)workspace, runtime_params, out,
+                     out_dtype == CUTHIP_F16, head_dim, nsplit);
+  return check_hip(hipGetLastError(), "attention merge launch");
+}
+
+int cuthip_silu_mul(const void *gate_up, int in_dtype, void *out, int out_dtype, uint32_t n, void *stream) {
+  if (!gate_up || !out || n == 0 || bad_dtype(in_dtype) || bad_dtype(out_dtype)) {
+    set_error("cuthip_silu_mul: bad argument");
+    return CUTHIP_ERR_INVALID;
+  }
+  hipLaunchKernelGGL(silu_mul_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, gate_up,
+                     in_dtype == CUTHIP_F16, out, out_dtype == CUTHIP_F16, n);
+  return check_hip(hipGetLastError(), "silu_mul launch");
+}
+
+int cuthip_argmax(const void *x, int x_dtype, uint32_t n, uint32_t *out_index, void *stream) {
+  if (!x || !out_index || n == 0 || bad_dtype(x_dtype)) {
+    set_error("cuthip_argmax: bad argument");
+    return CUTHIP_ERR_INVALID;
+  }
+  hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, x, x_dtype == CUTHIP_F16, n, out_index);
+  return check_hip(hipGetLastError(), "argmax launch");
+}
+
+}  // extern "C"

@@ -1,0 +1,103 @@
+"""One decode step of a Llama-style dense transformer on GGUF weights: the
+chain the reference's runner encodes per token (interface/runner/llama/
+llama.cpp, runLayer: RMSNorm -> q/k/v matmuls -> RoPE + KV write ->
+attention -> wo + residual -> RMSNorm -> fused gate+up -> SiLU * up ->
+w_down + residual; then the output norm, the head matmul and arg-max).
+
+Every launch goes through the C ABI on the current stream and allocates
+nothing, so `step()` can be captured once into a HIP graph and replayed:
+the position and sequence length live in a device buffer, as the reference's
+runtimeParams do.  The residual stream is fp32; matmul inputs are fp16.
+"""
+from __future__ import annotations
+
+import dataclasses
+import math
+
+import torch
+
+from . import ops
+
+
+@dataclasses.dataclass
+class DecodeConfig:
+    hidden: int = 4096
+    n_layers: int = 32
+    n_heads: int = 32
+    n_kv_heads: int = 8
+    head_dim: int = 128
+    ffn: int = 14336
+    vocab: int = 128256
+    max_ctx: int = 2048
+    rope_theta: float = 500000.0
+    eps: float = 1e-5
+    fmt_attn: str = "Q4_K"
+    fmt_v: str = "Q6_K"
+    fmt_ffn: str = "Q4_K"
+    fmt_head: str = "Q6_K"
+
+    @property
+    def q_dim(self) -> int:
+        return self.n_heads * self.head_dim
+
+    @property
+    def kv_dim(self) -> int:
+        return self.n_kv_heads * self.head_dim
+
+
+class DecodeStep:
+    """weights: per layer a dict with GGUF-block device tensors 'qk' ([q_dim + kv_dim, hidden], q rows first),
+    'v', 'o', 'gate_up' ([2 * ffn, hidden], gate rows first), 'down' and fp32 'attn_norm', 'ffn_norm';
+    plus 'out_norm' (fp32) and 'head' at the top level."""
+
+    def __init__(self, cfg: DecodeConfig, layers: list[dict], out_norm: torch.Tensor, head: torch.Tensor, device="cuda:0"):
+        self.cfg, self.layers, self.out_norm, self.head = cfg, layers, out_norm, head
+        dev = torch.device(device)
+        c = cfg
+        f16, f32 = torch.float16, torch.float32
+        self.x = torch.zeros(c.hidden, dtype=f32, device=dev)            # residual stream
+        self.xn = torch.empty(c.hidden, dtype=f16, device=dev)
+        self.qk = torch.empty(c.q_dim + c.kv_dim, dtype=f32, device=dev)
+        self.v = torch.empty(c.kv_dim, dtype=f32, device=dev)
+        self.q_rot = torch.empty(c.q_dim, dtype=f32, device=dev)
+        self.attn = torch.empty(c.q_dim, dtype=f16, device=dev)
+        self.gu = torch.empty(2 * c.ffn, dtype=f16, device=dev)
+        self.act = torch.empty(c.ffn, dtype=f16, device=dev)
+        self.logits = torch.empty(c.vocab, dtype=f32, device=dev)
+        self.token = torch.zeros(1, dtype=torch.int32, device=dev)
+        self.params = torch.zeros(2, dtype=torch.int32, device=dev)      # {position, sequence length}
+        self.k_cache = [torch.zeros((c.max_ctx, c.kv_dim), dtype=f16, device=dev) for _ in layers]
+        self.v_cache = [torch.zeros((c.max_ctx, c.kv_dim), dtype=f16, device=dev) for _ in layers]
+        half = c.head_dim // 2
+        inv = 1.0 / (c.rope_theta ** (torch.arange(half, dtype=torch.float64) * 2.0 / c.head_dim))
+        ang = torch.arange(c.max_ctx, dtype=torch.float64)[:, None] * inv[None, :]
+        self.cos_t = torch.cos(ang).to(f32).to(dev).contiguous()
+        self.sin_t = torch.sin(ang).to(f32).to(dev).contiguous()
+        self.ws = ops.attn_decode_workspace(c.n_heads, c.head_dim, c.max_ctx, dev)
+        self.scale = 1.0 / math.sqrt(c.head_dim)
+
+    def set_position(self, pos: int) -> None:
+        """Host-side update between graph replays (a 8-byte copy; the kernels read it on the device)."""
+        self.params.copy_(torch.tensor([pos, pos + 1], dtype=torch.int32))
+
+    def step(self) -> None:
+        """Consumes self.x (the embedding of the current token), leaves logits and the arg-max token."""
+        c = self.cfg
+        for i, L in enumerate(self.layers):
+            ops.rmsnorm(self.x, L["attn_norm"], c.eps, out=self.xn.view(1, -1))
+            ops.matmul_gguf(self.xn, L["qk"], c.fmt_attn, c.q_dim + c.kv_dim, c.hidden, out=self.qk.view(1, -1))
+            ops.matmul_gguf(self.xn, L["v"], c.fmt_v, c.kv_dim, c.hidden, out=self.v.view(1, -1))
+            ops.rope_kv_write(self.qk[:c.q_dim], self.qk[c.q_dim:], self.v, self.params, self.cos_t, self.sin_t,
+                              self.k_cache[i], self.v_cache[i], c.head_dim, self.q_rot)
+            ops.attn_decode(self.q_rot, self.k_cache[i], self.v_cache[i], self.params, c.n_heads, c.n_kv_heads, c.head_dim,
+                            self.scale, self.ws, self.attn)
+            ops.matmul_gguf(self.attn, L["o"], c.fmt_attn, c.hidden, c.q_dim, out=self.x.view(1, -1), binary="add",
+                            d=self.x.view(1, -1))
+            ops.rmsnorm(self.x, L["ffn_norm"], c.eps, out=self.xn.view(1, -1))
+            ops.matmul_gguf(self.xn, L["gate_up"], c.fmt_ffn, 2 * c.ffn, c.hidden, out=self.gu.view(1, -1))
+            ops.silu_mul(self.gu, self.act)
+            ops.matmul_gguf(self.act, L["down"], c.fmt_ffn, c.hidden, c.ffn, out=self.x.view(1, -1), binary="add",
+                            d=self.x.view(1, -1))
+        ops.rmsnorm(self.x, self.out_norm, c.eps, out=self.xn.view(1, -1))
+        ops.matmul_gguf(self.xn, self.head, c.fmt_head, c.vocab, c.hidden, out=self.logits.view(1, -1))
+        ops.argmax(self.logits, self.token)

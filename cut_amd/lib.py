@@ -30,6 +30,8 @@ EXPORTS = [
     "cuthip_event_create", "cuthip_event_destroy", "cuthip_event_record", "cuthip_event_sync", "cuthip_event_elapsed_ms",
     "cuthip_variant_count", "cuthip_variant_default", "cuthip_variant_info", "cuthip_variant_lookup",
     "cuthip_dequant", "cuthip_matmul_gguf",
+    "cuthip_rmsnorm", "cuthip_rope_kv_write", "cuthip_attn_decode_workspace_bytes", "cuthip_attn_decode",
+    "cuthip_silu_mul", "cuthip_argmax",
 ]
 
 
@@ -85,9 +87,17 @@ def load() -> C.CDLL:
     lib.cuthip_variant_lookup.argtypes = [i, C.c_char_p]
     lib.cuthip_dequant.argtypes = [i, vp, vp, i, u32, u32, u32, vp]
     lib.cuthip_matmul_gguf.argtypes = [i, vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, i, vp]
+    f32 = C.c_float
+    lib.cuthip_rmsnorm.argtypes = [vp, i, vp, vp, i, u32, u32, u32, f32, vp]
+    lib.cuthip_rope_kv_write.argtypes = [vp, vp, vp, i, vp, vp, vp, vp, vp, vp, i, u32, u32, u32, u32, vp]
+    lib.cuthip_attn_decode_workspace_bytes.argtypes = [u32, u32, u32]
+    lib.cuthip_attn_decode.argtypes = [vp, i, vp, vp, vp, vp, i, u32, u32, u32, u32, f32, u32, vp, C.c_size_t, vp]
+    lib.cuthip_silu_mul.argtypes = [vp, i, vp, i, u32, vp]
+    lib.cuthip_argmax.argtypes = [vp, i, u32, vp, vp]
     for n in EXPORTS:
-        if n != "cuthip_last_error":
+        if n not in ("cuthip_last_error", "cuthip_attn_decode_workspace_bytes"):
             getattr(lib, n).restype = i
+    lib.cuthip_attn_decode_workspace_bytes.restype = C.c_size_t
     _lib = lib
     return lib
 

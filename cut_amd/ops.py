@@ -87,3 +87,63 @@ def matmul_gguf(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: int, ou
         _l.F16 if out.dtype == torch.float16 else _l.F32, M, K, N, a2.stride(0), out.stride(0), epi, op, dptr,
         variant, _stream_ptr()))
     return out if a.dim() == 2 else out
+
+
+# ---- operators between the matmuls of a decode step ---------------------------------------------------
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == torch.float16:
+        return _l.F16
+    if t.dtype == torch.float32:
+        return _l.F32
+    raise _l.CutHipError(f"activations must be float16 or float32, got {t.dtype}")
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor | None = None,
+            out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """x: [rows, dim] or [dim]; weight: fp32 [dim] (RMSNormOpNode of the reference)."""
+    x2 = x if x.dim() == 2 else x.reshape(1, -1)
+    if weight.dtype != torch.float32 or weight.numel() != x2.shape[1] or x2.stride(1) != 1:
+        raise _l.CutHipError("rmsnorm: weight must be fp32 [dim] and x rows contiguous")
+    if out is None:
+        out = torch.empty(x2.shape, dtype=out_dtype or x.dtype, device=x.device)
+    _l.check(_l.load().cuthip_rmsnorm(x2.data_ptr(), _dt(x2), weight.data_ptr(), out.data_ptr(), _dt(out), x2.shape[0],
+                                      x2.shape[1], x2.stride(0), eps, _stream_ptr()))
+    return out
+
+
+def rope_kv_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, runtime_params: torch.Tensor, cos_t: torch.Tensor,
+                  sin_t: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, head_dim: int,
+                  q_out: torch.Tensor) -> torch.Tensor:
+    """q [q_dim], k, v [kv_dim] (same dtype); caches fp16 [max_ctx, aligned_kv_dim]; runtime_params int32/uint32[2] on device."""
+    if k_cache.dtype != torch.float16 or v_cache.dtype != torch.float16 or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise _l.CutHipError("rope_kv_write: caches must be fp16 and q, k, v of one dtype")
+    _l.check(_l.load().cuthip_rope_kv_write(q.data_ptr(), k.data_ptr(), v.data_ptr(), _dt(q), runtime_params.data_ptr(),
+                                            cos_t.data_ptr(), sin_t.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                            q_out.data_ptr(), _dt(q_out), q.numel(), k.numel(), head_dim, k_cache.stride(0),
+                                            _stream_ptr()))
+    return q_out
+
+
+def attn_decode_workspace(n_heads: int, head_dim: int, max_seq_len: int, device) -> torch.Tensor:
+    n = _l.load().cuthip_attn_decode_workspace_bytes(n_heads, head_dim, max_seq_len)
+    return torch.empty(n, dtype=torch.uint8, device=device)
+
+
+def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, runtime_params: torch.Tensor, n_heads: int,
+                n_kv_heads: int, head_dim: int, scale: float, workspace: torch.Tensor, out: torch.Tensor,
+                max_seq_len: int | None = None) -> torch.Tensor:
+    _l.check(_l.load().cuthip_attn_decode(q.data_ptr(), _dt(q), k_cache.data_ptr(), v_cache.data_ptr(),
+                                          runtime_params.data_ptr(), out.data_ptr(), _dt(out), n_heads, n_kv_heads, head_dim,
+                                          k_cache.stride(0), scale, max_seq_len or k_cache.shape[0], workspace.data_ptr(),
+                                          workspace.numel(), _stream_ptr()))
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _l.check(_l.load().cuthip_silu_mul(gate_up.data_ptr(), _dt(gate_up), out.data_ptr(), _dt(out), out.numel(), _stream_ptr()))
+    return out
+
+
+def argmax(x: torch.Tensor, out_index: torch.Tensor) -> torch.Tensor:
+    _l.check(_l.load().cuthip_argmax(x.data_ptr(), _dt(x), x.numel(), out_index.data_ptr(), _stream_ptr()))
+    return out_index

@@ -146,6 +146,46 @@ int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void 
                        uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D,
                        int variant, void *stream);
 
+/* ---- the operators between the matmuls of a decode step --------------------
+ * What the runner chains around the quantized matmuls for one token
+ * (interface/runner/llama/llama.cpp, runLayer / decode graph).  All take
+ * fp32 or fp16 activations (cuthip_dtype) and compute in fp32.
+ * runtime_params: device uint32[2] = {position of this token, sequence
+ * length including it}, the reference's runtimeParams buffer: read on the
+ * device so that a captured graph can be replayed for the next token. */
+
+/* out[r,c] = x[r,c] * rsqrt(mean_c(x[r,:]^2) + eps) * weight[c]
+ * (operators/impl/rmsnorm/RMSNorm.cu:15-37). stride: elements between rows. */
+int cuthip_rmsnorm(const void *x, int x_dtype, const float *weight, void *out, int out_dtype, uint32_t rows, uint32_t dim,
+                   uint32_t stride, float eps, void *stream);
+
+/* Half-split RoPE on q [q_dim] and k [kv_dim] with tables [pos][head_dim/2];
+ * k (rotated) and v are stored as fp16 to cache row `position`
+ * (rows of aligned_kv_dim elements); q (rotated) goes to q_out
+ * (operators/impl/attention/FusedRoPEKVWrite.cu:12-81). */
+int cuthip_rope_kv_write(const void *q, const void *k, const void *v, int in_dtype, const uint32_t *runtime_params,
+                         const float *cos_table, const float *sin_table, void *k_cache, void *v_cache, void *q_out,
+                         int q_out_dtype, uint32_t q_dim, uint32_t kv_dim, uint32_t head_dim, uint32_t aligned_kv_dim,
+                         void *stream);
+
+/* Scaled dot-product attention of one token over an fp16 KV cache with GQA:
+ * out[h,:] = softmax(scale * q[h,:] . K[0:seq, h/nRep, :]) . V[0:seq, h/nRep, :]
+ * (operators/impl/attention/Attention.cu:35-106; head_dim <= 128 as there).
+ * workspace: device scratch of cuthip_attn_decode_workspace_bytes(); the
+ * call allocates nothing.  max_seq_len sizes the launch (cache capacity). */
+size_t cuthip_attn_decode_workspace_bytes(uint32_t n_heads, uint32_t head_dim, uint32_t max_seq_len);
+int cuthip_attn_decode(const void *q, int q_dtype, const void *k_cache, const void *v_cache, const uint32_t *runtime_params,
+                       void *out, int out_dtype, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                       uint32_t aligned_kv_dim, float scale, uint32_t max_seq_len, void *workspace, size_t workspace_bytes,
+                       void *stream);
+
+/* out[i] = silu(gate_up[i]) * gate_up[n + i]: the SwiGLU combine after a fused
+ * gate+up matmul (llama.cpp:1832-1857: unary SiLU, then BinaryMul). */
+int cuthip_silu_mul(const void *gate_up, int in_dtype, void *out, int out_dtype, uint32_t n, void *stream);
+
+/* Index of the first maximum of x[0:n] (greedy sampling), written to device memory. */
+int cuthip_argmax(const void *x, int x_dtype, uint32_t n, uint32_t *out_index, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

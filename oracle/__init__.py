@@ -64,6 +64,10 @@ def _load():
         "orc_matmul_dense_f32": (None, [f32p, f32p, u32, u32, u32, f32p]),
         "orc_quantize_act_q8": (None, [f32p, sz, i8p, f32p]),
         "orc_quantize": (C.c_int, [C.c_int, f32p, sz, u8p]),
+        "orc_rmsnorm": (None, [f32p, f32p, u32, u32, C.c_float, f32p]),
+        "orc_rope_kv_write": (None, [f32p, f32p, f32p, u32, f32p, f32p, u32, u32, u32, u32, f32p, u16p, u16p]),
+        "orc_attention_decode": (None, [f32p, u16p, u16p, u32, u32, u32, u32, u32, C.c_float, f32p]),
+        "orc_silu_mul": (None, [f32p, u32, f32p]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -254,6 +258,43 @@ def quantize_act_q8(a):
 
 
 # ---- the reference's own reader (only where oracle/_ref was built) ----------
+
+def rmsnorm(x, weight, eps: float) -> np.ndarray:
+    x = _c(x, np.float32)
+    x2 = x.reshape(-1, x.shape[-1])
+    w = _c(weight, np.float32)
+    out = np.empty_like(x2)
+    _lib.orc_rmsnorm(_p(x2), _p(w), x2.shape[0], x2.shape[1], eps, _p(out))
+    return out.reshape(x.shape)
+
+
+def rope_kv_write(q, k, v, pos: int, cos_t, sin_t, head_dim: int, k_cache, v_cache) -> np.ndarray:
+    """Rotates q (returned) and k; writes k, v into row `pos` of the uint16 (fp16 bits) caches in place."""
+    q, k, v = _c(q, np.float32).reshape(-1), _c(k, np.float32).reshape(-1), _c(v, np.float32).reshape(-1)
+    cos_t, sin_t = _c(cos_t, np.float32), _c(sin_t, np.float32)
+    assert k_cache.dtype == np.uint16 and v_cache.dtype == np.uint16 and k_cache.flags.c_contiguous
+    q_out = np.empty_like(q)
+    _lib.orc_rope_kv_write(_p(q), _p(k), _p(v), pos, _p(cos_t), _p(sin_t), q.size, k.size, head_dim,
+                           k_cache.shape[1], _p(q_out), _p(k_cache), _p(v_cache))
+    return q_out
+
+
+def attention_decode(q, k_cache, v_cache, seq_len: int, n_heads: int, n_kv_heads: int, head_dim: int,
+                     scale: float) -> np.ndarray:
+    q = _c(q, np.float32).reshape(-1)
+    assert k_cache.dtype == np.uint16 and v_cache.dtype == np.uint16
+    out = np.empty(n_heads * head_dim, np.float32)
+    _lib.orc_attention_decode(_p(q), _p(k_cache), _p(v_cache), seq_len, n_heads, n_kv_heads, head_dim,
+                              k_cache.shape[1], scale, _p(out))
+    return out
+
+
+def silu_mul(gate_up) -> np.ndarray:
+    g = _c(gate_up, np.float32).reshape(-1)
+    out = np.empty(g.size // 2, np.float32)
+    _lib.orc_silu_mul(_p(g), g.size // 2, _p(out))
+    return out
+
 
 def have_ref() -> bool:
     return os.path.exists(_REF_PATH)

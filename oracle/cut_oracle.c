@@ -743,3 +743,97 @@ int orc_quantize(int fmt, const float *x, size_t n, uint8_t *blocks) {
   }
   return -1;
 }
+
+/* ---- operators between the matmuls of a decode step ------------------------ */
+
+/* operators/impl/rmsnorm/RMSNorm.cu:15-37 */
+void orc_rmsnorm(const float *x, const float *weight, uint32_t rows, uint32_t dim,
+                 float eps, float *out) {
+  for (uint32_t r = 0; r < rows; ++r) {
+    const float *xr = x + (size_t)r * dim;
+    double ss = 0.0; /* the kernel sums in fp32 over 256 strided lanes; double is the order-free anchor */
+    for (uint32_t i = 0; i < dim; ++i)
+      ss += (double)xr[i] * xr[i];
+    float scale = (float)(1.0 / sqrt(ss / dim + (double)eps));
+    for (uint32_t i = 0; i < dim; ++i)
+      out[(size_t)r * dim + i] = xr[i] * scale * weight[i];
+  }
+}
+
+/* fp32 -> fp16 bits, round to nearest even (what __float2half does; the KV
+ * cache store of AttentionCommon.cuh:17).  Built on the exact f16->f32 map. */
+static uint16_t f32_to_f16_rne(float v) {
+  uint16_t up = orc_f32_to_f16(v); /* round-half-away: differs from RNE only on exact ties */
+  uint32_t b;
+  memcpy(&b, &v, 4);
+  if ((b & 0x7F800000u) == 0x7F800000u)
+    return up;
+  uint16_t dn = (uint16_t)(up - 1);
+  float fu = orc_f16_to_f32(up), fd = orc_f16_to_f32(dn);
+  /* a tie: v is exactly halfway between dn and up (same sign) -> pick the even one */
+  if ((up & 0x7FFF) != 0 && (double)fu - (double)v == (double)v - (double)fd && (up & 1))
+    return dn;
+  return up;
+}
+
+/* operators/impl/attention/FusedRoPEKVWrite.cu:27-80 */
+void orc_rope_kv_write(const float *q, const float *k, const float *v, uint32_t pos,
+                       const float *cos_t, const float *sin_t, uint32_t q_dim,
+                       uint32_t kv_dim, uint32_t head_dim, uint32_t aligned_kv_dim,
+                       float *q_out, uint16_t *k_cache, uint16_t *v_cache) {
+  uint32_t half = head_dim / 2;
+  const float *c = cos_t + (size_t)pos * half, *s = sin_t + (size_t)pos * half;
+  for (uint32_t i = 0; i < q_dim; ++i) {
+    uint32_t d = i % head_dim;
+    q_out[i] = d < half ? q[i] * c[d] - q[i + half] * s[d]
+                        : q[i - half] * s[d - half] + q[i] * c[d - half];
+  }
+  for (uint32_t i = 0; i < kv_dim; ++i) {
+    uint32_t d = i % head_dim;
+    float r = d < half ? k[i] * c[d] - k[i + half] * s[d]
+                       : k[i - half] * s[d - half] + k[i] * c[d - half];
+    k_cache[(size_t)pos * aligned_kv_dim + i] = f32_to_f16_rne(r);
+    v_cache[(size_t)pos * aligned_kv_dim + i] = f32_to_f16_rne(v[i]);
+  }
+}
+
+/* operators/impl/attention/Attention.cu:35-106 */
+void orc_attention_decode(const float *q, const uint16_t *k_cache, const uint16_t *v_cache,
+                          uint32_t seq_len, uint32_t n_heads, uint32_t n_kv_heads,
+                          uint32_t head_dim, uint32_t aligned_kv_dim, float scale, float *out) {
+  uint32_t n_rep = n_heads / n_kv_heads;
+  double *sc = (double *)malloc(sizeof(double) * (seq_len ? seq_len : 1));
+  for (uint32_t h = 0; h < n_heads; ++h) {
+    uint32_t kvh = h / n_rep;
+    double mx = -1e300;
+    for (uint32_t t = 0; t < seq_len; ++t) {
+      double dot = 0.0;
+      for (uint32_t d = 0; d < head_dim; ++d)
+        dot += (double)q[(size_t)h * head_dim + d] *
+               orc_f16_to_f32(k_cache[(size_t)t * aligned_kv_dim + kvh * head_dim + d]);
+      sc[t] = dot * scale;
+      if (sc[t] > mx)
+        mx = sc[t];
+    }
+    double sum = 0.0;
+    for (uint32_t t = 0; t < seq_len; ++t) {
+      sc[t] = exp(sc[t] - mx);
+      sum += sc[t];
+    }
+    for (uint32_t d = 0; d < head_dim; ++d) {
+      double acc = 0.0;
+      for (uint32_t t = 0; t < seq_len; ++t)
+        acc += sc[t] / sum * orc_f16_to_f32(v_cache[(size_t)t * aligned_kv_dim + kvh * head_dim + d]);
+      out[(size_t)h * head_dim + d] = (float)acc;
+    }
+  }
+  free(sc);
+}
+
+/* interface/runner/llama/llama.cpp:1832-1857 (unary SiLU then BinaryMul) */
+void orc_silu_mul(const float *gate_up, uint32_t n, float *out) {
+  for (uint32_t i = 0; i < n; ++i) {
+    float g = gate_up[i];
+    out[i] = (float)(g / (1.0 + exp(-(double)g))) * gate_up[(size_t)n + i];
+  }
+}

@@ -117,6 +117,25 @@ void orc_quantize_q4_k(const float *x, size_t n, uint8_t *blocks);
 void orc_quantize_q6_k(const float *x, size_t n, uint8_t *blocks);
 int orc_quantize(int fmt, const float *x, size_t n, uint8_t *blocks);
 
+/* ---- operators between the matmuls of a decode step (fp32, as the reference kernels compute) ---- */
+/* RMSNorm.cu:15-37: out = x * rsqrt(sum(x^2)/dim + eps) * weight, per row */
+void orc_rmsnorm(const float *x, const float *weight, uint32_t rows, uint32_t dim,
+                 float eps, float *out);
+/* FusedRoPEKVWrite.cu:27-80: half-split rotation of q and k at `pos` with
+ * tables [pos][head_dim/2]; k (rotated) and v go to cache row pos as fp16 bits
+ * (host narrowing = round to nearest even here, as __float2half). */
+void orc_rope_kv_write(const float *q, const float *k, const float *v, uint32_t pos,
+                       const float *cos_t, const float *sin_t, uint32_t q_dim,
+                       uint32_t kv_dim, uint32_t head_dim, uint32_t aligned_kv_dim,
+                       float *q_out, uint16_t *k_cache, uint16_t *v_cache);
+/* Attention.cu:35-106: per head, scores = scale * q.K over seq_len cache rows,
+ * softmax, weighted sum of V; GQA: kv head = h / (n_heads / n_kv_heads) */
+void orc_attention_decode(const float *q, const uint16_t *k_cache, const uint16_t *v_cache,
+                          uint32_t seq_len, uint32_t n_heads, uint32_t n_kv_heads,
+                          uint32_t head_dim, uint32_t aligned_kv_dim, float scale, float *out);
+/* llama.cpp:1832-1857: silu(gate) * up on a fused [gate | up] vector */
+void orc_silu_mul(const float *gate_up, uint32_t n, float *out);
+
 #ifdef __cplusplus
 }
 #endif

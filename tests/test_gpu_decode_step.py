@@ -1,0 +1,183 @@
+"""GPU parity of the operators between the matmuls of a decode step (RMSNorm,
+RoPE + KV write, GQA decode attention, SiLU * up, arg-max) through the C ABI
+against the CPU oracle, and of a whole small decode step (two layers + head)
+against the same chain composed from oracle calls.  Floating point: each
+assert states its tolerance; the KV cache write is bit-exact."""
+import math
+
+import numpy as np
+import pytest
+
+import oracle
+from helpers import normwise_rel_err
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from cut_amd import lib, ops as _ops
+    lib.check(lib.load().cuthip_init(0))
+    return _ops
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("rows,dim", [(1, 4096), (3, 1000), (2, 64)])
+def test_rmsnorm(ops, dtype, rows, dim):
+    rng = np.random.default_rng(rows * dim)
+    x = rng.standard_normal((rows, dim)).astype(dtype)
+    w = rng.uniform(0.5, 1.5, dim).astype(np.float32)
+    got = ops.rmsnorm(dev(x), dev(w), 1e-5, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    want = oracle.rmsnorm(x.astype(np.float32), w, 1e-5)
+    np.testing.assert_allclose(got.cpu().numpy(), want, rtol=2e-6, atol=1e-7)
+    got16 = ops.rmsnorm(dev(x), dev(w), 1e-5, out_dtype=torch.float16)
+    assert normwise_rel_err(got16.float().cpu().numpy(), want) < 4e-4   # one fp16 rounding of the output
+
+
+def _tables(max_pos, head_dim, theta=500000.0):
+    half = head_dim // 2
+    inv = 1.0 / theta ** (np.arange(half, dtype=np.float64) * 2 / head_dim)
+    ang = np.arange(max_pos, dtype=np.float64)[:, None] * inv[None]
+    return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd,pos", [(32, 8, 128, 2047), (8, 2, 64, 3), (4, 4, 16, 0)])
+def test_rope_kv_write(ops, n_heads, n_kv, hd, pos):
+    max_ctx = pos + 2
+    rng = np.random.default_rng(pos + hd)
+    q = rng.standard_normal(n_heads * hd).astype(np.float32)
+    k = rng.standard_normal(n_kv * hd).astype(np.float32)
+    v = rng.standard_normal(n_kv * hd).astype(np.float32)
+    cos_t, sin_t = _tables(max_ctx, hd)
+    kc = np.zeros((max_ctx, n_kv * hd), np.uint16)
+    vc = np.zeros((max_ctx, n_kv * hd), np.uint16)
+    want_q = oracle.rope_kv_write(q, k, v, pos, cos_t, sin_t, hd, kc, vc)
+    kcd = torch.zeros((max_ctx, n_kv * hd), dtype=torch.float16, device="cuda")
+    vcd = torch.zeros_like(kcd)
+    params = dev(np.array([pos, pos + 1], np.int32))
+    q_out = torch.empty(n_heads * hd, dtype=torch.float32, device="cuda")
+    ops.rope_kv_write(dev(q), dev(k), dev(v), params, dev(cos_t), dev(sin_t), kcd, vcd, hd, q_out)
+    torch.cuda.synchronize()
+    # same fp32 expression: the rotated q may differ by fma contraction only
+    np.testing.assert_allclose(q_out.cpu().numpy(), want_q, rtol=1e-6, atol=1e-6)
+    got_k = kcd.cpu().numpy().view(np.uint16)
+    assert np.array_equal(vcd.cpu().numpy().view(np.uint16), vc)          # v: bit-exact fp16 store
+    assert np.max(np.abs(got_k.astype(np.int32) - kc.astype(np.int32))) <= 1   # k: at most one fp16 ulp (fma contraction)
+    assert not got_k[:pos].any() and not got_k[pos + 1:].any()
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd,seq,max_ctx", [(32, 8, 128, 2048, 2048), (32, 8, 128, 1, 2048), (8, 2, 64, 77, 128),
+                                                       (6, 1, 128, 130, 256), (4, 4, 16, 64, 64)])
+def test_attention_decode(ops, n_heads, n_kv, hd, seq, max_ctx):
+    rng = np.random.default_rng(seq)
+    q = rng.standard_normal(n_heads * hd).astype(np.float32)
+    K = (rng.standard_normal((max_ctx, n_kv * hd)) * 0.5).astype(np.float16)
+    V = rng.standard_normal((max_ctx, n_kv * hd)).astype(np.float16)
+    scale = 1 / math.sqrt(hd)
+    want = oracle.attention_decode(q, K.view(np.uint16), V.view(np.uint16), seq, n_heads, n_kv, hd, scale)
+    ws = ops.attn_decode_workspace(n_heads, hd, max_ctx, "cuda")
+    params = dev(np.array([seq - 1, seq], np.int32))
+    for out_dtype, tol in ((torch.float32, 2e-6), (torch.float16, 4e-4)):
+        out = torch.empty(n_heads * hd, dtype=out_dtype, device="cuda")
+        ops.attn_decode(dev(q), dev(K), dev(V), params, n_heads, n_kv, hd, scale, ws, out)
+        torch.cuda.synchronize()
+        assert normwise_rel_err(out.float().cpu().numpy(), want) < tol
+    # rows past seq_len must not matter: poison them
+    K2, V2 = K.copy(), V.copy()
+    K2[seq:] = np.float16(60000.0)
+    V2[seq:] = np.float16(np.nan)
+    out = torch.empty(n_heads * hd, dtype=torch.float32, device="cuda")
+    ops.attn_decode(dev(q), dev(K2), dev(V2), params, n_heads, n_kv, hd, scale, ws, out)
+    torch.cuda.synchronize()
+    assert normwise_rel_err(out.cpu().numpy(), want) < 2e-6
+
+
+def test_silu_mul_and_argmax(ops):
+    rng = np.random.default_rng(5)
+    gu = (rng.standard_normal(2 * 14336) * 3).astype(np.float16)
+    out = torch.empty(14336, dtype=torch.float32, device="cuda")
+    ops.silu_mul(dev(gu), out)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(out.cpu().numpy(), oracle.silu_mul(gu.astype(np.float32)), rtol=2e-6, atol=1e-7)
+    logits = rng.standard_normal(128256).astype(np.float32)
+    logits[[77, 90001]] = 9.5    # a tie: the first index wins
+    idx = torch.zeros(1, dtype=torch.int32, device="cuda")
+    ops.argmax(dev(logits), idx)
+    torch.cuda.synchronize()
+    assert int(idx.item()) == 77
+    ops.argmax(dev(logits.astype(np.float16)[:1000]), idx)
+    torch.cuda.synchronize()
+    assert int(idx.item()) == int(np.argmax(logits.astype(np.float16)[:1000]))
+
+
+def _oracle_step(cfg, layers_h, out_norm, head, x, pos, kc, vc, cos_t, sin_t):
+    """The same chain from oracle calls; activations rounded to fp16 where the GPU chain stores fp16."""
+    f16 = lambda a: a.astype(np.float16).astype(np.float32)
+    for i, L in enumerate(layers_h):
+        xn = f16(oracle.rmsnorm(x, L["attn_norm"], cfg.eps))
+        qk = oracle.matmul_gguf(oracle.Q4_K, L["qk"], xn[None], cfg.q_dim + cfg.kv_dim, f64=True)[0].astype(np.float32)
+        v = oracle.matmul_gguf(oracle.Q6_K, L["v"], xn[None], cfg.kv_dim, f64=True)[0].astype(np.float32)
+        q_rot = oracle.rope_kv_write(qk[:cfg.q_dim], qk[cfg.q_dim:], v, pos, cos_t, sin_t, cfg.head_dim, kc[i], vc[i])
+        attn = f16(oracle.attention_decode(q_rot, kc[i], vc[i], pos + 1, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim,
+                                           1 / math.sqrt(cfg.head_dim)))
+        x = x + oracle.matmul_gguf(oracle.Q4_K, L["o"], attn[None], cfg.hidden, f64=True)[0].astype(np.float32)
+        hn = f16(oracle.rmsnorm(x, L["ffn_norm"], cfg.eps))
+        gu = f16(oracle.matmul_gguf(oracle.Q4_K, L["gate_up"], hn[None], 2 * cfg.ffn, f64=True)[0].astype(np.float32))
+        act = f16(oracle.silu_mul(gu))
+        x = x + oracle.matmul_gguf(oracle.Q4_K, L["down"], act[None], cfg.hidden, f64=True)[0].astype(np.float32)
+    xn = f16(oracle.rmsnorm(x, out_norm, cfg.eps))
+    return oracle.matmul_gguf(oracle.Q6_K, head, xn[None], cfg.vocab, f64=True)[0].astype(np.float32)
+
+
+def test_small_decode_step_against_oracle_chain(ops):
+    from cut_amd.decode import DecodeConfig, DecodeStep
+    cfg = DecodeConfig(hidden=512, n_layers=2, n_heads=8, n_kv_heads=2, head_dim=64, ffn=1024, vocab=2048, max_ctx=64)
+    rng = np.random.default_rng(11)
+
+    def qw(fmt, n, k):
+        return oracle.quantize(fmt, (rng.standard_normal(n * k) * 0.05).astype(np.float32))
+    layers_h = [{"qk": qw(oracle.Q4_K, cfg.q_dim + cfg.kv_dim, cfg.hidden), "v": qw(oracle.Q6_K, cfg.kv_dim, cfg.hidden),
+                 "o": qw(oracle.Q4_K, cfg.hidden, cfg.q_dim), "gate_up": qw(oracle.Q4_K, 2 * cfg.ffn, cfg.hidden),
+                 "down": qw(oracle.Q4_K, cfg.hidden, cfg.ffn),
+                 "attn_norm": rng.uniform(0.5, 1.5, cfg.hidden).astype(np.float32),
+                 "ffn_norm": rng.uniform(0.5, 1.5, cfg.hidden).astype(np.float32)} for _ in range(cfg.n_layers)]
+    out_norm = rng.uniform(0.5, 1.5, cfg.hidden).astype(np.float32)
+    head = qw(oracle.Q6_K, cfg.vocab, cfg.hidden)
+    step = DecodeStep(cfg, [{k: dev(v) for k, v in L.items()} for L in layers_h], dev(out_norm), dev(head))
+    # a context of 9 earlier tokens already in the caches (same bits on both sides), then token 9
+    pos = 9
+    kc = [np.zeros((cfg.max_ctx, cfg.kv_dim), np.uint16) for _ in range(cfg.n_layers)]
+    vc = [np.zeros((cfg.max_ctx, cfg.kv_dim), np.uint16) for _ in range(cfg.n_layers)]
+    for i in range(cfg.n_layers):
+        kc[i][:pos] = (rng.standard_normal((pos, cfg.kv_dim)) * 0.5).astype(np.float16).view(np.uint16)
+        vc[i][:pos] = rng.standard_normal((pos, cfg.kv_dim)).astype(np.float16).view(np.uint16)
+        step.k_cache[i].copy_(dev(kc[i].view(np.float16)))
+        step.v_cache[i].copy_(dev(vc[i].view(np.float16)))
+    x = rng.standard_normal(cfg.hidden).astype(np.float32)
+    cos_t, sin_t = step.cos_t.cpu().numpy(), step.sin_t.cpu().numpy()
+    want = _oracle_step(cfg, layers_h, out_norm, head, x.copy(), pos, kc, vc, cos_t, sin_t)
+
+    step.x.copy_(dev(x))
+    step.set_position(pos)
+    step.step()
+    torch.cuda.synchronize()
+    got = step.logits.cpu().numpy()
+    assert normwise_rel_err(got, want) < 1e-3
+    assert int(step.token.item()) == int(np.argmax(got))
+    # the step captured in a HIP graph and replayed twice (with eager work in between) gives the eager result
+    step.x.copy_(dev(x))
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step.step()
+    for _ in range(2):
+        step.x.copy_(dev(x))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(step.logits.cpu().numpy(), got)
