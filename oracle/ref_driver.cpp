@@ -113,4 +113,37 @@ int ref_split_q4(const uint8_t *data, size_t nbytes, uint64_t rows,
   unlink(path.c_str());
   return rc;
 }
+
+// Opens `path` with the reference reader and copies the raw bytes of tensor
+// `name` to out (cap bytes).  Returns the tensor's byte size, or -1.
+// dims_out (if not null) receives up to 4 dimensions, innermost first; type_out the GGML type.
+long ref_read_raw(const char *path, const char *name, uint8_t *out, size_t cap,
+                  uint64_t *dims_out, uint32_t *type_out) {
+  try {
+    gguf::GGUFReader reader(path);
+    std::vector<uint8_t> raw = reader.read_tensor_raw(name);
+    if (raw.size() > cap)
+      return -1;
+    memcpy(out, raw.data(), raw.size());
+    const auto &info = reader.tensors().at(name);
+    if (dims_out)
+      for (size_t i = 0; i < info.dimensions.size() && i < 4; ++i)
+        dims_out[i] = info.dimensions[i];
+    if (type_out)
+      *type_out = static_cast<uint32_t>(info.type);
+    return (long)raw.size();
+  } catch (...) {
+    return -1;
+  }
+}
+
+// A uint32 metadata value read by the reference reader (0xFFFFFFFF if absent or of another type).
+uint32_t ref_meta_u32(const char *path, const char *key) {
+  try {
+    gguf::GGUFReader reader(path);
+    return reader.metadata().get_as<uint32_t>(key, 0xFFFFFFFFu);
+  } catch (...) {
+    return 0xFFFFFFFFu;
+  }
+}
 }

@@ -48,3 +48,39 @@ def normwise_rel_err(got, ref) -> float:
     got = np.asarray(got, np.float64).reshape(-1)
     ref = np.asarray(ref, np.float64).reshape(-1)
     return float(np.linalg.norm(got - ref) / max(np.linalg.norm(ref), 1e-300))
+
+
+def write_gguf(path, metadata: dict, tensors: list, alignment: int = 32, version: int = 3):
+    """Minimal GGUF writer for tests (the reference ships none): metadata values are (type_code, value) pairs
+    with type codes of gguf_types.hpp:56-70; tensors are (name, dims_innermost_first, ggml_type, bytes)."""
+    import struct
+
+    def s(b):
+        b = b.encode() if isinstance(b, str) else b
+        return struct.pack("<Q", len(b)) + b
+    fmt = {0: "B", 1: "b", 2: "H", 3: "h", 4: "I", 5: "i", 6: "f", 7: "?", 10: "Q", 11: "q", 12: "d"}
+
+    def val(t, v):
+        if t in fmt:
+            return struct.pack("<" + fmt[t], v)
+        if t == 8:
+            return s(v)
+        et, items = v   # array: (element type, list)
+        return struct.pack("<IQ", et, len(items)) + b"".join(val(et, x) for x in items)
+    out = struct.pack("<IIQQ", 0x46554747, version, len(tensors), len(metadata))
+    for k, (t, v) in metadata.items():
+        out += s(k) + struct.pack("<I", t) + val(t, v)
+    offset, blobs = 0, []
+    for name, dims, gt, data in tensors:
+        data = bytes(data)
+        out += s(name) + struct.pack("<I", len(dims)) + b"".join(struct.pack("<Q", d) for d in dims)
+        out += struct.pack("<IQ", gt, offset)
+        blobs.append((offset, data))
+        offset = (offset + len(data) + alignment - 1) // alignment * alignment
+    pad = (len(out) + alignment - 1) // alignment * alignment - len(out)
+    out += b"\0" * pad
+    body = bytearray(offset)
+    for off, data in blobs:
+        body[off:off + len(data)] = data
+    with open(path, "wb") as f:
+        f.write(out + bytes(body))
