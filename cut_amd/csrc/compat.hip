@@ -1,0 +1,258 @@
+// Quantized matmul on the reference's own ("separated") weight layout, for
+// callers that keep the tensors the reference's loader produced:
+//   Q8: values int8 [K, strideB] (row k holds the N columns), scales fp16 [K/32, scaleStride]
+//   Q4: nibbles [K, strideB bytes], even column in the low nibble, value nibble - 8;
+//       scales fp16 [K/32, scaleStride]; affine: per-block minima appended as rows
+//       [K/32 .. 2K/32) of the scale tensor, value (nibble - 8) * scale + min
+//   C[m,n] = sum_k A[m,k] * w[k,n]          (MatMulQ8Common.cuh / MatMulQ4Common.cuh:126-153)
+// A, C, D are fp32 as in the reference.
+//
+// The layout is column-major in n, so a wave streams whole k-rows: each lane
+// owns 16 consecutive columns (one 16-byte load of int8, or 8 bytes of
+// nibbles), a wave 1024 columns, and the k range is split over the four waves
+// of a workgroup and over workgroups (grid.y).  Per 32-row block a lane
+// accumulates sum(x * q) per column and applies the block's scale once; the
+// "- 8" and the affine minimum become multiples of the block's sum(x).  The
+// waves of a workgroup are reduced through LDS; if the k range is split over
+// several workgroups the partial sums go to a caller-provided workspace and a
+// second kernel adds them and applies the epilogue.
+#include <cstdint>
+
+#include "common.hpp"
+
+namespace cuthip {
+
+constexpr int kSepCols = 16;            // columns per lane
+constexpr int kSepTile = 64 * kSepCols; // columns per wave
+constexpr int kSepKC = 32;              // k-rows per wave (one quantization block)
+constexpr int kSepWaves = 4;
+
+struct SepParams {
+  const float *A;
+  const uint8_t *B;
+  const uint16_t *S;
+  float *C;         // output, or the workspace [nsplit][M][N] when nsplit > 1
+  Epilogue epi;
+  uint32_t M, K, N, strideA, strideB, strideC, scaleStride;
+  uint32_t m0;      // first row of A handled by this launch
+  uint32_t nsplit;
+  int affine;
+};
+
+template <bool Q4, int MT>
+__global__ void __launch_bounds__(64 * kSepWaves, 2) sep_gemv_kernel(SepParams p) {
+  __shared__ float xs[MT][kSepWaves * kSepKC];
+  __shared__ float red[MT][kSepTile];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t c0 = blockIdx.x * kSepTile + lane * kSepCols;
+  const uint32_t kwg = blockIdx.y * (kSepWaves * kSepKC);   // first k-row of this workgroup
+  const uint32_t k0 = kwg + wave * kSepKC;                  // this wave's block
+  const uint32_t blocksK = p.K / 32;
+
+  // activations of the workgroup's k range
+  for (int i = tid; i < MT * kSepWaves * kSepKC; i += 64 * kSepWaves) {
+    int m = i / (kSepWaves * kSepKC), kk = i % (kSepWaves * kSepKC);
+    uint32_t row = p.m0 + m, k = kwg + kk;
+    xs[m][kk] = (row < p.M && k < p.K) ? p.A[(size_t)row * p.strideA + k] : 0.0f;
+  }
+  __syncthreads();
+
+  // a wave handles exactly one quantization block of k, so the per-block sums become the result in place
+  float bs[MT][kSepCols], sx[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    sx[m] = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kSepCols; ++c) bs[m][c] = 0.0f;
+  }
+
+  const uint32_t ncols = c0 < p.N ? min((uint32_t)kSepCols, p.N - c0) : 0u;
+  if (k0 < p.K && ncols) {
+    const float *xw = &xs[0][wave * kSepKC];
+    for (int kk = 0; kk < kSepKC; ++kk) {
+      float q[kSepCols];
+      if (Q4) {
+        const uint8_t *src = p.B + (size_t)(k0 + kk) * p.strideB + c0 / 2;
+        uint32_t w0, w1;
+        if (ncols == kSepCols) {
+          u32x2 w = ld_u32x2(src);
+          w0 = w.x;
+          w1 = w.y;
+        } else {   // last lane of a ragged row: byte loads inside the row
+          w0 = w1 = 0;
+          for (uint32_t b = 0; b < (ncols + 1) / 2; ++b) {
+            uint32_t v = src[b];
+            if (b < 4) w0 |= v << (8 * b);
+            else w1 |= v << (8 * (b - 4));
+          }
+        }
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          q[c] = (float)((w0 >> (4 * c)) & 0xF);
+          q[8 + c] = (float)((w1 >> (4 * c)) & 0xF);
+        }
+      } else {
+        const uint8_t *src = p.B + (size_t)(k0 + kk) * p.strideB + c0;
+        u32x4 w;
+        if (ncols == kSepCols) {
+          w = ld_u32x4(src);
+        } else {
+          w = u32x4{0, 0, 0, 0};
+          for (uint32_t b = 0; b < ncols; ++b) w[b >> 2] |= (uint32_t)src[b] << (8 * (b & 3));
+        }
+#pragma unroll
+        for (int c = 0; c < kSepCols; ++c) q[c] = (float)(int)(int8_t)((w[c >> 2] >> (8 * (c & 3))) & 0xFF);
+      }
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        float x = xw[m * (kSepWaves * kSepKC) + kk];
+        sx[m] += x;
+#pragma unroll
+        for (int c = 0; c < kSepCols; ++c) bs[m][c] = fmaf(x, q[c], bs[m][c]);
+      }
+    }
+    // the block's scales (and minima): fp16 [k/32][scaleStride]
+    const uint32_t blk = k0 / 32;
+#pragma unroll
+    for (int c = 0; c < kSepCols; ++c) {
+      if ((uint32_t)c < ncols) {
+        float s = f16bits_to_f32(p.S[(size_t)blk * p.scaleStride + c0 + c]);
+        float mn = (Q4 && p.affine) ? f16bits_to_f32(p.S[(size_t)(blocksK + blk) * p.scaleStride + c0 + c]) : 0.0f;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          float v = Q4 ? fmaf(-8.0f, sx[m], bs[m][c]) : bs[m][c];
+          bs[m][c] = fmaf(v, s, mn * sx[m]);
+        }
+      }
+    }
+  }
+
+  // fold the four waves (k blocks) of the workgroup into wave 0, one wave at a time through LDS
+  for (int w = 1; w < kSepWaves; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int c = 0; c < kSepCols; ++c) red[m][lane * kSepCols + c] = bs[m][c];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int c = 0; c < kSepCols; ++c) bs[m][c] += red[m][lane * kSepCols + c];
+    }
+    __syncthreads();
+  }
+  if (wave == 0 && ncols) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const uint32_t row = p.m0 + m;
+#pragma unroll
+      for (int c = 0; c < kSepCols; ++c) {
+        if (row < p.M && (uint32_t)c < ncols) {
+          if (p.nsplit == 1)
+            store_out(p.C, p.epi, 0, (size_t)row * p.strideC + c0 + c, bs[m][c]);
+          else
+            p.C[((size_t)blockIdx.y * p.M + row) * p.N + c0 + c] = bs[m][c];   // workspace [split][M][N]
+        }
+      }
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256) sep_reduce_kernel(const float *ws, float *C, Epilogue epi, uint32_t M, uint32_t N,
+                                                         uint32_t strideC, uint32_t m0, uint32_t mcount, uint32_t nsplit) {
+  uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= mcount * N) return;
+  uint32_t row = m0 + i / N, n = i % N;
+  float v = 0.0f;
+  for (uint32_t s = 0; s < nsplit; ++s) v += ws[((size_t)s * M + row) * N + n];
+  store_out(C, epi, 0, (size_t)row * strideC + n, v);
+}
+
+template <bool Q4, int MT> static int launch_sep(SepParams p, uint32_t mcount, float *C, void *workspace, hipStream_t stream) {
+  dim3 grid((p.N + kSepTile - 1) / kSepTile, p.nsplit);
+  float *out = p.nsplit == 1 ? C : reinterpret_cast<float *>(workspace);
+  p.C = out;
+  hipLaunchKernelGGL((sep_gemv_kernel<Q4, MT>), grid, dim3(64 * kSepWaves), 0, stream, p);
+  if (int rc = check_hip(hipGetLastError(), "separated-layout matmul launch")) return rc;
+  if (p.nsplit > 1) {
+    hipLaunchKernelGGL(sep_reduce_kernel, dim3((mcount * p.N + 255) / 256), dim3(256), 0, stream,
+                       reinterpret_cast<const float *>(workspace), C, p.epi, p.M, p.N, p.strideC, p.m0, mcount, p.nsplit);
+    return check_hip(hipGetLastError(), "separated-layout reduce launch");
+  }
+  return CUTHIP_OK;
+}
+
+static int matmul_sep(bool q4, const float *A, const void *B, const void *S, const float *D, float *C, uint32_t M, uint32_t K,
+                      uint32_t N, uint32_t strideA, uint32_t strideB, uint32_t strideC, uint32_t scaleStride, int epilogue,
+                      int epilogue_op, int affine, void *workspace, size_t workspace_bytes, hipStream_t stream) {
+  const char *who = q4 ? "cuthip_matmul_q4_sep" : "cuthip_matmul_q8_sep";
+  if (!A || !B || !S || !C || M == 0 || K == 0 || N == 0 || K % 32 || strideA < K || strideC < N || scaleStride < N ||
+      strideB < (q4 ? (N + 1) / 2 : N) || (q4 && (N & 1))) {
+    set_error("%s: bad argument (M %u, K %u (multiple of 32), N %u%s, strides %u %u %u %u)", who, M, K, N,
+              q4 ? " (even)" : "", strideA, strideB, strideC, scaleStride);
+    return CUTHIP_ERR_INVALID;
+  }
+  if (epilogue < CUTHIP_EPI_NONE || epilogue > CUTHIP_EPI_BINARY || (epilogue == CUTHIP_EPI_BINARY && !D)) {
+    set_error("%s: bad epilogue %d (a binary epilogue needs D)", who, epilogue);
+    return CUTHIP_ERR_INVALID;
+  }
+  SepParams p;
+  p.A = A;
+  p.B = reinterpret_cast<const uint8_t *>(B);
+  p.S = reinterpret_cast<const uint16_t *>(S);
+  p.C = C;
+  p.epi = Epilogue{epilogue, epilogue_op, D};
+  p.M = M; p.K = K; p.N = N; p.strideA = strideA; p.strideB = strideB; p.strideC = strideC; p.scaleStride = scaleStride;
+  p.affine = affine;
+  p.nsplit = (K + kSepWaves * kSepKC - 1) / (kSepWaves * kSepKC);
+  if (p.nsplit > 1 && (!workspace || workspace_bytes < (size_t)p.nsplit * M * N * sizeof(float))) {
+    set_error("%s: workspace of %zu bytes, need %zu", who, workspace_bytes, (size_t)p.nsplit * M * N * sizeof(float));
+    return CUTHIP_ERR_INVALID;
+  }
+  // passes of up to 4 rows of A (each pass streams the weights once; 8 rows would spill registers)
+  for (uint32_t m0 = 0; m0 < M; m0 += 4) {
+    uint32_t mc = min(4u, M - m0);
+    p.m0 = m0;
+    int rc;
+    if (q4) {
+      rc = mc == 1 ? launch_sep<true, 1>(p, mc, C, workspace, stream) : mc == 2 ? launch_sep<true, 2>(p, mc, C, workspace, stream)
+                                                                                 : launch_sep<true, 4>(p, mc, C, workspace, stream);
+    } else {
+      rc = mc == 1 ? launch_sep<false, 1>(p, mc, C, workspace, stream) : mc == 2 ? launch_sep<false, 2>(p, mc, C, workspace, stream)
+                                                                                  : launch_sep<false, 4>(p, mc, C, workspace, stream);
+    }
+    if (rc) return rc;
+  }
+  return CUTHIP_OK;
+}
+
+}  // namespace cuthip
+
+using namespace cuthip;
+
+extern "C" {
+
+size_t cuthip_matmul_sep_workspace_bytes(uint32_t M, uint32_t K, uint32_t N) {
+  size_t nsplit = (K + kSepWaves * kSepKC - 1) / (kSepWaves * kSepKC);
+  return nsplit > 1 ? nsplit * M * N * sizeof(float) : 0;
+}
+
+int cuthip_matmul_q8_sep(const float *A, const int8_t *B, const uint16_t *scales, const float *D, float *C, uint32_t M,
+                         uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideB, uint32_t strideC, uint32_t scaleStride,
+                         int epilogue, int epilogue_op, void *workspace, size_t workspace_bytes, void *stream) {
+  return matmul_sep(false, A, B, scales, D, C, M, K, N, strideA, strideB, strideC, scaleStride, epilogue, epilogue_op, 0,
+                    workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int cuthip_matmul_q4_sep(const float *A, const uint8_t *packedB, const uint16_t *scales, const float *D, float *C, uint32_t M,
+                         uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideBNpacked, uint32_t strideC,
+                         uint32_t scaleStride, int epilogue, int epilogue_op, int affine, void *workspace,
+                         size_t workspace_bytes, void *stream) {
+  return matmul_sep(true, A, packedB, scales, D, C, M, K, N, strideA, strideBNpacked, strideC, scaleStride, epilogue,
+                    epilogue_op, affine, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+}  // extern "C"

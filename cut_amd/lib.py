@@ -32,6 +32,7 @@ EXPORTS = [
     "cuthip_dequant", "cuthip_matmul_gguf",
     "cuthip_rmsnorm", "cuthip_rope_kv_write", "cuthip_attn_decode_workspace_bytes", "cuthip_attn_decode",
     "cuthip_silu_mul", "cuthip_argmax",
+    "cuthip_matmul_sep_workspace_bytes", "cuthip_matmul_q8_sep", "cuthip_matmul_q4_sep",
 ]
 
 
@@ -94,10 +95,15 @@ def load() -> C.CDLL:
     lib.cuthip_attn_decode.argtypes = [vp, i, vp, vp, vp, vp, i, u32, u32, u32, u32, f32, u32, vp, C.c_size_t, vp]
     lib.cuthip_silu_mul.argtypes = [vp, i, vp, i, u32, vp]
     lib.cuthip_argmax.argtypes = [vp, i, u32, vp, vp]
+    lib.cuthip_matmul_sep_workspace_bytes.argtypes = [u32, u32, u32]
+    lib.cuthip_matmul_q8_sep.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, u32, i, i, vp, C.c_size_t, vp]
+    lib.cuthip_matmul_q4_sep.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, u32, i, i, i, vp, C.c_size_t, vp]
+    sized = ("cuthip_attn_decode_workspace_bytes", "cuthip_matmul_sep_workspace_bytes")
     for n in EXPORTS:
-        if n not in ("cuthip_last_error", "cuthip_attn_decode_workspace_bytes"):
+        if n != "cuthip_last_error" and n not in sized:
             getattr(lib, n).restype = i
-    lib.cuthip_attn_decode_workspace_bytes.restype = C.c_size_t
+    for n in sized:
+        getattr(lib, n).restype = C.c_size_t
     _lib = lib
     return lib
 

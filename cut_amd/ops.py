@@ -147,3 +147,37 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
 def argmax(x: torch.Tensor, out_index: torch.Tensor) -> torch.Tensor:
     _l.check(_l.load().cuthip_argmax(x.data_ptr(), _dt(x), x.numel(), out_index.data_ptr(), _stream_ptr()))
     return out_index
+
+
+# ---- the reference's separated weight layout ----------------------------------------------------------
+def matmul_sep(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, N: int, q4: bool = False, affine: bool = False,
+               out: torch.Tensor | None = None, unary: str | None = None, binary: str | None = None,
+               d: torch.Tensor | None = None) -> torch.Tensor:
+    """Operations::matmul(a, packedB, scalesB) of the reference on its own layout: a fp32 [M, K]; b int8 [K, N]
+    (q4: uint8 [K, N/2], even column in the low nibble); scales fp16 [K/32, N] ([2K/32, N] when affine)."""
+    a2 = a if a.dim() == 2 else a.reshape(1, -1)
+    M, K = a2.shape
+    if a2.dtype != torch.float32 or scales.dtype != torch.float16 or b.element_size() != 1 or b.dim() != 2 or scales.dim() != 2:
+        raise _l.CutHipError("matmul_sep: a must be fp32, b a 2-D 1-byte tensor and scales a 2-D fp16 tensor")
+    rows_s = (2 if affine else 1) * (K // 32)
+    if b.shape[0] != K or scales.shape[0] != rows_s or b.shape[1] < ((N + 1) // 2 if q4 else N) or scales.shape[1] < N:
+        raise _l.CutHipError(f"matmul_sep: shapes do not match K = {K}, N = {N} (b {tuple(b.shape)}, scales {tuple(scales.shape)})")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=a.device)
+    epi, op, dptr = _l.EPI_NONE, 0, None
+    if unary is not None:
+        epi, op = _l.EPI_UNARY, _l.UNARY[unary]
+    elif binary is not None:
+        if d is None or d.shape != out.shape or d.dtype != torch.float32 or d.stride(0) != out.stride(0):
+            raise _l.CutHipError("matmul_sep: binary epilogue needs an fp32 D with the shape and stride of C")
+        epi, op, dptr = _l.EPI_BINARY, _l.BINARY[binary], d.data_ptr()
+    lib = _l.load()
+    ws_bytes = lib.cuthip_matmul_sep_workspace_bytes(M, K, N)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=a.device)
+    common = (a2.data_ptr(), b.data_ptr(), scales.data_ptr(), dptr, out.data_ptr(), M, K, N, a2.stride(0), b.stride(0),
+              out.stride(0), scales.stride(0), epi, op)
+    if q4:
+        _l.check(lib.cuthip_matmul_q4_sep(*common, int(affine), ws.data_ptr(), ws_bytes, _stream_ptr()))
+    else:
+        _l.check(lib.cuthip_matmul_q8_sep(*common, ws.data_ptr(), ws_bytes, _stream_ptr()))
+    return out

@@ -146,6 +146,31 @@ int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void 
                        uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D,
                        int variant, void *stream);
 
+/* ---- quantized matmul on the reference's separated weight layout ----------
+ * Drop-in for the 3-input MatMulOpNode (operators/impl/matmul/MatMulOp.cpp:271-383)
+ * on the tensors the reference's loader produces (read_tensor_q8_separated /
+ * read_tensor_q4_separated, gguf_reader.cpp:389-501; affine Q4 from
+ * requantizeQ4KToAffine, llama.cpp:573-619); arguments are its PushConstants
+ * {M, K, N, strideA, strideB, strideC, scaleStride} (MatMulOp.cpp:514-541):
+ *   Q8: B int8 [K, strideB], scales fp16 [K/32, scaleStride]
+ *   Q4: packedB bytes [K, strideBNpacked], even column in the low nibble,
+ *       value nibble - 8; affine != 0: minima in rows [K/32, 2K/32) of scales
+ *       (MatMulQ4Common.cuh:126-153)
+ * A [M, strideA], C and D [M, strideC] are fp32; K must be a multiple of 32.
+ * epilogue / epilogue_op / D as in cuthip_matmul_gguf (MatMulFusion).
+ * workspace: device scratch of cuthip_matmul_sep_workspace_bytes(M, K, N)
+ * bytes (split-K partial sums; may be NULL when that is 0).  Streams the
+ * weights once per 4 rows of A: meant for decode and small batches; prefill
+ * belongs on cuthip_matmul_gguf with the native blocks. */
+size_t cuthip_matmul_sep_workspace_bytes(uint32_t M, uint32_t K, uint32_t N);
+int cuthip_matmul_q8_sep(const float *A, const int8_t *B, const uint16_t *scales, const float *D, float *C, uint32_t M,
+                         uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideB, uint32_t strideC, uint32_t scaleStride,
+                         int epilogue, int epilogue_op, void *workspace, size_t workspace_bytes, void *stream);
+int cuthip_matmul_q4_sep(const float *A, const uint8_t *packedB, const uint16_t *scales, const float *D, float *C, uint32_t M,
+                         uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideBNpacked, uint32_t strideC,
+                         uint32_t scaleStride, int epilogue, int epilogue_op, int affine, void *workspace,
+                         size_t workspace_bytes, void *stream);
+
 /* ---- the operators between the matmuls of a decode step --------------------
  * What the runner chains around the quantized matmuls for one token
  * (interface/runner/llama/llama.cpp, runLayer / decode graph).  All take
