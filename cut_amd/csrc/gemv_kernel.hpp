@@ -166,10 +166,7 @@ __device__ inline void x_store(const GemvParams &p, uint32_t sb, half_t *xs, flo
 // CNT > 0: every wave owns exactly CNT*KP steps (nsteps == WAVES*KP*CNT up to
 // the last part's tail, which is masked), CNT <= TB, and TileCfg::PIPE holds.
 template <int FMT, int MT, int WAVES, int KP, int CNT>
-#ifndef CUTHIP_GEMV_OCC
-#define CUTHIP_GEMV_OCC 2
-#endif
-__global__ void __launch_bounds__(64 * WAVES, CUTHIP_GEMV_OCC) gemv_kernel(GemvParams p) {
+__global__ void __launch_bounds__(64 * WAVES, 2) gemv_kernel(GemvParams p) {
   using S = Step<FMT>;
   using T = TileCfg<MT, KP>;
   constexpr int R = T::R, TB = T::TB, D = T::D, XROW = T::XROW, SXROW = TB * S::NSUB;
@@ -204,10 +201,7 @@ __global__ void __launch_bounds__(64 * WAVES, CUTHIP_GEMV_OCC) gemv_kernel(GemvP
 
   if constexpr (CNT > 0) {
     constexpr int XI = (T::ROWS * CNT * 32 + kWave - 1) / kWave;
-#ifndef CUTHIP_GEMV_DD
-#define CUTHIP_GEMV_DD 4
-#endif
-    constexpr int DD = CNT < CUTHIP_GEMV_DD ? CNT : CUTHIP_GEMV_DD;
+    constexpr int DD = CNT < 4 ? CNT : 4;   // ring depth: measured flat between 1 and 4
     XTile<XI> xt;
     x_load<KP, CNT, XI>(p, sb, lane, xt);
     typename S::Raw buf[DD];
