@@ -188,3 +188,32 @@ def test_reference_known_answers_on_native_blocks(ops):
     W = q8_rows(np.full((2, 64), 4, np.int8), [[0.5, 1.0], [2.0, 0.25]])
     got = gpu_matmul(ops, oracle.Q8_0, W, np.ones((1, 64), np.float32), 2, 64)
     assert np.array_equal(got, [[192.0, 288.0]])
+
+
+@pytest.mark.parametrize("name", list(oracle.FORMATS))
+@pytest.mark.parametrize("M,N,K", [(1, 1, 256), (1, 7, 512), (2, 9, 256), (3, 1030, 1024), (5, 64, 4096), (8, 40, 2048),
+                                  (1, 96, 14336), (2, 24, 14336), (1, 4100, 512)])
+def test_rows8_kernel_shapes(ops, name, M, N, K):
+    """The 8-row GEMV (variant 3) at its corner shapes: one row, fewer rows than a wave, a single K step, K split over
+    2/4/8 waves, every batch size class (dot path, 4/8/16 accumulators), long K; it agrees with the oracle and with
+    the fallback kernel (variant 0)."""
+    fmt = oracle.FORMATS[name]
+    W = quantized_weights(fmt, N, K, seed=N + K)
+    A = gauss_acts((M, K), seed=M, dtype=np.float16)
+    want = oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)
+    got3 = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=3)
+    got0 = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=0)
+    assert normwise_rel_err(got3, want) < TOL_F16_ACT
+    assert normwise_rel_err(got0, want) < TOL_F16_ACT
+
+
+def test_rows8_refuses_what_does_not_fit_and_auto_falls_back(ops):
+    from cut_amd import lib
+    fmt = oracle.Q4_K
+    N, K, M = 64, 14336, 8      # 8 rows of 14336 fp16 activations exceed the LDS budget of the 8-row kernel
+    W = quantized_weights(fmt, N, K, seed=1)
+    A = gauss_acts((M, K), seed=2, dtype=np.float16)
+    with pytest.raises(lib.CutHipError, match="variant 3"):
+        gpu_matmul(ops, fmt, W, A, N, K, variant=3)
+    want = oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)
+    assert normwise_rel_err(gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32), want) < TOL_F16_ACT
