@@ -165,3 +165,55 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
   }
   return launch_gemv(fmt, p, reinterpret_cast<hipStream_t>(stream));
 }
+extern "C" {
+
+int cuthip_matmul_gguf_pro(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t K, uint32_t N,
+                           int epilogue, int epilogue_op, const void *D, int prologue, const float *norm_weight, float eps,
+                           void *stream) {
+  using namespace cuthip;
+  if (prologue == CUTHIP_PRO_NONE)
+    return cuthip_matmul_gguf(fmt, W, A, a_dtype, C, c_dtype, 1, K, N, K, N, epilogue, epilogue_op, D, 3, stream);
+  if (fmt < CUTHIP_Q8_0 || fmt > CUTHIP_Q6_K || (a_dtype != CUTHIP_F32 && a_dtype != CUTHIP_F16) ||
+      (c_dtype != CUTHIP_F32 && c_dtype != CUTHIP_F16) || !W || !A || !C || N == 0 || K == 0 || K % fmt_elems(fmt) != 0 ||
+      epilogue < CUTHIP_EPI_NONE || epilogue > CUTHIP_EPI_BINARY || (epilogue == CUTHIP_EPI_BINARY && !D)) {
+    set_error("cuthip_matmul_gguf_pro: bad argument (format %d, K %u, N %u, epilogue %d)", fmt, K, N, epilogue);
+    return CUTHIP_ERR_INVALID;
+  }
+  if (prologue == CUTHIP_PRO_RMSNORM) {
+    if (!norm_weight || (uintptr_t)norm_weight % 16 != 0 || K % 8 != 0 || (uintptr_t)A % 16 != 0) {
+      set_error("cuthip_matmul_gguf_pro: the RMSNorm prologue needs a 16-byte aligned fp32 norm_weight[K] and A");
+      return CUTHIP_ERR_INVALID;
+    }
+  } else if (prologue == CUTHIP_PRO_SWIGLU) {
+    if (a_dtype != CUTHIP_F16 || K % 8 != 0 || (uintptr_t)A % 16 != 0) {
+      set_error("cuthip_matmul_gguf_pro: the SwiGLU prologue takes 16-byte aligned fp16 [gate | up] with K a multiple of 8");
+      return CUTHIP_ERR_INVALID;
+    }
+  } else {
+    set_error("cuthip_matmul_gguf_pro: unknown prologue %d", prologue);
+    return CUTHIP_ERR_INVALID;
+  }
+  GemvParams p;
+  p.W = reinterpret_cast<const uint8_t *>(W);
+  p.A = A;
+  p.C = C;
+  p.epi = Epilogue{epilogue, epilogue_op, D};
+  p.M = 1; p.K = K; p.N = N; p.strideA = K; p.strideC = N;
+  p.nsteps = (K + 255) / 256;
+  p.row_bytes = (uint32_t)((uint64_t)(K / fmt_elems(fmt)) * fmt_bytes(fmt));
+  p.a_f16 = a_dtype == CUTHIP_F16;
+  p.c_f16 = c_dtype == CUTHIP_F16;
+  p.pro = prologue;
+  p.norm_w = norm_weight;
+  p.eps = eps;
+  bool taken = false;
+  int rc = launch_rows8_any(fmt, p, reinterpret_cast<hipStream_t>(stream), &taken);
+  if (!taken) {
+    set_error("cuthip_matmul_gguf_pro: K = %u does not fit the LDS budget of the 8-row GEMV", K);
+    return CUTHIP_ERR_INVALID;
+  }
+  return rc;
+}
+
+}  // extern "C"
+

@@ -15,6 +15,11 @@ struct GemvParams {
   uint32_t nsteps;   // ceil(K / 256)
   uint32_t row_bytes;
   int a_f16, c_f16;
+  // prologue on the activations (8-row GEMV, batch 1): CUTHIP_PRO_RMSNORM: A is x, the product is taken with
+  // x * norm_w and scaled by rsqrt(mean(x^2) + eps); CUTHIP_PRO_SWIGLU: A is [gate(K) | up(K)], input silu(gate) * up
+  int pro = 0;
+  const float *norm_w = nullptr;
+  float eps = 0.0f;
 };
 
 // ---- per-tile configuration -------------------------------------------------

@@ -404,8 +404,16 @@ template <> struct Rows8<CUTHIP_Q4_0> {
 // / stored later (XStage::store), so the caller can put the weight loads in
 // between: memory returns in issue order, hence the wait for the activations
 // leaves the weight loads in flight.
-template <int SUBK, int THREADS, int MT, int XR> struct XStage {
+// PRO: the kernel instance also implements the activation prologues (RMSNorm, SiLU(gate) * up): extra
+// registers for the norm weights and the sum of squares, so only batch-1 decode kernels are built with it.
+template <int SUBK, int THREADS, int MT, int XR, bool PRO> struct XStage {
   u32x4 ra[MT * XR], rb[MT * XR];
+  u32x4 wa[PRO ? MT * XR : 1], wb[PRO ? MT * XR : 1];   // norm weights of the group (fp32 x 8)
+  float ssq[MT];                                        // this thread's share of sum(x^2) per batch row
+  __device__ void init() {
+#pragma unroll
+    for (int m = 0; m < MT; ++m) ssq[m] = 0.0f;
+  }
   // base: first group (of a row) of this batch; gpr: groups per padded row
   __device__ void load(const GemvParams &p, uint32_t base, int tid, uint32_t gpr) {
     const uint32_t esz = p.a_f16 ? 2u : 4u;
@@ -416,25 +424,56 @@ template <int SUBK, int THREADS, int MT, int XR> struct XStage {
       if (m < p.M && k < p.K) {
         const uint8_t *src = reinterpret_cast<const uint8_t *>(p.A) + ((size_t)m * p.strideA + k) * esz;
         ra[u] = ld_u32x4(src);
-        if (!p.a_f16) rb[u] = ld_u32x4(src + 16);
+        if (PRO && p.pro == CUTHIP_PRO_SWIGLU) {
+          rb[u] = ld_u32x4(src + (size_t)p.K * 2);   // the "up" half of [gate | up] (fp16 only)
+        } else {
+          if (!p.a_f16) rb[u] = ld_u32x4(src + 16);
+          if (PRO && p.pro == CUTHIP_PRO_RMSNORM) {
+            const uint8_t *w = reinterpret_cast<const uint8_t *>(p.norm_w + k);
+            wa[u] = ld_u32x4(w);
+            wb[u] = ld_u32x4(w + 16);
+          }
+        }
       }
     }
   }
   __device__ void store(const GemvParams &p, uint32_t base, int tid, uint32_t gpr, half_t *xs, float *sxs, int xrow,
-                        int sxrow) const {
+                        int sxrow) {
 #pragma unroll
     for (int u = 0; u < MT * XR; ++u) {
       const uint32_t m = u / XR, gi = base + (u % XR) * THREADS + tid, k = gi * 8;
       const bool active = m < p.M && gi < gpr, ok = active && k < p.K;
       half_t h[8];
-      if (p.a_f16) {
-        half8_t v = __builtin_bit_cast(half8_t, ra[u]);
+      if (PRO && p.pro == CUTHIP_PRO_SWIGLU) {
+        half8_t g = __builtin_bit_cast(half8_t, ra[u]), up = __builtin_bit_cast(half8_t, rb[u]);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) h[i] = v[i];
+        for (int i = 0; i < 8; ++i) {
+          float gf = (float)g[i];
+          h[i] = (half_t)(gf / (1.0f + __expf(-gf)) * (float)up[i]);
+        }
       } else {
-        f32x4 lo = __builtin_bit_cast(f32x4, ra[u]), hi = __builtin_bit_cast(f32x4, rb[u]);
-        h[0] = (half_t)lo.x; h[1] = (half_t)lo.y; h[2] = (half_t)lo.z; h[3] = (half_t)lo.w;
-        h[4] = (half_t)hi.x; h[5] = (half_t)hi.y; h[6] = (half_t)hi.z; h[7] = (half_t)hi.w;
+        float x[8];
+        if (p.a_f16) {
+          half8_t v = __builtin_bit_cast(half8_t, ra[u]);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) x[i] = (float)v[i];
+        } else {
+          f32x4 lo = __builtin_bit_cast(f32x4, ra[u]), hi = __builtin_bit_cast(f32x4, rb[u]);
+          x[0] = lo.x; x[1] = lo.y; x[2] = lo.z; x[3] = lo.w; x[4] = hi.x; x[5] = hi.y; x[6] = hi.z; x[7] = hi.w;
+        }
+        if (PRO && p.pro == CUTHIP_PRO_RMSNORM) {
+          f32x4 w0 = __builtin_bit_cast(f32x4, wa[u]), w1 = __builtin_bit_cast(f32x4, wb[u]);
+          const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+          float q = 0.0f;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            q = fmaf(x[i], x[i], q);
+            x[i] *= w[i];
+          }
+          if (ok) ssq[m] += q;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) h[i] = (half_t)x[i];
       }
       float s = 0.0f;
 #pragma unroll
@@ -459,7 +498,7 @@ template <int SUBK, int THREADS, int MT, int XR> struct XStage {
 // MT == 1 takes the lane-local dot-product path (v_dot2_f32_f16 on the same
 // subnormal operands: a quarter of the issue cycles of the matrix-core path,
 // whose 32 A-rows would be 7/8 padding); MT > 1 goes through the matrix core.
-template <int FMT, int MT, int RWG, int KW, int D, int XWANT>
+template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO>
 __global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_kernel(GemvParams p) {
   using S = Rows8<FMT>;
   constexpr bool DOT = MT <= kRows8DotMax;
@@ -482,6 +521,7 @@ __global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_kernel(GemvParams
   const int xrow = (int)(p.nsteps * kXStep), sxrow = (int)(p.nsteps * S::NSUB);
   half_t *xs = reinterpret_cast<half_t *>(lds);
   float *sxs = reinterpret_cast<float *>(lds + (size_t)MT * xrow * 2);
+  float *nrm = sxs + MT * sxrow;   // [MT][WAVES] per-wave shares of sum(x^2) (RMSNorm prologue)
 
   const uint32_t n0 = (blockIdx.x * RWG + rg) * 8u;
   const uint32_t n = min(n0 + (uint32_t)r8, p.N - 1);
@@ -496,7 +536,8 @@ __global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_kernel(GemvParams
   // second batch (every further batch is one more memory round trip before the first step can start)
   constexpr int XCAP = 8 / MT, XR = XWANT < XCAP ? XWANT : XCAP;
   const uint32_t gpr = kpad / 8;   // 8-element groups per padded row
-  XStage<S::SUBK, THREADS, MT, XR> xst;
+  XStage<S::SUBK, THREADS, MT, XR, PRO> xst;
+  xst.init();
   xst.load(p, 0, tid, gpr);
   typename S::Raw buf[D];
 #pragma unroll
@@ -509,7 +550,27 @@ __global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_kernel(GemvParams
     xst.load(p, base, tid, gpr);
     xst.store(p, base, tid, gpr, xs, sxs, xrow, sxrow);
   }
+  if (PRO && p.pro == CUTHIP_PRO_RMSNORM) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      float t = xst.ssq[m];
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o);
+      if (lane == 0) nrm[m * WAVES + wave] = t;
+    }
+  }
   __syncthreads();
+  // RMSNorm prologue: the scalar rsqrt(mean(x^2) + eps) multiplies the finished dot products
+  float xscale[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    xscale[m] = 1.0f;
+    if (PRO && p.pro == CUTHIP_PRO_RMSNORM) {
+      float t = 0.0f;
+      for (int w = 0; w < WAVES; ++w) t += nrm[m * WAVES + w];
+      xscale[m] = 1.0f / sqrtf(t / (float)p.K + p.eps);
+    }
+  }
 
   // Matrix-core path: A-row j of this lane is batch row j>>2 (clamped), piece j&3, and accumulator quad q
   // holds batch row 2q + kg.  Dot path: the lane's own slice of every batch row, accumulator q = batch row q.
@@ -569,7 +630,7 @@ __global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_kernel(GemvParams
       v += __shfl_xor(v, 1);
       v += __shfl_xor(v, 2);
       v += __shfl_xor(v, 32);
-      out[q] = v;
+      out[q] = PRO ? v * xscale[q] : v;   // linear in the partial sums, so it may be applied before the K ranges are folded
     }
     writer = c.g == 0 && c.kg == 0;
   } else {
@@ -616,15 +677,18 @@ __global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_kernel(GemvParams
 }
 
 template <int FMT> static size_t rows8_lds_bytes(const GemvParams &p, int mt) {
-  return (size_t)mt * ((size_t)p.nsteps * kXStep * 2 + (size_t)p.nsteps * Rows8<FMT>::NSUB * 4);
+  return (size_t)mt * ((size_t)p.nsteps * kXStep * 2 + (size_t)p.nsteps * Rows8<FMT>::NSUB * 4 + 8 * 4);   // + [8 waves] floats
 }
 
-template <int FMT, int MT, int RWG, int KW, int D, int XWANT>
+template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO = false>
 static int launch_rows8(const GemvParams &p, hipStream_t stream) {
+  if constexpr (MT == 1 && !PRO) {
+    if (p.pro) return launch_rows8<FMT, MT, RWG, KW, D, XWANT, true>(p, stream);
+  }
   size_t lds = rows8_lds_bytes<FMT>(p, MT);
   size_t red = (size_t)RWG * KW * MT * 8 * 4;
   if (red > lds) lds = red;
-  auto kern = gemv_rows8_kernel<FMT, MT, RWG, KW, D, XWANT>;
+  auto kern = gemv_rows8_kernel<FMT, MT, RWG, KW, D, XWANT, PRO>;
   if (lds > 64 * 1024) {
     if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),

@@ -50,8 +50,15 @@ class DecodeStep:
     'v', 'o', 'gate_up' ([2 * ffn, hidden], gate rows first), 'down' and fp32 'attn_norm', 'ffn_norm';
     plus 'out_norm' (fp32) and 'head' at the top level."""
 
-    def __init__(self, cfg: DecodeConfig, layers: list[dict], out_norm: torch.Tensor, head: torch.Tensor, device="cuda:0"):
-        self.cfg, self.layers, self.out_norm, self.head = cfg, layers, out_norm, head
+    def __init__(self, cfg: DecodeConfig, layers: list[dict], out_norm: torch.Tensor, head: torch.Tensor, device="cuda:0",
+                 fuse: int = 0):
+        """fuse: 0 = every operator is its own launch; 1 = SiLU(gate) * up runs inside the staging of w_down;
+        2 = RMSNorm is fused into the following matmuls as well.  Level 2 saves three more launches per layer but
+        every workgroup of those matmuls then stages fp32 x and the norm weights (4x the bytes of fp16 x), which
+        lengthens their start-up; likewise every workgroup of w_down recomputes SiLU * up for its whole input.  On
+        MI355X both levels measured slower than separate launches (2.43 / 2.70 / 2.85 ms per token for 0 / 1 / 2 at
+        the 8B shape), so 0 is the default; the fused entry point stays for shapes where launches dominate."""
+        self.cfg, self.layers, self.out_norm, self.head, self.fuse = cfg, layers, out_norm, head, fuse
         dev = torch.device(device)
         c = cfg
         f16, f32 = torch.float16, torch.float32
@@ -83,8 +90,12 @@ class DecodeStep:
     def step(self) -> None:
         """Consumes self.x (the embedding of the current token), leaves logits and the arg-max token."""
         c = self.cfg
+        if self.fuse >= 2:
+            return self._step_fused()
         for i, L in enumerate(self.layers):
             ops.rmsnorm(self.x, L["attn_norm"], c.eps, out=self.xn.view(1, -1))
+            # (running v beside q+k on a second stream was measured slower: the fork / join nodes of the graph cost
+            # more than the 6 us the small matmul takes)
             ops.matmul_gguf(self.xn, L["qk"], c.fmt_attn, c.q_dim + c.kv_dim, c.hidden, out=self.qk.view(1, -1))
             ops.matmul_gguf(self.xn, L["v"], c.fmt_v, c.kv_dim, c.hidden, out=self.v.view(1, -1))
             ops.rope_kv_write(self.qk[:c.q_dim], self.qk[c.q_dim:], self.v, self.params, self.cos_t, self.sin_t,
@@ -95,9 +106,28 @@ class DecodeStep:
                             d=self.x.view(1, -1))
             ops.rmsnorm(self.x, L["ffn_norm"], c.eps, out=self.xn.view(1, -1))
             ops.matmul_gguf(self.xn, L["gate_up"], c.fmt_ffn, 2 * c.ffn, c.hidden, out=self.gu.view(1, -1))
-            ops.silu_mul(self.gu, self.act)
-            ops.matmul_gguf(self.act, L["down"], c.fmt_ffn, c.hidden, c.ffn, out=self.x.view(1, -1), binary="add",
-                            d=self.x.view(1, -1))
+            if self.fuse >= 1:
+                ops.matmul_gguf_pro(self.gu, L["down"], c.fmt_ffn, c.hidden, c.ffn, self.x, "swiglu", binary="add", d=self.x)
+            else:
+                ops.silu_mul(self.gu, self.act)
+                ops.matmul_gguf(self.act, L["down"], c.fmt_ffn, c.hidden, c.ffn, out=self.x.view(1, -1), binary="add",
+                                d=self.x.view(1, -1))
         ops.rmsnorm(self.x, self.out_norm, c.eps, out=self.xn.view(1, -1))
         ops.matmul_gguf(self.xn, self.head, c.fmt_head, c.vocab, c.hidden, out=self.logits.view(1, -1))
+        ops.argmax(self.logits, self.token)
+
+    def _step_fused(self) -> None:
+        c = self.cfg
+        for i, L in enumerate(self.layers):
+            ops.matmul_gguf_pro(self.x, L["qk"], c.fmt_attn, c.q_dim + c.kv_dim, c.hidden, self.qk, "rmsnorm", L["attn_norm"], c.eps)
+            ops.matmul_gguf_pro(self.x, L["v"], c.fmt_v, c.kv_dim, c.hidden, self.v, "rmsnorm", L["attn_norm"], c.eps)
+            ops.rope_kv_write(self.qk[:c.q_dim], self.qk[c.q_dim:], self.v, self.params, self.cos_t, self.sin_t,
+                              self.k_cache[i], self.v_cache[i], c.head_dim, self.q_rot)
+            ops.attn_decode(self.q_rot, self.k_cache[i], self.v_cache[i], self.params, c.n_heads, c.n_kv_heads, c.head_dim,
+                            self.scale, self.ws, self.attn)
+            ops.matmul_gguf(self.attn, L["o"], c.fmt_attn, c.hidden, c.q_dim, out=self.x.view(1, -1), binary="add",
+                            d=self.x.view(1, -1))
+            ops.matmul_gguf_pro(self.x, L["gate_up"], c.fmt_ffn, 2 * c.ffn, c.hidden, self.gu, "rmsnorm", L["ffn_norm"], c.eps)
+            ops.matmul_gguf_pro(self.gu, L["down"], c.fmt_ffn, c.hidden, c.ffn, self.x, "swiglu", binary="add", d=self.x)
+        ops.matmul_gguf_pro(self.x, self.head, c.fmt_head, c.vocab, c.hidden, self.logits, "rmsnorm", self.out_norm, c.eps)
         ops.argmax(self.logits, self.token)

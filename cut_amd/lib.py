@@ -29,7 +29,7 @@ EXPORTS = [
     "cuthip_stream_create", "cuthip_stream_destroy", "cuthip_stream_sync",
     "cuthip_event_create", "cuthip_event_destroy", "cuthip_event_record", "cuthip_event_sync", "cuthip_event_elapsed_ms",
     "cuthip_variant_count", "cuthip_variant_default", "cuthip_variant_info", "cuthip_variant_lookup",
-    "cuthip_dequant", "cuthip_matmul_gguf",
+    "cuthip_dequant", "cuthip_matmul_gguf", "cuthip_matmul_gguf_pro",
     "cuthip_rmsnorm", "cuthip_rope_kv_write", "cuthip_attn_decode_workspace_bytes", "cuthip_attn_decode",
     "cuthip_silu_mul", "cuthip_argmax",
     "cuthip_matmul_sep_workspace_bytes", "cuthip_matmul_q8_sep", "cuthip_matmul_q4_sep",
@@ -89,6 +89,7 @@ def load() -> C.CDLL:
     lib.cuthip_dequant.argtypes = [i, vp, vp, i, u32, u32, u32, vp]
     lib.cuthip_matmul_gguf.argtypes = [i, vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, i, vp]
     f32 = C.c_float
+    lib.cuthip_matmul_gguf_pro.argtypes = [i, vp, vp, i, vp, i, u32, u32, i, i, vp, i, vp, f32, vp]
     lib.cuthip_rmsnorm.argtypes = [vp, i, vp, vp, i, u32, u32, u32, f32, vp]
     lib.cuthip_rope_kv_write.argtypes = [vp, vp, vp, i, vp, vp, vp, vp, vp, vp, i, u32, u32, u32, u32, vp]
     lib.cuthip_attn_decode_workspace_bytes.argtypes = [u32, u32, u32]

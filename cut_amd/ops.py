@@ -181,3 +181,25 @@ def matmul_sep(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, N: int, q
     else:
         _l.check(lib.cuthip_matmul_q8_sep(*common, ws.data_ptr(), ws_bytes, _stream_ptr()))
     return out
+
+
+def matmul_gguf_pro(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: int, out: torch.Tensor, prologue: str,
+                    norm_weight: torch.Tensor | None = None, eps: float = 0.0, unary: str | None = None,
+                    binary: str | None = None, d: torch.Tensor | None = None) -> torch.Tensor:
+    """Batch-1 matmul with the preceding operator fused into the activation staging:
+    prologue "rmsnorm": a = x [K] (fp32 or fp16), norm_weight fp32 [K];  "swiglu": a = [gate | up] fp16 [2K]."""
+    pro = {"rmsnorm": 1, "swiglu": 2}[prologue]
+    need = K if pro == 1 else 2 * K
+    if a.numel() != need or not a.is_contiguous() or out.numel() != N:
+        raise _l.CutHipError(f"matmul_gguf_pro: a must hold {need} contiguous elements and out {N}")
+    epi, op, dptr = _l.EPI_NONE, 0, None
+    if unary is not None:
+        epi, op = _l.EPI_UNARY, _l.UNARY[unary]
+    elif binary is not None:
+        if d is None or d.numel() != N or d.dtype != out.dtype:
+            raise _l.CutHipError("matmul_gguf_pro: binary epilogue needs D like C")
+        epi, op, dptr = _l.EPI_BINARY, _l.BINARY[binary], d.data_ptr()
+    _l.check(_l.load().cuthip_matmul_gguf_pro(_fmt(fmt), w_blocks.data_ptr(), a.data_ptr(), _dt(a), out.data_ptr(), _dt(out), K, N,
+                                              epi, op, dptr, pro, norm_weight.data_ptr() if norm_weight is not None else None,
+                                              eps, _stream_ptr()))
+    return out

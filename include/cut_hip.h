@@ -46,6 +46,9 @@ typedef enum { CUTHIP_EPI_NONE = 0, CUTHIP_EPI_UNARY = 1, CUTHIP_EPI_BINARY = 2 
 typedef enum { CUTHIP_UNARY_SILU = 0, CUTHIP_UNARY_RELU = 1, CUTHIP_UNARY_GELU_TANH = 2, CUTHIP_UNARY_SIGMOID = 3, CUTHIP_UNARY_TANH = 4, CUTHIP_UNARY_NEG = 5 } cuthip_unary_op;
 typedef enum { CUTHIP_BINARY_ADD = 0, CUTHIP_BINARY_SUB = 1, CUTHIP_BINARY_MUL = 2, CUTHIP_BINARY_DIV = 3, CUTHIP_BINARY_MIN = 4, CUTHIP_BINARY_MAX = 5 } cuthip_binary_op;
 
+/* Prologues on the activations of cuthip_matmul_gguf_pro. */
+typedef enum { CUTHIP_PRO_NONE = 0, CUTHIP_PRO_RMSNORM = 1, CUTHIP_PRO_SWIGLU = 2 } cuthip_prologue;
+
 typedef struct {
   char name[64];
   char arch[32];
@@ -145,6 +148,20 @@ int cuthip_dequant(int fmt, const void *blocks, void *out, int out_dtype, uint32
 int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M, uint32_t K,
                        uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D,
                        int variant, void *stream);
+
+/* The same matmul at batch 1 with the operator in front of it fused into the
+ * staging of the activations, which saves a launch per use in a decode step
+ * (the reference fuses RMSNorm into its consumers in ExtendedRMSNormFusion /
+ * RMSNormFusion, runtime/graph/GraphOptimizer.cpp:46-70):
+ *   CUTHIP_PRO_RMSNORM: A = x [K]; C = (x * rsqrt(mean(x^2) + eps) * norm_weight) . dequant(W)^T
+ *                       (RMSNorm.cu:15-37 followed by the matmul; norm_weight fp32 [K], 16-byte aligned)
+ *   CUTHIP_PRO_SWIGLU : A = [gate(K) | up(K)] fp16; C = (silu(gate) * up) . dequant(W)^T
+ *                       (llama.cpp:1832-1860: SiLU, BinaryMul, then w_down)
+ * M must be 1 and the activations must fit the 8-row GEMV's LDS budget (K <= ~40k);
+ * other arguments as cuthip_matmul_gguf (no variant choice: always the 8-row GEMV). */
+int cuthip_matmul_gguf_pro(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t K, uint32_t N,
+                           int epilogue, int epilogue_op, const void *D, int prologue, const float *norm_weight, float eps,
+                           void *stream);
 
 /* ---- quantized matmul on the reference's separated weight layout ----------
  * Drop-in for the 3-input MatMulOpNode (operators/impl/matmul/MatMulOp.cpp:271-383)

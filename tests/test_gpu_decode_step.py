@@ -135,7 +135,38 @@ def _oracle_step(cfg, layers_h, out_norm, head, x, pos, kc, vc, cos_t, sin_t):
     return oracle.matmul_gguf(oracle.Q6_K, head, xn[None], cfg.vocab, f64=True)[0].astype(np.float32)
 
 
-def test_small_decode_step_against_oracle_chain(ops):
+@pytest.mark.parametrize("name", list(oracle.FORMATS))
+@pytest.mark.parametrize("N,K", [(200, 512), (64, 4096), (1000, 14336)])
+def test_matmul_with_fused_prologues(ops, name, N, K):
+    """RMSNorm and SiLU(gate) * up fused into the activation staging of the batch-1 matmul against the oracle chain
+    (norm -> fp16 -> matmul).  The fused kernel rounds x * w to fp16 and applies rsqrt(mean + eps) in fp32 to the
+    result, the chain rounds x * scale * w: both one fp16 rounding per activation, hence the 4e-4 bound."""
+    fmt = oracle.FORMATS[name]
+    rng = np.random.default_rng(N + K)
+    W = oracle.quantize(fmt, (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    x = (rng.standard_normal(K) * 3).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, K).astype(np.float32)
+    xn = oracle.rmsnorm(x, w, 1e-5)
+    want = oracle.matmul_gguf(fmt, W, xn[None], N, f64=True)[0]
+    for xin in (x, x.astype(np.float16)):
+        if xin.dtype == np.float16:
+            want = oracle.matmul_gguf(fmt, W, oracle.rmsnorm(xin.astype(np.float32), w, 1e-5)[None], N, f64=True)[0]
+        out = torch.empty(N, dtype=torch.float32, device="cuda")
+        ops.matmul_gguf_pro(dev(xin), dev(W), fmt, N, K, out, "rmsnorm", dev(w), 1e-5)
+        torch.cuda.synchronize()
+        assert normwise_rel_err(out.cpu().numpy(), want) < 4e-4
+    gu = (rng.standard_normal(2 * K) * 2).astype(np.float16)
+    act = oracle.silu_mul(gu.astype(np.float32)).astype(np.float16).astype(np.float32)
+    want = oracle.matmul_gguf(fmt, W, act[None], N, f64=True)[0]
+    res = rng.standard_normal(N).astype(np.float32)
+    out = dev(res.copy())
+    ops.matmul_gguf_pro(dev(gu), dev(W), fmt, N, K, out, "swiglu", binary="add", d=out)   # in-place residual add
+    torch.cuda.synchronize()
+    assert normwise_rel_err(out.cpu().numpy() - res, want) < 4e-4
+
+
+@pytest.mark.parametrize("fuse", [0, 1, 2])
+def test_small_decode_step_against_oracle_chain(ops, fuse):
     from cut_amd.decode import DecodeConfig, DecodeStep
     cfg = DecodeConfig(hidden=512, n_layers=2, n_heads=8, n_kv_heads=2, head_dim=64, ffn=1024, vocab=2048, max_ctx=64)
     rng = np.random.default_rng(11)
@@ -149,7 +180,7 @@ def test_small_decode_step_against_oracle_chain(ops):
                  "ffn_norm": rng.uniform(0.5, 1.5, cfg.hidden).astype(np.float32)} for _ in range(cfg.n_layers)]
     out_norm = rng.uniform(0.5, 1.5, cfg.hidden).astype(np.float32)
     head = qw(oracle.Q6_K, cfg.vocab, cfg.hidden)
-    step = DecodeStep(cfg, [{k: dev(v) for k, v in L.items()} for L in layers_h], dev(out_norm), dev(head))
+    step = DecodeStep(cfg, [{k: dev(v) for k, v in L.items()} for L in layers_h], dev(out_norm), dev(head), fuse=fuse)
     # a context of 9 earlier tokens already in the caches (same bits on both sides), then token 9
     pos = 9
     kc = [np.zeros((cfg.max_ctx, cfg.kv_dim), np.uint16) for _ in range(cfg.n_layers)]
