@@ -159,8 +159,8 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_
                                                            float scale, uint32_t nsplit) {
   __shared__ __attribute__((aligned(16))) half_t Ks[kAttnChunk * kAttnRow];
   __shared__ __attribute__((aligned(16))) half_t Vs[kAttnChunk * kAttnRow];
-  __shared__ float Qs[4 * kAttnMaxHd];
-  __shared__ float Ps[4 * kAttnChunk];
+  __shared__ __attribute__((aligned(16))) float Qs[4 * kAttnMaxHd];
+  __shared__ __attribute__((aligned(16))) float Ps[4 * kAttnChunk];
   const uint32_t kvH = blockIdx.x, split = blockIdx.y, nRep = nHeads / nKvHeads;
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t seqLen = params[1];
@@ -188,28 +188,42 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_
     __syncthreads();   // K, V staged (first pass) / Qs, Ps free again (later passes)
     for (uint32_t d = lane; d < headDim; d += 64) Qs[wave * kAttnMaxHd + d] = ld_act(q, q_f16, (size_t)h * headDim + d);
     __syncthreads();
-    // score of position t0 + lane
+    // score of position t0 + lane: q is read as broadcast 16-byte pieces
     float sc = 0.0f;
     const half_t *krow = Ks + lane * kAttnRow;
-    const float *qv = Qs + wave * kAttnMaxHd;
+    const f32x4 *qv = reinterpret_cast<const f32x4 *>(Qs + wave * kAttnMaxHd);
     for (uint32_t d = 0; d < headDim; d += 8) {
       half8_t k8 = *reinterpret_cast<const half8_t *>(krow + d);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) sc = fmaf(qv[d + e], (float)k8[e], sc);
+      f32x4 qa = qv[d / 4], qb = qv[d / 4 + 1];
+      sc = fmaf(qa.x, (float)k8[0], sc); sc = fmaf(qa.y, (float)k8[1], sc);
+      sc = fmaf(qa.z, (float)k8[2], sc); sc = fmaf(qa.w, (float)k8[3], sc);
+      sc = fmaf(qb.x, (float)k8[4], sc); sc = fmaf(qb.y, (float)k8[5], sc);
+      sc = fmaf(qb.z, (float)k8[6], sc); sc = fmaf(qb.w, (float)k8[7], sc);
     }
     sc = lane < nvalid ? sc * scale : -INFINITY;
     float m = wave_max(sc);
     float p = lane < nvalid ? expf(sc - m) : 0.0f;
     float l = wave_sum(p);
-    Ps[wave * kAttnChunk + lane] = p;
+    Ps[wave * kAttnChunk + lane] = p;   // zero for positions past the sequence
     __builtin_amdgcn_wave_barrier();
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    // weighted V: lane owns dims lane and lane + 64
+    // weighted V: lane owns the adjacent dims 2 * lane and 2 * lane + 1 (one 4-byte LDS read per position),
+    // four weights per 16-byte read; rows past the sequence are zero and carry zero weight
     float o0 = 0.0f, o1 = 0.0f;
-    for (uint32_t t = 0; t < nvalid; ++t) {
-      float pt = Ps[wave * kAttnChunk + t];
-      o0 = fmaf(pt, (float)Vs[t * kAttnRow + lane], o0);
-      if (headDim > 64) o1 = fmaf(pt, (float)Vs[t * kAttnRow + 64 + lane], o1);
+    typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+    const f32x4 *pv = reinterpret_cast<const f32x4 *>(Ps + wave * kAttnChunk);
+    const uint32_t dcol = min(2 * lane, (uint32_t)kAttnMaxHd - 2);
+#pragma unroll 4
+    for (uint32_t t = 0; t < (uint32_t)kAttnChunk; t += 4) {
+      f32x4 p4 = pv[t / 4];
+      half2v v0 = *reinterpret_cast<const half2v *>(Vs + (t + 0) * kAttnRow + dcol);
+      half2v v1 = *reinterpret_cast<const half2v *>(Vs + (t + 1) * kAttnRow + dcol);
+      half2v v2 = *reinterpret_cast<const half2v *>(Vs + (t + 2) * kAttnRow + dcol);
+      half2v v3 = *reinterpret_cast<const half2v *>(Vs + (t + 3) * kAttnRow + dcol);
+      o0 = fmaf(p4.x, (float)v0.x, o0); o1 = fmaf(p4.x, (float)v0.y, o1);
+      o0 = fmaf(p4.y, (float)v1.x, o0); o1 = fmaf(p4.y, (float)v1.y, o1);
+      o0 = fmaf(p4.z, (float)v2.x, o0); o1 = fmaf(p4.z, (float)v2.y, o1);
+      o0 = fmaf(p4.w, (float)v3.x, o0); o1 = fmaf(p4.w, (float)v3.y, o1);
     }
     if (live) {
       float *dst = partial + ((size_t)h * nsplit + split) * (2 + headDim);
@@ -217,8 +231,10 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_
         dst[0] = nvalid ? m : -INFINITY;
         dst[1] = l;
       }
-      if (lane < headDim) dst[2 + lane] = o0;
-      if (64 + lane < headDim) dst[2 + 64 + lane] = o1;
+      if (2 * lane + 1 < headDim) {
+        dst[2 + 2 * lane] = o0;
+        dst[2 + 2 * lane + 1] = o1;
+      }
     }
   }
 }
