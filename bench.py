@@ -304,7 +304,7 @@ def main():
             oracle.matmul_gguf(oracle.Q4_K, w_up_h, a1, N_FF)
             oracle.matmul_gguf(oracle.Q4_K, w_down_h, h1, N_EMBD)
             reps += 1
-            if time.perf_counter() - t0 > 10.0 or reps >= 40:
+            if time.perf_counter() - t0 > 12.0 or reps >= 100:
                 break
         cpu_s = (time.perf_counter() - t0) / reps
         result["cpu_baseline"] = {
