@@ -113,6 +113,27 @@ def bench_decode_step(torch, np, ops, dev, x_h, steps=5):
             "decode_step_8b_bytes_per_token": int(w_bytes_tok + kv_bytes_tok)}
 
 
+def bench_dequant(torch, ops, dev, reps=20):
+    """config 2: dequant of 256 Mi elements to fp16 (a 4 Mi-element tile of quantized N(0, 0.02) weights repeated
+    64 times); GB/s = (block bytes in + fp16 bytes out) / kernel time from events."""
+    res = {}
+    n_el = 256 * 1024 * 1024
+    out = torch.empty((n_el // 4096, 4096), dtype=torch.float16, device=dev)
+    for name in ("Q8_0", "Q4_0", "Q4_K", "Q6_K"):
+        tile = make_q_weights(name, 1024, 4096, 2)
+        raw = torch.from_numpy(tile).to(dev).repeat(64)
+        in_bytes = raw.numel()
+
+        def dq(_s, raw=raw, name=name):
+            ops.dequantize(raw, name, n_el // 4096, 4096, torch.float16, out=out)
+        wall_d, ev_d, _ = timed_graph(torch, dq, reps, 3)
+        res[f"dequant_{name}_to_f16_256Mi_GBps"] = round((in_bytes + n_el * 2) * reps / (ev_d * 1e-3) / 1e9, 1)
+        del raw
+    del out
+    torch.cuda.empty_cache()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -124,6 +145,8 @@ def main():
                     help="only run a plain 1 GiB device copy 5 times (reference traffic for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--gemm-only", type=int, default=0, metavar="M",
                     help="only run the Q4_K prefill GEMM (M x 4096) . (14336 x 4096)^T twelve times (target of rocprofv3 runs)")
+    ap.add_argument("--dequant-only", action="store_true",
+                    help="only run the 256 Mi-element dequant of the four formats (target of rocprofv3 runs)")
     ap.add_argument("--decode-only", action="store_true",
                     help="only run the 8B-shape decode step (target of rocprofv3 runs)")
     args = ap.parse_args()
@@ -145,6 +168,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4, "launches": 5}))
+        return
+    if args.dequant_only:
+        print(json.dumps(bench_dequant(torch, ops, dev, reps=5)))
         return
     if args.decode_only:
         x_h = np.random.default_rng(1).standard_normal((8, N_EMBD), dtype=np.float32).astype(np.float16)
@@ -251,21 +277,7 @@ def main():
         torch.cuda.empty_cache()
         extras.update(bench_decode_step(torch, np, ops, dev, x_h))
         torch.cuda.empty_cache()
-        # config 2: dequant of 256 Mi elements to fp16 (a 4 Mi-element tile repeated 64 times)
-        n_el = 256 * 1024 * 1024
-        out = torch.empty((n_el // 4096, 4096), dtype=torch.float16, device=dev)
-        for name in ("Q8_0", "Q4_0", "Q4_K", "Q6_K"):
-            tile = make_q_weights(name, 1024, 4096, 2)
-            raw = torch.from_numpy(tile).to(dev).repeat(64)
-            in_bytes = raw.numel()
-
-            def dq(_s, raw=raw, name=name):
-                ops.dequantize(raw, name, n_el // 4096, 4096, torch.float16, out=out)
-            wall_d, ev_d, _ = timed_graph(torch, dq, 20, 3)
-            extras[f"dequant_{name}_to_f16_256Mi_GBps"] = round((in_bytes + n_el * 2) * 20 / (ev_d * 1e-3) / 1e9, 1)
-            del raw
-        del out
-        torch.cuda.empty_cache()
+        extras.update(bench_dequant(torch, ops, dev))
         # LM head: Q6_K 128256 x 4096, batch 1 (431 MB per launch: streams from HBM by itself)
         head = torch.from_numpy(make_q_weights("Q6_K", 4008, 4096, 3)).to(dev).repeat(32)
         logits = torch.empty((1, 128256), dtype=torch.float16, device=dev)
