@@ -37,12 +37,15 @@ static const cuthip_variant_info_t kMatMulGgufVariants[] = {
     {"MatMulGgufGemvRows8", 64, 4, 8, 8,
      "decode GEMV (M <= 8): 8 weight rows x 128-byte runs per wave instruction, four 64-element pieces per row as "
      "MFMA columns, register ring of loads, no cross-wave reduction unless K is split"},
+    {"MatMulGgufDequantGemm", 256, 1, 256, 256,
+     "large-M prefill in two launches: the weights are dequantized once to an fp16 workspace, then a dense fp16 MFMA GEMM "
+     "with LDS-direct loads and 128x128 accumulators per wave (needs cuthip_matmul_gguf_ws)"},
 };
 
 static const cuthip_variant_info_t *table(int op, int *count) {
   switch (op) {
   case CUTHIP_OP_DEQUANT: *count = 1; return kDequantVariants;
-  case CUTHIP_OP_MATMUL_GGUF: *count = 4; return kMatMulGgufVariants;
+  case CUTHIP_OP_MATMUL_GGUF: *count = 5; return kMatMulGgufVariants;
   }
   *count = 0;
   return nullptr;

@@ -178,6 +178,17 @@ static int launch_dequant(const void *blocks, void *out, int out_dtype, uint32_t
   return check_hip(hipGetLastError(), "dequant launch");
 }
 
+// Internal entry for other translation units (the two-pass prefill matmul): arguments already validated.
+int launch_dequant_any(int fmt, const void *blocks, void *out, int out_dtype, uint32_t rows, uint32_t cols,
+                       uint32_t out_stride, hipStream_t stream) {
+  switch (fmt) {
+  case CUTHIP_Q8_0: return launch_dequant<CUTHIP_Q8_0>(blocks, out, out_dtype, rows, cols, out_stride, stream);
+  case CUTHIP_Q4_0: return launch_dequant<CUTHIP_Q4_0>(blocks, out, out_dtype, rows, cols, out_stride, stream);
+  case CUTHIP_Q4_K: return launch_dequant<CUTHIP_Q4_K>(blocks, out, out_dtype, rows, cols, out_stride, stream);
+  default: return launch_dequant<CUTHIP_Q6_K>(blocks, out, out_dtype, rows, cols, out_stride, stream);
+  }
+}
+
 }  // namespace cuthip
 
 extern "C" int cuthip_dequant(int fmt, const void *blocks, void *out, int out_dtype, uint32_t rows, uint32_t cols,

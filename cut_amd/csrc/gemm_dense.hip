@@ -1,0 +1,273 @@
+// Two-pass prefill matmul for gfx950 (variant MatMulGgufDequantGemm):
+//   pass 1  dequantizes the GGUF weight tensor once into an fp16 [N, K] workspace
+//           (the dequant kernel of this library, HBM-bound: ~25 us for 14336 x 4096),
+//   pass 2  C[m,n] = sum_k A[m,k] * W16[n,k] as a dense fp16 MFMA GEMM.
+// The single-launch GEMM (gemm.hip) decodes every weight once per 256 rows of
+// activations, i.e. M/256 times; for M in the thousands the decode ALU work, not
+// the MFMA, bounds it.  Here each weight is decoded exactly once and the GEMM's
+// inner loop contains nothing but MFMAs, LDS fragment reads and copy instructions.
+// Supersedes MatMulQ{4,8}CoopMatTiled.cu (operators/impl/matmul) for large M.
+//
+// The GEMM: a workgroup of four waves owns a BM x 256 tile of C (BM = 256 or 128),
+// each wave a (BM/2) x 128 sub-tile in fp32 accumulators (AGPRs), K walked in slices
+// of 64.  Both operands go global -> LDS with global_load_lds_dwordx4 (no VGPR
+// round trip): one instruction fills 8 tile rows x 128 bytes = 1 KB of LDS, lane i
+// at byte 16 i; the lane reads the 16-byte chunk (i & 7) ^ (i >> 3) of its row, so
+// that the LDS image is XOR-swizzled and the MFMA fragment reads (lane l: row l & 31,
+// chunk 2 s + (l >> 5) of k-step s) spread over all banks.  Two LDS stages; the
+// loads of slice t+1 are in flight while slice t is multiplied.
+//
+// Issue order is explicit.  A wave has the SIMD to itself (one wave per SIMD), so a
+// burst of memory instructions stalls its MFMA stream: 16 loads in a row cost ~1000
+// cycles per slice, 8 LDS reads in a row ~90.  Every MFMA is therefore followed by
+// at most one LDS read and one global load, the loads spread over the slice at the
+// rate the texture path sustains (64 B/clk per CU), and the fragment reads of k-step
+// s+1 are issued under the MFMAs of k-step s.  The LDS reads are inline asm with
+// hand-placed s_waitcnt, because the compiler's own counter tracking waits for all
+// outstanding LDS-direct loads before any LDS read.  The last k-step of a slice is
+// multiplied after the barrier, under the first fragment reads of the next slice.
+//
+// Numerics: weights rounded to fp16 once (2^-11 relative), fp32 activations rounded
+// to fp16 once, fp32 accumulation: the same error budget as the single-launch GEMM.
+#include <type_traits>
+#include <utility>
+
+#include "common.hpp"
+
+namespace cuthip {
+
+int launch_dequant_any(int fmt, const void *blocks, void *out, int out_dtype, uint32_t rows, uint32_t cols,
+                       uint32_t out_stride, hipStream_t stream);
+
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) uint8_t lds_u8;
+
+template <int... Is, class F> __device__ inline void static_for_impl(std::integer_sequence<int, Is...>, F &&f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F> __device__ inline void static_for(F &&f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F &&>(f));
+}
+
+struct DenseParams {
+  const uint8_t *A, *W;  // fp16 [M, strideA], fp16 [N, K]
+  void *C;
+  Epilogue epi;
+  uint32_t M, N, K, strideA, strideC, mtiles, ntiles;
+  int c_f16;
+};
+
+constexpr int kDBN = 256, kDBK = 64;
+
+template <int BM>
+__global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)  // LDS address-space casts and AMDGPU inline asm: the host pass only needs the stub
+  constexpr int MI = BM / 64, NJ = kDBN / 64;  // 32 x 32 MFMA tiles per wave: MI x NJ
+  constexpr int NM = MI * NJ;                  // MFMAs per k-step of 16
+  constexpr int NLA = BM / 32, NL = (BM + kDBN) / 32;  // LDS-direct loads per wave per slice (A, total)
+  constexpr int LSTEP = MI == 4 ? 3 : 2;       // one load every LSTEP-th MFMA slot
+  static_assert(NJ == 4 && (MI == 4 || MI == 2), "tile shape");
+  static_assert((NL - 1) * LSTEP < 3 * NM, "the last load must be issued before the last k-step of the slice");
+  __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * 128];
+  __shared__ __attribute__((aligned(1024))) uint8_t sA1[BM * 128];
+  __shared__ __attribute__((aligned(1024))) uint8_t sB0[kDBN * 128];
+  __shared__ __attribute__((aligned(1024))) uint8_t sB1[kDBN * 128];
+
+  // XCD-aware tile order: ids id, id+8, id+16, ... share an XCD and its L2; give
+  // them the M-tiles of the same weight panels.
+  uint32_t id = blockIdx.x, mt, nt;
+  if (p.ntiles % 8 == 0) {
+    uint32_t xcd = id & 7, slot = id >> 3;
+    nt = (slot / p.mtiles) * 8 + xcd;
+    mt = slot % p.mtiles;
+  } else {
+    nt = id / p.mtiles;
+    mt = id % p.mtiles;
+  }
+  const uint32_t m0 = mt * BM, n0 = nt * kDBN;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // copy assignment: load v of wave w fills the 8-row group 4 v + w of its tile
+  uint32_t aoff[NLA], boff[kDBN / 32];
+  const uint32_t chunk = ((lane & 7) ^ (lane >> 3)) * 16;
+#pragma unroll
+  for (int v = 0; v < NLA; ++v) {
+    uint32_t r = min(m0 + 8 * (4 * v + wave) + (lane >> 3), p.M - 1);
+    aoff[v] = r * p.strideA * 2 + chunk;
+  }
+#pragma unroll
+  for (int v = 0; v < kDBN / 32; ++v) {
+    uint32_t r = min(n0 + 8 * (4 * v + wave) + (lane >> 3), p.N - 1);
+    boff[v] = r * p.K * 2 + chunk;
+  }
+  auto load_one = [&](int l, uint8_t *na, uint8_t *nb, uint32_t k0) {
+    const uint8_t *ga = p.A + (size_t)k0 * 2, *gb = p.W + (size_t)k0 * 2;
+    if (l < NLA)
+      __builtin_amdgcn_global_load_lds(ga + aoff[l], na + (4 * l + wave) * 1024, 16, 0, 0);
+    else
+      __builtin_amdgcn_global_load_lds(gb + boff[l - NLA], nb + (4 * (l - NLA) + wave) * 1024, 16, 0, 0);
+  };
+
+  f32x16 acc[MI][NJ];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) acc[i][j] = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+  const uint32_t arow = (wm * (BM / 2) + (lane & 31)) * 128, brow = (wn * 128 + (lane & 31)) * 128;
+  uint32_t xs[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) xs[s] = ((2 * s + (lane >> 5)) ^ (lane & 7)) * 16;
+
+  half8v fa[2][MI], fb[2][NJ];
+  // Waits until at most n of this wave's LDS reads are outstanding; the fragment registers pass through the
+  // statement so that no MFMA that uses them can be scheduled above it.
+#define CUTHIP_WAIT_FRAGS(f, n)                                                                                  \
+  asm volatile("s_waitcnt lgkmcnt(" #n ")"                                                                         \
+               : "+v"(fa[f][0]), "+v"(fa[f][1]), "+v"(fa[f][MI - 2]), "+v"(fa[f][MI - 1]), "+v"(fb[f][0]),         \
+                 "+v"(fb[f][1]), "+v"(fb[f][2]), "+v"(fb[f][3]))
+
+  // The NM MFMAs of one k-step on fragment set f.  After MFMA idx: the idx-th fragment read of k-step s of
+  // (sa, sb) into the other set, and, in every LSTEP-th slot of the slice (g = position of the group in the
+  // slice), one load of the next slice (k0) into (na, nb).
+  auto group = [&](int g, int f, const uint8_t *sa, const uint8_t *sb, int s, uint8_t *na, uint8_t *nb, uint32_t k0) {
+    const uint32_t pa = (uint32_t)(uintptr_t)(lds_u8 *)(sa) + arow + xs[s];
+    const uint32_t pb = (uint32_t)(uintptr_t)(lds_u8 *)(sb) + brow + xs[s];
+#pragma unroll
+    for (int idx = 0; idx < NM; ++idx) {
+      const int i = idx / NJ, j = idx % NJ;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[f][i], fb[f][j], acc[i][j], 0, 0, 0);
+      if (idx < MI)
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa[f ^ 1][idx]) : "v"(pa), "n"(idx * 4096) : "memory");
+      else if (idx < MI + NJ)
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[f ^ 1][idx - MI]) : "v"(pb), "n"((idx - MI) * 4096) : "memory");
+      const int q = g * NM + idx;
+      if (q % LSTEP == 0 && q / LSTEP < NL) load_one(q / LSTEP, na, nb, k0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  const uint32_t nsl = p.K / kDBK, klast = p.K - kDBK;
+  // One slice, entered right after a barrier with nothing in flight.  Set 1 holds the fragments of the previous
+  // slice's last k-step; its MFMAs run under the first fragment reads of this slice.  The loads of the slice
+  // after the last one re-read the last slice (never used) instead of branching around the MFMAs.
+  auto slice = [&](uint8_t *sa, uint8_t *sb, uint8_t *na, uint8_t *nb, uint32_t t) {
+    const uint32_t k0 = min((t + 1) * kDBK, klast);
+    group(0, 1, sa, sb, 0, na, nb, k0);
+    CUTHIP_WAIT_FRAGS(0, 0);
+    group(1, 0, sa, sb, 1, na, nb, k0);
+    CUTHIP_WAIT_FRAGS(1, 0);
+    group(2, 1, sa, sb, 2, na, nb, k0);
+    CUTHIP_WAIT_FRAGS(0, 0);
+    group(3, 0, sa, sb, 3, na, nb, k0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next slice has landed in (na, nb)
+    CUTHIP_WAIT_FRAGS(1, 0);                           // and this wave is done reading (sa, sb)
+    __syncthreads();
+  };
+
+#pragma unroll
+  for (int l = 0; l < NL; ++l) load_one(l, sA0, sB0, 0);
+#pragma unroll
+  for (int i = 0; i < MI; ++i) fa[1][i] = half8v{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) fb[1][j] = half8v{0, 0, 0, 0, 0, 0, 0, 0};
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  for (uint32_t t = 0; t < nsl; t += 2) {  // nsl is even (host check)
+    slice(sA0, sB0, sA1, sB1, t);
+    slice(sA1, sB1, sA0, sB0, t + 1);
+  }
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[1][i], fb[1][j], acc[i][j], 0, 0, 0);
+#undef CUTHIP_WAIT_FRAGS
+
+  // C tile: register r of lane l holds row 8*(r/4) + 4*(l>>5) + r%4, column l & 31 of its 32x32 block.
+  // Compile-time tile indices: a rolled loop would index the accumulators dynamically and copy them to scratch.
+  static_for<MI * NJ>([&](auto ij) {
+    constexpr int i = decltype(ij)::value / NJ, j = decltype(ij)::value % NJ;
+    const uint32_t col = n0 + wn * 128 + 32 * j + (lane & 31);
+    const uint32_t row0 = m0 + wm * (BM / 2) + 32 * i + 4 * (lane >> 5);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const uint32_t row = row0 + 8 * (r >> 2) + (r & 3);
+      if (row < p.M && col < p.N) store_out(p.C, p.epi, p.c_f16, (size_t)row * p.strideC + col, acc[i][j][r]);
+    }
+  });
+#endif
+}
+
+// fp32 [M, strideA] -> fp16 [M, K] (round to nearest even), 8 elements per thread
+__global__ void __launch_bounds__(256) cvt_rows_kernel(const float *src, half_t *dst, uint32_t K, uint32_t strideA,
+                                                       uint32_t chunks) {
+  uint32_t row = blockIdx.x / chunks, c = (blockIdx.x % chunks) * 256 + threadIdx.x;
+  if (c * 8 >= K) return;
+  const float *s = src + (size_t)row * strideA + c * 8;
+  f32x4 lo = *reinterpret_cast<const f32x4 *>(s), hi = *reinterpret_cast<const f32x4 *>(s + 4);
+  half8v o{(half_t)lo.x, (half_t)lo.y, (half_t)lo.z, (half_t)lo.w, (half_t)hi.x, (half_t)hi.y, (half_t)hi.z, (half_t)hi.w};
+  *reinterpret_cast<half8v *>(dst + (size_t)row * K + c * 8) = o;
+}
+
+template <int BM> static int launch_dense_bm(DenseParams p, hipStream_t stream) {
+  p.mtiles = (p.M + BM - 1) / BM;
+  p.ntiles = (p.N + kDBN - 1) / kDBN;
+  uint64_t grid = (uint64_t)p.mtiles * p.ntiles;
+  if (grid > 0x7FFFFFFFull) {
+    set_error("cuthip_matmul_gguf_ws: problem too large for one launch");
+    return CUTHIP_ERR_INVALID;
+  }
+  auto kern = gemm_dense_kernel<BM>;
+  hipLaunchKernelGGL(kern, dim3((uint32_t)grid), dim3(256), 0, stream, p);
+  return check_hip(hipGetLastError(), "dense gemm launch");
+}
+
+// Shapes the two-pass path takes: K a multiple of 128 (two LDS stages per loop trip), 16-byte aligned rows of A,
+// and operands small enough for 32-bit byte offsets.
+bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a_f16, const void *A) {
+  if (K % 128 != 0 || M == 0 || N == 0) return false;
+  if ((uint64_t)N * K * 2 >= (1ull << 32)) return false;
+  if (a_f16) {
+    if ((uintptr_t)A % 16 != 0 || strideA % 8 != 0 || (uint64_t)M * strideA * 2 >= (1ull << 32)) return false;
+  } else {
+    if ((uintptr_t)A % 16 != 0 || strideA % 4 != 0 || (uint64_t)M * K * 2 >= (1ull << 32)) return false;
+  }
+  return true;
+}
+
+size_t dense_gemm_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
+  size_t w = ((size_t)N * K * 2 + 255) & ~(size_t)255;
+  return w + (a_f16 ? 0 : (size_t)M * K * 2);
+}
+
+int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K,
+                      uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream) {
+  uint8_t *w16 = reinterpret_cast<uint8_t *>(workspace);
+  if (int rc = launch_dequant_any(fmt, W, w16, CUTHIP_F16, N, K, K, stream)) return rc;
+  DenseParams p;
+  p.W = w16;
+  p.A = reinterpret_cast<const uint8_t *>(A);
+  p.strideA = strideA;
+  if (!a_f16) {
+    half_t *a16 = reinterpret_cast<half_t *>(w16 + (((size_t)N * K * 2 + 255) & ~(size_t)255));
+    uint32_t chunks = (K / 8 + 255) / 256;
+    hipLaunchKernelGGL(cvt_rows_kernel, dim3(M * chunks), dim3(256), 0, stream, reinterpret_cast<const float *>(A), a16, K,
+                       strideA, chunks);
+    if (int rc = check_hip(hipGetLastError(), "activation convert launch")) return rc;
+    p.A = reinterpret_cast<const uint8_t *>(a16);
+    p.strideA = K;
+  }
+  p.C = C;
+  p.epi = epi;
+  p.M = M; p.N = N; p.K = K; p.strideC = strideC;
+  p.mtiles = p.ntiles = 0;
+  p.c_f16 = c_f16;
+  // 256-row tiles when they give every CU a workgroup, else 128-row tiles
+  uint64_t tiles256 = (uint64_t)((M + 255) / 256) * ((N + kDBN - 1) / kDBN);
+  if (tiles256 >= 256) return launch_dense_bm<256>(p, stream);
+  return launch_dense_bm<128>(p, stream);
+}
+
+}  // namespace cuthip

@@ -71,6 +71,11 @@ GemvShape pick_gemv_shape(uint32_t N, uint32_t nsteps, int mt) {
 int launch_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K, uint32_t N,
                 uint32_t strideA, uint32_t strideC, Epilogue epi, hipStream_t stream);
 
+bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a_f16, const void *A);
+size_t dense_gemm_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16);
+int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K,
+                      uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream);
+
 static int launch_gemv(int fmt, const GemvParams &p, hipStream_t stream) {
   switch (fmt) {
   case CUTHIP_Q8_0: return launch_fmt<CUTHIP_Q8_0>(p, stream);
@@ -82,9 +87,9 @@ static int launch_gemv(int fmt, const GemvParams &p, hipStream_t stream) {
 
 }  // namespace cuthip
 
-extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M,
-                                  uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue,
-                                  int epilogue_op, const void *D, int variant, void *stream) {
+// Argument checks shared by the matmul entry points: 0 = go on, 1 = empty problem (success), < 0 = error.
+static int check_matmul_args(int fmt, const void *W, const void *A, int a_dtype, const void *C, int c_dtype, uint32_t M,
+                             uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, const void *D) {
   using namespace cuthip;
   if (fmt < CUTHIP_Q8_0 || fmt > CUTHIP_Q6_K) {
     set_error("cuthip_matmul_gguf: unknown format %d", fmt);
@@ -94,7 +99,7 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
     set_error("cuthip_matmul_gguf: unsupported dtype (a %d, c %d)", a_dtype, c_dtype);
     return CUTHIP_ERR_INVALID;
   }
-  if (M == 0 || N == 0) return CUTHIP_OK;
+  if (M == 0 || N == 0) return 1;  // nothing to do
   if (K == 0 || K % fmt_elems(fmt) != 0) {
     set_error("cuthip_matmul_gguf: K (%u) must be a positive multiple of the block size %d", K, fmt_elems(fmt));
     return CUTHIP_ERR_INVALID;
@@ -119,6 +124,15 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
     set_error("cuthip_matmul_gguf: misaligned W or A pointer");
     return CUTHIP_ERR_INVALID;
   }
+  return 0;
+}
+
+extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M,
+                                  uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue,
+                                  int epilogue_op, const void *D, int variant, void *stream) {
+  using namespace cuthip;
+  if (int rc = check_matmul_args(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, D))
+    return rc > 0 ? CUTHIP_OK : rc;
   int nvar = cuthip_variant_count(CUTHIP_OP_MATMUL_GGUF);
   if (variant < -1 || variant >= nvar) {
     set_error("cuthip_matmul_gguf: unknown variant index %d (table has %d)", variant, nvar);
@@ -131,6 +145,10 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
   }
   // variant table: 0 streaming GEMV (M <= 8), 1 skinny passes of 32 rows, 2 LDS-tiled GEMM
   Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
+  if (variant == 4) {
+    set_error("cuthip_matmul_gguf: variant 4 (dequantize, then dense GEMM) needs a workspace: call cuthip_matmul_gguf_ws");
+    return CUTHIP_ERR_INVALID;
+  }
   if (variant == 0 && M > 8) {
     set_error("cuthip_matmul_gguf: variant 0 (GEMV) handles M <= 8, got M = %u", M);
     return CUTHIP_ERR_INVALID;
@@ -166,6 +184,42 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
   return launch_gemv(fmt, p, reinterpret_cast<hipStream_t>(stream));
 }
 extern "C" {
+
+size_t cuthip_matmul_gguf_workspace_bytes(int fmt, uint32_t M, uint32_t K, uint32_t N, int a_dtype) {
+  (void)fmt;
+  return cuthip::dense_gemm_workspace(M, K, N, a_dtype == CUTHIP_F16);
+}
+
+int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M, uint32_t K,
+                          uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D,
+                          int variant, void *workspace, size_t workspace_bytes, void *stream) {
+  using namespace cuthip;
+  if (variant != 4 && variant != -1)
+    return cuthip_matmul_gguf(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, variant,
+                              stream);
+  if (int rc = check_matmul_args(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, D))
+    return rc > 0 ? CUTHIP_OK : rc;
+  const int a_f16 = a_dtype == CUTHIP_F16;
+  const bool fits = dense_gemm_fits(M, K, N, strideA, a_f16, A);
+  const size_t need = dense_gemm_workspace(M, K, N, a_f16);
+  const bool ws_ok = workspace && (uintptr_t)workspace % 256 == 0 && workspace_bytes >= need;
+  if (variant == -1 && !(M >= 512 && fits && ws_ok))
+    return cuthip_matmul_gguf(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, -1,
+                              stream);
+  if (!fits) {
+    set_error("cuthip_matmul_gguf_ws: variant 4 needs K a multiple of 128, 16-byte aligned rows of A and operands below "
+              "4 GiB (M %u, K %u, N %u, strideA %u)", M, K, N, strideA);
+    return CUTHIP_ERR_INVALID;
+  }
+  if (!ws_ok) {
+    set_error("cuthip_matmul_gguf_ws: variant 4 needs a 256-byte aligned workspace of %zu bytes, got %zu", need,
+              workspace ? workspace_bytes : (size_t)0);
+    return CUTHIP_ERR_INVALID;
+  }
+  Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
+  return launch_dense_gemm(fmt, W, A, a_f16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC, epi, workspace,
+                           reinterpret_cast<hipStream_t>(stream));
+}
 
 int cuthip_matmul_gguf_pro(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t K, uint32_t N,
                            int epilogue, int epilogue_op, const void *D, int prologue, const float *norm_weight, float eps,

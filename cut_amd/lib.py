@@ -30,6 +30,7 @@ EXPORTS = [
     "cuthip_event_create", "cuthip_event_destroy", "cuthip_event_record", "cuthip_event_sync", "cuthip_event_elapsed_ms",
     "cuthip_variant_count", "cuthip_variant_default", "cuthip_variant_info", "cuthip_variant_lookup",
     "cuthip_dequant", "cuthip_matmul_gguf", "cuthip_matmul_gguf_pro",
+    "cuthip_matmul_gguf_workspace_bytes", "cuthip_matmul_gguf_ws",
     "cuthip_rmsnorm", "cuthip_rope_kv_write", "cuthip_attn_decode_workspace_bytes", "cuthip_attn_decode",
     "cuthip_silu_mul", "cuthip_argmax",
     "cuthip_matmul_sep_workspace_bytes", "cuthip_matmul_q8_sep", "cuthip_matmul_q4_sep",
@@ -88,6 +89,8 @@ def load() -> C.CDLL:
     lib.cuthip_variant_lookup.argtypes = [i, C.c_char_p]
     lib.cuthip_dequant.argtypes = [i, vp, vp, i, u32, u32, u32, vp]
     lib.cuthip_matmul_gguf.argtypes = [i, vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, i, vp]
+    lib.cuthip_matmul_gguf_workspace_bytes.argtypes = [i, u32, u32, u32, i]
+    lib.cuthip_matmul_gguf_ws.argtypes = [i, vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, i, vp, C.c_size_t, vp]
     f32 = C.c_float
     lib.cuthip_matmul_gguf_pro.argtypes = [i, vp, vp, i, vp, i, u32, u32, i, i, vp, i, vp, f32, vp]
     lib.cuthip_rmsnorm.argtypes = [vp, i, vp, vp, i, u32, u32, u32, f32, vp]
@@ -99,7 +102,8 @@ def load() -> C.CDLL:
     lib.cuthip_matmul_sep_workspace_bytes.argtypes = [u32, u32, u32]
     lib.cuthip_matmul_q8_sep.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, u32, i, i, vp, C.c_size_t, vp]
     lib.cuthip_matmul_q4_sep.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, u32, i, i, i, vp, C.c_size_t, vp]
-    sized = ("cuthip_attn_decode_workspace_bytes", "cuthip_matmul_sep_workspace_bytes")
+    sized = ("cuthip_attn_decode_workspace_bytes", "cuthip_matmul_sep_workspace_bytes",
+             "cuthip_matmul_gguf_workspace_bytes")
     for n in EXPORTS:
         if n != "cuthip_last_error" and n not in sized:
             getattr(lib, n).restype = i

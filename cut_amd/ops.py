@@ -55,9 +55,11 @@ def dequantize(raw: torch.Tensor, fmt, rows: int, cols: int, dtype: torch.dtype 
 
 def matmul_gguf(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: int, out_dtype: torch.dtype | None = None,
                 out: torch.Tensor | None = None, unary: str | None = None, binary: str | None = None,
-                d: torch.Tensor | None = None, variant: int = -1) -> torch.Tensor:
+                d: torch.Tensor | None = None, variant: int = -1, workspace: torch.Tensor | None = None) -> torch.Tensor:
     """C = A . dequant(W)^T.  a: [M, K] or [K] (fp32 or fp16); w_blocks: N rows
-    of K/blk GGUF blocks as a 1-byte device tensor."""
+    of K/blk GGUF blocks as a 1-byte device tensor.  With `workspace` (a device
+    byte tensor from matmul_gguf_workspace) the call goes through
+    cuthip_matmul_gguf_ws, which opens variant 4 (dequantize once, dense GEMM)."""
     f = _fmt(fmt)
     if a.dim() == 1:
         a2 = a.unsqueeze(0)
@@ -82,11 +84,23 @@ def matmul_gguf(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: int, ou
         if d is None or d.shape != out.shape or d.dtype != out.dtype or d.stride(0) != out.stride(0):
             raise _l.CutHipError("matmul: binary epilogue needs D with the shape, dtype and stride of C")
         epi, op, dptr = _l.EPI_BINARY, _l.BINARY[binary], d.data_ptr()
-    _l.check(_l.load().cuthip_matmul_gguf(
-        f, w_blocks.data_ptr(), a2.data_ptr(), _l.F16 if a2.dtype == torch.float16 else _l.F32, out.data_ptr(),
-        _l.F16 if out.dtype == torch.float16 else _l.F32, M, K, N, a2.stride(0), out.stride(0), epi, op, dptr,
-        variant, _stream_ptr()))
-    return out if a.dim() == 2 else out
+    adt = _l.F16 if a2.dtype == torch.float16 else _l.F32
+    cdt = _l.F16 if out.dtype == torch.float16 else _l.F32
+    if workspace is not None:
+        _l.check(_l.load().cuthip_matmul_gguf_ws(
+            f, w_blocks.data_ptr(), a2.data_ptr(), adt, out.data_ptr(), cdt, M, K, N, a2.stride(0), out.stride(0), epi, op,
+            dptr, variant, workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream_ptr()))
+    else:
+        _l.check(_l.load().cuthip_matmul_gguf(
+            f, w_blocks.data_ptr(), a2.data_ptr(), adt, out.data_ptr(), cdt, M, K, N, a2.stride(0), out.stride(0), epi, op,
+            dptr, variant, _stream_ptr()))
+    return out
+
+
+def matmul_gguf_workspace(fmt, M: int, K: int, N: int, a_dtype: torch.dtype, device) -> torch.Tensor:
+    """Scratch for the two-pass prefill matmul (variant 4): N*K fp16 (+ M*K fp16 for fp32 activations)."""
+    n = _l.load().cuthip_matmul_gguf_workspace_bytes(_fmt(fmt), M, K, N, _l.F16 if a_dtype == torch.float16 else _l.F32)
+    return torch.empty(max(int(n), 256), dtype=torch.uint8, device=device)
 
 
 # ---- operators between the matmuls of a decode step ---------------------------------------------------

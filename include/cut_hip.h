@@ -144,10 +144,30 @@ int cuthip_dequant(int fmt, const void *blocks, void *out, int out_dtype, uint32
  *          epilogue (residual add etc.), else NULL
  * K must be a multiple of the block size; fp32 accumulation throughout.
  * variant: index into the CUTHIP_OP_MATMUL_GGUF table, or -1 = choose by shape
- *          (M <= 8 -> streaming GEMV, else the LDS-tiled MFMA GEMM). */
+ *          (M <= 8 -> streaming GEMV, else the LDS-tiled MFMA GEMM); variant 4 needs
+ *          cuthip_matmul_gguf_ws. */
 int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M, uint32_t K,
                        uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D,
                        int variant, void *stream);
+
+/* The same matmul with a caller-provided device workspace, which opens variant 4
+ * (MatMulGgufDequantGemm) for large M: the weight tensor is dequantized once to
+ * fp16 in the workspace (cuthip_dequant's kernel) and multiplied by a dense fp16
+ * MFMA GEMM, two launches on `stream`, no allocation.  It replaces the M > 1
+ * default MatMulQ{4,8}CoopMatTiled.cu (MatMulOp.cpp:363-374), which re-decodes
+ * the weights for every tile of activations.
+ * workspace: device, 256-byte aligned, at least
+ *            cuthip_matmul_gguf_workspace_bytes(fmt, M, K, N, a_dtype) bytes
+ *            (N*K fp16, plus M*K fp16 when A is fp32); contents are scratch.
+ * variant  : 4 = the two-pass path (an error if K is not a multiple of 128, the
+ *            rows of A are not 16-byte aligned or the workspace is too small);
+ *            -1 = choose by shape: variant 4 when M >= 512 and it applies, else
+ *            as cuthip_matmul_gguf; 0..3 = as cuthip_matmul_gguf (workspace unused).
+ * Other arguments and numerics as cuthip_matmul_gguf. */
+size_t cuthip_matmul_gguf_workspace_bytes(int fmt, uint32_t M, uint32_t K, uint32_t N, int a_dtype);
+int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M, uint32_t K,
+                          uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D,
+                          int variant, void *workspace, size_t workspace_bytes, void *stream);
 
 /* The same matmul at batch 1 with the operator in front of it fused into the
  * staging of the activations, which saves a launch per use in a decode step

@@ -99,3 +99,119 @@ def test_prefill_shape_sampled(ops, M):
     want = oracle.matmul_gguf(fmt, Ws, A[rows].astype(np.float32), len(cols), f64=True)
     err = normwise_rel_err(got[np.ix_(rows, cols)], want)
     assert err < 8e-4, err  # fp16 weights (3e-4) and fp16 output rounding (3e-4)
+
+
+# ---- variant 4: dequantize once to an fp16 workspace, then a dense fp16 MFMA GEMM --------------------------------
+
+def gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=None, variant=4, **kw):
+    a = torch.from_numpy(A).cuda()
+    ws = ops.matmul_gguf_workspace(fmt, a.shape[0], K, N, a.dtype, "cuda")
+    ws.fill_(0xFF)  # the workspace is scratch: stale contents (NaN patterns) must not leak into C
+    c = ops.matmul_gguf(a, torch.from_numpy(W).cuda(), fmt, N, K, out_dtype=out_dtype, variant=variant, workspace=ws, **kw)
+    torch.cuda.synchronize()
+    return c.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("name", list(oracle.FORMATS))
+@pytest.mark.parametrize("M,N,K", [(1, 1, 256), (70, 130, 256), (300, 520, 1024), (512, 768, 512), (129, 2056, 256)])
+def test_dense_gemm_vs_oracle(ops, name, M, N, K):
+    """Ragged tiles on both sides (M, N not multiples of 128 / 256), one to eight slices of K, N-tile counts that are
+    and are not multiples of 8 (both workgroup orders), 128- and 256-row tiles."""
+    fmt = oracle.FORMATS[name]
+    W = quantized_weights(fmt, N, K, seed=41)
+    A = gauss_acts((M, K), seed=42, dtype=np.float16)
+    got = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32)
+    want = oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)
+    err = normwise_rel_err(got, want)
+    assert err < (TOL_GEMM if M * N >= 1024 else TOL), err  # a single output has no averaging over elements
+    assert normwise_rel_err(got, oracle.matmul_gguf(fmt, W, A.astype(np.float32), N)) < TOL
+
+
+def test_dense_gemm_256_row_tiles_and_single_launch_gemm_agree(ops):
+    """Enough tiles for the 256-row kernel (>= 256 tiles of 256 x 256), checked on sampled rows / columns against the
+    oracle and everywhere against the single-launch GEMM (fp16 weights and activations, fp32 accumulation in both)."""
+    fmt = oracle.Q4_K
+    M, N, K = 2100, 8200, 256
+    W = quantized_weights(fmt, N, K, seed=43)
+    A = gauss_acts((M, K), seed=44, dtype=np.float16)
+    got = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32)
+    ref = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=2)
+    # the dequant kernel rounds the reference's exact fp32 expression, the single-launch GEMM a contracted one: a few
+    # weights differ by one fp16 ulp
+    assert normwise_rel_err(got, ref) < 2e-4
+    assert np.all(np.abs(got - ref) <= 2e-3 * np.abs(ref) + 1e-3)
+    rng = np.random.default_rng(5)
+    rows = np.unique(np.concatenate([[0, 255, 256, M - 1], rng.integers(0, M, 12)]))
+    cols = np.unique(np.concatenate([[0, 255, 256, N - 1], rng.integers(0, N, 200)]))
+    Ws = np.ascontiguousarray(W.reshape(N, oracle.n_bytes(fmt, K))[cols]).reshape(-1)
+    want = oracle.matmul_gguf(fmt, Ws, A[rows].astype(np.float32), len(cols), f64=True)
+    assert normwise_rel_err(got[np.ix_(rows, cols)], want) < TOL_GEMM
+
+
+def test_dense_gemm_fp32_activations_strides_epilogues(ops):
+    fmt = oracle.Q6_K
+    M, N, K = 200, 300, 512
+    W = quantized_weights(fmt, N, K, seed=45)
+    A = gauss_acts((M, K), seed=46)
+    want = oracle.matmul_gguf(fmt, W, A, N, f64=True)
+    w = torch.from_numpy(W).cuda()
+    a_buf = torch.zeros((M, K + 8), dtype=torch.float32, device="cuda")
+    a_buf[:, :K] = torch.from_numpy(A).cuda()
+    c_buf = torch.full((M, N + 4), 7.0, dtype=torch.float32, device="cuda")
+    ws = ops.matmul_gguf_workspace(fmt, M, K, N, torch.float32, "cuda")
+    ops.matmul_gguf(a_buf[:, :K], w, fmt, N, K, out=c_buf[:, :N], variant=4, workspace=ws)
+    torch.cuda.synchronize()
+    plain = c_buf[:, :N].cpu().numpy()
+    assert normwise_rel_err(plain, want) < 8e-4  # activations and weights both rounded to fp16
+    assert torch.all(c_buf[:, N:] == 7.0)
+    D = gauss_acts((M, N), seed=47)
+    add = ops.matmul_gguf(torch.from_numpy(A).cuda(), w, fmt, N, K, binary="add", d=torch.from_numpy(D).cuda(), variant=4,
+                          workspace=ws)
+    silu = ops.matmul_gguf(torch.from_numpy(A).cuda(), w, fmt, N, K, unary="silu", variant=4, workspace=ws)
+    h = ops.matmul_gguf(torch.from_numpy(A).cuda(), w, fmt, N, K, out_dtype=torch.float16, variant=4, workspace=ws)
+    torch.cuda.synchronize()
+    assert np.array_equal(add.cpu().numpy(), plain + D)
+    assert np.allclose(silu.cpu().numpy(), plain / (1 + np.exp(-plain.astype(np.float64))), rtol=2e-6, atol=1e-7)
+    assert np.array_equal(h.float().cpu().numpy(), plain.astype(np.float16).astype(np.float32))
+
+
+def test_dense_gemm_refusals_and_automatic_choice(ops):
+    from cut_amd import lib
+    fmt = oracle.Q8_0
+    M, N, K = 64, 64, 192  # K not a multiple of 128
+    W = quantized_weights(fmt, N, K, seed=48)
+    A = gauss_acts((M, K), seed=49, dtype=np.float16)
+    with pytest.raises(lib.CutHipError, match="multiple of 128"):
+        gpu_matmul_ws(ops, fmt, W, A, N, K)
+    # the automatic choice falls back to the single-launch kernels for the same call
+    got = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=-1)
+    assert normwise_rel_err(got, oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)) < TOL_GEMM
+    K = 256
+    W = quantized_weights(fmt, N, K, seed=48)
+    A = gauss_acts((M, K), seed=49, dtype=np.float16)
+    a, w = torch.from_numpy(A).cuda(), torch.from_numpy(W).cuda()
+    with pytest.raises(lib.CutHipError, match="workspace"):
+        ops.matmul_gguf(a, w, fmt, N, K, variant=4, workspace=torch.empty(1024, dtype=torch.uint8, device="cuda"))
+    with pytest.raises(lib.CutHipError, match="cuthip_matmul_gguf_ws"):
+        ops.matmul_gguf(a, w, fmt, N, K, variant=4)
+    # automatic: M >= 512 with a workspace takes the two-pass path, and agrees with the single-launch GEMM
+    M = 600
+    A = gauss_acts((M, K), seed=50, dtype=np.float16)
+    auto = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=-1)
+    assert normwise_rel_err(auto, oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)) < TOL_GEMM
+
+
+@pytest.mark.parametrize("M,N,K", [(2048, 14336, 4096), (512, 14336, 4096), (2048, 4096, 14336)])
+def test_dense_gemm_prefill_shapes_sampled(ops, M, N, K):
+    """BASELINE config 5 geometry through the two-pass path, on a sample of output rows and columns."""
+    fmt = oracle.Q4_K
+    W = quantized_weights(fmt, N, K, seed=0)
+    A = gauss_acts((M, K), seed=1, dtype=np.float16)
+    got = gpu_matmul_ws(ops, fmt, W, A, N, K)  # fp16 out
+    rng = np.random.default_rng(3)
+    rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 14)]))
+    cols = np.unique(np.concatenate([np.arange(0, 32), np.arange(N - 32, N), rng.integers(0, N, 192)]))
+    Ws = np.ascontiguousarray(W.reshape(N, oracle.n_bytes(fmt, K))[cols]).reshape(-1)
+    want = oracle.matmul_gguf(fmt, Ws, A[rows].astype(np.float32), len(cols), f64=True)
+    err = normwise_rel_err(got[np.ix_(rows, cols)], want)
+    assert err < 8e-4, err
