@@ -143,6 +143,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (reference traffic for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--gemm-variant", type=int, default=4, choices=(2, 4),
+                    help="with --gemm-only: 4 = dequantize once + dense GEMM (default), 2 = single-launch GEMM")
     ap.add_argument("--gemm-only", type=int, default=0, metavar="M",
                     help="only run the Q4_K prefill GEMM (M x 4096) . (14336 x 4096)^T twelve times (target of rocprofv3 runs)")
     ap.add_argument("--dequant-only", action="store_true",
@@ -181,18 +183,20 @@ def main():
         wq = torch.from_numpy(make_q_weights("Q4_K", N_FF, N_EMBD, 0)).to(dev)
         a = torch.randn((M, N_EMBD), dtype=torch.float16, device=dev)
         c = torch.empty((M, N_FF), dtype=torch.float16, device=dev)
+        # variant 4 = dequantize once + dense GEMM (two launches, both inside the timed region); 2 = single launch
+        ws = ops.matmul_gguf_workspace("Q4_K", M, N_EMBD, N_FF, a.dtype, dev) if args.gemm_variant == 4 else None
         for _ in range(2):
-            ops.matmul_gguf(a, wq, "Q4_K", N_FF, N_EMBD, out=c)
+            ops.matmul_gguf(a, wq, "Q4_K", N_FF, N_EMBD, out=c, variant=args.gemm_variant, workspace=ws)
         torch.cuda.synchronize()
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         ev0.record()
         for _ in range(10):
-            ops.matmul_gguf(a, wq, "Q4_K", N_FF, N_EMBD, out=c)
+            ops.matmul_gguf(a, wq, "Q4_K", N_FF, N_EMBD, out=c, variant=args.gemm_variant, workspace=ws)
         ev1.record()
         torch.cuda.synchronize()
         us = ev0.elapsed_time(ev1) * 1e3 / 10
-        print(json.dumps({"gemm": f"Q4_K M={M} N={N_FF} K={N_EMBD}", "us_per_launch": round(us, 1),
-                          "TFLOPs": round(2.0 * M * N_FF * N_EMBD / us / 1e6, 1)}))
+        print(json.dumps({"gemm": f"Q4_K M={M} N={N_FF} K={N_EMBD}", "variant": args.gemm_variant,
+                          "us_per_matmul": round(us, 1), "TFLOPs": round(2.0 * M * N_FF * N_EMBD / us / 1e6, 1)}))
         return
     log(f"[bench] {info['name']} {info['arch']} CUs={info['compute_units']}")
 
@@ -295,12 +299,20 @@ def main():
             a = torch.randn((M, K), dtype=torch.float16, device=dev)
             c = torch.empty((M, N), dtype=torch.float16, device=dev)
 
-            def gemm(_s, a=a, wq=wq, c=c, N=N, K=K):
-                ops.matmul_gguf(a, wq, "Q4_K", N, K, out=c)
+            ws = ops.matmul_gguf_workspace("Q4_K", M, K, N, a.dtype, dev)
+
+            def gemm(_s, a=a, wq=wq, c=c, N=N, K=K, ws=ws):  # with a workspace: dequantize once + dense GEMM
+                ops.matmul_gguf(a, wq, "Q4_K", N, K, out=c, workspace=ws)
+
+            def gemm1(_s, a=a, wq=wq, c=c, N=N, K=K):  # the single-launch GEMM on the blocks
+                ops.matmul_gguf(a, wq, "Q4_K", N, K, out=c, variant=2)
             wall_g, ev_g, _ = timed_graph(torch, gemm, 10, 2)
             tflops = 2.0 * M * N * K * 10 / (ev_g * 1e-3) / 1e12
             extras[f"q4k_prefill_gemm_M{M}_N{N}_K{K}_TFLOPs"] = round(tflops, 1)
             extras[f"q4k_prefill_gemm_M{M}_N{N}_K{K}_pct_of_f16_mfma_peak"] = round(tflops / 2500.0 * 100, 1)
+            wall_g, ev_g, _ = timed_graph(torch, gemm1, 10, 2)
+            extras[f"q4k_prefill_gemm_M{M}_N{N}_K{K}_single_launch_TFLOPs"] = round(2.0 * M * N * K * 10 / (ev_g * 1e-3) / 1e12, 1)
+            del ws
             del wq, a, c
     result["extras"] = extras
 

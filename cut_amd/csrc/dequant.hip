@@ -108,7 +108,7 @@ template <> struct Deq8<CUTHIP_Q6_K> {
 template <int FMT, bool F16OUT, bool VEC>
 __global__ void __launch_bounds__(256)
 dequant_kernel(const uint8_t *__restrict__ blocks, void *__restrict__ out, uint32_t cols, uint32_t out_stride,
-               uint32_t chunks_per_row, size_t row_bytes) {
+               uint32_t chunks_per_row, size_t row_bytes, int keep_cached) {
   uint32_t row = blockIdx.x / chunks_per_row;
   uint32_t chunk = blockIdx.x - row * chunks_per_row;
   uint32_t col = (chunk * 256u + threadIdx.x) * 8u;
@@ -128,7 +128,12 @@ dequant_kernel(const uint8_t *__restrict__ blocks, void *__restrict__ out, uint3
     uint16_t *dst = reinterpret_cast<uint16_t *>(out) + idx;
     if (VEC) {
       u32x4 v{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
-      __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst));
+      // streaming stores for a tensor that leaves the GPU's caches alone; plain stores when the next kernel on
+      // the stream reads the output back (the fp16 workspace of the two-pass matmul fits the last-level cache)
+      if (keep_cached)
+        *reinterpret_cast<u32x4 *>(dst) = v;
+      else
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst));
     } else {
 #pragma unroll
       for (int i = 0; i < 8; ++i) dst[i] = (uint16_t)h[i];
@@ -147,7 +152,7 @@ dequant_kernel(const uint8_t *__restrict__ blocks, void *__restrict__ out, uint3
 
 template <int FMT>
 static int launch_dequant(const void *blocks, void *out, int out_dtype, uint32_t rows, uint32_t cols,
-                          uint32_t out_stride, hipStream_t stream) {
+                          uint32_t out_stride, hipStream_t stream, int keep_cached = 0) {
   size_t row_bytes = (size_t)(cols / Fmt<FMT>::elems) * Fmt<FMT>::bytes;
   // A contiguous output is one long row: no partially filled workgroups.
   if (out_stride == cols && (uint64_t)rows * cols < (1ull << 32)) {
@@ -168,7 +173,8 @@ static int launch_dequant(const void *blocks, void *out, int out_dtype, uint32_t
   dim3 g((uint32_t)grid), b(256);
   const uint8_t *src = reinterpret_cast<const uint8_t *>(blocks);
 #define CUTHIP_LAUNCH(F16, VEC) \
-  hipLaunchKernelGGL((dequant_kernel<FMT, F16, VEC>), g, b, 0, stream, src, out, cols, out_stride, chunks, row_bytes)
+  hipLaunchKernelGGL((dequant_kernel<FMT, F16, VEC>), g, b, 0, stream, src, out, cols, out_stride, chunks, row_bytes, \
+                     keep_cached)
   if (f16) {
     if (vec) CUTHIP_LAUNCH(true, true); else CUTHIP_LAUNCH(true, false);
   } else {
@@ -178,14 +184,15 @@ static int launch_dequant(const void *blocks, void *out, int out_dtype, uint32_t
   return check_hip(hipGetLastError(), "dequant launch");
 }
 
-// Internal entry for other translation units (the two-pass prefill matmul): arguments already validated.
+// Internal entry for other translation units (the two-pass prefill matmul): arguments already validated; the
+// output is written with plain stores because the caller reads it back at once.
 int launch_dequant_any(int fmt, const void *blocks, void *out, int out_dtype, uint32_t rows, uint32_t cols,
                        uint32_t out_stride, hipStream_t stream) {
   switch (fmt) {
-  case CUTHIP_Q8_0: return launch_dequant<CUTHIP_Q8_0>(blocks, out, out_dtype, rows, cols, out_stride, stream);
-  case CUTHIP_Q4_0: return launch_dequant<CUTHIP_Q4_0>(blocks, out, out_dtype, rows, cols, out_stride, stream);
-  case CUTHIP_Q4_K: return launch_dequant<CUTHIP_Q4_K>(blocks, out, out_dtype, rows, cols, out_stride, stream);
-  default: return launch_dequant<CUTHIP_Q6_K>(blocks, out, out_dtype, rows, cols, out_stride, stream);
+  case CUTHIP_Q8_0: return launch_dequant<CUTHIP_Q8_0>(blocks, out, out_dtype, rows, cols, out_stride, stream, 1);
+  case CUTHIP_Q4_0: return launch_dequant<CUTHIP_Q4_0>(blocks, out, out_dtype, rows, cols, out_stride, stream, 1);
+  case CUTHIP_Q4_K: return launch_dequant<CUTHIP_Q4_K>(blocks, out, out_dtype, rows, cols, out_stride, stream, 1);
+  default: return launch_dequant<CUTHIP_Q6_K>(blocks, out, out_dtype, rows, cols, out_stride, stream, 1);
   }
 }
 

@@ -203,7 +203,7 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   const bool fits = dense_gemm_fits(M, K, N, strideA, a_f16, A);
   const size_t need = dense_gemm_workspace(M, K, N, a_f16);
   const bool ws_ok = workspace && (uintptr_t)workspace % 256 == 0 && workspace_bytes >= need;
-  if (variant == -1 && !(M >= 512 && fits && ws_ok))
+  if (variant == -1 && !(M >= 1024 && fits && ws_ok))  // below ~1000 rows the single-launch GEMM is faster
     return cuthip_matmul_gguf(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, -1,
                               stream);
   if (!fits) {

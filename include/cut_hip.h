@@ -161,7 +161,7 @@ int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void 
  *            (N*K fp16, plus M*K fp16 when A is fp32); contents are scratch.
  * variant  : 4 = the two-pass path (an error if K is not a multiple of 128, the
  *            rows of A are not 16-byte aligned or the workspace is too small);
- *            -1 = choose by shape: variant 4 when M >= 512 and it applies, else
+ *            -1 = choose by shape: variant 4 when M >= 1024 and it applies, else
  *            as cuthip_matmul_gguf; 0..3 = as cuthip_matmul_gguf (workspace unused).
  * Other arguments and numerics as cuthip_matmul_gguf. */
 size_t cuthip_matmul_gguf_workspace_bytes(int fmt, uint32_t M, uint32_t K, uint32_t N, int a_dtype);

@@ -194,8 +194,8 @@ def test_dense_gemm_refusals_and_automatic_choice(ops):
         ops.matmul_gguf(a, w, fmt, N, K, variant=4, workspace=torch.empty(1024, dtype=torch.uint8, device="cuda"))
     with pytest.raises(lib.CutHipError, match="cuthip_matmul_gguf_ws"):
         ops.matmul_gguf(a, w, fmt, N, K, variant=4)
-    # automatic: M >= 512 with a workspace takes the two-pass path, and agrees with the single-launch GEMM
-    M = 600
+    # automatic: M >= 1024 with a workspace takes the two-pass path
+    M = 1100
     A = gauss_acts((M, K), seed=50, dtype=np.float16)
     auto = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=-1)
     assert normwise_rel_err(auto, oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)) < TOL_GEMM
