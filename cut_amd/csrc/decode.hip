@@ -291,13 +291,39 @@ __global__ void __launch_bounds__(1024) argmax_kernel(const void *x, int x_f16, 
   const uint32_t tid = threadIdx.x;
   float best = -INFINITY;
   uint32_t idx = 0xFFFFFFFFu;
-  for (uint32_t i = tid; i < n; i += 1024) {
-    float v = ld_act(x, x_f16, i);
+  auto consider = [&](float v, uint32_t i) {
     if (v > best || (v == best && i < idx)) {
       best = v;
       idx = i;
     }
+  };
+  // 16-byte loads, four per thread in flight: with one scalar load per trip every trip pays a memory latency
+  uint32_t done = 0;
+  if ((uintptr_t)x % 16 == 0) {
+    const uint32_t per = x_f16 ? 8 : 4, nvec = n / per;
+    const u32x4 *xv = reinterpret_cast<const u32x4 *>(x);
+    for (uint32_t b = tid; b < nvec; b += 4 * 1024) {
+      u32x4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = xv[min(b + u * 1024, nvec - 1)];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const uint32_t vi = b + u * 1024;
+        if (vi >= nvec) break;
+        if (x_f16) {
+          half8_t h = __builtin_bit_cast(half8_t, v[u]);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) consider((float)h[e], vi * 8 + e);
+        } else {
+          f32x4 f = __builtin_bit_cast(f32x4, v[u]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) consider(f[e], vi * 4 + e);
+        }
+      }
+    }
+    done = nvec * per;
   }
+  for (uint32_t i = done + tid; i < n; i += 1024) consider(ld_act(x, x_f16, i), i);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
     float ov = __shfl_xor(best, o);

@@ -114,6 +114,17 @@ def test_silu_mul_and_argmax(ops):
     ops.argmax(dev(logits.astype(np.float16)[:1000]), idx)
     torch.cuda.synchronize()
     assert int(idx.item()) == int(np.argmax(logits.astype(np.float16)[:1000]))
+    # vector body and scalar tail, unaligned base, maximum in the tail / at the ends, fewer elements than one vector
+    big = dev(logits)
+    for dt in (np.float32, np.float16):
+        for n, off, hot in ((128256, 0, 128255), (4099, 1, 4098), (4099, 3, 0), (70001, 2, 69999), (3, 1, 2), (1, 0, 0),
+                            (8191, 0, 4096)):
+            h = rng.standard_normal(n + off).astype(dt)
+            h[off + hot] = 40.0
+            ops.argmax(dev(h)[off:], idx)
+            torch.cuda.synchronize()
+            assert int(idx.item()) == hot, (dt, n, off)
+    del big
 
 
 def _oracle_step(cfg, layers_h, out_norm, head, x, pos, kc, vc, cos_t, sin_t):
