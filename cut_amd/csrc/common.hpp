@@ -134,6 +134,13 @@ __device__ inline void store_out(void *C, const Epilogue &e, int c_f16, size_t i
     reinterpret_cast<float *>(C)[idx] = v;
 }
 
+__device__ inline void store_plain(void *C, int c_f16, size_t idx, float v) {
+  if (c_f16)
+    reinterpret_cast<half_t *>(C)[idx] = (half_t)v;
+  else
+    reinterpret_cast<float *>(C)[idx] = v;
+}
+
 void set_error(const char *fmt, ...);
 int check_hip(hipError_t e, const char *what);
 

@@ -36,6 +36,14 @@ Rows8Shape pick_rows8_shape(uint32_t N, uint32_t nsteps) {
   return Rows8Shape{groups >= 8192 ? 8 : 4, kw};
 }
 
+#define CUTHIP_EXTERN_PAIR(FA, FB) \
+  extern template bool launch_rows8_pair_fmt<FA, FB>(const GemvParams &, const GemvParams &, hipStream_t, int *);
+CUTHIP_EXTERN_PAIR(CUTHIP_Q4_K, CUTHIP_Q4_K)
+CUTHIP_EXTERN_PAIR(CUTHIP_Q4_K, CUTHIP_Q6_K)
+CUTHIP_EXTERN_PAIR(CUTHIP_Q6_K, CUTHIP_Q4_K)
+CUTHIP_EXTERN_PAIR(CUTHIP_Q6_K, CUTHIP_Q6_K)
+#undef CUTHIP_EXTERN_PAIR
+
 static int launch_rows8_any(int fmt, const GemvParams &p, hipStream_t stream, bool *taken) {
   *taken = true;
   switch (fmt) {
@@ -108,12 +116,17 @@ static int check_matmul_args(int fmt, const void *W, const void *A, int a_dtype,
     set_error("cuthip_matmul_gguf: null device pointer");
     return CUTHIP_ERR_INVALID;
   }
-  if (strideA < K || strideC < N) {
-    set_error("cuthip_matmul_gguf: strideA (%u) < K (%u) or strideC (%u) < N (%u)", strideA, K, strideC, N);
+  if (epilogue < CUTHIP_EPI_NONE || epilogue > CUTHIP_EPI_SWIGLU_PAIRS) {
+    set_error("cuthip_matmul_gguf: unknown epilogue %d", epilogue);
     return CUTHIP_ERR_INVALID;
   }
-  if (epilogue < CUTHIP_EPI_NONE || epilogue > CUTHIP_EPI_BINARY) {
-    set_error("cuthip_matmul_gguf: unknown epilogue %d", epilogue);
+  const uint32_t n_out = epilogue == CUTHIP_EPI_SWIGLU_PAIRS ? N / 2 : N;
+  if (strideA < K || strideC < n_out) {
+    set_error("cuthip_matmul_gguf: strideA (%u) < K (%u) or strideC (%u) < N (%u)", strideA, K, strideC, n_out);
+    return CUTHIP_ERR_INVALID;
+  }
+  if (epilogue == CUTHIP_EPI_SWIGLU_PAIRS && (N % 2 != 0 || M > 8)) {
+    set_error("cuthip_matmul_gguf: the SwiGLU row-pair epilogue needs an even N and M <= 8 (N %u, M %u)", N, M);
     return CUTHIP_ERR_INVALID;
   }
   if (epilogue == CUTHIP_EPI_BINARY && !D) {
@@ -145,6 +158,10 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
   }
   // variant table: 0 streaming GEMV (M <= 8), 1 skinny passes of 32 rows, 2 LDS-tiled GEMM
   Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
+  if (epilogue == CUTHIP_EPI_SWIGLU_PAIRS && variant != -1 && variant != 3) {
+    set_error("cuthip_matmul_gguf: the SwiGLU row-pair epilogue exists in variant 3 only (got variant %d)", variant);
+    return CUTHIP_ERR_INVALID;
+  }
   if (variant == 4) {
     set_error("cuthip_matmul_gguf: variant 4 (dequantize, then dense GEMM) needs a workspace: call cuthip_matmul_gguf_ws");
     return CUTHIP_ERR_INVALID;
@@ -176,14 +193,54 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
     bool taken = false;
     int rc = launch_rows8_any(fmt, p, reinterpret_cast<hipStream_t>(stream), &taken);
     if (taken) return rc;
-    if (variant == 3) {
+    if (variant == 3 || epilogue == CUTHIP_EPI_SWIGLU_PAIRS) {
       set_error("cuthip_matmul_gguf: variant 3 needs M <= 8 and the activations to fit in LDS (M = %u, K = %u)", M, K);
       return CUTHIP_ERR_INVALID;
     }
   }
+  if (epilogue == CUTHIP_EPI_SWIGLU_PAIRS) {
+    set_error("cuthip_matmul_gguf: the SwiGLU row-pair epilogue exists in variant 3 only (got variant %d)", variant);
+    return CUTHIP_ERR_INVALID;
+  }
   return launch_gemv(fmt, p, reinterpret_cast<hipStream_t>(stream));
 }
 extern "C" {
+
+int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, int fmt_b, const void *Wb, uint32_t Nb,
+                            void *Cb, const void *A, int a_dtype, int c_dtype, uint32_t K, void *stream) {
+  using namespace cuthip;
+  if (int rc = check_matmul_args(fmt_a, Wa, A, a_dtype, Ca, c_dtype, 1, K, Na, K, Na, CUTHIP_EPI_NONE, nullptr))
+    return rc > 0 ? cuthip_matmul_gguf(fmt_b, Wb, A, a_dtype, Cb, c_dtype, 1, K, Nb, K, Nb, 0, 0, nullptr, -1, stream) : rc;
+  if (int rc = check_matmul_args(fmt_b, Wb, A, a_dtype, Cb, c_dtype, 1, K, Nb, K, Nb, CUTHIP_EPI_NONE, nullptr))
+    return rc > 0 ? cuthip_matmul_gguf(fmt_a, Wa, A, a_dtype, Ca, c_dtype, 1, K, Na, K, Na, 0, 0, nullptr, -1, stream) : rc;
+  auto params = [&](int fmt, const void *W, uint32_t N, void *C) {
+    GemvParams p;
+    p.W = reinterpret_cast<const uint8_t *>(W);
+    p.A = A;
+    p.C = C;
+    p.epi = Epilogue{CUTHIP_EPI_NONE, 0, nullptr};
+    p.M = 1; p.K = K; p.N = N; p.strideA = K; p.strideC = N;
+    p.nsteps = (K + 255) / 256;
+    p.row_bytes = (uint32_t)((uint64_t)(K / fmt_elems(fmt)) * fmt_bytes(fmt));
+    p.a_f16 = a_dtype == CUTHIP_F16;
+    p.c_f16 = c_dtype == CUTHIP_F16;
+    return p;
+  };
+  if ((uint64_t)(K / fmt_elems(fmt_a)) * fmt_bytes(fmt_a) <= 0xFFFFFFFFull && (uint64_t)Na + Nb <= 0x7FFFFFFFull) {
+    const GemvParams pa = params(fmt_a, Wa, Na, Ca), pb = params(fmt_b, Wb, Nb, Cb);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    int rc = CUTHIP_OK;
+    bool taken = false;
+    if (fmt_a == CUTHIP_Q4_K && fmt_b == CUTHIP_Q4_K) taken = launch_rows8_pair_fmt<CUTHIP_Q4_K, CUTHIP_Q4_K>(pa, pb, s, &rc);
+    else if (fmt_a == CUTHIP_Q4_K && fmt_b == CUTHIP_Q6_K) taken = launch_rows8_pair_fmt<CUTHIP_Q4_K, CUTHIP_Q6_K>(pa, pb, s, &rc);
+    else if (fmt_a == CUTHIP_Q6_K && fmt_b == CUTHIP_Q4_K) taken = launch_rows8_pair_fmt<CUTHIP_Q6_K, CUTHIP_Q4_K>(pa, pb, s, &rc);
+    else if (fmt_a == CUTHIP_Q6_K && fmt_b == CUTHIP_Q6_K) taken = launch_rows8_pair_fmt<CUTHIP_Q6_K, CUTHIP_Q6_K>(pa, pb, s, &rc);
+    if (taken) return rc;
+  }
+  // other formats or shapes: the same two products as two launches
+  if (int rc = cuthip_matmul_gguf(fmt_a, Wa, A, a_dtype, Ca, c_dtype, 1, K, Na, K, Na, 0, 0, nullptr, -1, stream)) return rc;
+  return cuthip_matmul_gguf(fmt_b, Wb, A, a_dtype, Cb, c_dtype, 1, K, Nb, K, Nb, 0, 0, nullptr, -1, stream);
+}
 
 size_t cuthip_matmul_gguf_workspace_bytes(int fmt, uint32_t M, uint32_t K, uint32_t N, int a_dtype) {
   (void)fmt;
@@ -194,7 +251,7 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
                           uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D,
                           int variant, void *workspace, size_t workspace_bytes, void *stream) {
   using namespace cuthip;
-  if (variant != 4 && variant != -1)
+  if ((variant != 4 && variant != -1) || epilogue == CUTHIP_EPI_SWIGLU_PAIRS)
     return cuthip_matmul_gguf(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, variant,
                               stream);
   if (int rc = check_matmul_args(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, D))

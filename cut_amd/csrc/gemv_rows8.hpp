@@ -499,7 +499,7 @@ template <int SUBK, int THREADS, int MT, int XR, bool PRO> struct XStage {
 // subnormal operands: a quarter of the issue cycles of the matrix-core path,
 // whose 32 A-rows would be 7/8 padding); MT > 1 goes through the matrix core.
 template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO>
-__global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_kernel(GemvParams p) {
+__device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t bid) {
   using S = Rows8<FMT>;
   constexpr bool DOT = MT <= kRows8DotMax;
   constexpr int WAVES = RWG * KW, THREADS = 64 * WAVES;
@@ -523,7 +523,7 @@ __global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_kernel(GemvParams
   float *sxs = reinterpret_cast<float *>(lds + (size_t)MT * xrow * 2);
   float *nrm = sxs + MT * sxrow;   // [MT][WAVES] per-wave shares of sum(x^2) (RMSNorm prologue)
 
-  const uint32_t n0 = (blockIdx.x * RWG + rg) * 8u;
+  const uint32_t n0 = (bid * RWG + rg) * 8u;
   const uint32_t n = min(n0 + (uint32_t)r8, p.N - 1);
   const uint8_t *row = p.W + (size_t)n * p.row_bytes;
   const uint32_t sb = (uint32_t)(((uint64_t)p.nsteps * kw) / KW);
@@ -644,8 +644,19 @@ __global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_kernel(GemvParams
     }
     writer = c.g == 0;
   }
+  // SwiGLU over row pairs: weight rows 2i / 2i+1 are gate_i / up_i, C[m, i] = silu(gate) * up.  The partner row
+  // sits four lanes up (same piece, same K half); in the folded path it is the next thread.
+  const bool swiglu = p.epi.kind == CUTHIP_EPI_SWIGLU_PAIRS;
   if (KW == 1) {
-    if (writer && n0 + r8 < p.N) {
+    if (swiglu) {
+#pragma unroll
+      for (int q = 0; q < RQ; ++q) {
+        float up = __shfl_down(out[q], 4);
+        int m = DOT ? q : 2 * q + c.kg;
+        if (writer && (r8 & 1) == 0 && n0 + r8 + 1 < p.N && m < (int)p.M)
+          store_plain(p.C, p.c_f16, (size_t)m * p.strideC + (n0 + r8) / 2, apply_unary(CUTHIP_UNARY_SILU, out[q]) * up);
+      }
+    } else if (writer && n0 + r8 < p.N) {
 #pragma unroll
       for (int q = 0; q < RQ; ++q) {
         int m = DOT ? q : 2 * q + c.kg;
@@ -665,15 +676,35 @@ __global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_kernel(GemvParams
     __syncthreads();
     if (tid < RWG * MT * 8) {
       int rgi = tid / (MT * 8), m = (tid / 8) % MT, rr = tid & 7;
-      uint32_t nn = (blockIdx.x * RWG + rgi) * 8u + rr;
-      if (m < (int)p.M && nn < p.N) {
-        float v = 0.0f;
+      uint32_t nn = (bid * RWG + rgi) * 8u + rr;
+      float v = 0.0f;
 #pragma unroll
-        for (int k = 0; k < KW; ++k) v += red[((rgi * KW + k) * MT + m) * 8 + rr];
+      for (int k = 0; k < KW; ++k) v += red[((rgi * KW + k) * MT + m) * 8 + rr];
+      if (swiglu) {
+        float up = __shfl_down(v, 1);
+        if (m < (int)p.M && (rr & 1) == 0 && nn + 1 < p.N)
+          store_plain(p.C, p.c_f16, (size_t)m * p.strideC + nn / 2, apply_unary(CUTHIP_UNARY_SILU, v) * up);
+      } else if (m < (int)p.M && nn < p.N) {
         store_out(p.C, p.epi, p.c_f16, (size_t)m * p.strideC + nn, v);
       }
     }
   }
+}
+
+template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO>
+__global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_kernel(GemvParams p) {
+  rows8_body<FMT, MT, RWG, KW, D, XWANT, PRO>(p, blockIdx.x);
+}
+
+// Two weight tensors (formats FA, FB) against the same batch-1 activations in one launch: workgroups
+// [0, blocks_a) take the rows of the first, the rest the rows of the second.  Saves a launch and a kernel
+// start where a small projection (w_v) sits next to a larger one (w_q | w_k) of another format.
+template <int FA, int FB, int RWG, int KW, int D, int XWANT>
+__global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_pair_kernel(GemvParams pa, GemvParams pb, uint32_t blocks_a) {
+  if (blockIdx.x < blocks_a)
+    rows8_body<FA, 1, RWG, KW, D, XWANT, false>(pa, blockIdx.x);
+  else
+    rows8_body<FB, 1, RWG, KW, D, XWANT, false>(pb, blockIdx.x - blocks_a);
 }
 
 template <int FMT> static size_t rows8_lds_bytes(const GemvParams &p, int mt) {
@@ -720,6 +751,23 @@ template <int FMT, int MT> static int launch_rows8_shape(const GemvParams &p, in
   return launch_rows8<FMT, MT, 1, 8, D, 4>(p, stream);
 }
 
+template <int FA, int FB, int RWG, int KW, int D, int XWANT>
+static int launch_rows8_pair(const GemvParams &pa, const GemvParams &pb, hipStream_t stream) {
+  size_t la = rows8_lds_bytes<FA>(pa, 1), lb = rows8_lds_bytes<FB>(pb, 1), red = (size_t)RWG * KW * 8 * 4;
+  size_t lds = la > lb ? la : lb;
+  if (red > lds) lds = red;
+  auto kern = gemv_rows8_pair_kernel<FA, FB, RWG, KW, D, XWANT>;
+  if (lds > 64 * 1024) {
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                           "hipFuncSetAttribute"))
+      return rc;
+  }
+  uint32_t blocks_a = ((pa.N + 7) / 8 + RWG - 1) / RWG, blocks_b = ((pb.N + 7) / 8 + RWG - 1) / RWG;
+  hipLaunchKernelGGL(kern, dim3(blocks_a + blocks_b), dim3(64 * RWG * KW), lds, stream, pa, pb, blocks_a);
+  return check_hip(hipGetLastError(), "gemv pair launch");
+}
+
 struct Rows8Shape { int rwg, kw; };
 Rows8Shape pick_rows8_shape(uint32_t N, uint32_t nsteps);
 
@@ -736,6 +784,20 @@ template <int FMT> int launch_rows8_fmt(const GemvParams &p, hipStream_t stream)
   if (p.M <= 2) return launch_rows8_shape<FMT, 2>(p, s.rwg, s.kw, stream);
   if (p.M <= 4) return launch_rows8_shape<FMT, 4>(p, s.rwg, s.kw, stream);
   return launch_rows8_shape<FMT, 8>(p, s.rwg, s.kw, stream);
+}
+
+// Pair launch for the K-quant formats at the shapes a decode step uses; returns false (nothing launched) for
+// anything else, and the caller issues two launches.
+template <int FA, int FB> bool launch_rows8_pair_fmt(const GemvParams &pa, const GemvParams &pb, hipStream_t stream, int *rc) {
+  if (pa.M != 1 || pb.M != 1 || pa.K != pb.K || pa.pro || pb.pro) return false;
+  if (rows8_lds_bytes<FA>(pa, 1) > 96 * 1024 || rows8_lds_bytes<FB>(pb, 1) > 96 * 1024) return false;
+  Rows8Shape s = pick_rows8_shape(pa.N + pb.N, pa.nsteps);
+  constexpr int D = 4;
+  if (s.kw == 1 && s.rwg < 8) *rc = launch_rows8_pair<FA, FB, 4, 1, D, 2>(pa, pb, stream);
+  else if (s.kw == 2) *rc = launch_rows8_pair<FA, FB, 2, 2, D, 4>(pa, pb, stream);
+  else if (s.kw == 4 && pa.nsteps <= 16) *rc = launch_rows8_pair<FA, FB, 1, 4, D, 2>(pa, pb, stream);
+  else return false;
+  return true;
 }
 
 }  // namespace cuthip

@@ -45,19 +45,32 @@ class DecodeConfig:
         return self.n_kv_heads * self.head_dim
 
 
+def interleave_gate_up(gate_up: torch.Tensor, ffn: int) -> torch.Tensor:
+    """[gate rows | up rows] of GGUF blocks -> rows gate_0, up_0, gate_1, up_1, ... (the layout the SwiGLU row-pair
+    epilogue reads); rows are whole numbers of blocks, so this is a permutation of byte ranges."""
+    rb = gate_up.numel() // (2 * ffn)
+    g = gate_up.view(2, ffn, rb)
+    return torch.stack((g[0], g[1]), dim=1).reshape(-1).contiguous()
+
+
 class DecodeStep:
     """weights: per layer a dict with GGUF-block device tensors 'qk' ([q_dim + kv_dim, hidden], q rows first),
     'v', 'o', 'gate_up' ([2 * ffn, hidden], gate rows first), 'down' and fp32 'attn_norm', 'ffn_norm';
     plus 'out_norm' (fp32) and 'head' at the top level."""
 
     def __init__(self, cfg: DecodeConfig, layers: list[dict], out_norm: torch.Tensor, head: torch.Tensor, device="cuda:0",
-                 fuse: int = 0):
-        """fuse: 0 = every operator is its own launch; 1 = SiLU(gate) * up runs inside the staging of w_down;
+                 fuse: int = 3):
+        """fuse: 3 (default) = SiLU(gate) * up runs in the epilogue of the gate+up matmul (the producer), whose rows
+        are interleaved gate_0, up_0, gate_1, ... for it: 'gate_up' is re-laid out once, here, and the layer dicts are
+        copied; 0 = every operator is its own launch; 1 = SiLU(gate) * up runs inside the staging of w_down;
         2 = RMSNorm is fused into the following matmuls as well.  Level 2 saves three more launches per layer but
         every workgroup of those matmuls then stages fp32 x and the norm weights (4x the bytes of fp16 x), which
         lengthens their start-up; likewise every workgroup of w_down recomputes SiLU * up for its whole input.  On
         MI355X both levels measured slower than separate launches (2.43 / 2.70 / 2.85 ms per token for 0 / 1 / 2 at
-        the 8B shape), so 0 is the default; the fused entry point stays for shapes where launches dominate."""
+        the 8B shape); fusing into the producer has no such cost.  The fused entry point stays for shapes where
+        launches dominate."""
+        if fuse == 3:
+            layers = [dict(L, gate_up=interleave_gate_up(L["gate_up"], cfg.ffn)) for L in layers]
         self.cfg, self.layers, self.out_norm, self.head, self.fuse = cfg, layers, out_norm, head, fuse
         dev = torch.device(device)
         c = cfg
@@ -90,14 +103,15 @@ class DecodeStep:
     def step(self) -> None:
         """Consumes self.x (the embedding of the current token), leaves logits and the arg-max token."""
         c = self.cfg
-        if self.fuse >= 2:
+        if self.fuse == 2:
             return self._step_fused()
         for i, L in enumerate(self.layers):
             ops.rmsnorm(self.x, L["attn_norm"], c.eps, out=self.xn.view(1, -1))
             # (running v beside q+k on a second stream was measured slower: the fork / join nodes of the graph cost
             # more than the 6 us the small matmul takes)
-            ops.matmul_gguf(self.xn, L["qk"], c.fmt_attn, c.q_dim + c.kv_dim, c.hidden, out=self.qk.view(1, -1))
-            ops.matmul_gguf(self.xn, L["v"], c.fmt_v, c.kv_dim, c.hidden, out=self.v.view(1, -1))
+            # q | k and v in one launch although their formats differ
+            ops.matmul_gguf_pair(self.xn, L["qk"], c.fmt_attn, c.q_dim + c.kv_dim, self.qk, L["v"], c.fmt_v, c.kv_dim, self.v,
+                                 c.hidden)
             ops.rope_kv_write(self.qk[:c.q_dim], self.qk[c.q_dim:], self.v, self.params, self.cos_t, self.sin_t,
                               self.k_cache[i], self.v_cache[i], c.head_dim, self.q_rot)
             ops.attn_decode(self.q_rot, self.k_cache[i], self.v_cache[i], self.params, c.n_heads, c.n_kv_heads, c.head_dim,
@@ -105,6 +119,12 @@ class DecodeStep:
             ops.matmul_gguf(self.attn, L["o"], c.fmt_attn, c.hidden, c.q_dim, out=self.x.view(1, -1), binary="add",
                             d=self.x.view(1, -1))
             ops.rmsnorm(self.x, L["ffn_norm"], c.eps, out=self.xn.view(1, -1))
+            if self.fuse == 3:
+                ops.matmul_gguf(self.xn, L["gate_up"], c.fmt_ffn, 2 * c.ffn, c.hidden, out=self.act.view(1, -1),
+                                swiglu_pairs=True)
+                ops.matmul_gguf(self.act, L["down"], c.fmt_ffn, c.hidden, c.ffn, out=self.x.view(1, -1), binary="add",
+                                d=self.x.view(1, -1))
+                continue
             ops.matmul_gguf(self.xn, L["gate_up"], c.fmt_ffn, 2 * c.ffn, c.hidden, out=self.gu.view(1, -1))
             if self.fuse >= 1:
                 ops.matmul_gguf_pro(self.gu, L["down"], c.fmt_ffn, c.hidden, c.ffn, self.x, "swiglu", binary="add", d=self.x)

@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(_HERE, "libcut_hip.so")
 Q8_0, Q4_0, Q4_K, Q6_K = 0, 1, 2, 3
 F32, F16 = 0, 1
 OP_DEQUANT, OP_MATMUL_GGUF, OP_MATMUL_Q8, OP_MATMUL_Q4 = 0, 1, 2, 3
-EPI_NONE, EPI_UNARY, EPI_BINARY = 0, 1, 2
+EPI_NONE, EPI_UNARY, EPI_BINARY, EPI_SWIGLU_PAIRS = 0, 1, 2, 3
 UNARY = {"silu": 0, "relu": 1, "gelu_tanh": 2, "sigmoid": 3, "tanh": 4, "neg": 5}
 BINARY = {"add": 0, "sub": 1, "mul": 2, "div": 3, "min": 4, "max": 5}
 FORMATS = {"Q8_0": Q8_0, "Q4_0": Q4_0, "Q4_K": Q4_K, "Q6_K": Q6_K}
@@ -30,7 +30,7 @@ EXPORTS = [
     "cuthip_event_create", "cuthip_event_destroy", "cuthip_event_record", "cuthip_event_sync", "cuthip_event_elapsed_ms",
     "cuthip_variant_count", "cuthip_variant_default", "cuthip_variant_info", "cuthip_variant_lookup",
     "cuthip_dequant", "cuthip_matmul_gguf", "cuthip_matmul_gguf_pro",
-    "cuthip_matmul_gguf_workspace_bytes", "cuthip_matmul_gguf_ws",
+    "cuthip_matmul_gguf_workspace_bytes", "cuthip_matmul_gguf_ws", "cuthip_matmul_gguf_pair",
     "cuthip_rmsnorm", "cuthip_rope_kv_write", "cuthip_attn_decode_workspace_bytes", "cuthip_attn_decode",
     "cuthip_silu_mul", "cuthip_argmax",
     "cuthip_matmul_sep_workspace_bytes", "cuthip_matmul_q8_sep", "cuthip_matmul_q4_sep",
@@ -91,6 +91,7 @@ def load() -> C.CDLL:
     lib.cuthip_matmul_gguf.argtypes = [i, vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, i, vp]
     lib.cuthip_matmul_gguf_workspace_bytes.argtypes = [i, u32, u32, u32, i]
     lib.cuthip_matmul_gguf_ws.argtypes = [i, vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, i, vp, C.c_size_t, vp]
+    lib.cuthip_matmul_gguf_pair.argtypes = [i, vp, u32, vp, i, vp, u32, vp, vp, i, i, u32, vp]
     f32 = C.c_float
     lib.cuthip_matmul_gguf_pro.argtypes = [i, vp, vp, i, vp, i, u32, u32, i, i, vp, i, vp, f32, vp]
     lib.cuthip_rmsnorm.argtypes = [vp, i, vp, vp, i, u32, u32, u32, f32, vp]

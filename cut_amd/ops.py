@@ -55,11 +55,13 @@ def dequantize(raw: torch.Tensor, fmt, rows: int, cols: int, dtype: torch.dtype 
 
 def matmul_gguf(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: int, out_dtype: torch.dtype | None = None,
                 out: torch.Tensor | None = None, unary: str | None = None, binary: str | None = None,
-                d: torch.Tensor | None = None, variant: int = -1, workspace: torch.Tensor | None = None) -> torch.Tensor:
+                d: torch.Tensor | None = None, variant: int = -1, workspace: torch.Tensor | None = None,
+                swiglu_pairs: bool = False) -> torch.Tensor:
     """C = A . dequant(W)^T.  a: [M, K] or [K] (fp32 or fp16); w_blocks: N rows
     of K/blk GGUF blocks as a 1-byte device tensor.  With `workspace` (a device
     byte tensor from matmul_gguf_workspace) the call goes through
-    cuthip_matmul_gguf_ws, which opens variant 4 (dequantize once, dense GEMM)."""
+    cuthip_matmul_gguf_ws, which opens variant 4 (dequantize once, dense GEMM).
+    swiglu_pairs: weight rows 2i / 2i+1 are gate_i / up_i and the result is [M, N/2] = silu(gate) * up (M <= 8)."""
     f = _fmt(fmt)
     if a.dim() == 1:
         a2 = a.unsqueeze(0)
@@ -76,9 +78,11 @@ def matmul_gguf(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: int, ou
         raise _l.CutHipError("matmul: weight tensor too small for [N, K]")
     odt = out_dtype or a2.dtype
     if out is None:
-        out = torch.empty((M, N), dtype=odt, device=a.device)
+        out = torch.empty((M, N // 2 if swiglu_pairs else N), dtype=odt, device=a.device)
     epi, op, dptr = _l.EPI_NONE, 0, None
-    if unary is not None:
+    if swiglu_pairs:
+        epi = _l.EPI_SWIGLU_PAIRS
+    elif unary is not None:
         epi, op = _l.EPI_UNARY, _l.UNARY[unary]
     elif binary is not None:
         if d is None or d.shape != out.shape or d.dtype != out.dtype or d.stride(0) != out.stride(0):
@@ -95,6 +99,22 @@ def matmul_gguf(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: int, ou
             f, w_blocks.data_ptr(), a2.data_ptr(), adt, out.data_ptr(), cdt, M, K, N, a2.stride(0), out.stride(0), epi, op,
             dptr, variant, _stream_ptr()))
     return out
+
+
+def matmul_gguf_pair(a: torch.Tensor, wa: torch.Tensor, fmt_a, Na: int, out_a: torch.Tensor, wb: torch.Tensor, fmt_b, Nb: int,
+                     out_b: torch.Tensor, K: int) -> None:
+    """out_a = a . dequant(wa)^T and out_b = a . dequant(wb)^T for one activation vector a [K], in one launch where the
+    formats allow it (cuthip_matmul_gguf_pair)."""
+    fa, fb = _fmt(fmt_a), _fmt(fmt_b)
+    if a.numel() != K or a.dtype not in (torch.float32, torch.float16) or not a.is_contiguous():
+        raise _l.CutHipError("matmul_pair: A must be a contiguous float32/float16 vector of K elements")
+    if wa.numel() < n_bytes(fa, Na, K) or wb.numel() < n_bytes(fb, Nb, K):
+        raise _l.CutHipError("matmul_pair: weight tensor too small for [N, K]")
+    if out_a.dtype != out_b.dtype or out_a.numel() != Na or out_b.numel() != Nb or not (out_a.is_contiguous() and out_b.is_contiguous()):
+        raise _l.CutHipError("matmul_pair: outputs must be contiguous [Na] and [Nb] of one dtype")
+    _l.check(_l.load().cuthip_matmul_gguf_pair(
+        fa, wa.data_ptr(), Na, out_a.data_ptr(), fb, wb.data_ptr(), Nb, out_b.data_ptr(), a.data_ptr(), _dt(a), _dt(out_a), K,
+        _stream_ptr()))
 
 
 def matmul_gguf_workspace(fmt, M: int, K: int, N: int, a_dtype: torch.dtype, device) -> torch.Tensor:

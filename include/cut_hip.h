@@ -42,7 +42,16 @@ typedef enum { CUTHIP_OP_DEQUANT = 0, CUTHIP_OP_MATMUL_GGUF = 1, CUTHIP_OP_MATMU
 
 /* Fused epilogues of the matmul (operators/impl/matmul/MatMulQ8Common.cuh:58-109;
  * MatMulOp.h:14 "MatMulFusion { None, Unary, Binary }"). */
-typedef enum { CUTHIP_EPI_NONE = 0, CUTHIP_EPI_UNARY = 1, CUTHIP_EPI_BINARY = 2 } cuthip_epilogue;
+typedef enum {
+  CUTHIP_EPI_NONE = 0,
+  CUTHIP_EPI_UNARY = 1,
+  CUTHIP_EPI_BINARY = 2,
+  /* SwiGLU over interleaved rows: weight rows 2i and 2i+1 are gate_i and up_i, C is [M, N/2] with
+   * C[m, i] = silu(A . gate_i) * (A . up_i): the fused gate+up matmul, SiLU and BinaryMul of the runner
+   * (interface/runner/llama/llama.cpp:1832-1857) in one launch.  M <= 8 only (the 8-row GEMV), N even;
+   * strideC counts the N/2 outputs; epilogue_op and D unused. */
+  CUTHIP_EPI_SWIGLU_PAIRS = 3
+} cuthip_epilogue;
 typedef enum { CUTHIP_UNARY_SILU = 0, CUTHIP_UNARY_RELU = 1, CUTHIP_UNARY_GELU_TANH = 2, CUTHIP_UNARY_SIGMOID = 3, CUTHIP_UNARY_TANH = 4, CUTHIP_UNARY_NEG = 5 } cuthip_unary_op;
 typedef enum { CUTHIP_BINARY_ADD = 0, CUTHIP_BINARY_SUB = 1, CUTHIP_BINARY_MUL = 2, CUTHIP_BINARY_DIV = 3, CUTHIP_BINARY_MIN = 4, CUTHIP_BINARY_MAX = 5 } cuthip_binary_op;
 
@@ -168,6 +177,18 @@ size_t cuthip_matmul_gguf_workspace_bytes(int fmt, uint32_t M, uint32_t K, uint3
 int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M, uint32_t K,
                           uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D,
                           int variant, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Two batch-1 matmuls on the same activations in one launch:
+ *   Ca[Na] = A . dequant(Wa)^T,  Cb[Nb] = A . dequant(Wb)^T,  A [K].
+ * For the q/k and v projections of a decode step, whose weights differ in format
+ * (Q4_K and Q6_K in the common GGUF mixes) and so cannot be concatenated like
+ * gate and up; the reference fuses wqkv only when the loader could concatenate
+ * them and otherwise issues one matmul per projection
+ * (interface/runner/llama/llama.cpp:1710-1756).  One launch for the K-quant
+ * formats at decode shapes, otherwise the same two products as two launches.
+ * No epilogue; dtypes and alignment as cuthip_matmul_gguf. */
+int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, int fmt_b, const void *Wb, uint32_t Nb,
+                            void *Cb, const void *A, int a_dtype, int c_dtype, uint32_t K, void *stream);
 
 /* The same matmul at batch 1 with the operator in front of it fused into the
  * staging of the activations, which saves a launch per use in a decode step

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import normwise_rel_err
+from helpers import gauss_acts, normwise_rel_err, quantized_weights
 
 torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
@@ -176,7 +176,7 @@ def test_matmul_with_fused_prologues(ops, name, N, K):
     assert normwise_rel_err(out.cpu().numpy() - res, want) < 4e-4
 
 
-@pytest.mark.parametrize("fuse", [0, 1, 2])
+@pytest.mark.parametrize("fuse", [0, 1, 2, 3])
 def test_small_decode_step_against_oracle_chain(ops, fuse):
     from cut_amd.decode import DecodeConfig, DecodeStep
     cfg = DecodeConfig(hidden=512, n_layers=2, n_heads=8, n_kv_heads=2, head_dim=64, ffn=1024, vocab=2048, max_ctx=64)
@@ -223,3 +223,38 @@ def test_small_decode_step_against_oracle_chain(ops, fuse):
         g.replay()
         torch.cuda.synchronize()
         assert np.array_equal(step.logits.cpu().numpy(), got)
+
+
+@pytest.mark.parametrize("name", ["Q4_K", "Q6_K", "Q8_0", "Q4_0"])
+@pytest.mark.parametrize("M,ffn,K", [(1, 14336, 4096), (1, 44, 512), (2, 300, 1024), (8, 64, 2048), (1, 4, 256), (1, 1024, 256)])
+def test_swiglu_row_pair_epilogue(ops, name, M, ffn, K):
+    """Interleaved gate / up rows, SiLU(gate) * up in the matmul's epilogue, against the oracle's two matmuls and
+    silu_mul; covers the direct (one K range) and folded (split K) epilogues and every batch size class."""
+    from cut_amd.decode import interleave_gate_up
+    fmt = oracle.FORMATS[name]
+    W = quantized_weights(fmt, 2 * ffn, K, seed=70)           # [gate rows | up rows]
+    A = gauss_acts((M, K), seed=71, dtype=np.float16)
+    w_il = interleave_gate_up(dev(W), ffn)
+    got = ops.matmul_gguf(dev(A), w_il, fmt, 2 * ffn, K, out_dtype=torch.float32, swiglu_pairs=True)
+    torch.cuda.synchronize()
+    assert tuple(got.shape) == (M, ffn)
+    gu = oracle.matmul_gguf(fmt, W, A.astype(np.float32), 2 * ffn, f64=True).astype(np.float32)
+    want = np.stack([oracle.silu_mul(gu[m]) for m in range(M)])
+    assert normwise_rel_err(got.cpu().numpy(), want) < 5e-5
+    # and the permutation itself: row 2i of the interleaved tensor is gate row i, row 2i+1 is up row i
+    rb = oracle.n_bytes(fmt, K)
+    il = w_il.cpu().numpy().reshape(2 * ffn, rb)
+    Wr = W.reshape(2, ffn, rb)
+    assert np.array_equal(il[0::2], Wr[0]) and np.array_equal(il[1::2], Wr[1])
+
+
+def test_swiglu_row_pair_epilogue_refusals(ops):
+    from cut_amd import lib
+    fmt = oracle.Q4_K
+    W = dev(quantized_weights(fmt, 64, 256, seed=72))
+    with pytest.raises(lib.CutHipError, match="M <= 8"):
+        ops.matmul_gguf(dev(gauss_acts((9, 256), seed=1, dtype=np.float16)), W, fmt, 64, 256, swiglu_pairs=True)
+    with pytest.raises(lib.CutHipError, match="variant 3 only"):
+        ops.matmul_gguf(dev(gauss_acts((2, 256), seed=1, dtype=np.float16)), W, fmt, 64, 256, swiglu_pairs=True, variant=2)
+    with pytest.raises(lib.CutHipError, match="even N"):
+        ops.matmul_gguf(dev(gauss_acts((1, 256), seed=1, dtype=np.float16)), W, fmt, 63, 256, swiglu_pairs=True)

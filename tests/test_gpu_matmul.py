@@ -217,3 +217,29 @@ def test_rows8_refuses_what_does_not_fit_and_auto_falls_back(ops):
         gpu_matmul(ops, fmt, W, A, N, K, variant=3)
     want = oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)
     assert normwise_rel_err(gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32), want) < TOL_F16_ACT
+
+
+@pytest.mark.parametrize("fa,fb", [("Q4_K", "Q6_K"), ("Q6_K", "Q4_K"), ("Q4_K", "Q4_K"), ("Q6_K", "Q6_K"), ("Q8_0", "Q4_K"),
+                                   ("Q4_0", "Q8_0")])
+@pytest.mark.parametrize("Na,Nb,K", [(5120, 1024, 4096), (70, 9, 1024), (1, 1, 256), (20000, 8, 2048)])
+def test_pair_launch_equals_two_matmuls(ops, fa, fb, Na, Nb, K):
+    """Two weight tensors on one activation vector: one launch for the K-quant pairs at decode shapes, two launches
+    otherwise; either way each output must match the oracle and the single matmul (same kernel body; only the
+    split of K may differ)."""
+    A = gauss_acts((1, K), seed=60, dtype=np.float16)
+    a = torch.from_numpy(A).cuda()
+    outs, singles = [], []
+    ws = [torch.from_numpy(quantized_weights(oracle.FORMATS[f], n, K, seed=61 + i)).cuda() for i, (f, n) in
+          enumerate(((fa, Na), (fb, Nb)))]
+    ca = torch.full((Na,), 7.0, dtype=torch.float32, device="cuda")
+    cb = torch.full((Nb,), 7.0, dtype=torch.float32, device="cuda")
+    ops.matmul_gguf_pair(a.view(-1), ws[0], oracle.FORMATS[fa], Na, ca, ws[1], oracle.FORMATS[fb], Nb, cb, K)
+    torch.cuda.synchronize()
+    for f, n, w, c in ((fa, Na, ws[0], ca), (fb, Nb, ws[1], cb)):
+        fmt = oracle.FORMATS[f]
+        want = oracle.matmul_gguf(fmt, w.cpu().numpy(), A.astype(np.float32), n, f64=True)
+        assert normwise_rel_err(c.cpu().numpy()[None, :], want) < (TOL_F16_ACT if n > 4 else 1e-4)
+        single = ops.matmul_gguf(a, w, fmt, n, K, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        # the pair may pick another split of K than the single launch (it sizes the grid for both tensors)
+        assert normwise_rel_err(c.cpu().numpy()[None, :], single.cpu().numpy()) < 2e-6
