@@ -105,10 +105,10 @@ template <> struct Deq8<CUTHIP_Q6_K> {
   }
 };
 
-template <int FMT, bool F16OUT, bool VEC>
+template <int FMT, bool F16OUT, bool VEC, bool KEEP = false>
 __global__ void __launch_bounds__(256)
 dequant_kernel(const uint8_t *__restrict__ blocks, void *__restrict__ out, uint32_t cols, uint32_t out_stride,
-               uint32_t chunks_per_row, size_t row_bytes, int keep_cached) {
+               uint32_t chunks_per_row, size_t row_bytes) {
   uint32_t row = blockIdx.x / chunks_per_row;
   uint32_t chunk = blockIdx.x - row * chunks_per_row;
   uint32_t col = (chunk * 256u + threadIdx.x) * 8u;
@@ -130,7 +130,7 @@ dequant_kernel(const uint8_t *__restrict__ blocks, void *__restrict__ out, uint3
       u32x4 v{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
       // streaming stores for a tensor that leaves the GPU's caches alone; plain stores when the next kernel on
       // the stream reads the output back (the fp16 workspace of the two-pass matmul fits the last-level cache)
-      if (keep_cached)
+      if (KEEP)
         *reinterpret_cast<u32x4 *>(dst) = v;
       else
         __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst));
@@ -173,9 +173,10 @@ static int launch_dequant(const void *blocks, void *out, int out_dtype, uint32_t
   dim3 g((uint32_t)grid), b(256);
   const uint8_t *src = reinterpret_cast<const uint8_t *>(blocks);
 #define CUTHIP_LAUNCH(F16, VEC) \
-  hipLaunchKernelGGL((dequant_kernel<FMT, F16, VEC>), g, b, 0, stream, src, out, cols, out_stride, chunks, row_bytes, \
-                     keep_cached)
-  if (f16) {
+  hipLaunchKernelGGL((dequant_kernel<FMT, F16, VEC>), g, b, 0, stream, src, out, cols, out_stride, chunks, row_bytes)
+  if (f16 && vec && keep_cached) {
+    hipLaunchKernelGGL((dequant_kernel<FMT, true, true, true>), g, b, 0, stream, src, out, cols, out_stride, chunks, row_bytes);
+  } else if (f16) {
     if (vec) CUTHIP_LAUNCH(true, true); else CUTHIP_LAUNCH(true, false);
   } else {
     if (vec) CUTHIP_LAUNCH(false, true); else CUTHIP_LAUNCH(false, false);
