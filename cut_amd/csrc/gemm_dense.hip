@@ -12,9 +12,10 @@
 // each wave a (BM/2) x 128 sub-tile in fp32 accumulators (AGPRs), K walked in slices
 // of 64.  Both operands go global -> LDS with global_load_lds_dwordx4 (no VGPR
 // round trip): one instruction fills 8 tile rows x 128 bytes = 1 KB of LDS, lane i
-// at byte 16 i; the lane reads the 16-byte chunk (i & 7) ^ (i >> 3) of its row, so
-// that the LDS image is XOR-swizzled and the MFMA fragment reads (lane l: row l & 31,
-// chunk 2 s + (l >> 5) of k-step s) spread over all banks.  Two LDS stages; the
+// at byte 16 i; the lane fetches the chunk of its row that belongs at that position
+// of an XOR-swizzled image (chunk c of row r sits at c ^ ((r >> 1) & 7)), so that the
+// MFMA fragment reads (lane l: row l & 31, chunk 2 s + (l >> 5) of k-step s) spread
+// over all 64 banks.  Two LDS stages; the
 // loads of slice t+1 are in flight while slice t is multiplied.
 //
 // Issue order is explicit.  A wave has the SIMD to itself (one wave per SIMD), so a
@@ -90,7 +91,10 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
 
   // copy assignment: load v of wave w fills the 8-row group 4 v + w of its tile
   uint32_t aoff[NLA], boff[kDBN / 32];
-  const uint32_t chunk = ((lane & 7) ^ (lane >> 3)) * 16;
+  // tile row r keeps its 16-byte chunk c at position c ^ ((r >> 1) & 7): the 16 lanes the LDS serves per cycle
+  // (16 consecutive rows, one chunk index) then cover all 64 banks.  For the row 8 g + (lane >> 3) of 8-row group
+  // g = 4 v + wave that key is (4 (wave & 1) + (lane >> 4)) & 7, the same for every v.
+  const uint32_t chunk = ((lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7)) * 16;
 #pragma unroll
   for (int v = 0; v < NLA; ++v) {
     uint32_t r = min(m0 + 8 * (4 * v + wave) + (lane >> 3), p.M - 1);
@@ -118,7 +122,7 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
   const uint32_t arow = (wm * (BM / 2) + (lane & 31)) * 128, brow = (wn * 128 + (lane & 31)) * 128;
   uint32_t xs[4];
 #pragma unroll
-  for (int s = 0; s < 4; ++s) xs[s] = ((2 * s + (lane >> 5)) ^ (lane & 7)) * 16;
+  for (int s = 0; s < 4; ++s) xs[s] = ((2 * s + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
 
   half8v fa[2][MI], fb[2][NJ];
   // Waits until at most n of this wave's LDS reads are outstanding; the fragment registers pass through the
