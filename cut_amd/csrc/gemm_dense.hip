@@ -56,6 +56,8 @@ struct DenseParams {
   Epilogue epi;
   uint32_t M, N, K, strideA, strideC, mtiles, ntiles;
   int c_f16;
+  uint32_t ksplit, kper;  // K is cut into ksplit ranges of kper (a multiple of 128); a workgroup multiplies one range
+  float *partial;         // ksplit > 1: fp32 [ksplit][M][N] partial products instead of C
 };
 
 constexpr int kDBN = 256, kDBK = 64;
@@ -76,7 +78,8 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
 
   // XCD-aware tile order: ids id, id+8, id+16, ... share an XCD and its L2; give
   // them the M-tiles of the same weight panels.
-  uint32_t id = blockIdx.x, mt, nt;
+  const uint32_t tiles = p.mtiles * p.ntiles, split = blockIdx.x / tiles;
+  uint32_t id = blockIdx.x - split * tiles, mt, nt;
   if (p.ntiles % 8 == 0) {
     uint32_t xcd = id & 7, slot = id >> 3;
     nt = (slot / p.mtiles) * 8 + xcd;
@@ -152,12 +155,12 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
     }
   };
 
-  const uint32_t nsl = p.K / kDBK, klast = p.K - kDBK;
+  const uint32_t kbeg = split * p.kper, nsl = p.kper / kDBK, klast = kbeg + p.kper - kDBK;
   // One slice, entered right after a barrier with nothing in flight.  Set 1 holds the fragments of the previous
   // slice's last k-step; its MFMAs run under the first fragment reads of this slice.  The loads of the slice
   // after the last one re-read the last slice (never used) instead of branching around the MFMAs.
   auto slice = [&](uint8_t *sa, uint8_t *sb, uint8_t *na, uint8_t *nb, uint32_t t) {
-    const uint32_t k0 = min((t + 1) * kDBK, klast);
+    const uint32_t k0 = min(kbeg + (t + 1) * kDBK, klast);
     group(0, 1, sa, sb, 0, na, nb, k0);
     CUTHIP_WAIT_FRAGS(0, 0);
     group(1, 0, sa, sb, 1, na, nb, k0);
@@ -171,7 +174,7 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
   };
 
 #pragma unroll
-  for (int l = 0; l < NL; ++l) load_one(l, sA0, sB0, 0);
+  for (int l = 0; l < NL; ++l) load_one(l, sA0, sB0, kbeg);
 #pragma unroll
   for (int i = 0; i < MI; ++i) fa[1][i] = half8v{0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
@@ -198,7 +201,12 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const uint32_t row = row0 + 8 * (r >> 2) + (r & 3);
-      if (row < p.M && col < p.N) store_out(p.C, p.epi, p.c_f16, (size_t)row * p.strideC + col, acc[i][j][r]);
+      if (row < p.M && col < p.N) {
+        if (p.ksplit > 1)
+          p.partial[((size_t)split * p.M + row) * p.N + col] = acc[i][j][r];
+        else
+          store_out(p.C, p.epi, p.c_f16, (size_t)row * p.strideC + col, acc[i][j][r]);
+      }
     }
   });
 #endif
@@ -215,10 +223,21 @@ __global__ void __launch_bounds__(256) cvt_rows_kernel(const float *src, half_t 
   *reinterpret_cast<half8v *>(dst + (size_t)row * K + c * 8) = o;
 }
 
+// C = epilogue(sum over the K ranges of the fp32 partial products), one output per thread
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *partial, uint32_t ksplit, uint32_t M, uint32_t N,
+                                                            void *C, uint32_t strideC, Epilogue epi, int c_f16) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, mn = (size_t)M * N;
+  if (i >= mn) return;
+  float v = 0.0f;
+  for (uint32_t s = 0; s < ksplit; ++s) v += partial[s * mn + i];
+  const uint32_t row = (uint32_t)(i / N), col = (uint32_t)(i - (size_t)row * N);
+  store_out(C, epi, c_f16, (size_t)row * strideC + col, v);
+}
+
 template <int BM> static int launch_dense_bm(DenseParams p, hipStream_t stream) {
   p.mtiles = (p.M + BM - 1) / BM;
   p.ntiles = (p.N + kDBN - 1) / kDBN;
-  uint64_t grid = (uint64_t)p.mtiles * p.ntiles;
+  uint64_t grid = (uint64_t)p.mtiles * p.ntiles * p.ksplit;
   if (grid > 0x7FFFFFFFull) {
     set_error("cuthip_matmul_gguf_ws: problem too large for one launch");
     return CUTHIP_ERR_INVALID;
@@ -241,9 +260,32 @@ bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a
   return true;
 }
 
+// Tile height and number of K ranges: 256-row tiles when they give every CU a workgroup, else 128-row tiles if
+// those do, else 256-row tiles with K split (partials in the workspace, summed by a second kernel).
+struct DenseShape { int bm; uint32_t ksplit; };
+static DenseShape pick_dense_shape(uint32_t M, uint32_t K, uint32_t N) {
+  const uint64_t nt = (N + kDBN - 1) / kDBN, tiles256 = (uint64_t)((M + 255) / 256) * nt, tiles128 = (uint64_t)((M + 127) / 128) * nt;
+  if (tiles256 >= 256) return DenseShape{256, 1};
+  if (tiles128 >= 224) return DenseShape{128, 1};
+  uint32_t s = 1;
+  while (s < 8 && tiles256 * s < 192 && K % (2 * s * 128) == 0) s *= 2;
+  if (s == 1) return DenseShape{tiles128 > tiles256 ? 128 : 256, 1};
+  return DenseShape{256, s};
+}
+
+static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
 size_t dense_gemm_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
-  size_t w = ((size_t)N * K * 2 + 255) & ~(size_t)255;
-  return w + (a_f16 ? 0 : (size_t)M * K * 2);
+  DenseShape sh = pick_dense_shape(M, K, N);
+  return align256((size_t)N * K * 2) + align256(a_f16 ? 0 : (size_t)M * K * 2) +
+         (sh.ksplit > 1 ? (size_t)sh.ksplit * M * N * 4 : 0);
+}
+
+// true where the two-pass path beats the single-launch GEMM: from about a thousand rows, or earlier when the
+// single-launch kernel's 128 x 128 tiles would leave most of the chip idle
+bool dense_gemm_preferred(uint32_t M, uint32_t N) {
+  if (M >= 1024) return true;
+  return M >= 256 && (uint64_t)((M + 127) / 128) * ((N + 127) / 128) < 200;
 }
 
 int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K,
@@ -255,7 +297,7 @@ int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C,
   p.A = reinterpret_cast<const uint8_t *>(A);
   p.strideA = strideA;
   if (!a_f16) {
-    half_t *a16 = reinterpret_cast<half_t *>(w16 + (((size_t)N * K * 2 + 255) & ~(size_t)255));
+    half_t *a16 = reinterpret_cast<half_t *>(w16 + align256((size_t)N * K * 2));
     uint32_t chunks = (K / 8 + 255) / 256;
     hipLaunchKernelGGL(cvt_rows_kernel, dim3(M * chunks), dim3(256), 0, stream, reinterpret_cast<const float *>(A), a16, K,
                        strideA, chunks);
@@ -268,10 +310,18 @@ int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C,
   p.M = M; p.N = N; p.K = K; p.strideC = strideC;
   p.mtiles = p.ntiles = 0;
   p.c_f16 = c_f16;
-  // 256-row tiles when they give every CU a workgroup, else 128-row tiles
-  uint64_t tiles256 = (uint64_t)((M + 255) / 256) * ((N + kDBN - 1) / kDBN);
-  if (tiles256 >= 256) return launch_dense_bm<256>(p, stream);
-  return launch_dense_bm<128>(p, stream);
+  const DenseShape sh = pick_dense_shape(M, K, N);
+  p.ksplit = sh.ksplit;
+  p.kper = K / sh.ksplit;
+  p.partial = reinterpret_cast<float *>(w16 + align256((size_t)N * K * 2) + align256(a_f16 ? 0 : (size_t)M * K * 2));
+  if (int rc = sh.bm == 256 ? launch_dense_bm<256>(p, stream) : launch_dense_bm<128>(p, stream)) return rc;
+  if (sh.ksplit > 1) {
+    const uint64_t mn = (uint64_t)M * N;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((uint32_t)((mn + 255) / 256)), dim3(256), 0, stream, p.partial, sh.ksplit, M,
+                       N, C, strideC, epi, c_f16);
+    return check_hip(hipGetLastError(), "split-K reduce launch");
+  }
+  return CUTHIP_OK;
 }
 
 }  // namespace cuthip

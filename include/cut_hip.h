@@ -167,10 +167,13 @@ int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void 
  * the weights for every tile of activations.
  * workspace: device, 256-byte aligned, at least
  *            cuthip_matmul_gguf_workspace_bytes(fmt, M, K, N, a_dtype) bytes
- *            (N*K fp16, plus M*K fp16 when A is fp32); contents are scratch.
+ *            (N*K fp16, plus M*K fp16 when A is fp32, plus fp32 partial products
+ *            when K is split); contents are scratch.
  * variant  : 4 = the two-pass path (an error if K is not a multiple of 128, the
  *            rows of A are not 16-byte aligned or the workspace is too small);
- *            -1 = choose by shape: variant 4 when M >= 1024 and it applies, else
+ *            -1 = choose by shape: variant 4 when it applies and M >= 1024 (or M >= 256
+ *            with so few output tiles that the single-launch GEMM would leave most
+ *            of the chip idle; K is then split and the partial products summed), else
  *            as cuthip_matmul_gguf; 0..3 = as cuthip_matmul_gguf (workspace unused).
  * Other arguments and numerics as cuthip_matmul_gguf. */
 size_t cuthip_matmul_gguf_workspace_bytes(int fmt, uint32_t M, uint32_t K, uint32_t N, int a_dtype);

@@ -213,7 +213,23 @@ public:
   std::vector<uint32_t> outputShape() const { return output_.shape; }
   std::string displayName() const { return "MatMulGguf"; }
   const Tensor &output() const { return output_; }
+  // Scratch for the two-pass prefill variant (MatMulGgufDequantGemm): the weights are dequantized into it once
+  // per dispatch.  With a workspace set, large M takes that variant automatically; the buffer may be shared by
+  // every node of a prefill graph (dispatches on one stream run in order).
+  size_t workspaceBytes() const { return cuthip_matmul_gguf_workspace_bytes((int)format_, M_, K_, N_, (int)a_.dtype); }
+  void setWorkspace(DeviceBuffer *workspace) {
+    if (workspace && workspace->bytes() < workspaceBytes())
+      throw std::runtime_error("MatMulGgufOpNode::setWorkspace: buffer smaller than workspaceBytes()");
+    workspace_ = workspace;
+  }
   void dispatch(void *stream = nullptr) const {
+    if (workspace_) {
+      check(cuthip_matmul_gguf_ws((int)format_, w_.data(), a_.data(), (int)a_.dtype, output_.data(), (int)outDtype_, M_, K_, N_,
+                                  a_.stride(), N_, (int)fusion_, fusionOp_, d_.data(), spec_, workspace_->data(),
+                                  workspace_->bytes(), stream),
+            "cuthip_matmul_gguf_ws");
+      return;
+    }
     check(cuthip_matmul_gguf((int)format_, w_.data(), a_.data(), (int)a_.dtype, output_.data(), (int)outDtype_, M_, K_, N_,
                              a_.stride(), N_, (int)fusion_, fusionOp_, d_.data(), spec_, stream),
           "cuthip_matmul_gguf");
@@ -227,6 +243,7 @@ private:
   int spec_ = -1;   // -1: chosen by shape at dispatch
   MatMulFusion fusion_ = MatMulFusion::None;
   int fusionOp_ = 0;
+  DeviceBuffer *workspace_ = nullptr;
   DeviceBuffer storage_;
   Tensor output_;
 };

@@ -45,6 +45,7 @@ static void test_tables() {
   EXPECT(getMatMulGgufVariantName(1) == "MatMulGgufSkinnyMfma");
   EXPECT(getMatMulGgufVariantName(2) == "MatMulGgufGemmLds");
   EXPECT(getMatMulGgufVariantName(3) == "MatMulGgufGemvRows8");
+  EXPECT(getMatMulGgufVariantName(4) == "MatMulGgufDequantGemm");
   for (uint32_t i = 0; i < n; ++i) EXPECT(lookupVariant(CUTHIP_OP_MATMUL_GGUF, variantInfo(CUTHIP_OP_MATMUL_GGUF, i).name) == i);
   EXPECT(throws([] { lookupVariant(CUTHIP_OP_MATMUL_GGUF, "NoSuchVariant"); }));
   EXPECT(throws([&] { variantInfo(CUTHIP_OP_MATMUL_GGUF, n); }));
@@ -126,6 +127,37 @@ static void test_gpu() {
       for (size_t i = 0; i < cf.size() && ok; ++i) ok = std::fabs(cf[i] - (c[i] + 0.5f)) <= 1e-5f * (1.0f + std::fabs(c[i]));
       EXPECT(ok);
     }
+  }
+  // prefill with a workspace: M = 1100 takes the two-pass variant (dequantize once, dense GEMM); variant 4 without a
+  // workspace is refused
+  {
+    const GgufFormat f = GgufFormat::Q4_K;
+    const uint32_t M = 1100, N = 136, K = 512;
+    std::vector<float> w((size_t)N * K), a((size_t)M * K);
+    for (auto &v : w) v = gw(rng);
+    for (auto &v : a) v = ga(rng);
+    std::vector<uint8_t> blocks(ggufBytes(f, (uint64_t)N * K));
+    EXPECT(orc_quantize((int)f, w.data(), (size_t)N * K, blocks.data()) == 0);
+    DeviceBuffer wdev(blocks.data(), blocks.size()), adev(a.data(), a.size() * 4);
+    Tensor wt{&wdev, {(uint32_t)blocks.size()}, DataType::Float32, 0}, at{&adev, {M, K}, DataType::Float32, 0};
+    MatMulGgufOpNode mm(at, wt, f, N);
+    EXPECT(mm.workspaceBytes() >= (size_t)N * K * 2 + (size_t)M * K * 2);
+    DeviceBuffer small(1024), ws(mm.workspaceBytes());
+    EXPECT(throws([&] { mm.setWorkspace(&small); }));
+    mm.setWorkspace(&ws);
+    mm.dispatch();
+    std::vector<float> c((size_t)M * N);
+    mm.output().buffer->download(c.data(), c.size() * 4);
+    std::vector<double> ref((size_t)M * N);
+    EXPECT(orc_matmul_gguf_f64((int)f, blocks.data(), a.data(), M, K, N, ref.data()) == 0);
+    EXPECT(normwise(c, ref) < 1e-3);
+    MatMulGgufOpNode m4(at, wt, f, N, DataType::Float32, lookupVariant(CUTHIP_OP_MATMUL_GGUF, "MatMulGgufDequantGemm"));
+    EXPECT(throws([&] { m4.dispatch(); }));
+    m4.setWorkspace(&ws);
+    m4.dispatch();
+    std::vector<float> c4((size_t)M * N);
+    m4.output().buffer->download(c4.data(), c4.size() * 4);
+    EXPECT(std::memcmp(c.data(), c4.data(), c.size() * 4) == 0);
   }
   // an explicit variant that cannot take the shape is an error, not a silent fallback
   {

@@ -201,7 +201,7 @@ def test_dense_gemm_refusals_and_automatic_choice(ops):
     assert normwise_rel_err(auto, oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)) < TOL_GEMM
 
 
-@pytest.mark.parametrize("M,N,K", [(2048, 14336, 4096), (512, 14336, 4096), (2048, 4096, 14336)])
+@pytest.mark.parametrize("M,N,K", [(2048, 14336, 4096), (512, 14336, 4096), (2048, 4096, 14336), (512, 4096, 14336)])
 def test_dense_gemm_prefill_shapes_sampled(ops, M, N, K):
     """BASELINE config 5 geometry through the two-pass path, on a sample of output rows and columns."""
     fmt = oracle.Q4_K
