@@ -94,7 +94,7 @@ def bench_decode_step(torch, np, ops, dev, x_h, steps=5):
     ones = torch.ones(cfg.hidden, dtype=torch.float32, device=dev)
     layers = [dict({k: v.clone() for k, v in base.items()}, attn_norm=ones, ffn_norm=ones) for _ in range(cfg.n_layers)]
     head = torch.from_numpy(make_q_weights(cfg.fmt_head, 4008, cfg.hidden, 3)).to(dev).repeat(32)
-    dstep = DecodeStep(cfg, layers, ones, head, dev, fuse=int(os.environ.get("CUT_DECODE_FUSE", "3")))
+    dstep = DecodeStep(cfg, layers, ones, head, dev, fuse=int(os.environ.get("CUT_DECODE_FUSE", "4")))
     for kc, vc in zip(dstep.k_cache, dstep.v_cache):
         kc.normal_(0.0, 0.5)
         vc.normal_(0.0, 1.0)

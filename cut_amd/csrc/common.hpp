@@ -134,6 +134,21 @@ __device__ inline void store_out(void *C, const Epilogue &e, int c_f16, size_t i
     reinterpret_cast<float *>(C)[idx] = v;
 }
 
+// store_out that also returns the fp32 value it stored (before any narrowing to fp16)
+__device__ inline float store_out_value(void *C, const Epilogue &e, int c_f16, size_t idx, float v) {
+  if (e.kind == CUTHIP_EPI_UNARY) {
+    v = apply_unary(e.op, v);
+  } else if (e.kind == CUTHIP_EPI_BINARY) {
+    float d = c_f16 ? (float)reinterpret_cast<const half_t *>(e.D)[idx] : reinterpret_cast<const float *>(e.D)[idx];
+    v = apply_binary(e.op, v, d);
+  }
+  if (c_f16)
+    reinterpret_cast<half_t *>(C)[idx] = (half_t)v;
+  else
+    reinterpret_cast<float *>(C)[idx] = v;
+  return v;
+}
+
 __device__ inline void store_plain(void *C, int c_f16, size_t idx, float v) {
   if (c_f16)
     reinterpret_cast<half_t *>(C)[idx] = (half_t)v;

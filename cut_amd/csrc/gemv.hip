@@ -207,9 +207,57 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
 }
 extern "C" {
 
-int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, int fmt_b, const void *Wb, uint32_t Nb,
-                            void *Cb, const void *A, int a_dtype, int c_dtype, uint32_t K, void *stream) {
+// Copies the consumer / producer fields of a carried RMSNorm into the launch parameters; false = malformed.
+static bool apply_carry(cuthip::GemvParams &p, const cuthip_norm_carry_t *carry, bool producer_allowed) {
+  if (!carry) return true;
+  const bool producer = carry->next_norm_weight || carry->next_x16 || carry->next_sumsq_parts;
+  if (producer && !(producer_allowed && carry->next_norm_weight && carry->next_x16 && carry->next_sumsq_parts)) return false;
+  if ((uintptr_t)carry->next_x16 % 2 != 0) return false;
+  p.sumsq_parts = carry->sumsq_parts;
+  p.eps = carry->eps;
+  p.next_norm_w = carry->next_norm_weight;
+  p.next_x16 = reinterpret_cast<cuthip::half_t *>(carry->next_x16);
+  p.next_sumsq_parts = carry->next_sumsq_parts;
+  return true;
+}
+
+int cuthip_matmul_gguf_carry(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t K, uint32_t N,
+                             int epilogue, int epilogue_op, const void *D, const cuthip_norm_carry_t *carry, void *stream) {
   using namespace cuthip;
+  const uint32_t n_out = epilogue == CUTHIP_EPI_SWIGLU_PAIRS ? N / 2 : N;
+  if (int rc = check_matmul_args(fmt, W, A, a_dtype, C, c_dtype, 1, K, N, K, n_out, epilogue, D)) return rc > 0 ? CUTHIP_OK : rc;
+  GemvParams p;
+  p.W = reinterpret_cast<const uint8_t *>(W);
+  p.A = A;
+  p.C = C;
+  p.epi = Epilogue{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
+  p.M = 1; p.K = K; p.N = N; p.strideA = K; p.strideC = n_out;
+  p.nsteps = (K + 255) / 256;
+  p.row_bytes = (uint32_t)((uint64_t)(K / fmt_elems(fmt)) * fmt_bytes(fmt));
+  p.a_f16 = a_dtype == CUTHIP_F16;
+  p.c_f16 = c_dtype == CUTHIP_F16;
+  if (!apply_carry(p, carry, epilogue != CUTHIP_EPI_SWIGLU_PAIRS)) {
+    set_error("cuthip_matmul_gguf_carry: the producer fields (next_norm_weight, next_x16, next_sumsq_parts) come together, "
+              "next_x16 2-byte aligned, and not with the SwiGLU row-pair epilogue");
+    return CUTHIP_ERR_INVALID;
+  }
+  bool taken = false;
+  int rc = launch_rows8_any(fmt, p, reinterpret_cast<hipStream_t>(stream), &taken);
+  if (!taken) {
+    set_error("cuthip_matmul_gguf_carry: K = %u does not fit the LDS budget of the 8-row GEMV", K);
+    return CUTHIP_ERR_INVALID;
+  }
+  return rc;
+}
+
+int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, int fmt_b, const void *Wb, uint32_t Nb,
+                            void *Cb, const void *A, int a_dtype, int c_dtype, uint32_t K,
+                            const cuthip_norm_carry_t *carry, void *stream) {
+  using namespace cuthip;
+  if (carry && (carry->next_norm_weight || carry->next_x16 || carry->next_sumsq_parts)) {
+    set_error("cuthip_matmul_gguf_pair: only the consumer fields of the carried RMSNorm apply here");
+    return CUTHIP_ERR_INVALID;
+  }
   if (int rc = check_matmul_args(fmt_a, Wa, A, a_dtype, Ca, c_dtype, 1, K, Na, K, Na, CUTHIP_EPI_NONE, nullptr))
     return rc > 0 ? cuthip_matmul_gguf(fmt_b, Wb, A, a_dtype, Cb, c_dtype, 1, K, Nb, K, Nb, 0, 0, nullptr, -1, stream) : rc;
   if (int rc = check_matmul_args(fmt_b, Wb, A, a_dtype, Cb, c_dtype, 1, K, Nb, K, Nb, CUTHIP_EPI_NONE, nullptr))
@@ -225,6 +273,7 @@ int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, in
     p.row_bytes = (uint32_t)((uint64_t)(K / fmt_elems(fmt)) * fmt_bytes(fmt));
     p.a_f16 = a_dtype == CUTHIP_F16;
     p.c_f16 = c_dtype == CUTHIP_F16;
+    apply_carry(p, carry, false);
     return p;
   };
   if ((uint64_t)(K / fmt_elems(fmt_a)) * fmt_bytes(fmt_a) <= 0xFFFFFFFFull && (uint64_t)Na + Nb <= 0x7FFFFFFFull) {
@@ -239,6 +288,10 @@ int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, in
     if (taken) return rc;
   }
   // other formats or shapes: the same two products as two launches
+  if (carry) {
+    if (int rc = cuthip_matmul_gguf_carry(fmt_a, Wa, A, a_dtype, Ca, c_dtype, K, Na, 0, 0, nullptr, carry, stream)) return rc;
+    return cuthip_matmul_gguf_carry(fmt_b, Wb, A, a_dtype, Cb, c_dtype, K, Nb, 0, 0, nullptr, carry, stream);
+  }
   if (int rc = cuthip_matmul_gguf(fmt_a, Wa, A, a_dtype, Ca, c_dtype, 1, K, Na, K, Na, 0, 0, nullptr, -1, stream)) return rc;
   return cuthip_matmul_gguf(fmt_b, Wb, A, a_dtype, Cb, c_dtype, 1, K, Nb, K, Nb, 0, 0, nullptr, -1, stream);
 }

@@ -20,6 +20,14 @@ struct GemvParams {
   int pro = 0;
   const float *norm_w = nullptr;
   float eps = 0.0f;
+  // RMSNorm carried across matmuls (8-row GEMV, batch 1).  Producer side, after the epilogue: next_x16[n] =
+  // fp16(C[n] * next_norm_w[n]) and the sum of C[n]^2 over each group of 8 rows goes to next_sumsq_parts[n / 8].
+  // Consumer side (the activations are such a next_x16): the result is multiplied by
+  // rsqrt(sum(sumsq_parts[0 .. K/8)) / K + eps).  Fixed summation order, no atomics.
+  const float *sumsq_parts = nullptr;
+  const float *next_norm_w = nullptr;
+  half_t *next_x16 = nullptr;
+  float *next_sumsq_parts = nullptr;
 };
 
 // ---- per-tile configuration -------------------------------------------------

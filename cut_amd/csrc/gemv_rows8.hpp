@@ -70,6 +70,12 @@ struct LaneCtx {
   uint32_t c0, c1, c2, c3;  // per-lane constants of the format
 };
 
+__device__ inline float wave_sum_all(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
 template <int FMT> struct Rows8;
 
 // ---- Q4_K -------------------------------------------------------------------
@@ -571,6 +577,15 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
       xscale[m] = 1.0f / sqrtf(t / (float)p.K + p.eps);
     }
   }
+  // RMSNorm carried over from the producer of the activations: every wave adds the K / 8 partial sums of squares in
+  // the same order and scales the whole (batch-1) product by one scalar.  (Requesting the partial sums ahead of the
+  // activations and the weight ring measured slower.)
+  float carry_scale = 1.0f;
+  if (p.sumsq_parts) {
+    float t = 0.0f;
+    for (uint32_t i = lane; i < (p.K + 7) / 8; i += 64) t += p.sumsq_parts[i];
+    carry_scale = 1.0f / sqrtf(wave_sum_all(t) / (float)p.K + p.eps);
+  }
 
   // Matrix-core path: A-row j of this lane is batch row j>>2 (clamped), piece j&3, and accumulator quad q
   // holds batch row 2q + kg.  Dot path: the lane's own slice of every batch row, accumulator q = batch row q.
@@ -630,7 +645,7 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
       v += __shfl_xor(v, 1);
       v += __shfl_xor(v, 2);
       v += __shfl_xor(v, 32);
-      out[q] = PRO ? v * xscale[q] : v;   // linear in the partial sums, so it may be applied before the K ranges are folded
+      out[q] = (PRO ? v * xscale[q] : v) * carry_scale;   // linear in the partial sums: applied before the K ranges are folded
     }
     writer = c.g == 0 && c.kg == 0;
   } else {
@@ -640,10 +655,11 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
       v = S::finish(v, cacc[q]);
       v += __shfl_xor(v, 1);
       v += __shfl_xor(v, 2);
-      out[q] = v;   // batch row 2q + kg
+      out[q] = v * carry_scale;   // batch row 2q + kg
     }
     writer = c.g == 0;
   }
+  float carry_sq = 0.0f;
   // SwiGLU over row pairs: weight rows 2i / 2i+1 are gate_i / up_i, C[m, i] = silu(gate) * up.  The partner row
   // sits four lanes up (same piece, same K half); in the folded path it is the next thread.
   const bool swiglu = p.epi.kind == CUTHIP_EPI_SWIGLU_PAIRS;
@@ -660,7 +676,13 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
 #pragma unroll
       for (int q = 0; q < RQ; ++q) {
         int m = DOT ? q : 2 * q + c.kg;
-        if (m < (int)p.M) store_out(p.C, p.epi, p.c_f16, (size_t)m * p.strideC + n0 + r8, out[q]);
+        if (m < (int)p.M) {
+          float v = store_out_value(p.C, p.epi, p.c_f16, (size_t)m * p.strideC + n0 + r8, out[q]);
+          if (p.next_sumsq_parts && m == 0) {
+            p.next_x16[n0 + r8] = (half_t)(v * p.next_norm_w[n0 + r8]);
+            carry_sq = v * v;
+          }
+        }
       }
     }
   } else {
@@ -685,8 +707,25 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
         if (m < (int)p.M && (rr & 1) == 0 && nn + 1 < p.N)
           store_plain(p.C, p.c_f16, (size_t)m * p.strideC + nn / 2, apply_unary(CUTHIP_UNARY_SILU, v) * up);
       } else if (m < (int)p.M && nn < p.N) {
-        store_out(p.C, p.epi, p.c_f16, (size_t)m * p.strideC + nn, v);
+        v = store_out_value(p.C, p.epi, p.c_f16, (size_t)m * p.strideC + nn, v);
+        if (p.next_sumsq_parts && m == 0) {
+          p.next_x16[nn] = (half_t)(v * p.next_norm_w[nn]);
+          carry_sq = v * v;
+        }
       }
+    }
+  }
+  // producer side of the carried RMSNorm: sum(C^2) of each group of 8 rows to its own slot
+  if (p.next_sumsq_parts) {
+    if (KW == 1) {   // one row group per wave, its writers are 8 of the lanes
+      carry_sq = wave_sum_all(carry_sq);
+      if (lane == 0 && n0 < p.N) p.next_sumsq_parts[n0 / 8] = carry_sq;
+    } else {         // folded epilogue: thread 8 g + r of the workgroup holds row r of its g-th row group
+      carry_sq += __shfl_xor(carry_sq, 1);
+      carry_sq += __shfl_xor(carry_sq, 2);
+      carry_sq += __shfl_xor(carry_sq, 4);
+      const uint32_t grp = bid * RWG + (uint32_t)tid / 8;
+      if (tid < RWG * 8 && (tid & 7) == 0 && grp * 8 < p.N) p.next_sumsq_parts[grp] = carry_sq;
     }
   }
 }
@@ -780,6 +819,7 @@ template <int FMT> bool rows8_fits(const GemvParams &p) {
 
 template <int FMT> int launch_rows8_fmt(const GemvParams &p, hipStream_t stream) {
   Rows8Shape s = pick_rows8_shape(p.N, p.nsteps);
+  if (FMT == CUTHIP_Q6_K && s.rwg > 4) s.rwg = 4;   // measured on the 128256 x 4096 head: 103 us against 110-114 with 8 row groups
   if (p.M <= 1) return launch_rows8_shape<FMT, 1>(p, s.rwg, s.kw, stream);
   if (p.M <= 2) return launch_rows8_shape<FMT, 2>(p, s.rwg, s.kw, stream);
   if (p.M <= 4) return launch_rows8_shape<FMT, 4>(p, s.rwg, s.kw, stream);

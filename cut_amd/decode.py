@@ -59,8 +59,10 @@ class DecodeStep:
     plus 'out_norm' (fp32) and 'head' at the top level."""
 
     def __init__(self, cfg: DecodeConfig, layers: list[dict], out_norm: torch.Tensor, head: torch.Tensor, device="cuda:0",
-                 fuse: int = 3):
-        """fuse: 3 (default) = SiLU(gate) * up runs in the epilogue of the gate+up matmul (the producer), whose rows
+                 fuse: int = 4):
+        """fuse: 4 (default) = 3 plus RMSNorm carried across the matmuls (see _step_carry): the producer of the
+        residual stream stores x * norm_weight and partial sums of x^2, the consumer scales its result, so neither
+        repeats the norm per workgroup and the RMSNorm launches disappear; 3 = SiLU(gate) * up runs in the epilogue of the gate+up matmul (the producer), whose rows
         are interleaved gate_0, up_0, gate_1, ... for it: 'gate_up' is re-laid out once, here, and the layer dicts are
         copied; 0 = every operator is its own launch; 1 = SiLU(gate) * up runs inside the staging of w_down;
         2 = RMSNorm is fused into the following matmuls as well.  Level 2 saves three more launches per layer but
@@ -69,7 +71,7 @@ class DecodeStep:
         MI355X both levels measured slower than separate launches (2.43 / 2.70 / 2.85 ms per token for 0 / 1 / 2 at
         the 8B shape); fusing into the producer has no such cost.  The fused entry point stays for shapes where
         launches dominate."""
-        if fuse == 3:
+        if fuse >= 3:
             layers = [dict(L, gate_up=interleave_gate_up(L["gate_up"], cfg.ffn)) for L in layers]
         self.cfg, self.layers, self.out_norm, self.head, self.fuse = cfg, layers, out_norm, head, fuse
         dev = torch.device(device)
@@ -86,6 +88,7 @@ class DecodeStep:
         self.logits = torch.empty(c.vocab, dtype=f32, device=dev)
         self.token = torch.zeros(1, dtype=torch.int32, device=dev)
         self.params = torch.zeros(2, dtype=torch.int32, device=dev)      # {position, sequence length}
+        self.sumsq_parts = torch.zeros((c.hidden + 7) // 8, dtype=f32, device=dev)   # carried RMSNorm: sum(x^2) per 8 outputs
         self.k_cache = [torch.zeros((c.max_ctx, c.kv_dim), dtype=f16, device=dev) for _ in layers]
         self.v_cache = [torch.zeros((c.max_ctx, c.kv_dim), dtype=f16, device=dev) for _ in layers]
         half = c.head_dim // 2
@@ -105,6 +108,8 @@ class DecodeStep:
         c = self.cfg
         if self.fuse == 2:
             return self._step_fused()
+        if self.fuse == 4:
+            return self._step_carry()
         for i, L in enumerate(self.layers):
             ops.rmsnorm(self.x, L["attn_norm"], c.eps, out=self.xn.view(1, -1))
             # (running v beside q+k on a second stream was measured slower: the fork / join nodes of the graph cost
@@ -134,6 +139,33 @@ class DecodeStep:
                                 d=self.x.view(1, -1))
         ops.rmsnorm(self.x, self.out_norm, c.eps, out=self.xn.view(1, -1))
         ops.matmul_gguf(self.xn, self.head, c.fmt_head, c.vocab, c.hidden, out=self.logits.view(1, -1))
+        ops.argmax(self.logits, self.token)
+
+    def _step_carry(self) -> None:
+        """Seven launches per layer: only the first RMSNorm of the step is a kernel.  Every matmul that forms the
+        residual stream (wo, w_down) also stores x * next_norm_weight as fp16 and the sum of x^2 over each group of 8
+        outputs; the matmul that consumes it adds those partial sums (fixed order) and scales its result by
+        rsqrt(sum / hidden + eps).  Producers and consumers alternate, so one array of partial sums serves all."""
+        c = self.cfg
+        n_layers = len(self.layers)
+        consume = ops.norm_carry(sumsq_parts=self.sumsq_parts, eps=c.eps)
+        ops.rmsnorm(self.x, self.layers[0]["attn_norm"], c.eps, out=self.xn.view(1, -1))
+        for i, L in enumerate(self.layers):
+            # layer 0 reads the output of the RMSNorm kernel (already scaled); the others the carried form
+            ops.matmul_gguf_pair(self.xn, L["qk"], c.fmt_attn, c.q_dim + c.kv_dim, self.qk, L["v"], c.fmt_v, c.kv_dim, self.v,
+                                 c.hidden, carry=consume if i > 0 else None)
+            ops.rope_kv_write(self.qk[:c.q_dim], self.qk[c.q_dim:], self.v, self.params, self.cos_t, self.sin_t,
+                              self.k_cache[i], self.v_cache[i], c.head_dim, self.q_rot)
+            ops.attn_decode(self.q_rot, self.k_cache[i], self.v_cache[i], self.params, c.n_heads, c.n_kv_heads, c.head_dim,
+                            self.scale, self.ws, self.attn)
+            ops.matmul_gguf_carry(self.attn, L["o"], c.fmt_attn, c.hidden, c.q_dim, self.x, binary="add", d=self.x,
+                                  carry=ops.norm_carry(next_norm_weight=L["ffn_norm"], next_x16=self.xn,
+                                                       next_sumsq_parts=self.sumsq_parts))
+            ops.matmul_gguf_carry(self.xn, L["gate_up"], c.fmt_ffn, 2 * c.ffn, c.hidden, self.act, swiglu_pairs=True, carry=consume)
+            nxt = self.layers[i + 1]["attn_norm"] if i + 1 < n_layers else self.out_norm
+            ops.matmul_gguf_carry(self.act, L["down"], c.fmt_ffn, c.hidden, c.ffn, self.x, binary="add", d=self.x,
+                                  carry=ops.norm_carry(next_norm_weight=nxt, next_x16=self.xn, next_sumsq_parts=self.sumsq_parts))
+        ops.matmul_gguf_carry(self.xn, self.head, c.fmt_head, c.vocab, c.hidden, self.logits, carry=consume)
         ops.argmax(self.logits, self.token)
 
     def _step_fused(self) -> None:

@@ -30,11 +30,17 @@ EXPORTS = [
     "cuthip_event_create", "cuthip_event_destroy", "cuthip_event_record", "cuthip_event_sync", "cuthip_event_elapsed_ms",
     "cuthip_variant_count", "cuthip_variant_default", "cuthip_variant_info", "cuthip_variant_lookup",
     "cuthip_dequant", "cuthip_matmul_gguf", "cuthip_matmul_gguf_pro",
-    "cuthip_matmul_gguf_workspace_bytes", "cuthip_matmul_gguf_ws", "cuthip_matmul_gguf_pair",
+    "cuthip_matmul_gguf_workspace_bytes", "cuthip_matmul_gguf_ws", "cuthip_matmul_gguf_pair", "cuthip_matmul_gguf_carry",
     "cuthip_rmsnorm", "cuthip_rope_kv_write", "cuthip_attn_decode_workspace_bytes", "cuthip_attn_decode",
     "cuthip_silu_mul", "cuthip_argmax",
     "cuthip_matmul_sep_workspace_bytes", "cuthip_matmul_q8_sep", "cuthip_matmul_q4_sep",
 ]
+
+
+class NormCarry(C.Structure):
+    """cuthip_norm_carry_t: device pointers as integers (0 = NULL)."""
+    _fields_ = [("sumsq_parts", C.c_void_p), ("eps", C.c_float), ("next_norm_weight", C.c_void_p), ("next_x16", C.c_void_p),
+                ("next_sumsq_parts", C.c_void_p)]
 
 
 class CutHipError(RuntimeError):
@@ -91,7 +97,8 @@ def load() -> C.CDLL:
     lib.cuthip_matmul_gguf.argtypes = [i, vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, i, vp]
     lib.cuthip_matmul_gguf_workspace_bytes.argtypes = [i, u32, u32, u32, i]
     lib.cuthip_matmul_gguf_ws.argtypes = [i, vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, i, vp, C.c_size_t, vp]
-    lib.cuthip_matmul_gguf_pair.argtypes = [i, vp, u32, vp, i, vp, u32, vp, vp, i, i, u32, vp]
+    lib.cuthip_matmul_gguf_pair.argtypes = [i, vp, u32, vp, i, vp, u32, vp, vp, i, i, u32, C.POINTER(NormCarry), vp]
+    lib.cuthip_matmul_gguf_carry.argtypes = [i, vp, vp, i, vp, i, u32, u32, i, i, vp, C.POINTER(NormCarry), vp]
     f32 = C.c_float
     lib.cuthip_matmul_gguf_pro.argtypes = [i, vp, vp, i, vp, i, u32, u32, i, i, vp, i, vp, f32, vp]
     lib.cuthip_rmsnorm.argtypes = [vp, i, vp, vp, i, u32, u32, u32, f32, vp]

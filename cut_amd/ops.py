@@ -101,8 +101,42 @@ def matmul_gguf(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: int, ou
     return out
 
 
+def norm_carry(sumsq_parts: torch.Tensor | None = None, eps: float = 0.0, next_norm_weight: torch.Tensor | None = None,
+               next_x16: torch.Tensor | None = None, next_sumsq_parts: torch.Tensor | None = None) -> "_l.NormCarry":
+    """cuthip_norm_carry_t from device tensors (float32 [K/8] / [N] / [N/8], fp16 [N] output)."""
+    def ptr(t, dtype):
+        if t is None:
+            return None
+        if t.dtype != dtype or not t.is_contiguous():
+            raise _l.CutHipError("norm_carry: wrong dtype or non-contiguous tensor")
+        return t.data_ptr()
+    return _l.NormCarry(ptr(sumsq_parts, torch.float32), eps, ptr(next_norm_weight, torch.float32), ptr(next_x16, torch.float16),
+                        ptr(next_sumsq_parts, torch.float32))
+
+
+def matmul_gguf_carry(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: int, out: torch.Tensor, carry, binary: str | None = None,
+                      d: torch.Tensor | None = None, swiglu_pairs: bool = False) -> torch.Tensor:
+    """Batch-1 matmul taking part in a carried RMSNorm (cuthip_matmul_gguf_carry); a [K], out [N] (or [N/2])."""
+    f = _fmt(fmt)
+    if a.numel() != K or a.dtype not in (torch.float32, torch.float16) or not a.is_contiguous() or not out.is_contiguous():
+        raise _l.CutHipError("matmul_carry: A must be a contiguous float32/float16 vector of K elements, out contiguous")
+    if w_blocks.numel() < n_bytes(f, N, K) or out.numel() != (N // 2 if swiglu_pairs else N):
+        raise _l.CutHipError("matmul_carry: weight tensor too small or output of the wrong size")
+    epi, op, dptr = _l.EPI_NONE, 0, None
+    if swiglu_pairs:
+        epi = _l.EPI_SWIGLU_PAIRS
+    elif binary is not None:
+        if d is None or d.numel() != N or d.dtype != out.dtype:
+            raise _l.CutHipError("matmul_carry: binary epilogue needs D with the size and dtype of C")
+        epi, op, dptr = _l.EPI_BINARY, _l.BINARY[binary], d.data_ptr()
+    import ctypes
+    _l.check(_l.load().cuthip_matmul_gguf_carry(f, w_blocks.data_ptr(), a.data_ptr(), _dt(a), out.data_ptr(), _dt(out), K, N, epi,
+                                                op, dptr, ctypes.byref(carry) if carry is not None else None, _stream_ptr()))
+    return out
+
+
 def matmul_gguf_pair(a: torch.Tensor, wa: torch.Tensor, fmt_a, Na: int, out_a: torch.Tensor, wb: torch.Tensor, fmt_b, Nb: int,
-                     out_b: torch.Tensor, K: int) -> None:
+                     out_b: torch.Tensor, K: int, carry=None) -> None:
     """out_a = a . dequant(wa)^T and out_b = a . dequant(wb)^T for one activation vector a [K], in one launch where the
     formats allow it (cuthip_matmul_gguf_pair)."""
     fa, fb = _fmt(fmt_a), _fmt(fmt_b)
@@ -112,9 +146,10 @@ def matmul_gguf_pair(a: torch.Tensor, wa: torch.Tensor, fmt_a, Na: int, out_a: t
         raise _l.CutHipError("matmul_pair: weight tensor too small for [N, K]")
     if out_a.dtype != out_b.dtype or out_a.numel() != Na or out_b.numel() != Nb or not (out_a.is_contiguous() and out_b.is_contiguous()):
         raise _l.CutHipError("matmul_pair: outputs must be contiguous [Na] and [Nb] of one dtype")
+    import ctypes
     _l.check(_l.load().cuthip_matmul_gguf_pair(
         fa, wa.data_ptr(), Na, out_a.data_ptr(), fb, wb.data_ptr(), Nb, out_b.data_ptr(), a.data_ptr(), _dt(a), _dt(out_a), K,
-        _stream_ptr()))
+        ctypes.byref(carry) if carry is not None else None, _stream_ptr()))
 
 
 def matmul_gguf_workspace(fmt, M: int, K: int, N: int, a_dtype: torch.dtype, device) -> torch.Tensor:

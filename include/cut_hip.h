@@ -181,6 +181,15 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
                           uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D,
                           int variant, void *workspace, size_t workspace_bytes, void *stream);
 
+/* Fields of an RMSNorm carried across batch-1 matmuls (cuthip_matmul_gguf_carry). */
+typedef struct {
+  const float *sumsq_parts;      /* consumer: device [ceil(K/8)], partial sums of squares of the un-normalised activations */
+  float eps;
+  const float *next_norm_weight; /* producer: weight [N] of the norm that follows this matmul */
+  void *next_x16;                /* producer: fp16 [N] out */
+  float *next_sumsq_parts;       /* producer: device [ceil(N/8)] out, sum of C^2 over each group of 8 outputs */
+} cuthip_norm_carry_t;
+
 /* Two batch-1 matmuls on the same activations in one launch:
  *   Ca[Na] = A . dequant(Wa)^T,  Cb[Nb] = A . dequant(Wb)^T,  A [K].
  * For the q/k and v projections of a decode step, whose weights differ in format
@@ -191,7 +200,26 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
  * formats at decode shapes, otherwise the same two products as two launches.
  * No epilogue; dtypes and alignment as cuthip_matmul_gguf. */
 int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, int fmt_b, const void *Wb, uint32_t Nb,
-                            void *Cb, const void *A, int a_dtype, int c_dtype, uint32_t K, void *stream);
+                            void *Cb, const void *A, int a_dtype, int c_dtype, uint32_t K,
+                            const cuthip_norm_carry_t *carry /* consumer fields only, or NULL */, void *stream);
+
+/* Batch-1 matmul that takes part in an RMSNorm carried across matmuls, which removes
+ * the RMSNorm launches of a decode step (the reference fuses RMSNorm into its
+ * consumers, runtime/graph/GraphOptimizer.cpp:46-70; here the work is split between
+ * producer and consumer so that neither repeats it per workgroup):
+ *   producer (the matmul whose epilogue forms the residual stream, C = A.W^T + D):
+ *     also stores next_x16[n] = fp16(C[n] * next_norm_weight[n]) and the sum of
+ *     C[n]^2 over each group of 8 outputs in next_sumsq_parts[n / 8];
+ *   consumer (the matmul that reads next_x16 as its activations, so its K is the
+ *     producer's N): multiplies its result by rsqrt(sum(sumsq_parts) / K + eps)
+ *     before the epilogue, i.e. computes RMSNorm(x) . W^T with the rounding to fp16
+ *     taken before the scaling.
+ * The partial sums are added in a fixed order (no atomics): results are
+ * reproducible from run to run.
+ * Any field group may be NULL.  M = 1, the 8-row GEMV only; other arguments as
+ * cuthip_matmul_gguf (strideA = K, strideC = N, or N/2 with CUTHIP_EPI_SWIGLU_PAIRS). */
+int cuthip_matmul_gguf_carry(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t K, uint32_t N,
+                             int epilogue, int epilogue_op, const void *D, const cuthip_norm_carry_t *carry, void *stream);
 
 /* The same matmul at batch 1 with the operator in front of it fused into the
  * staging of the activations, which saves a launch per use in a decode step

@@ -176,7 +176,7 @@ def test_matmul_with_fused_prologues(ops, name, N, K):
     assert normwise_rel_err(out.cpu().numpy() - res, want) < 4e-4
 
 
-@pytest.mark.parametrize("fuse", [0, 1, 2, 3])
+@pytest.mark.parametrize("fuse", [0, 1, 2, 3, 4])
 def test_small_decode_step_against_oracle_chain(ops, fuse):
     from cut_amd.decode import DecodeConfig, DecodeStep
     cfg = DecodeConfig(hidden=512, n_layers=2, n_heads=8, n_kv_heads=2, head_dim=64, ffn=1024, vocab=2048, max_ctx=64)
@@ -258,3 +258,72 @@ def test_swiglu_row_pair_epilogue_refusals(ops):
         ops.matmul_gguf(dev(gauss_acts((2, 256), seed=1, dtype=np.float16)), W, fmt, 64, 256, swiglu_pairs=True, variant=2)
     with pytest.raises(lib.CutHipError, match="even N"):
         ops.matmul_gguf(dev(gauss_acts((1, 256), seed=1, dtype=np.float16)), W, fmt, 63, 256, swiglu_pairs=True)
+
+
+@pytest.mark.parametrize("name", ["Q4_K", "Q6_K", "Q8_0"])
+@pytest.mark.parametrize("N,K", [(4096, 14336), (4096, 4096), (14336, 4096), (40, 512), (9, 256)])
+def test_carried_rmsnorm_producer_and_consumer(ops, name, N, K):
+    """Producer: C = A . W^T + D as the plain matmul gives it, next_x16 = fp16(C * g), sum(C^2) of every group of 8
+    outputs in its slot.  Consumer: the plain matmul times 1 / sqrt(sum(parts) / K + eps).  Shapes cover the direct and
+    the folded (split K) epilogues and a ragged last group."""
+    fmt = oracle.FORMATS[name]
+    W = dev(quantized_weights(fmt, N, K, seed=80))
+    A = gauss_acts((1, K), seed=81, dtype=np.float16)
+    D = gauss_acts((1, N), seed=82)
+    g = np.random.default_rng(83).uniform(0.5, 1.5, N).astype(np.float32)
+    plain = ops.matmul_gguf(dev(A), W, fmt, N, K, out_dtype=torch.float32, binary="add", d=dev(D))
+    c = torch.empty(N, dtype=torch.float32, device="cuda")
+    x16 = torch.zeros(N, dtype=torch.float16, device="cuda")
+    ng = (N + 7) // 8
+    parts = torch.full((ng + 3,), -1.0, dtype=torch.float32, device="cuda")   # stale contents are overwritten, the tail is not touched
+    ops.matmul_gguf_carry(dev(A).view(-1), W, fmt, N, K, c, binary="add", d=dev(D).view(-1),
+                          carry=ops.norm_carry(next_norm_weight=dev(g), next_x16=x16, next_sumsq_parts=parts))
+    torch.cuda.synchronize()
+    cn = c.cpu().numpy()
+    assert np.array_equal(cn, plain.cpu().numpy()[0])
+    # the device rounds the exact product once (mixed-precision multiply), numpy rounds to fp32 first: at most one ulp apart
+    d16 = x16.cpu().numpy().view(np.uint16).astype(np.int32) - (cn * g).astype(np.float16).view(np.uint16).astype(np.int32)
+    assert np.max(np.abs(d16)) <= 1 and np.mean(d16 != 0) < 0.01
+    sq = np.zeros(ng * 8, np.float64)
+    sq[:N] = cn.astype(np.float64) ** 2
+    pn = parts.cpu().numpy()
+    np.testing.assert_allclose(pn[:ng], sq.reshape(ng, 8).sum(1), rtol=2e-6, atol=1e-30)
+    assert np.all(pn[ng:] == -1.0)
+    # consumer: K / 8 partial sums of some earlier producer
+    A2 = gauss_acts((1, K), seed=84, dtype=np.float16)
+    pk = np.random.default_rng(85).uniform(0.0, 2.0, (K + 7) // 8).astype(np.float32)
+    base = ops.matmul_gguf(dev(A2), W, fmt, N, K, out_dtype=torch.float32).cpu().numpy()[0]
+    out = torch.empty(N, dtype=torch.float32, device="cuda")
+    ops.matmul_gguf_carry(dev(A2).view(-1), W, fmt, N, K, out, carry=ops.norm_carry(sumsq_parts=dev(pk), eps=1e-5))
+    torch.cuda.synchronize()
+    scale = 1.0 / np.sqrt(pk.astype(np.float64).sum() / K + 1e-5)
+    # the scale multiplies the partial sums of the K ranges before they are folded: errors relative to those, not to the result
+    np.testing.assert_allclose(out.cpu().numpy(), base * np.float32(scale), rtol=3e-6, atol=3e-6 * float(np.abs(base).max() * scale))
+    again = torch.empty(N, dtype=torch.float32, device="cuda")
+    ops.matmul_gguf_carry(dev(A2).view(-1), W, fmt, N, K, again, carry=ops.norm_carry(sumsq_parts=dev(pk), eps=1e-5))
+    torch.cuda.synchronize()
+    assert np.array_equal(again.cpu().numpy(), out.cpu().numpy())   # fixed summation order: reproducible
+
+
+def test_carried_rmsnorm_equals_rmsnorm_then_matmul(ops):
+    """producer -> consumer against RMSNorm kernel -> matmul on the same data (the fp16 rounding of the activations is
+    taken before the scaling instead of after it: 2^-11 relative per element, well inside 1e-3 normwise)."""
+    fmt = oracle.Q4_K
+    hidden, N = 4096, 512
+    rng = np.random.default_rng(90)
+    x = rng.standard_normal(hidden).astype(np.float32)
+    g = rng.uniform(0.5, 1.5, hidden).astype(np.float32)
+    Wp = dev(quantized_weights(fmt, hidden, hidden, seed=91))   # producer weights (square)
+    Wc = dev(quantized_weights(fmt, N, hidden, seed=92))
+    a = gauss_acts((1, hidden), seed=93, dtype=np.float16)
+    xs = torch.from_numpy(x).cuda()
+    x16 = torch.empty(hidden, dtype=torch.float16, device="cuda")
+    parts = torch.zeros(hidden // 8, dtype=torch.float32, device="cuda")
+    ops.matmul_gguf_carry(dev(a).view(-1), Wp, fmt, hidden, hidden, xs, binary="add", d=xs,
+                          carry=ops.norm_carry(next_norm_weight=dev(g), next_x16=x16, next_sumsq_parts=parts))
+    got = torch.empty(N, dtype=torch.float32, device="cuda")
+    ops.matmul_gguf_carry(x16, Wc, fmt, N, hidden, got, carry=ops.norm_carry(sumsq_parts=parts, eps=1e-5))
+    xn = ops.rmsnorm(xs.view(1, -1), dev(g), 1e-5, out_dtype=torch.float16)
+    want = ops.matmul_gguf(xn, Wc, fmt, N, hidden, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    assert normwise_rel_err(got.cpu().numpy()[None, :], want.cpu().numpy()) < 5e-4
