@@ -536,6 +536,17 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
   const uint32_t se = (uint32_t)(((uint64_t)p.nsteps * (kw + 1)) / KW);
   const uint32_t cnt = se - sb, last = min(se > sb ? se - 1 : sb, p.nsteps - 1);
 
+  // Batch 1: the epilogue's operands for this thread's output row (D of a binary epilogue, the weight of a carried
+  // norm) are requested now, ahead of everything else, so that the end of the workgroup does not wait for them.
+  // Valid because each output element is read (as D) and written (as C) by the same thread only.
+  float pre_d = 0.0f, pre_g = 0.0f;
+  const uint32_t prow = KW == 1 ? n0 + (uint32_t)r8 : (bid * RWG + (uint32_t)tid / 8) * 8u + ((uint32_t)tid & 7u);
+  const bool pre_ok = MT == 1 && (KW == 1 || tid < RWG * 8) && prow < p.N;
+  if (pre_ok) {
+    if (p.epi.kind == CUTHIP_EPI_BINARY)
+      pre_d = p.c_f16 ? (float)reinterpret_cast<const half_t *>(p.epi.D)[prow] : reinterpret_cast<const float *>(p.epi.D)[prow];
+    if (p.next_norm_w) pre_g = p.next_norm_w[prow];
+  }
   // activation loads first (they must not queue behind the weight loads), then the weight ring, then the
   // conversion of the activations; batches beyond the first (large M * K only) are staged behind the ring
   // groups of 8 activations per thread and batch row in the first batch: sized so that typical shapes need no
@@ -677,10 +688,19 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
       for (int q = 0; q < RQ; ++q) {
         int m = DOT ? q : 2 * q + c.kg;
         if (m < (int)p.M) {
-          float v = store_out_value(p.C, p.epi, p.c_f16, (size_t)m * p.strideC + n0 + r8, out[q]);
-          if (p.next_sumsq_parts && m == 0) {
-            p.next_x16[n0 + r8] = (half_t)(v * p.next_norm_w[n0 + r8]);
-            carry_sq = v * v;
+          if (MT == 1 && p.epi.kind == CUTHIP_EPI_BINARY) {
+            float v = apply_binary(p.epi.op, out[q], pre_d);
+            store_plain(p.C, p.c_f16, n0 + r8, v);
+            if (p.next_sumsq_parts) {
+              p.next_x16[n0 + r8] = (half_t)(v * pre_g);
+              carry_sq = v * v;
+            }
+          } else {
+            float v = store_out_value(p.C, p.epi, p.c_f16, (size_t)m * p.strideC + n0 + r8, out[q]);
+            if (p.next_sumsq_parts && m == 0) {
+              p.next_x16[n0 + r8] = (half_t)(v * p.next_norm_w[n0 + r8]);
+              carry_sq = v * v;
+            }
           }
         }
       }
@@ -707,10 +727,19 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
         if (m < (int)p.M && (rr & 1) == 0 && nn + 1 < p.N)
           store_plain(p.C, p.c_f16, (size_t)m * p.strideC + nn / 2, apply_unary(CUTHIP_UNARY_SILU, v) * up);
       } else if (m < (int)p.M && nn < p.N) {
-        v = store_out_value(p.C, p.epi, p.c_f16, (size_t)m * p.strideC + nn, v);
-        if (p.next_sumsq_parts && m == 0) {
-          p.next_x16[nn] = (half_t)(v * p.next_norm_w[nn]);
-          carry_sq = v * v;
+        if (MT == 1 && p.epi.kind == CUTHIP_EPI_BINARY) {   // nn == prow here
+          v = apply_binary(p.epi.op, v, pre_d);
+          store_plain(p.C, p.c_f16, nn, v);
+          if (p.next_sumsq_parts) {
+            p.next_x16[nn] = (half_t)(v * pre_g);
+            carry_sq = v * v;
+          }
+        } else {
+          v = store_out_value(p.C, p.epi, p.c_f16, (size_t)m * p.strideC + nn, v);
+          if (p.next_sumsq_parts && m == 0) {
+            p.next_x16[nn] = (half_t)(v * p.next_norm_w[nn]);
+            carry_sq = v * v;
+          }
         }
       }
     }
