@@ -556,6 +556,17 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
   XStage<S::SUBK, THREADS, MT, XR, PRO> xst;
   xst.init();
   xst.load(p, 0, tid, gpr);
+  // carried RMSNorm, consumer side: the K / 8 partial sums of squares travel like the activations: requested ahead of
+  // the weight ring, one share per thread, folded per wave and across the waves through LDS at the staging barrier
+  // (the order of the additions depends on the launch shape only)
+  constexpr int CP = 4;
+  const uint32_t nparts = p.sumsq_parts ? (p.K + 7) / 8 : 0u;
+  float cpart[CP];
+#pragma unroll
+  for (int jj = 0; jj < CP; ++jj) {
+    const uint32_t i = (uint32_t)tid + (uint32_t)jj * THREADS;
+    cpart[jj] = i < nparts ? p.sumsq_parts[i] : 0.0f;
+  }
   typename S::Raw buf[D];
 #pragma unroll
   for (int i = 0; i < D; ++i) {
@@ -566,6 +577,12 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
   for (uint32_t base = THREADS * XR; base < gpr; base += THREADS * XR) {
     xst.load(p, base, tid, gpr);
     xst.store(p, base, tid, gpr, xs, sxs, xrow, sxrow);
+  }
+  if (!PRO && nparts) {
+    float t = (cpart[0] + cpart[1]) + (cpart[2] + cpart[3]);
+    for (uint32_t i = (uint32_t)tid + CP * THREADS; i < nparts; i += THREADS) t += p.sumsq_parts[i];
+    t = wave_sum_all(t);
+    if (lane == 0) nrm[wave] = t;
   }
   if (PRO && p.pro == CUTHIP_PRO_RMSNORM) {
 #pragma unroll
@@ -588,14 +605,12 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
       xscale[m] = 1.0f / sqrtf(t / (float)p.K + p.eps);
     }
   }
-  // RMSNorm carried over from the producer of the activations: every wave adds the K / 8 partial sums of squares in
-  // the same order and scales the whole (batch-1) product by one scalar.  (Requesting the partial sums ahead of the
-  // activations and the weight ring measured slower.)
+  // RMSNorm carried over from the producer of the activations: one scalar for the whole (batch-1) product
   float carry_scale = 1.0f;
-  if (p.sumsq_parts) {
+  if (!PRO && nparts) {
     float t = 0.0f;
-    for (uint32_t i = lane; i < (p.K + 7) / 8; i += 64) t += p.sumsq_parts[i];
-    carry_scale = 1.0f / sqrtf(wave_sum_all(t) / (float)p.K + p.eps);
+    for (int w = 0; w < WAVES; ++w) t += nrm[w];
+    carry_scale = 1.0f / sqrtf(t / (float)p.K + p.eps);
   }
 
   // Matrix-core path: A-row j of this lane is batch row j>>2 (clamped), piece j&3, and accumulator quad q
