@@ -252,8 +252,35 @@ int cuthip_matmul_gguf_carry(int fmt, const void *W, const void *A, int a_dtype,
 
 int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, int fmt_b, const void *Wb, uint32_t Nb,
                             void *Cb, const void *A, int a_dtype, int c_dtype, uint32_t K,
-                            const cuthip_norm_carry_t *carry, void *stream) {
+                            const cuthip_norm_carry_t *carry, const cuthip_rope_append_t *rope, void *stream) {
   using namespace cuthip;
+  RopeAppend ra, rb;
+  if (rope) {
+    const uint32_t hd = rope->head_dim;
+    if (!rope->runtime_params || !rope->cos_table || !rope->sin_table || !rope->q_out || !rope->k_cache || !rope->v_cache ||
+        hd == 0 || hd % 2 || rope->q_dim == 0 || rope->q_dim % hd || Na <= rope->q_dim || (Na - rope->q_dim) % hd ||
+        Nb != Na - rope->q_dim || rope->aligned_kv_dim < Nb ||
+        (rope->q_out_dtype != CUTHIP_F32 && rope->q_out_dtype != CUTHIP_F16)) {
+      set_error("cuthip_matmul_gguf_pair: bad RoPE / cache-append arguments (q_dim %u, head_dim %u, Na %u, Nb %u)",
+                rope ? rope->q_dim : 0u, hd, Na, Nb);
+      return CUTHIP_ERR_INVALID;
+    }
+    ra.mode = 1;
+    ra.params = rope->runtime_params;
+    ra.cosT = rope->cos_table;
+    ra.sinT = rope->sin_table;
+    ra.q_out = rope->q_out;
+    ra.q_out_f16 = rope->q_out_dtype == CUTHIP_F16;
+    ra.k_cache = reinterpret_cast<half_t *>(rope->k_cache);
+    ra.v_cache = reinterpret_cast<half_t *>(rope->v_cache);
+    ra.q_dim = rope->q_dim;
+    ra.head_dim = hd;
+    ra.kv_stride = rope->aligned_kv_dim;
+    rb = ra;
+    rb.mode = 2;
+    if (!Ca) Ca = rope->q_out;   // the plain outputs are not written in this mode
+    if (!Cb) Cb = rope->q_out;
+  }
   if (carry && (carry->next_norm_weight || carry->next_x16 || carry->next_sumsq_parts)) {
     set_error("cuthip_matmul_gguf_pair: only the consumer fields of the carried RMSNorm apply here");
     return CUTHIP_ERR_INVALID;
@@ -262,8 +289,9 @@ int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, in
     return rc > 0 ? cuthip_matmul_gguf(fmt_b, Wb, A, a_dtype, Cb, c_dtype, 1, K, Nb, K, Nb, 0, 0, nullptr, -1, stream) : rc;
   if (int rc = check_matmul_args(fmt_b, Wb, A, a_dtype, Cb, c_dtype, 1, K, Nb, K, Nb, CUTHIP_EPI_NONE, nullptr))
     return rc > 0 ? cuthip_matmul_gguf(fmt_a, Wa, A, a_dtype, Ca, c_dtype, 1, K, Na, K, Na, 0, 0, nullptr, -1, stream) : rc;
-  auto params = [&](int fmt, const void *W, uint32_t N, void *C) {
+  auto params = [&](int fmt, const void *W, uint32_t N, void *C, const RopeAppend &r) {
     GemvParams p;
+    p.rope = r;
     p.W = reinterpret_cast<const uint8_t *>(W);
     p.A = A;
     p.C = C;
@@ -277,7 +305,7 @@ int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, in
     return p;
   };
   if ((uint64_t)(K / fmt_elems(fmt_a)) * fmt_bytes(fmt_a) <= 0xFFFFFFFFull && (uint64_t)Na + Nb <= 0x7FFFFFFFull) {
-    const GemvParams pa = params(fmt_a, Wa, Na, Ca), pb = params(fmt_b, Wb, Nb, Cb);
+    const GemvParams pa = params(fmt_a, Wa, Na, Ca, ra), pb = params(fmt_b, Wb, Nb, Cb, rb);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     int rc = CUTHIP_OK;
     bool taken = false;
@@ -288,6 +316,18 @@ int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, in
     if (taken) return rc;
   }
   // other formats or shapes: the same two products as two launches
+  if (rope) {
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const GemvParams pa = params(fmt_a, Wa, Na, Ca, ra), pb = params(fmt_b, Wb, Nb, Cb, rb);
+    bool taken = false;
+    int rc = launch_rows8_any(fmt_a, pa, s, &taken);
+    if (taken && rc == CUTHIP_OK) rc = launch_rows8_any(fmt_b, pb, s, &taken);
+    if (!taken) {
+      set_error("cuthip_matmul_gguf_pair: K = %u does not fit the LDS budget of the 8-row GEMV", K);
+      return CUTHIP_ERR_INVALID;
+    }
+    return rc;
+  }
   if (carry) {
     if (int rc = cuthip_matmul_gguf_carry(fmt_a, Wa, A, a_dtype, Ca, c_dtype, K, Na, 0, 0, nullptr, carry, stream)) return rc;
     return cuthip_matmul_gguf_carry(fmt_b, Wb, A, a_dtype, Cb, c_dtype, K, Nb, 0, 0, nullptr, carry, stream);

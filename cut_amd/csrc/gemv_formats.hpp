@@ -6,6 +6,20 @@
 
 namespace cuthip {
 
+// RoPE and KV-cache append in the epilogue of a batch-1 matmul (the q | k and v projections of a decode step).
+// mode 1: the weight rows are [q heads | k heads], inside each head interleaved as d = 0, half, 1, half + 1, ... so
+// that the two partners of the half-split rotation are neighbouring rows; rotated q goes to q_out, rotated k as
+// fp16 to cache row params[0].  mode 2: the rows are v and go to the cache row as fp16.  mode 0: off.
+struct RopeAppend {
+  int mode = 0;
+  const uint32_t *params = nullptr;
+  const float *cosT = nullptr, *sinT = nullptr;   // [position][head_dim / 2]
+  void *q_out = nullptr;
+  int q_out_f16 = 0;
+  half_t *k_cache = nullptr, *v_cache = nullptr;
+  uint32_t q_dim = 0, head_dim = 0, kv_stride = 0;
+};
+
 struct GemvParams {
   const uint8_t *W;
   const void *A;
@@ -24,6 +38,7 @@ struct GemvParams {
   // fp16(C[n] * next_norm_w[n]) and the sum of C[n]^2 over each group of 8 rows goes to next_sumsq_parts[n / 8].
   // Consumer side (the activations are such a next_x16): the result is multiplied by
   // rsqrt(sum(sumsq_parts[0 .. K/8)) / K + eps).  Fixed summation order, no atomics.
+  RopeAppend rope;
   const float *sumsq_parts = nullptr;
   const float *next_norm_w = nullptr;
   half_t *next_x16 = nullptr;

@@ -76,6 +76,25 @@ __device__ inline float wave_sum_all(float v) {
   return v;
 }
 
+// One output row of a matmul with the RoPE / cache-append epilogue: v = this row's product, partner = the
+// neighbouring row's (row ^ 1), cs / sn = the table entries of the pair at the current position.
+__device__ inline void rope_store(const RopeAppend &r, uint32_t row, float v, float partner, float cs, float sn, uint32_t pos) {
+  if (r.mode == 2) {
+    r.v_cache[(size_t)pos * r.kv_stride + row] = (half_t)v;
+    return;
+  }
+  const uint32_t hd = r.head_dim, w = row % hd, b = w & 1u, d = (w >> 1) + b * (hd / 2);
+  const float x0 = b ? partner : v, x1 = b ? v : partner;   // elements d and d + half of the head, un-rotated
+  const float o = b ? x0 * sn + x1 * cs : x0 * cs - x1 * sn;
+  if (row < r.q_dim) {
+    const size_t i = (size_t)(row - w) + d;
+    if (r.q_out_f16) reinterpret_cast<half_t *>(r.q_out)[i] = (half_t)o;
+    else reinterpret_cast<float *>(r.q_out)[i] = o;
+  } else {
+    r.k_cache[(size_t)pos * r.kv_stride + (row - r.q_dim - w) + d] = (half_t)o;
+  }
+}
+
 template <int FMT> struct Rows8;
 
 // ---- Q4_K -------------------------------------------------------------------
@@ -547,6 +566,13 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
       pre_d = p.c_f16 ? (float)reinterpret_cast<const half_t *>(p.epi.D)[prow] : reinterpret_cast<const float *>(p.epi.D)[prow];
     if (p.next_norm_w) pre_g = p.next_norm_w[prow];
   }
+  float pre_cs = 0.0f, pre_sn = 0.0f;
+  const uint32_t rope_pos = p.rope.mode ? p.rope.params[0] : 0u;
+  if (pre_ok && p.rope.mode == 1) {
+    const size_t ti = (size_t)rope_pos * (p.rope.head_dim / 2) + ((prow % p.rope.head_dim) >> 1);
+    pre_cs = p.rope.cosT[ti];
+    pre_sn = p.rope.sinT[ti];
+  }
   // activation loads first (they must not queue behind the weight loads), then the weight ring, then the
   // conversion of the activations; batches beyond the first (large M * K only) are staged behind the ring
   // groups of 8 activations per thread and batch row in the first batch: sized so that typical shapes need no
@@ -690,7 +716,10 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
   // sits four lanes up (same piece, same K half); in the folded path it is the next thread.
   const bool swiglu = p.epi.kind == CUTHIP_EPI_SWIGLU_PAIRS;
   if (KW == 1) {
-    if (swiglu) {
+    if (MT == 1 && p.rope.mode) {
+      float partner = __shfl_xor(out[0], 4);   // row r8 ^ 1 of this wave
+      if (writer && n0 + r8 < p.N) rope_store(p.rope, n0 + r8, out[0], partner, pre_cs, pre_sn, rope_pos);
+    } else if (swiglu) {
 #pragma unroll
       for (int q = 0; q < RQ; ++q) {
         float up = __shfl_down(out[q], 4);
@@ -737,7 +766,10 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
       float v = 0.0f;
 #pragma unroll
       for (int k = 0; k < KW; ++k) v += red[((rgi * KW + k) * MT + m) * 8 + rr];
-      if (swiglu) {
+      if (MT == 1 && p.rope.mode) {
+        float partner = __shfl_xor(v, 1);
+        if (nn < p.N) rope_store(p.rope, nn, v, partner, pre_cs, pre_sn, rope_pos);
+      } else if (swiglu) {
         float up = __shfl_down(v, 1);
         if (m < (int)p.M && (rr & 1) == 0 && nn + 1 < p.N)
           store_plain(p.C, p.c_f16, (size_t)m * p.strideC + nn / 2, apply_unary(CUTHIP_UNARY_SILU, v) * up);

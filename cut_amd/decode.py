@@ -73,6 +73,8 @@ class DecodeStep:
         launches dominate."""
         if fuse >= 3:
             layers = [dict(L, gate_up=interleave_gate_up(L["gate_up"], cfg.ffn)) for L in layers]
+        if fuse == 4:   # rows of q | k interleaved inside every head for the RoPE epilogue
+            layers = [dict(L, qk=ops.interleave_rope_rows(L["qk"], cfg.q_dim + cfg.kv_dim, cfg.head_dim)) for L in layers]
         self.cfg, self.layers, self.out_norm, self.head, self.fuse = cfg, layers, out_norm, head, fuse
         dev = torch.device(device)
         c = cfg
@@ -142,7 +144,8 @@ class DecodeStep:
         ops.argmax(self.logits, self.token)
 
     def _step_carry(self) -> None:
-        """Seven launches per layer: only the first RMSNorm of the step is a kernel.  Every matmul that forms the
+        """Six launches per layer (q|k|v with RoPE and cache append, attention, merge, wo, gate+up with SwiGLU, down);
+        only the first RMSNorm of the step is a kernel.  Every matmul that forms the
         residual stream (wo, w_down) also stores x * next_norm_weight as fp16 and the sum of x^2 over each group of 8
         outputs; the matmul that consumes it adds those partial sums (fixed order) and scales its result by
         rsqrt(sum / hidden + eps).  Producers and consumers alternate, so one array of partial sums serves all."""
@@ -152,10 +155,11 @@ class DecodeStep:
         ops.rmsnorm(self.x, self.layers[0]["attn_norm"], c.eps, out=self.xn.view(1, -1))
         for i, L in enumerate(self.layers):
             # layer 0 reads the output of the RMSNorm kernel (already scaled); the others the carried form
-            ops.matmul_gguf_pair(self.xn, L["qk"], c.fmt_attn, c.q_dim + c.kv_dim, self.qk, L["v"], c.fmt_v, c.kv_dim, self.v,
-                                 c.hidden, carry=consume if i > 0 else None)
-            ops.rope_kv_write(self.qk[:c.q_dim], self.qk[c.q_dim:], self.v, self.params, self.cos_t, self.sin_t,
-                              self.k_cache[i], self.v_cache[i], c.head_dim, self.q_rot)
+            # q | k | v projections, RoPE and the cache append in one launch
+            ops.matmul_gguf_pair(self.xn, L["qk"], c.fmt_attn, c.q_dim + c.kv_dim, None, L["v"], c.fmt_v, c.kv_dim, None,
+                                 c.hidden, carry=consume if i > 0 else None,
+                                 rope=ops.rope_append(self.params, self.cos_t, self.sin_t, self.q_rot, self.k_cache[i],
+                                                      self.v_cache[i], c.q_dim, c.head_dim))
             ops.attn_decode(self.q_rot, self.k_cache[i], self.v_cache[i], self.params, c.n_heads, c.n_kv_heads, c.head_dim,
                             self.scale, self.ws, self.attn)
             ops.matmul_gguf_carry(self.attn, L["o"], c.fmt_attn, c.hidden, c.q_dim, self.x, binary="add", d=self.x,

@@ -43,6 +43,13 @@ class NormCarry(C.Structure):
                 ("next_sumsq_parts", C.c_void_p)]
 
 
+class RopeAppend(C.Structure):
+    """cuthip_rope_append_t: device pointers as integers."""
+    _fields_ = [("runtime_params", C.c_void_p), ("cos_table", C.c_void_p), ("sin_table", C.c_void_p), ("q_out", C.c_void_p),
+                ("q_out_dtype", C.c_int), ("k_cache", C.c_void_p), ("v_cache", C.c_void_p), ("q_dim", C.c_uint32),
+                ("head_dim", C.c_uint32), ("aligned_kv_dim", C.c_uint32)]
+
+
 class CutHipError(RuntimeError):
     """A C-ABI call returned non-zero (the reference throws std::runtime_error)."""
 
@@ -97,7 +104,8 @@ def load() -> C.CDLL:
     lib.cuthip_matmul_gguf.argtypes = [i, vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, i, vp]
     lib.cuthip_matmul_gguf_workspace_bytes.argtypes = [i, u32, u32, u32, i]
     lib.cuthip_matmul_gguf_ws.argtypes = [i, vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, i, vp, C.c_size_t, vp]
-    lib.cuthip_matmul_gguf_pair.argtypes = [i, vp, u32, vp, i, vp, u32, vp, vp, i, i, u32, C.POINTER(NormCarry), vp]
+    lib.cuthip_matmul_gguf_pair.argtypes = [i, vp, u32, vp, i, vp, u32, vp, vp, i, i, u32, C.POINTER(NormCarry),
+                                            C.POINTER(RopeAppend), vp]
     lib.cuthip_matmul_gguf_carry.argtypes = [i, vp, vp, i, vp, i, u32, u32, i, i, vp, C.POINTER(NormCarry), vp]
     f32 = C.c_float
     lib.cuthip_matmul_gguf_pro.argtypes = [i, vp, vp, i, vp, i, u32, u32, i, i, vp, i, vp, f32, vp]

@@ -135,8 +135,26 @@ def matmul_gguf_carry(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: i
     return out
 
 
-def matmul_gguf_pair(a: torch.Tensor, wa: torch.Tensor, fmt_a, Na: int, out_a: torch.Tensor, wb: torch.Tensor, fmt_b, Nb: int,
-                     out_b: torch.Tensor, K: int, carry=None) -> None:
+def rope_append(runtime_params: torch.Tensor, cos_t: torch.Tensor, sin_t: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor,
+                v_cache: torch.Tensor, q_dim: int, head_dim: int) -> "_l.RopeAppend":
+    """cuthip_rope_append_t for matmul_gguf_pair: rotated q to q_out, rotated k and v to the cache row of the position."""
+    if k_cache.dtype != torch.float16 or v_cache.dtype != torch.float16 or k_cache.stride(0) != v_cache.stride(0):
+        raise _l.CutHipError("rope_append: caches must be fp16 with one row stride")
+    return _l.RopeAppend(runtime_params.data_ptr(), cos_t.data_ptr(), sin_t.data_ptr(), q_out.data_ptr(), _dt(q_out),
+                         k_cache.data_ptr(), v_cache.data_ptr(), q_dim, head_dim, k_cache.stride(0))
+
+
+def interleave_rope_rows(w_blocks: torch.Tensor, n_rows: int, head_dim: int) -> torch.Tensor:
+    """Rows of [heads * head_dim, K] GGUF blocks re-ordered inside every head to d = 0, half, 1, half + 1, ...: the
+    layout the RoPE epilogue of matmul_gguf_pair reads (a permutation of whole block rows)."""
+    rb = w_blocks.numel() // n_rows
+    half = head_dim // 2
+    w = w_blocks.view(n_rows // head_dim, 2, half, rb)
+    return w.permute(0, 2, 1, 3).reshape(-1).contiguous()
+
+
+def matmul_gguf_pair(a: torch.Tensor, wa: torch.Tensor, fmt_a, Na: int, out_a: torch.Tensor | None, wb: torch.Tensor, fmt_b,
+                     Nb: int, out_b: torch.Tensor | None, K: int, carry=None, rope=None) -> None:
     """out_a = a . dequant(wa)^T and out_b = a . dequant(wb)^T for one activation vector a [K], in one launch where the
     formats allow it (cuthip_matmul_gguf_pair)."""
     fa, fb = _fmt(fmt_a), _fmt(fmt_b)
@@ -144,12 +162,17 @@ def matmul_gguf_pair(a: torch.Tensor, wa: torch.Tensor, fmt_a, Na: int, out_a: t
         raise _l.CutHipError("matmul_pair: A must be a contiguous float32/float16 vector of K elements")
     if wa.numel() < n_bytes(fa, Na, K) or wb.numel() < n_bytes(fb, Nb, K):
         raise _l.CutHipError("matmul_pair: weight tensor too small for [N, K]")
+    import ctypes
+    if rope is not None:   # the epilogue writes q_out and the caches; the plain outputs are not used
+        _l.check(_l.load().cuthip_matmul_gguf_pair(
+            fa, wa.data_ptr(), Na, None, fb, wb.data_ptr(), Nb, None, a.data_ptr(), _dt(a), _l.F32, K,
+            ctypes.byref(carry) if carry is not None else None, ctypes.byref(rope), _stream_ptr()))
+        return
     if out_a.dtype != out_b.dtype or out_a.numel() != Na or out_b.numel() != Nb or not (out_a.is_contiguous() and out_b.is_contiguous()):
         raise _l.CutHipError("matmul_pair: outputs must be contiguous [Na] and [Nb] of one dtype")
-    import ctypes
     _l.check(_l.load().cuthip_matmul_gguf_pair(
         fa, wa.data_ptr(), Na, out_a.data_ptr(), fb, wb.data_ptr(), Nb, out_b.data_ptr(), a.data_ptr(), _dt(a), _dt(out_a), K,
-        ctypes.byref(carry) if carry is not None else None, _stream_ptr()))
+        ctypes.byref(carry) if carry is not None else None, None, _stream_ptr()))
 
 
 def matmul_gguf_workspace(fmt, M: int, K: int, N: int, a_dtype: torch.dtype, device) -> torch.Tensor:

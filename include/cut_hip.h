@@ -190,6 +190,21 @@ typedef struct {
   float *next_sumsq_parts;       /* producer: device [ceil(N/8)] out, sum of C^2 over each group of 8 outputs */
 } cuthip_norm_carry_t;
 
+/* RoPE and KV-cache append in the epilogue of cuthip_matmul_gguf_pair, which then is the whole of
+ * "q, k, v projections + FusedRoPEKVWrite" (operators/impl/attention/FusedRoPEKVWrite.cu:12-81) in one launch:
+ * tensor A holds the rows [q heads | k heads], inside every head interleaved as d = 0, head_dim/2, 1,
+ * head_dim/2 + 1, ... (a row permutation done once at load) so that the two partners of the half-split rotation
+ * are neighbouring rows; tensor B holds the v rows.  Rotated q goes to q_out [q_dim] in natural order, rotated k and
+ * v as fp16 to row runtime_params[0] of the caches.  Ca and Cb are not written (may be NULL). */
+typedef struct {
+  const uint32_t *runtime_params;   /* device uint32[2]: {position, sequence length} */
+  const float *cos_table, *sin_table; /* [position][head_dim / 2] */
+  void *q_out;
+  int q_out_dtype;
+  void *k_cache, *v_cache;          /* fp16 [max_ctx][aligned_kv_dim] */
+  uint32_t q_dim, head_dim, aligned_kv_dim;
+} cuthip_rope_append_t;
+
 /* Two batch-1 matmuls on the same activations in one launch:
  *   Ca[Na] = A . dequant(Wa)^T,  Cb[Nb] = A . dequant(Wb)^T,  A [K].
  * For the q/k and v projections of a decode step, whose weights differ in format
@@ -201,7 +216,8 @@ typedef struct {
  * No epilogue; dtypes and alignment as cuthip_matmul_gguf. */
 int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, int fmt_b, const void *Wb, uint32_t Nb,
                             void *Cb, const void *A, int a_dtype, int c_dtype, uint32_t K,
-                            const cuthip_norm_carry_t *carry /* consumer fields only, or NULL */, void *stream);
+                            const cuthip_norm_carry_t *carry /* consumer fields only, or NULL */,
+                            const cuthip_rope_append_t *rope /* or NULL */, void *stream);
 
 /* Batch-1 matmul that takes part in an RMSNorm carried across matmuls, which removes
  * the RMSNorm launches of a decode step (the reference fuses RMSNorm into its

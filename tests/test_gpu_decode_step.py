@@ -327,3 +327,46 @@ def test_carried_rmsnorm_equals_rmsnorm_then_matmul(ops):
     want = ops.matmul_gguf(xn, Wc, fmt, N, hidden, out_dtype=torch.float32)
     torch.cuda.synchronize()
     assert normwise_rel_err(got.cpu().numpy()[None, :], want.cpu().numpy()) < 5e-4
+
+
+@pytest.mark.parametrize("fa,fb", [("Q4_K", "Q6_K"), ("Q4_K", "Q4_K"), ("Q8_0", "Q8_0")])
+@pytest.mark.parametrize("n_heads,n_kv,hd,K,pos", [(32, 8, 128, 4096, 2047), (4, 2, 64, 256, 0), (8, 2, 64, 1024, 17),
+                                                   (2, 1, 16, 512, 3)])
+def test_pair_launch_with_rope_and_cache_append(ops, fa, fb, n_heads, n_kv, hd, K, pos):
+    """q | k | v projections with RoPE and the cache append in the epilogue (rows of q | k interleaved inside every
+    head) against the plain pair launch followed by the RoPE kernel: rotated q, the new cache rows, and nothing else
+    touched.  Shapes cover the direct and the folded epilogue and the two-launch fallback (Q8_0)."""
+    q_dim, kv_dim, max_ctx = n_heads * hd, n_kv * hd, pos + 2
+    fqa, fqb = oracle.FORMATS[fa], oracle.FORMATS[fb]
+    Wqk = dev(quantized_weights(fqa, q_dim + kv_dim, K, seed=100))
+    Wv = dev(quantized_weights(fqb, kv_dim, K, seed=101))
+    x = dev(gauss_acts((1, K), seed=102, dtype=np.float16)).view(-1)
+    cos_t, sin_t = _tables(max_ctx, hd)
+    params = dev(np.array([pos, pos + 1], np.int32))
+    # reference: plain pair launch, then the RoPE kernel
+    qk = torch.empty(q_dim + kv_dim, dtype=torch.float32, device="cuda")
+    v = torch.empty(kv_dim, dtype=torch.float32, device="cuda")
+    ops.matmul_gguf_pair(x, Wqk, fqa, q_dim + kv_dim, qk, Wv, fqb, kv_dim, v, K)
+    k1 = torch.full((max_ctx, kv_dim + 8), 3.0, dtype=torch.float16, device="cuda")
+    v1 = torch.full_like(k1, 5.0)
+    q1 = torch.empty(q_dim, dtype=torch.float32, device="cuda")
+    ops.rope_kv_write(qk[:q_dim], qk[q_dim:], v, params, dev(cos_t), dev(sin_t), k1[:, :kv_dim], v1[:, :kv_dim], hd, q1)
+    # fused
+    Wqk_il = ops.interleave_rope_rows(Wqk, q_dim + kv_dim, hd)
+    k2 = torch.full((max_ctx, kv_dim + 8), 3.0, dtype=torch.float16, device="cuda")
+    v2 = torch.full_like(k2, 5.0)
+    q2 = torch.empty(q_dim, dtype=torch.float32, device="cuda")
+    ops.matmul_gguf_pair(x, Wqk_il, fqa, q_dim + kv_dim, None, Wv, fqb, kv_dim, None, K,
+                         rope=ops.rope_append(params, dev(cos_t), dev(sin_t), q2, k2[:, :kv_dim], v2[:, :kv_dim], q_dim, hd))
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(q2.cpu().numpy(), q1.cpu().numpy(), rtol=2e-6, atol=2e-6)
+    kd = k2.cpu().numpy().view(np.uint16).astype(np.int32) - k1.cpu().numpy().view(np.uint16).astype(np.int32)
+    assert np.max(np.abs(kd)) <= 1   # fma contraction may differ between the two code sites: at most one fp16 ulp
+    assert np.array_equal(v2.cpu().numpy().view(np.uint16), v1.cpu().numpy().view(np.uint16))
+    assert torch.all(k2[:, kv_dim:] == 3.0) and torch.all(v2[:, kv_dim:] == 5.0)
+    assert torch.all(k2[:pos] == 3.0) and torch.all(k2[pos + 1:] == 3.0)
+    # the row permutation itself
+    rb = oracle.n_bytes(fqa, K)
+    il = Wqk_il.cpu().numpy().reshape(-1, hd, rb)
+    w = Wqk.cpu().numpy().reshape(-1, hd, rb)
+    assert np.array_equal(il[:, 0::2], w[:, :hd // 2]) and np.array_equal(il[:, 1::2], w[:, hd // 2:])
