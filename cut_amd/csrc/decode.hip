@@ -167,6 +167,15 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_
   const uint32_t t0 = split * kAttnChunk;
   const uint32_t nvalid = t0 < seqLen ? min((uint32_t)kAttnChunk, seqLen - t0) : 0u;
 
+  // the query of the first pass is requested before anything else: it does not depend on the sequence length, and
+  // loaded after the staging barrier it would cost a memory round trip of its own
+  float q_pre[2] = {0.0f, 0.0f};
+  {
+    const uint32_t h0 = kvH * nRep + (wave < nRep ? wave : 0);
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+      if (lane + 64 * e < headDim) q_pre[e] = ld_act(q, q_f16, (size_t)h0 * headDim + lane + 64 * e);
+  }
   // stage the chunk of K and V (16-byte pieces; rows past the sequence are zero)
   const uint32_t pieces = headDim / 8;
   for (uint32_t i = tid; i < kAttnChunk * pieces; i += 256) {
@@ -186,7 +195,13 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_
     const bool live = rep < nRep;
     const uint32_t h = kvH * nRep + (live ? rep : 0);
     __syncthreads();   // K, V staged (first pass) / Qs, Ps free again (later passes)
-    for (uint32_t d = lane; d < headDim; d += 64) Qs[wave * kAttnMaxHd + d] = ld_act(q, q_f16, (size_t)h * headDim + d);
+    if (rep0 == 0) {
+#pragma unroll
+      for (int e = 0; e < 2; ++e)
+        if (lane + 64 * e < headDim) Qs[wave * kAttnMaxHd + lane + 64 * e] = q_pre[e];
+    } else {
+      for (uint32_t d = lane; d < headDim; d += 64) Qs[wave * kAttnMaxHd + d] = ld_act(q, q_f16, (size_t)h * headDim + d);
+    }
     __syncthreads();
     // score of position t0 + lane: q is read as broadcast 16-byte pieces
     float sc = 0.0f;
