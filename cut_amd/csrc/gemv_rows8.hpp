@@ -886,11 +886,16 @@ static int launch_rows8_pair(const GemvParams &pa, const GemvParams &pb, hipStre
 struct Rows8Shape { int rwg, kw; };
 Rows8Shape pick_rows8_shape(uint32_t N, uint32_t nsteps);
 
+// LDS a workgroup may ask for.  More would fit (160 KB per CU), but every workgroup stages all of its activations:
+// at 129 KB (4 batch rows, K = 14336) the staging traffic makes this kernel slower than the 32-row fallback
+// (30 us against 23.5 us for 4096 x 14336), so such shapes stay with the fallback.
+constexpr size_t kRows8LdsBudget = 96 * 1024;
+
 // true if the rows8 kernel can take the problem (activations must fit in LDS)
 template <int FMT> bool rows8_fits(const GemvParams &p) {
   if (p.M > 8) return false;
   int mt = p.M <= 1 ? 1 : (p.M <= 2 ? 2 : (p.M <= 4 ? 4 : 8));
-  return rows8_lds_bytes<FMT>(p, mt) <= 96 * 1024;
+  return rows8_lds_bytes<FMT>(p, mt) <= kRows8LdsBudget;
 }
 
 template <int FMT> int launch_rows8_fmt(const GemvParams &p, hipStream_t stream) {
@@ -906,7 +911,7 @@ template <int FMT> int launch_rows8_fmt(const GemvParams &p, hipStream_t stream)
 // anything else, and the caller issues two launches.
 template <int FA, int FB> bool launch_rows8_pair_fmt(const GemvParams &pa, const GemvParams &pb, hipStream_t stream, int *rc) {
   if (pa.M != 1 || pb.M != 1 || pa.K != pb.K || pa.pro || pb.pro) return false;
-  if (rows8_lds_bytes<FA>(pa, 1) > 96 * 1024 || rows8_lds_bytes<FB>(pb, 1) > 96 * 1024) return false;
+  if (rows8_lds_bytes<FA>(pa, 1) > kRows8LdsBudget || rows8_lds_bytes<FB>(pb, 1) > kRows8LdsBudget) return false;
   Rows8Shape s = pick_rows8_shape(pa.N + pb.N, pa.nsteps);
   constexpr int D = 4;
   if (s.kw == 1 && s.rwg < 8) *rc = launch_rows8_pair<FA, FB, 4, 1, D, 2>(pa, pb, stream);
