@@ -860,6 +860,9 @@ template <int FMT, int MT> static int launch_rows8_shape(const GemvParams &p, in
   }
   if (kw == 2) return launch_rows8<FMT, MT, 2, 2, D, 4>(p, stream);
   if (kw == 4) {
+    if constexpr (MT == 1) {
+      if (rwg == 2) return launch_rows8<FMT, MT, 2, 4, D, 4>(p, stream);   // two row groups share one staging of a long x
+    }
     if (p.nsteps <= 16) return launch_rows8<FMT, MT, 1, 4, D, 2>(p, stream);
     return launch_rows8<FMT, MT, 1, 4, D, 8>(p, stream);
   }
