@@ -76,7 +76,7 @@ def timed_graph(torch, fn_step, steps, warmup):
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE (x 2.000, the factor a plain
 # 1 GiB copy gives on this part) + WRITE_SIZE (x 1.000), launch-weighted over gate, up, down
 # (profiles/gemv_q4k_ffn_batch1.md holds the counters and the commands)
-TRAFFIC_BYTES_PER_LAUNCH = 33690829
+TRAFFIC_BYTES_PER_LAUNCH = 33689600
 
 
 def bench_decode_step(torch, np, ops, dev, x_h, steps=5):
