@@ -156,7 +156,7 @@ constexpr int kAttnRow = kAttnMaxHd + 8;   // LDS row in halfs: +16 bytes keeps 
 __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_f16, const half_t *kCache, const half_t *vCache,
                                                            const uint32_t *params, float *partial, uint32_t nHeads,
                                                            uint32_t nKvHeads, uint32_t headDim, uint32_t alignedKvDim,
-                                                           float scale, uint32_t nsplit) {
+                                                           float scale, uint32_t nsplit, uint32_t maxSeqLen) {
   __shared__ __attribute__((aligned(16))) half_t Ks[kAttnChunk * kAttnRow];
   __shared__ __attribute__((aligned(16))) half_t Vs[kAttnChunk * kAttnRow];
   __shared__ __attribute__((aligned(16))) float Qs[4 * kAttnMaxHd];
@@ -180,11 +180,14 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_
   const uint32_t pieces = headDim / 8;
   for (uint32_t i = tid; i < kAttnChunk * pieces; i += 256) {
     uint32_t r = i / pieces, c8 = i % pieces;
-    u32x4 kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
-    if (r < nvalid) {
-      size_t off = (size_t)(t0 + r) * alignedKvDim + kvH * headDim + c8 * 8;
-      kv = ld_u32x4(reinterpret_cast<const uint8_t *>(kCache + off));
-      vv = ld_u32x4(reinterpret_cast<const uint8_t *>(vCache + off));
+    // the loads do not wait for the sequence length (every row below the cache capacity is readable); rows past
+    // the sequence are zeroed afterwards
+    size_t off = (size_t)min(t0 + r, maxSeqLen - 1) * alignedKvDim + kvH * headDim + c8 * 8;
+    u32x4 kv = ld_u32x4(reinterpret_cast<const uint8_t *>(kCache + off));
+    u32x4 vv = ld_u32x4(reinterpret_cast<const uint8_t *>(vCache + off));
+    if (r >= nvalid) {
+      kv = u32x4{0, 0, 0, 0};
+      vv = u32x4{0, 0, 0, 0};
     }
     *reinterpret_cast<u32x4 *>(Ks + r * kAttnRow + c8 * 8) = kv;
     *reinterpret_cast<u32x4 *>(Vs + r * kAttnRow + c8 * 8) = vv;
@@ -263,8 +266,10 @@ __global__ void __launch_bounds__(128) attn_merge_kernel(const float *partial, c
   __shared__ float Ws[kAttnMaxSplit];
   __shared__ float red[4];
   const uint32_t h = blockIdx.x, tid = threadIdx.x;
-  const uint32_t seqLen = params[1];
-  const uint32_t used = min(nsplit, (seqLen + kAttnChunk - 1) / kAttnChunk);
+  // every split has a record (empty ones carry max = -inf, sum = 0), so the merge does not need the sequence length
+  // and its loads do not wait for it
+  (void)params;
+  const uint32_t used = nsplit;
   const uint32_t rec = 2 + headDim;
   const float *base = partial + (size_t)h * nsplit * rec;
   float m = -INFINITY;
@@ -275,7 +280,8 @@ __global__ void __launch_bounds__(128) attn_merge_kernel(const float *partial, c
   const float M = fmaxf(red[0], red[1]);
   float l = 0.0f;
   for (uint32_t s = tid; s < used; s += 128) {
-    float w = expf(base[(size_t)s * rec] - M);
+    float ms = base[(size_t)s * rec];
+    float w = ms == -INFINITY ? 0.0f : expf(ms - M);   // an empty split (and an empty sequence: M = -inf) weighs nothing
     Ws[s] = w;
     l = fmaf(base[(size_t)s * rec + 1], w, l);
   }
@@ -287,7 +293,7 @@ __global__ void __launch_bounds__(128) attn_merge_kernel(const float *partial, c
     float o = 0.0f;
 #pragma unroll 8
     for (uint32_t s = 0; s < used; ++s) o = fmaf(base[(size_t)s * rec + 2 + tid], Ws[s], o);
-    st_act(out, out_f16, (size_t)h * headDim + tid, used ? o / L : 0.0f);
+    st_act(out, out_f16, (size_t)h * headDim + tid, L > 0.0f ? o / L : 0.0f);
   }
 }
 
@@ -432,7 +438,7 @@ int cuthip_attn_decode(const void *q, int q_dtype, const void *k_cache, const vo
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(attn_partial_kernel, dim3(n_kv_heads, nsplit), dim3(256), 0, s, q, q_dtype == CUTHIP_F16,
                      (const half_t *)k_cache, (const half_t *)v_cache, runtime_params, (float *)workspace, n_heads, n_kv_heads,
-                     head_dim, aligned_kv_dim, scale, nsplit);
+                     head_dim, aligned_kv_dim, scale, nsplit, max_seq_len);
   if (int rc = check_hip(hipGetLastError(), "attention launch")) return rc;
   hipLaunchKernelGGL(attn_merge_kernel, dim3(n_heads), dim3(128), 0, s, (const float *)workspace, runtime_params, out,
                      out_dtype == CUTHIP_F16, head_dim, nsplit);
