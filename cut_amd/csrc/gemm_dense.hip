@@ -30,6 +30,9 @@
 //
 // Numerics: weights rounded to fp16 once (2^-11 relative), fp32 activations rounded
 // to fp16 once, fp32 accumulation: the same error budget as the single-launch GEMM.
+#include <stdio.h>
+#include <stdlib.h>
+
 #include <type_traits>
 #include <utility>
 
@@ -62,19 +65,20 @@ struct DenseParams {
 
 constexpr int kDBN = 256, kDBK = 64;
 
-template <int BM>
+template <int BM, int BN>
 __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // LDS address-space casts and AMDGPU inline asm: the host pass only needs the stub
-  constexpr int MI = BM / 64, NJ = kDBN / 64;  // 32 x 32 MFMA tiles per wave: MI x NJ
+  constexpr int MI = BM / 64, NJ = BN / 64;  // 32 x 32 MFMA tiles per wave: MI x NJ
   constexpr int NM = MI * NJ;                  // MFMAs per k-step of 16
-  constexpr int NLA = BM / 32, NL = (BM + kDBN) / 32;  // LDS-direct loads per wave per slice (A, total)
-  constexpr int LSTEP = MI == 4 ? 3 : 2;       // one load every LSTEP-th MFMA slot
-  static_assert(NJ == 4 && (MI == 4 || MI == 2), "tile shape");
+  constexpr int NLA = BM / 32, NL = (BM + BN) / 32;  // LDS-direct loads per wave per slice (A, total)
+  constexpr int LSTEP = (NL - 1) * 3 < 3 * NM ? 3 : 2;   // one load every LSTEP-th MFMA slot
+  static_assert((NJ == 4 && (MI == 4 || MI == 2)) || (NJ == 7 && MI == 2), "tile shape");
+  static_assert((BM + BN) * 128 * 2 <= 160 * 1024, "two LDS stages");
   static_assert((NL - 1) * LSTEP < 3 * NM, "the last load must be issued before the last k-step of the slice");
   __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * 128];
   __shared__ __attribute__((aligned(1024))) uint8_t sA1[BM * 128];
-  __shared__ __attribute__((aligned(1024))) uint8_t sB0[kDBN * 128];
-  __shared__ __attribute__((aligned(1024))) uint8_t sB1[kDBN * 128];
+  __shared__ __attribute__((aligned(1024))) uint8_t sB0[BN * 128];
+  __shared__ __attribute__((aligned(1024))) uint8_t sB1[BN * 128];
 
   // XCD-aware tile order: ids id, id+8, id+16, ... share an XCD and its L2; give
   // them the M-tiles of the same weight panels.
@@ -88,12 +92,12 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
     nt = id / p.mtiles;
     mt = id % p.mtiles;
   }
-  const uint32_t m0 = mt * BM, n0 = nt * kDBN;
+  const uint32_t m0 = mt * BM, n0 = nt * BN;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
 
   // copy assignment: load v of wave w fills the 8-row group 4 v + w of its tile
-  uint32_t aoff[NLA], boff[kDBN / 32];
+  uint32_t aoff[NLA], boff[BN / 32];
   // tile row r keeps its 16-byte chunk c at position c ^ ((r >> 1) & 7): the 16 lanes the LDS serves per cycle
   // (16 consecutive rows, one chunk index) then cover all 64 banks.  For the row 8 g + (lane >> 3) of 8-row group
   // g = 4 v + wave that key is (4 (wave & 1) + (lane >> 4)) & 7, the same for every v.
@@ -104,7 +108,7 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
     aoff[v] = r * p.strideA * 2 + chunk;
   }
 #pragma unroll
-  for (int v = 0; v < kDBN / 32; ++v) {
+  for (int v = 0; v < BN / 32; ++v) {
     uint32_t r = min(n0 + 8 * (4 * v + wave) + (lane >> 3), p.N - 1);
     boff[v] = r * p.K * 2 + chunk;
   }
@@ -122,7 +126,7 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
 #pragma unroll
     for (int j = 0; j < NJ; ++j) acc[i][j] = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
-  const uint32_t arow = (wm * (BM / 2) + (lane & 31)) * 128, brow = (wn * 128 + (lane & 31)) * 128;
+  const uint32_t arow = (wm * (BM / 2) + (lane & 31)) * 128, brow = (wn * (BN / 2) + (lane & 31)) * 128;
   uint32_t xs[4];
 #pragma unroll
   for (int s = 0; s < 4; ++s) xs[s] = ((2 * s + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
@@ -133,7 +137,8 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
 #define CUTHIP_WAIT_FRAGS(f, n)                                                                                  \
   asm volatile("s_waitcnt lgkmcnt(" #n ")"                                                                         \
                : "+v"(fa[f][0]), "+v"(fa[f][1]), "+v"(fa[f][MI - 2]), "+v"(fa[f][MI - 1]), "+v"(fb[f][0]),         \
-                 "+v"(fb[f][1]), "+v"(fb[f][2]), "+v"(fb[f][3]))
+                 "+v"(fb[f][1]), "+v"(fb[f][2]), "+v"(fb[f][3]), "+v"(fb[f][NJ - 3]), "+v"(fb[f][NJ - 2]),           \
+                 "+v"(fb[f][NJ - 1]))
 
   // The NM MFMAs of one k-step on fragment set f.  After MFMA idx: the idx-th fragment read of k-step s of
   // (sa, sb) into the other set, and, in every LSTEP-th slot of the slice (g = position of the group in the
@@ -196,7 +201,7 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
   // Compile-time tile indices: a rolled loop would index the accumulators dynamically and copy them to scratch.
   static_for<MI * NJ>([&](auto ij) {
     constexpr int i = decltype(ij)::value / NJ, j = decltype(ij)::value % NJ;
-    const uint32_t col = n0 + wn * 128 + 32 * j + (lane & 31);
+    const uint32_t col = n0 + wn * (BN / 2) + 32 * j + (lane & 31);
     const uint32_t row0 = m0 + wm * (BM / 2) + 32 * i + 4 * (lane >> 5);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -234,15 +239,15 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *partial
   store_out(C, epi, c_f16, (size_t)row * strideC + col, v);
 }
 
-template <int BM> static int launch_dense_bm(DenseParams p, hipStream_t stream) {
+template <int BM, int BN> static int launch_dense_bm(DenseParams p, hipStream_t stream) {
   p.mtiles = (p.M + BM - 1) / BM;
-  p.ntiles = (p.N + kDBN - 1) / kDBN;
+  p.ntiles = (p.N + BN - 1) / BN;
   uint64_t grid = (uint64_t)p.mtiles * p.ntiles * p.ksplit;
   if (grid > 0x7FFFFFFFull) {
     set_error("cuthip_matmul_gguf_ws: problem too large for one launch");
     return CUTHIP_ERR_INVALID;
   }
-  auto kern = gemm_dense_kernel<BM>;
+  auto kern = gemm_dense_kernel<BM, BN>;
   hipLaunchKernelGGL(kern, dim3((uint32_t)grid), dim3(256), 0, stream, p);
   return check_hip(hipGetLastError(), "dense gemm launch");
 }
@@ -262,15 +267,24 @@ bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a
 
 // Tile height and number of K ranges: 256-row tiles when they give every CU a workgroup, else 128-row tiles if
 // those do, else 256-row tiles with K split (partials in the workspace, summed by a second kernel).
-struct DenseShape { int bm; uint32_t ksplit; };
+struct DenseShape { int bm, bn; uint32_t ksplit; };
 static DenseShape pick_dense_shape(uint32_t M, uint32_t K, uint32_t N) {
   const uint64_t nt = (N + kDBN - 1) / kDBN, tiles256 = (uint64_t)((M + 255) / 256) * nt, tiles128 = (uint64_t)((M + 127) / 128) * nt;
-  if (tiles256 >= 256) return DenseShape{256, 1};
-  if (tiles128 >= 224) return DenseShape{128, 1};
+  // 128 x 448 tiles when they come out as whole rounds over the 256 CUs where 256 x 256 tiles would leave a partial
+  // round (N = 14336 = 32 x 448 at M = 2048: 512 tiles = 2 rounds, against 448 tiles = 1.75 rounds)
+  if (const char *env = getenv("CUT_HIP_DENSE_TILE")) {   // "bm,bn" tuning aid: 256,256 / 128,256 / 128,448
+    int bm = 0, bn = 0;
+    if (sscanf(env, "%d,%d", &bm, &bn) == 2 && ((bn == 256 && (bm == 256 || bm == 128)) || (bn == 448 && bm == 128)))
+      return DenseShape{bm, bn, 1};
+  }
+  const uint64_t t448 = (uint64_t)((M + 127) / 128) * ((N + 447) / 448);
+  if (N % 448 == 0 && t448 >= 256 && t448 % 256 == 0 && tiles256 % 256 != 0) return DenseShape{128, 448, 1};
+  if (tiles256 >= 256) return DenseShape{256, 256, 1};
+  if (tiles128 >= 224) return DenseShape{128, 256, 1};
   uint32_t s = 1;
   while (s < 8 && tiles256 * s < 192 && K % (2 * s * 128) == 0) s *= 2;
-  if (s == 1) return DenseShape{tiles128 > tiles256 ? 128 : 256, 1};
-  return DenseShape{256, s};
+  if (s == 1) return DenseShape{tiles128 > tiles256 ? 128 : 256, 256, 1};
+  return DenseShape{256, 256, s};
 }
 
 static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
@@ -314,7 +328,11 @@ int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C,
   p.ksplit = sh.ksplit;
   p.kper = K / sh.ksplit;
   p.partial = reinterpret_cast<float *>(w16 + align256((size_t)N * K * 2) + align256(a_f16 ? 0 : (size_t)M * K * 2));
-  if (int rc = sh.bm == 256 ? launch_dense_bm<256>(p, stream) : launch_dense_bm<128>(p, stream)) return rc;
+  int rc;
+  if (sh.bn == 448) rc = launch_dense_bm<128, 448>(p, stream);
+  else if (sh.bm == 256) rc = launch_dense_bm<256, 256>(p, stream);
+  else rc = launch_dense_bm<128, 256>(p, stream);
+  if (rc) return rc;
   if (sh.ksplit > 1) {
     const uint64_t mn = (uint64_t)M * N;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((uint32_t)((mn + 255) / 256)), dim3(256), 0, stream, p.partial, sh.ksplit, M,

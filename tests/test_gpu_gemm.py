@@ -215,3 +215,22 @@ def test_dense_gemm_prefill_shapes_sampled(ops, M, N, K):
     want = oracle.matmul_gguf(fmt, Ws, A[rows].astype(np.float32), len(cols), f64=True)
     err = normwise_rel_err(got[np.ix_(rows, cols)], want)
     assert err < 8e-4, err
+
+
+def test_dense_gemm_128x448_tiles(ops):
+    """The tile shape chosen when it makes whole rounds over the CUs (N a multiple of 448, 256 tiles): sampled rows and
+    columns against the oracle, every output against the single-launch GEMM."""
+    fmt = oracle.Q4_K
+    M, N, K = 4096 - 5, 3584, 512   # ragged last row tile
+    W = quantized_weights(fmt, N, K, seed=51)
+    A = gauss_acts((M, K), seed=52, dtype=np.float16)
+    got = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32)
+    ref = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=2)
+    assert normwise_rel_err(got, ref) < 2e-4
+    assert np.all(np.abs(got - ref) <= 2e-3 * np.abs(ref) + 1e-3)
+    rng = np.random.default_rng(6)
+    rows = np.unique(np.concatenate([[0, 127, 128, M - 1], rng.integers(0, M, 12)]))
+    cols = np.unique(np.concatenate([[0, 223, 224, 447, 448, N - 1], rng.integers(0, N, 200)]))
+    Ws = np.ascontiguousarray(W.reshape(N, oracle.n_bytes(fmt, K))[cols]).reshape(-1)
+    want = oracle.matmul_gguf(fmt, Ws, A[rows].astype(np.float32), len(cols), f64=True)
+    assert normwise_rel_err(got[np.ix_(rows, cols)], want) < TOL_GEMM
