@@ -220,11 +220,14 @@ def main():
     w_bytes = ops.n_bytes("Q4_K", N_FF, N_EMBD)  # 33,030,144 for either shape
 
     def ffn_step(b):
+        # batch 3-8: with a workspace the long-row down projection splits K across workgroups
+        ws_down = ops.matmul_gguf_workspace("Q4_K", b, N_FF, N_EMBD, torch.float16, dev) if b > 2 else None
+
         def step(s):
             i = s % COPIES
             ops.matmul_gguf(x[:b], gate[i], "Q4_K", N_FF, N_EMBD, out=y_gate[:b])
             ops.matmul_gguf(x[:b], up[i], "Q4_K", N_FF, N_EMBD, out=y_up[:b])
-            ops.matmul_gguf(h[:b], down[i], "Q4_K", N_EMBD, N_FF, out=y_down[:b])
+            ops.matmul_gguf(h[:b], down[i], "Q4_K", N_EMBD, N_FF, out=y_down[:b], workspace=ws_down)
         return step
 
     def ffn_bytes(b):

@@ -39,6 +39,29 @@ Rows8Shape pick_rows8_shape(uint32_t N, uint32_t nsteps) {
   return Rows8Shape{groups >= 8192 ? 8 : 4, kw};
 }
 
+#define CUTHIP_EXTERN_KSPLIT(F) \
+  extern template int launch_rows8_ksplit<F>(const GemvParams &, float *, uint32_t *, hipStream_t);
+CUTHIP_EXTERN_KSPLIT(CUTHIP_Q8_0)
+CUTHIP_EXTERN_KSPLIT(CUTHIP_Q4_0)
+CUTHIP_EXTERN_KSPLIT(CUTHIP_Q4_K)
+CUTHIP_EXTERN_KSPLIT(CUTHIP_Q6_K)
+#undef CUTHIP_EXTERN_KSPLIT
+
+// defined with the two-pass GEMM: C = epilogue(sum of the fp32 partial products)
+__global__ void splitk_reduce_kernel(const float *partial, uint32_t ksplit, uint32_t M, uint32_t N, void *C, uint32_t strideC,
+                                     Epilogue epi, int c_f16);
+
+// The split across workgroups pays where one row group per workgroup would re-stage long activations for few rows:
+// batch 2-8, rows of at least 32 steps, and not enough row groups to fill the chip without splitting K.
+static bool ksplit_gemv_preferred(uint32_t M, uint32_t K, uint32_t N) {
+  // from 3 batch rows on (two rows of K = 14336 still fit the LDS budget of the unsplit kernel, which then measures
+  // faster: 13.3 us against 16 us for 4096 x 14336)
+  return M >= 3 && M <= 8 && K >= 8192 && (N + 7) / 8 < 1536;
+}
+static size_t ksplit_gemv_workspace(uint32_t M, uint32_t K, uint32_t N) {
+  return (size_t)rows8_ksplit_parts(N, (K + 255) / 256) * M * N * sizeof(float);
+}
+
 #define CUTHIP_EXTERN_PAIR(FA, FB) \
   extern template bool launch_rows8_pair_fmt<FA, FB>(const GemvParams &, const GemvParams &, hipStream_t, int *);
 CUTHIP_EXTERN_PAIR(CUTHIP_Q4_K, CUTHIP_Q4_K)
@@ -341,6 +364,7 @@ int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, in
 
 size_t cuthip_matmul_gguf_workspace_bytes(int fmt, uint32_t M, uint32_t K, uint32_t N, int a_dtype) {
   (void)fmt;
+  if (cuthip::ksplit_gemv_preferred(M, K, N)) return cuthip::ksplit_gemv_workspace(M, K, N);
   return cuthip::dense_gemm_workspace(M, K, N, a_dtype == CUTHIP_F16);
 }
 
@@ -354,6 +378,36 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   if (int rc = check_matmul_args(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, D))
     return rc > 0 ? CUTHIP_OK : rc;
   const int a_f16 = a_dtype == CUTHIP_F16;
+  // batch 2-8 on long rows: the 8-row GEMV with K split across workgroups, partial products in the workspace
+  if (variant == -1 && ksplit_gemv_preferred(M, K, N) && workspace && (uintptr_t)workspace % 16 == 0 &&
+      workspace_bytes >= ksplit_gemv_workspace(M, K, N) && (uintptr_t)A % 16 == 0 && (strideA * (a_f16 ? 2 : 4)) % 16 == 0) {
+    GemvParams p;
+    p.W = reinterpret_cast<const uint8_t *>(W);
+    p.A = A;
+    p.C = C;
+    p.epi = Epilogue{CUTHIP_EPI_NONE, 0, nullptr};
+    p.M = M; p.K = K; p.N = N; p.strideA = strideA; p.strideC = strideC;
+    p.nsteps = (K + 255) / 256;
+    p.row_bytes = (uint32_t)((uint64_t)(K / fmt_elems(fmt)) * fmt_bytes(fmt));
+    p.a_f16 = a_f16;
+    p.c_f16 = c_dtype == CUTHIP_F16;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    float *partial = reinterpret_cast<float *>(workspace);
+    uint32_t parts = 0;
+    int rc;
+    switch (fmt) {
+    case CUTHIP_Q8_0: rc = launch_rows8_ksplit<CUTHIP_Q8_0>(p, partial, &parts, s); break;
+    case CUTHIP_Q4_0: rc = launch_rows8_ksplit<CUTHIP_Q4_0>(p, partial, &parts, s); break;
+    case CUTHIP_Q4_K: rc = launch_rows8_ksplit<CUTHIP_Q4_K>(p, partial, &parts, s); break;
+    default: rc = launch_rows8_ksplit<CUTHIP_Q6_K>(p, partial, &parts, s); break;
+    }
+    if (rc) return rc;
+    Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
+    const uint64_t mn = (uint64_t)M * N;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((uint32_t)((mn + 255) / 256)), dim3(256), 0, s, partial, parts, M, N, C,
+                       strideC, epi, c_dtype == CUTHIP_F16);
+    return check_hip(hipGetLastError(), "split-K reduce launch");
+  }
   const bool fits = dense_gemm_fits(M, K, N, strideA, a_f16, A);
   const size_t need = dense_gemm_workspace(M, K, N, a_f16);
   const bool ws_ok = workspace && (uintptr_t)workspace % 256 == 0 && workspace_bytes >= need;

@@ -6,4 +6,5 @@ namespace cuthip {
 template int launch_fmt<CUTHIP_Q4_0>(GemvParams, hipStream_t);
 template int launch_rows8_fmt<CUTHIP_Q4_0>(const GemvParams &, hipStream_t);
 template bool rows8_fits<CUTHIP_Q4_0>(const GemvParams &);
+template int launch_rows8_ksplit<CUTHIP_Q4_0>(const GemvParams &, float *, uint32_t *, hipStream_t);
 }

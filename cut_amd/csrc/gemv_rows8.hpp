@@ -811,6 +811,28 @@ __global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_kernel(GemvParams
   rows8_body<FMT, MT, RWG, KW, D, XWANT, PRO>(p, blockIdx.x);
 }
 
+// K split across workgroups for long rows and few of them (the down projection at batch 2-8): workgroup
+// (part, block) multiplies the K range `part` of 8 row groups and writes fp32 partial products
+// partial[part][m][n]; a second kernel sums the parts and applies the epilogue.  Eight row groups per workgroup
+// keep the staging of the activations (all of a K range per workgroup) an eighth of what one row group per
+// workgroup would read, and the K ranges supply the workgroups that N / 64 alone would not.
+template <int FMT, int MT, int D>
+__global__ void __launch_bounds__(64 * 8, 2) gemv_rows8_ksplit_kernel(GemvParams p, uint32_t nblocks, uint32_t part_steps,
+                                                                       float *partial) {
+  const uint32_t part = blockIdx.x / nblocks, bid = blockIdx.x - part * nblocks;
+  const uint32_t k_lo = part * part_steps * 256u, k_hi = min(p.K, k_lo + part_steps * 256u);
+  if (k_lo >= p.K) return;   // the host launches no empty part (k_hi - k_lo would wrap around)
+  p.A = reinterpret_cast<const uint8_t *>(p.A) + (size_t)k_lo * (p.a_f16 ? 2 : 4);
+  p.W += (size_t)(k_lo / Fmt<FMT>::elems) * Fmt<FMT>::bytes;
+  p.K = k_hi - k_lo;
+  p.nsteps = (p.K + 255) / 256;
+  p.C = partial + (size_t)part * p.M * p.N;
+  p.strideC = p.N;
+  p.c_f16 = 0;
+  p.epi = Epilogue{CUTHIP_EPI_NONE, 0, nullptr};
+  rows8_body<FMT, MT, 8, 1, D, 1, false>(p, bid);
+}
+
 // Two weight tensors (formats FA, FB) against the same batch-1 activations in one launch: workgroups
 // [0, blocks_a) take the rows of the first, the rest the rows of the second.  Saves a launch and a kernel
 // start where a small projection (w_v) sits next to a larger one (w_q | w_k) of another format.
@@ -884,6 +906,50 @@ static int launch_rows8_pair(const GemvParams &pa, const GemvParams &pb, hipStre
   uint32_t blocks_a = ((pa.N + 7) / 8 + RWG - 1) / RWG, blocks_b = ((pb.N + 7) / 8 + RWG - 1) / RWG;
   hipLaunchKernelGGL(kern, dim3(blocks_a + blocks_b), dim3(64 * RWG * KW), lds, stream, pa, pb, blocks_a);
   return check_hip(hipGetLastError(), "gemv pair launch");
+}
+
+// parts of K for the split across workgroups: enough parts for two workgroups per CU, at least 4 steps per part
+inline uint32_t rows8_ksplit_parts(uint32_t N, uint32_t nsteps) {
+  const uint32_t blocks = ((N + 7) / 8 + 7) / 8;
+  uint32_t s = 1;
+  while (s < 16 && blocks * s < 512 && nsteps / (2 * s) >= 4) s *= 2;
+  return s;
+}
+
+// steps per part and the number of non-empty parts (rounding the steps up can leave the last of the wanted parts empty)
+inline void rows8_ksplit_layout(uint32_t N, uint32_t nsteps, uint32_t *part_steps, uint32_t *parts) {
+  const uint32_t want = rows8_ksplit_parts(N, nsteps);
+  *part_steps = (nsteps + want - 1) / want;
+  *parts = (nsteps + *part_steps - 1) / *part_steps;
+}
+
+template <int FMT, int MT> static int launch_rows8_ksplit_mt(const GemvParams &p, float *partial, hipStream_t stream) {
+  constexpr int D = 4;
+  uint32_t parts, part_steps;
+  rows8_ksplit_layout(p.N, p.nsteps, &part_steps, &parts);
+  GemvParams q = p;
+  q.K = min(p.K, part_steps * 256u);
+  q.nsteps = part_steps;
+  size_t lds = rows8_lds_bytes<FMT>(q, MT);
+  auto kern = gemv_rows8_ksplit_kernel<FMT, MT, D>;
+  if (lds > 64 * 1024) {
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                           "hipFuncSetAttribute"))
+      return rc;
+  }
+  const uint32_t nblocks = ((p.N + 7) / 8 + 7) / 8;
+  hipLaunchKernelGGL(kern, dim3(nblocks * parts), dim3(512), lds, stream, p, nblocks, part_steps, partial);
+  return check_hip(hipGetLastError(), "gemv split-K launch");
+}
+
+// M = 2..8; returns the number of parts through *parts_out (the caller sums them)
+template <int FMT> int launch_rows8_ksplit(const GemvParams &p, float *partial, uint32_t *parts_out, hipStream_t stream) {
+  uint32_t part_steps;
+  rows8_ksplit_layout(p.N, p.nsteps, &part_steps, parts_out);
+  if (p.M <= 2) return launch_rows8_ksplit_mt<FMT, 2>(p, partial, stream);
+  if (p.M <= 4) return launch_rows8_ksplit_mt<FMT, 4>(p, partial, stream);
+  return launch_rows8_ksplit_mt<FMT, 8>(p, partial, stream);
 }
 
 struct Rows8Shape { int rwg, kw; };

@@ -175,6 +175,9 @@ int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void 
  *            with so few output tiles that the single-launch GEMM would leave most
  *            of the chip idle; K is then split and the partial products summed), else
  *            as cuthip_matmul_gguf; 0..3 = as cuthip_matmul_gguf (workspace unused).
+ * With variant -1 the workspace also serves batch 3-8 on long rows (K >= 8192) of few (N < 12288): the 8-row GEMV
+ * then splits K across workgroups, writes fp32 partial products to the workspace and sums them in a second launch
+ * (the unsplit kernel would have to stage all of the activations in every workgroup).
  * Other arguments and numerics as cuthip_matmul_gguf. */
 size_t cuthip_matmul_gguf_workspace_bytes(int fmt, uint32_t M, uint32_t K, uint32_t N, int a_dtype);
 int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M, uint32_t K,

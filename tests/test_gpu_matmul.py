@@ -243,3 +243,31 @@ def test_pair_launch_equals_two_matmuls(ops, fa, fb, Na, Nb, K):
         torch.cuda.synchronize()
         # the pair may pick another split of K than the single launch (it sizes the grid for both tensors)
         assert normwise_rel_err(c.cpu().numpy()[None, :], single.cpu().numpy()) < 2e-6
+
+
+@pytest.mark.parametrize("name", list(oracle.FORMATS))
+@pytest.mark.parametrize("M,N,K", [(4, 4096, 14336), (8, 4096, 14336), (3, 4096, 14336), (3, 100, 8192), (5, 9, 8192 + 32)])
+def test_batched_gemv_with_k_split_across_workgroups(ops, name, M, N, K):
+    """Batch 3-8 on long rows with a workspace: K ranges go to different workgroups, fp32 partial products are summed by
+    a second kernel, which also applies the epilogue.  Against the oracle (sampled columns for the big shapes) and
+    against the launch without a workspace."""
+    fmt = oracle.FORMATS[name]
+    if K % oracle.BLOCK_ELEMS[fmt]:
+        pytest.skip("K is not a multiple of this format's block")
+    W = quantized_weights(fmt, N, K, seed=110)
+    A = gauss_acts((M, K), seed=111, dtype=np.float16)
+    D = gauss_acts((M, N), seed=112)
+    a, w, d = torch.from_numpy(A).cuda(), torch.from_numpy(W).cuda(), torch.from_numpy(D).cuda()
+    ws = ops.matmul_gguf_workspace(fmt, M, K, N, a.dtype, "cuda")
+    ws.fill_(0xFF)
+    got = ops.matmul_gguf(a, w, fmt, N, K, out_dtype=torch.float32, binary="add", d=d, workspace=ws)
+    ref = ops.matmul_gguf(a, w, fmt, N, K, out_dtype=torch.float32, binary="add", d=d)
+    h16 = ops.matmul_gguf(a, w, fmt, N, K, out_dtype=torch.float16, workspace=ws)
+    torch.cuda.synchronize()
+    got, ref = got.cpu().numpy(), ref.cpu().numpy()
+    assert normwise_rel_err(got - D, ref - D) < 2e-5
+    cols = np.unique(np.concatenate([[0, N - 1], np.random.default_rng(7).integers(0, N, min(N, 96))]))
+    Ws = np.ascontiguousarray(W.reshape(N, oracle.n_bytes(fmt, K))[cols]).reshape(-1)
+    want = oracle.matmul_gguf(fmt, Ws, A.astype(np.float32), len(cols), f64=True)
+    assert normwise_rel_err(got[:, cols] - D[:, cols], want) < TOL_F16_ACT
+    assert normwise_rel_err(h16.float().cpu().numpy(), ref - D) < 4e-4   # fp16 output rounding
