@@ -234,3 +234,40 @@ def test_dense_gemm_128x448_tiles(ops):
     Ws = np.ascontiguousarray(W.reshape(N, oracle.n_bytes(fmt, K))[cols]).reshape(-1)
     want = oracle.matmul_gguf(fmt, Ws, A[rows].astype(np.float32), len(cols), f64=True)
     assert normwise_rel_err(got[np.ix_(rows, cols)], want) < TOL_GEMM
+
+
+def test_workspace_paths_under_hip_graph_replay(ops):
+    """The two-pass GEMM (dequant + GEMM, with and without split K) and the K-split batched GEMV captured into one HIP
+    graph and replayed with eager work in between: every replay equals the eager result (no allocation, no host
+    dependence inside the calls)."""
+    fmt = oracle.Q4_K
+    cases = [(1100, 520, 512), (300, 256, 2048), (4, 200, 8192)]   # dense, dense with split K, K-split GEMV
+    bufs = []
+    for M, N, K in cases:
+        w = torch.from_numpy(quantized_weights(fmt, N, K, seed=120 + M)).cuda()
+        a = torch.from_numpy(gauss_acts((M, K), seed=121, dtype=np.float16)).cuda()
+        ws = ops.matmul_gguf_workspace(fmt, M, K, N, a.dtype, "cuda")
+        out = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        bufs.append((M, N, K, w, a, ws, out))
+
+    def run():
+        for M, N, K, w, a, ws, out in bufs:
+            ops.matmul_gguf(a, w, fmt, N, K, out=out, workspace=ws)
+    run()
+    torch.cuda.synchronize()
+    eager = [b[6].clone() for b in bufs]
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        run()
+    for rep in range(3):
+        for b in bufs:
+            b[6].zero_()
+            b[5].fill_(rep)   # the workspace is scratch: its contents between calls do not matter
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for b, e in zip(bufs, eager):
+            assert torch.equal(b[6], e)
+    for (M, N, K, w, a, ws, out), e in zip(bufs, eager):
+        want = oracle.matmul_gguf(fmt, w.cpu().numpy(), a.float().cpu().numpy(), N, f64=True)
+        assert normwise_rel_err(e.cpu().numpy(), want) < TOL_GEMM
