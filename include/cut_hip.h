@@ -153,7 +153,8 @@ int cuthip_dequant(int fmt, const void *blocks, void *out, int out_dtype, uint32
  *          epilogue (residual add etc.), else NULL
  * K must be a multiple of the block size; fp32 accumulation throughout.
  * variant: index into the CUTHIP_OP_MATMUL_GGUF table, or -1 = choose by shape
- *          (M <= 8 -> streaming GEMV, else the LDS-tiled MFMA GEMM); variant 4 needs
+ *          (M <= 8 -> streaming GEMV, 9..40 -> passes of 8 rows through it, else the
+ *          LDS-tiled MFMA GEMM); variant 4 needs
  *          cuthip_matmul_gguf_ws. */
 int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M, uint32_t K,
                        uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D,

@@ -271,3 +271,25 @@ def test_batched_gemv_with_k_split_across_workgroups(ops, name, M, N, K):
     want = oracle.matmul_gguf(fmt, Ws, A.astype(np.float32), len(cols), f64=True)
     assert normwise_rel_err(got[:, cols] - D[:, cols], want) < TOL_F16_ACT
     assert normwise_rel_err(h16.float().cpu().numpy(), ref - D) < 4e-4   # fp16 output rounding
+
+
+@pytest.mark.parametrize("name", list(oracle.FORMATS))
+@pytest.mark.parametrize("M", [9, 19, 40])
+def test_mid_size_batches_run_as_eight_row_passes(ops, name, M):
+    """9-40 rows with the automatic choice: passes of 8 rows through the decode kernel, with strided A / C / D and a
+    binary epilogue, so that a wrong row offset in any of the three operands shows."""
+    fmt = oracle.FORMATS[name]
+    N, K = 100, 1024
+    W = quantized_weights(fmt, N, K, seed=130)
+    A = gauss_acts((M, K), seed=131, dtype=np.float16)
+    D = gauss_acts((M, N), seed=132)
+    a_buf = torch.zeros((M, K + 8), dtype=torch.float16, device="cuda")
+    a_buf[:, :K] = torch.from_numpy(A).cuda()
+    d_buf = torch.zeros((M, N + 4), dtype=torch.float32, device="cuda")
+    d_buf[:, :N] = torch.from_numpy(D).cuda()
+    c_buf = torch.full((M, N + 4), 7.0, dtype=torch.float32, device="cuda")
+    ops.matmul_gguf(a_buf[:, :K], torch.from_numpy(W).cuda(), fmt, N, K, out=c_buf[:, :N], binary="add", d=d_buf[:, :N])
+    torch.cuda.synchronize()
+    want = oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)
+    assert normwise_rel_err(c_buf[:, :N].cpu().numpy() - D, want) < TOL_F16_ACT
+    assert torch.all(c_buf[:, N:] == 7.0)
