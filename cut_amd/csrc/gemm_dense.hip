@@ -295,11 +295,14 @@ size_t dense_gemm_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
          (sh.ksplit > 1 ? (size_t)sh.ksplit * M * N * 4 : 0);
 }
 
-// true where the two-pass path beats the single-launch GEMM: from about a thousand rows, or earlier when the
-// single-launch kernel's 128 x 128 tiles would leave most of the chip idle
-bool dense_gemm_preferred(uint32_t M, uint32_t N) {
+// true where the two-pass path beats the single-launch GEMM: from about a thousand rows; or when the single-launch
+// kernel's 128 x 128 tiles would leave most of the chip idle, from 256 rows, and already from 41 rows on long K, where
+// that kernel's time is the decode of a whole K-long tile row per workgroup (measured 4096 x 14336: 217-222 us for
+// any M up to 512, against 91-131 us for dequantize + dense GEMM with K split)
+bool dense_gemm_preferred(uint32_t M, uint32_t K, uint32_t N) {
   if (M >= 1024) return true;
-  return M >= 256 && (uint64_t)((M + 127) / 128) * ((N + 127) / 128) < 200;
+  if ((uint64_t)((M + 127) / 128) * ((N + 127) / 128) >= 200) return false;
+  return M >= 256 || (M > 40 && K >= 8192);
 }
 
 int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K,

@@ -107,7 +107,7 @@ int launch_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c
 
 bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a_f16, const void *A);
 size_t dense_gemm_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16);
-bool dense_gemm_preferred(uint32_t M, uint32_t N);
+bool dense_gemm_preferred(uint32_t M, uint32_t K, uint32_t N);
 int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K,
                       uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream);
 
@@ -440,7 +440,7 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   const bool fits = dense_gemm_fits(M, K, N, strideA, a_f16, A);
   const size_t need = dense_gemm_workspace(M, K, N, a_f16);
   const bool ws_ok = workspace && (uintptr_t)workspace % 256 == 0 && workspace_bytes >= need;
-  if (variant == -1 && !(dense_gemm_preferred(M, N) && fits && ws_ok))
+  if (variant == -1 && !(dense_gemm_preferred(M, K, N) && fits && ws_ok))
     return cuthip_matmul_gguf(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, -1,
                               stream);
   if (!fits) {

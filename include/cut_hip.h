@@ -172,9 +172,10 @@ int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void 
  *            when K is split); contents are scratch.
  * variant  : 4 = the two-pass path (an error if K is not a multiple of 128, the
  *            rows of A are not 16-byte aligned or the workspace is too small);
- *            -1 = choose by shape: variant 4 when it applies and M >= 1024 (or M >= 256
- *            with so few output tiles that the single-launch GEMM would leave most
- *            of the chip idle; K is then split and the partial products summed), else
+ *            -1 = choose by shape: variant 4 when it applies and M >= 1024 (or, with so
+ *            few output tiles that the single-launch GEMM would leave most of the chip
+ *            idle, from M = 256, and from M = 41 when K >= 8192; K is then split and
+ *            the partial products summed), else
  *            as cuthip_matmul_gguf; 0..3 = as cuthip_matmul_gguf (workspace unused).
  * With variant -1 the workspace also serves batch 3-8 on long rows (K >= 8192) of few (N < 12288): the 8-row GEMV
  * then splits K across workgroups, writes fp32 partial products to the workspace and sums them in a second launch
