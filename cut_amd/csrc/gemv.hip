@@ -122,6 +122,23 @@ static int launch_gemv(int fmt, const GemvParams &p, hipStream_t stream) {
 
 }  // namespace cuthip
 
+// Launch parameters of the GEMV kernels for C[M, strideC] = A[M, strideA] . dequant(W)^T.
+static cuthip::GemvParams gemv_params(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M,
+                                      uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideC, const cuthip::Epilogue &epi) {
+  using namespace cuthip;
+  GemvParams p;
+  p.W = reinterpret_cast<const uint8_t *>(W);
+  p.A = A;
+  p.C = C;
+  p.epi = epi;
+  p.M = M; p.K = K; p.N = N; p.strideA = strideA; p.strideC = strideC;
+  p.nsteps = (K + 255) / 256;
+  p.row_bytes = (uint32_t)((uint64_t)(K / fmt_elems(fmt)) * fmt_bytes(fmt));
+  p.a_f16 = a_dtype == CUTHIP_F16;
+  p.c_f16 = c_dtype == CUTHIP_F16;
+  return p;
+}
+
 constexpr uint32_t kPassesMaxRows = 40;   // up to here 8-row passes of the decode kernels beat one tiled GEMM launch
 
 // Argument checks shared by the matmul entry points: 0 = go on, 1 = empty problem (success), < 0 = error.
@@ -222,16 +239,7 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
     return launch_gemm(fmt, W, A, a_dtype == CUTHIP_F16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC, epi,
                        reinterpret_cast<hipStream_t>(stream));
   }
-  GemvParams p;
-  p.W = reinterpret_cast<const uint8_t *>(W);
-  p.A = A;
-  p.C = C;
-  p.epi = epi;
-  p.M = M; p.K = K; p.N = N; p.strideA = strideA; p.strideC = strideC;
-  p.nsteps = (K + 255) / 256;
-  p.row_bytes = (uint32_t)row_bytes;
-  p.a_f16 = a_dtype == CUTHIP_F16;
-  p.c_f16 = c_dtype == CUTHIP_F16;
+  GemvParams p = gemv_params(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epi);
   // variant 3 (and the automatic choice for M <= 8): 8 rows x 128-byte runs per wave instruction
   if (variant == 3 || (variant == -1 && M <= 8)) {
     bool taken = false;
@@ -269,16 +277,8 @@ int cuthip_matmul_gguf_carry(int fmt, const void *W, const void *A, int a_dtype,
   using namespace cuthip;
   const uint32_t n_out = epilogue == CUTHIP_EPI_SWIGLU_PAIRS ? N / 2 : N;
   if (int rc = check_matmul_args(fmt, W, A, a_dtype, C, c_dtype, 1, K, N, K, n_out, epilogue, D)) return rc > 0 ? CUTHIP_OK : rc;
-  GemvParams p;
-  p.W = reinterpret_cast<const uint8_t *>(W);
-  p.A = A;
-  p.C = C;
-  p.epi = Epilogue{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
-  p.M = 1; p.K = K; p.N = N; p.strideA = K; p.strideC = n_out;
-  p.nsteps = (K + 255) / 256;
-  p.row_bytes = (uint32_t)((uint64_t)(K / fmt_elems(fmt)) * fmt_bytes(fmt));
-  p.a_f16 = a_dtype == CUTHIP_F16;
-  p.c_f16 = c_dtype == CUTHIP_F16;
+  GemvParams p = gemv_params(fmt, W, A, a_dtype, C, c_dtype, 1, K, N, K, n_out,
+                             Epilogue{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr});
   if (!apply_carry(p, carry, epilogue != CUTHIP_EPI_SWIGLU_PAIRS)) {
     set_error("cuthip_matmul_gguf_carry: the producer fields (next_norm_weight, next_x16, next_sumsq_parts) come together, "
               "next_x16 2-byte aligned, and not with the SwiGLU row-pair epilogue");
@@ -333,17 +333,8 @@ int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, in
   if (int rc = check_matmul_args(fmt_b, Wb, A, a_dtype, Cb, c_dtype, 1, K, Nb, K, Nb, CUTHIP_EPI_NONE, nullptr))
     return rc > 0 ? cuthip_matmul_gguf(fmt_a, Wa, A, a_dtype, Ca, c_dtype, 1, K, Na, K, Na, 0, 0, nullptr, -1, stream) : rc;
   auto params = [&](int fmt, const void *W, uint32_t N, void *C, const RopeAppend &r) {
-    GemvParams p;
+    GemvParams p = gemv_params(fmt, W, A, a_dtype, C, c_dtype, 1, K, N, K, N, Epilogue{CUTHIP_EPI_NONE, 0, nullptr});
     p.rope = r;
-    p.W = reinterpret_cast<const uint8_t *>(W);
-    p.A = A;
-    p.C = C;
-    p.epi = Epilogue{CUTHIP_EPI_NONE, 0, nullptr};
-    p.M = 1; p.K = K; p.N = N; p.strideA = K; p.strideC = N;
-    p.nsteps = (K + 255) / 256;
-    p.row_bytes = (uint32_t)((uint64_t)(K / fmt_elems(fmt)) * fmt_bytes(fmt));
-    p.a_f16 = a_dtype == CUTHIP_F16;
-    p.c_f16 = c_dtype == CUTHIP_F16;
     apply_carry(p, carry, false);
     return p;
   };
@@ -410,16 +401,8 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   // batch 3-8 on long rows: the 8-row GEMV with K split across workgroups, partial products in the workspace
   if (variant == -1 && ksplit_gemv_preferred(M, K, N) && workspace && (uintptr_t)workspace % 16 == 0 &&
       workspace_bytes >= ksplit_gemv_workspace(M, K, N) && (uintptr_t)A % 16 == 0 && (strideA * (a_f16 ? 2 : 4)) % 16 == 0) {
-    GemvParams p;
-    p.W = reinterpret_cast<const uint8_t *>(W);
-    p.A = A;
-    p.C = C;
-    p.epi = Epilogue{CUTHIP_EPI_NONE, 0, nullptr};
-    p.M = M; p.K = K; p.N = N; p.strideA = strideA; p.strideC = strideC;
-    p.nsteps = (K + 255) / 256;
-    p.row_bytes = (uint32_t)((uint64_t)(K / fmt_elems(fmt)) * fmt_bytes(fmt));
-    p.a_f16 = a_f16;
-    p.c_f16 = c_dtype == CUTHIP_F16;
+    const GemvParams p = gemv_params(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC,
+                                     Epilogue{CUTHIP_EPI_NONE, 0, nullptr});
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     float *partial = reinterpret_cast<float *>(workspace);
     uint32_t parts = 0;
@@ -484,16 +467,7 @@ int cuthip_matmul_gguf_pro(int fmt, const void *W, const void *A, int a_dtype, v
     set_error("cuthip_matmul_gguf_pro: unknown prologue %d", prologue);
     return CUTHIP_ERR_INVALID;
   }
-  GemvParams p;
-  p.W = reinterpret_cast<const uint8_t *>(W);
-  p.A = A;
-  p.C = C;
-  p.epi = Epilogue{epilogue, epilogue_op, D};
-  p.M = 1; p.K = K; p.N = N; p.strideA = K; p.strideC = N;
-  p.nsteps = (K + 255) / 256;
-  p.row_bytes = (uint32_t)((uint64_t)(K / fmt_elems(fmt)) * fmt_bytes(fmt));
-  p.a_f16 = a_dtype == CUTHIP_F16;
-  p.c_f16 = c_dtype == CUTHIP_F16;
+  GemvParams p = gemv_params(fmt, W, A, a_dtype, C, c_dtype, 1, K, N, K, N, Epilogue{epilogue, epilogue_op, D});
   p.pro = prologue;
   p.norm_w = norm_weight;
   p.eps = eps;
