@@ -275,6 +275,45 @@ def matmul_sep(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, N: int, q
     return out
 
 
+def prepare_sep(w_blocks: torch.Tensor, fmt, N: int, K: int, stride_b: int | None = None, scale_stride: int | None = None):
+    """GGUF blocks [N rows of K/blk blocks] on the device -> (B, scales) in the reference's separated [K, N] layout:
+    Q8_0 -> int8 [K, N] + fp16 [K/32, N]; Q4_0 -> nibbles uint8 [K, N/2] + fp16 [K/32, N]; Q4_K -> affine Q4, nibbles
+    + fp16 [2K/32, N] (scales then minima: requantizeQ4KToAffine).  Row strides default to the reference's padding
+    to multiples of 4 elements (MatMulOp.cpp:514-541)."""
+    f = _fmt(fmt)
+    if f not in (_l.Q8_0, _l.Q4_0, _l.Q4_K):
+        raise _l.CutHipError("prepare_sep: only Q8_0, Q4_0 and Q4_K have a separated layout")
+    q4 = f != _l.Q8_0
+    width = (N // 2) if q4 else N
+    sb = stride_b if stride_b is not None else (width + 3) & ~3
+    ss = scale_stride if scale_stride is not None else (N + 3) & ~3
+    rows_s = (2 if f == _l.Q4_K else 1) * (K // 32)
+    B = torch.zeros((K, sb), dtype=torch.uint8 if q4 else torch.int8, device=w_blocks.device)
+    S = torch.zeros((rows_s, ss), dtype=torch.float16, device=w_blocks.device)
+    _l.check(_l.load().cuthip_prepare_sep(f, w_blocks.data_ptr(), N, K, B.data_ptr(), sb, S.data_ptr(), ss, _stream_ptr()))
+    return B, S
+
+
+def transpose_q4_nibble(packed: torch.Tensor, N: int, K: int) -> torch.Tensor:
+    """Operations::transposeQ4(packed, N, K) of the reference: GGML-order nibbles [N, K/2] -> [K, N/2]."""
+    if packed.dim() != 2 or packed.element_size() != 1 or packed.stride(1) != 1:
+        raise _l.CutHipError("transpose_q4_nibble: packed must be a 2-D 1-byte tensor with contiguous rows")
+    so = (N // 2 + 3) & ~3
+    out = torch.zeros((K, so), dtype=torch.uint8, device=packed.device)
+    _l.check(_l.load().cuthip_transpose_q4_nibble(packed.data_ptr(), out.data_ptr(), N, K, packed.stride(0), so, _stream_ptr()))
+    return out
+
+
+def quantize_rows_q8_0(x: torch.Tensor) -> torch.Tensor:
+    """quantizeRowsQ8_0 of the reference's runner on the device: fp32 [n] -> Q8_0 blocks (uint8 [n/32 * 34])."""
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise _l.CutHipError("quantize_rows_q8_0: x must be a contiguous fp32 tensor")
+    n = x.numel()
+    out = torch.empty(max(n // 32, 1) * 34, dtype=torch.uint8, device=x.device)
+    _l.check(_l.load().cuthip_quantize_rows_q8_0(x.data_ptr(), n, out.data_ptr(), _stream_ptr()))
+    return out
+
+
 def matmul_gguf_pro(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: int, out: torch.Tensor, prologue: str,
                     norm_weight: torch.Tensor | None = None, eps: float = 0.0, unary: str | None = None,
                     binary: str | None = None, d: torch.Tensor | None = None) -> torch.Tensor:

@@ -281,6 +281,39 @@ int cuthip_matmul_q4_sep(const float *A, const uint8_t *packedB, const uint16_t 
                          uint32_t scaleStride, int epilogue, int epilogue_op, int affine, void *workspace,
                          size_t workspace_bytes, void *stream);
 
+/* ---- load-time preparation of the separated layout, on the device ----------
+ * cuthip_prepare_sep: GGUF blocks (row n = K/blk consecutive blocks, as in the
+ * file) -> the tensors cuthip_matmul_q8_sep / cuthip_matmul_q4_sep take, in one
+ * launch.  Replaces the host split of read_tensor_q8_separated /
+ * read_tensor_q4_separated (gguf_reader.cpp:389-501) followed by the GPU
+ * transposes of uploadQ4 / uploadQ8 (llama.cpp:940-965, TransposeQ4Nibble.cu:17-61),
+ * and, for fmt = CUTHIP_Q4_K, requantizeQ4KToAffine (llama.cpp:573-619):
+ *   Q8_0: B int8 [K, strideB],        scales fp16 [K/32, scaleStride]
+ *   Q4_0: B nibbles [K, strideB bytes], even row n in the low nibble; scales as Q8_0
+ *   Q4_K: B nibbles as Q4_0; scales fp16 [2K/32, scaleStride]: rows [0, K/32) hold
+ *         f16(d*sc), rows [K/32, 2K/32) hold f16(8*(d*sc) - dmin*m); decode
+ *         (nibble - 8) * scale + min (pass affine = 1 to cuthip_matmul_q4_sep)
+ * N must be even for the nibble formats (the reference throws otherwise), K a
+ * multiple of the block size; B must be 4-byte aligned.  Bit-exact against the
+ * reference's host code for finite block scales. */
+int cuthip_prepare_sep(int fmt, const void *blocks, uint32_t N, uint32_t K, void *B, uint32_t strideB, uint16_t *scales,
+                       uint32_t scaleStride, void *stream);
+
+/* TransposeQ4NibbleOpNode (operators/impl/q4transpose/TransposeQ4NibbleOp.cpp:7-23,
+ * TransposeQ4Nibble.cu:17-61): packed [N, strideInHalf bytes] in GGML Q4_0 nibble
+ * order (low nibble of byte j of a 16-byte block = element j, high = j + 16) ->
+ * packedT [K, strideOutHalf bytes], even n in the low nibble.  N even, K a
+ * multiple of 32, strideInHalf even. */
+int cuthip_transpose_q4_nibble(const void *packed, void *packedT, uint32_t N, uint32_t K, uint32_t strideInHalf,
+                               uint32_t strideOutHalf, void *stream);
+
+/* quantizeRowsQ8_0 (llama.cpp:488-505): fp32 x[n] -> n/32 Q8_0 blocks (34 bytes:
+ * fp16 scale, 32 int8).  d = absmax/127, q = lroundf(x * (1/d)) from the
+ * unrounded d, stored scale = f32ToF16(d).  The reference returns values and
+ * scales as two vectors; the blocks written here hold the same numbers in GGUF
+ * order, ready for cuthip_matmul_gguf or cuthip_prepare_sep.  x 16-byte aligned. */
+int cuthip_quantize_rows_q8_0(const float *x, uint64_t n, void *blocks, void *stream);
+
 /* ---- the operators between the matmuls of a decode step --------------------
  * What the runner chains around the quantized matmuls for one token
  * (interface/runner/llama/llama.cpp, runLayer / decode graph).  All take
