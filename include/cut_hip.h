@@ -281,6 +281,22 @@ int cuthip_matmul_q4_sep(const float *A, const uint8_t *packedB, const uint16_t 
                          uint32_t scaleStride, int epilogue, int epilogue_op, int affine, void *workspace,
                          size_t workspace_bytes, void *stream);
 
+/* ---- Q8_0 weights x int8 activations on the int8 matrix core -----------------
+ * The arithmetic of the reference's int8 dot-product GEMV (MatMulQ8GemvDot.cu:60-85)
+ * for prefill-sized M: A is quantized per 32 elements (a_scale = amax / 127,
+ * q = clamp(round(a * (127 / amax)), -127, 127)) and
+ *   C[m,n] = sum_b float(sum_{k in b} qa[m,k] * qw[n,k]) * a_scale[m,b] * d_w[n,b]
+ * with W in GGUF Q8_0 blocks [N][K/32].  The 8-bit activations put the result
+ * about 5e-3 (normwise) from the fp32 path, so this is its own entry point and
+ * cuthip_matmul_gguf never selects it.  workspace: device scratch of
+ * cuthip_matmul_q8_i8_workspace_bytes(M, K) bytes (the quantized activations),
+ * 16-byte aligned.  A: fp32 or fp16, aligned to 4 elements, strideA a multiple
+ * of 4; epilogue / epilogue_op / D as in cuthip_matmul_gguf (none, unary, binary). */
+size_t cuthip_matmul_q8_i8_workspace_bytes(uint32_t M, uint32_t K);
+int cuthip_matmul_q8_i8(const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M, uint32_t K, uint32_t N,
+                        uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D, void *workspace,
+                        size_t workspace_bytes, void *stream);
+
 /* ---- load-time preparation of the separated layout, on the device ----------
  * cuthip_prepare_sep: GGUF blocks (row n = K/blk consecutive blocks, as in the
  * file) -> the tensors cuthip_matmul_q8_sep / cuthip_matmul_q4_sep take, in one

@@ -63,6 +63,7 @@ def _load():
         "orc_matmul_gguf_f64": (C.c_int, [C.c_int, u8p, f32p, u32, u32, u32, f64p]),
         "orc_matmul_dense_f32": (None, [f32p, f32p, u32, u32, u32, f32p]),
         "orc_quantize_act_q8": (None, [f32p, sz, i8p, f32p]),
+        "orc_matmul_q8_i8": (C.c_int, [u8p, f32p, u32, u32, u32, f32p, f64p]),
         "orc_quantize": (C.c_int, [C.c_int, f32p, sz, u8p]),
         "orc_rmsnorm": (None, [f32p, f32p, u32, u32, C.c_float, f32p]),
         "orc_rope_kv_write": (None, [f32p, f32p, f32p, u32, f32p, f32p, u32, u32, u32, u32, f32p, u16p, u16p]),
@@ -255,6 +256,20 @@ def quantize_act_q8(a):
     s = np.empty(a.size // 32, np.float32)
     _lib.orc_quantize_act_q8(_p(a), a.size, _p(q), _p(s))
     return q, s
+
+
+def matmul_q8_i8(W, A, N: int, f64: bool = False) -> np.ndarray:
+    """The reference's int8-activation arithmetic (MatMulQ8GemvDot.cu:60-85) on Q8_0 blocks W [N][K/32]."""
+    A = _c(A, np.float32)
+    A = A.reshape(1, -1) if A.ndim == 1 else A
+    M, K = A.shape
+    W = _c(W, np.uint8).reshape(-1)
+    assert W.size == N * (K // 32) * 34
+    c32 = np.empty((M, N), np.float32)
+    c64 = np.empty((M, N), np.float64)
+    rc = _lib.orc_matmul_q8_i8(_p(W), _p(A), M, K, N, _p(c32), _p(c64))
+    assert rc == 0
+    return c64 if f64 else c32
 
 
 # ---- the reference's own reader (only where oracle/_ref was built) ----------

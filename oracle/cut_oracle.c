@@ -571,6 +571,54 @@ void orc_quantize_act_q8(const float *a, size_t n, int8_t *q, float *scale) {
   }
 }
 
+/* MatMulQ8GemvDot.cu:60-85 on GGUF Q8_0 blocks W [N][K/32]: activations
+ * quantized per 32 (orc_quantize_act_q8), integer dot per block, then
+ * acc += (float)dot * a_scale * b_scale in fp32, blocks in order.  C64 (may be
+ * NULL) receives the same sum with the scaling and the accumulation in double:
+ * the two differ by fp32 rounding only. */
+int orc_matmul_q8_i8(const uint8_t *W, const float *A, uint32_t M, uint32_t K,
+                     uint32_t N, float *C32, double *C64) {
+  if (K % 32 != 0)
+    return -1;
+  uint32_t nb = K / 32;
+  int8_t *qa = (int8_t *)malloc((size_t)M * K);
+  float *sa = (float *)malloc((size_t)M * nb * sizeof(float));
+  if (!qa || !sa) {
+    free(qa);
+    free(sa);
+    return -2;
+  }
+  for (uint32_t m = 0; m < M; ++m)
+    orc_quantize_act_q8(A + (size_t)m * K, K, qa + (size_t)m * K,
+                        sa + (size_t)m * nb);
+  for (uint32_t m = 0; m < M; ++m)
+    for (uint32_t n = 0; n < N; ++n) {
+      float acc = 0.0f;
+      double acc64 = 0.0;
+      for (uint32_t b = 0; b < nb; ++b) {
+        const uint8_t *blk = W + ((size_t)n * nb + b) * 34;
+        uint16_t dbits;
+        memcpy(&dbits, blk, 2);
+        float d = orc_f16_to_f32(dbits);
+        const int8_t *qw = (const int8_t *)(blk + 2);
+        const int8_t *x = qa + (size_t)m * K + (size_t)b * 32;
+        int dot = 0;
+        for (int i = 0; i < 32; ++i)
+          dot += (int)x[i] * (int)qw[i];
+        float a_scale = sa[(size_t)m * nb + b];
+        acc += (float)dot * a_scale * d;
+        acc64 += (double)dot * (double)a_scale * (double)d;
+      }
+      if (C32)
+        C32[(size_t)m * N + n] = acc;
+      if (C64)
+        C64[(size_t)m * N + n] = acc64;
+    }
+  free(qa);
+  free(sa);
+  return 0;
+}
+
 /* ---- own encoders (test inputs only) ----------------------------------- */
 
 static inline int nearest_int(float f) { return (int)lrintf(f); }

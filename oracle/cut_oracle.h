@@ -14,7 +14,8 @@
  *           orc_get_scale_min_k4, orc_dequant_q8_0/q4_0/q4_k/q6_k,
  *           orc_quantize_rows_q8_0, orc_requantize_q4k_to_affine,
  *           orc_split_q8_0/q4_0, orc_matmul_sep_*, orc_matmul_gguf_*,
- *           orc_transpose_q4_nibble, orc_quantize_act_q8
+ *           orc_transpose_q4_nibble, orc_quantize_act_q8,
+ *           orc_matmul_q8_i8
  *   no function here is "parity unpinned".
  */
 #ifndef CUT_ORACLE_H
@@ -110,6 +111,8 @@ void orc_matmul_dense_f32(const float *Wf, const float *A, uint32_t M,
 /* MatMulQ8GemvDot.cu:60-64: per-32 activation quantizer, a_scale = amax/127,
  * q = clamp(round-half-away(a*127/amax), -127, 127) */
 void orc_quantize_act_q8(const float *a, size_t n, int8_t *q, float *scale);
+int orc_matmul_q8_i8(const uint8_t *W, const float *A, uint32_t M, uint32_t K,
+                     uint32_t N, float *C32, double *C64);
 
 /* own encoders (test inputs only; the reference has none for these) */
 void orc_quantize_q4_0(const float *x, size_t n, uint8_t *blocks);

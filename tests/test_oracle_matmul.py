@@ -144,3 +144,67 @@ def test_quantize_act_q8():
     assert np.all(np.abs(q.astype(np.int32)) <= 127)
     back = q.reshape(-1, 32) * s[:, None]
     assert np.max(np.abs(back - ab)) <= np.max(s) * 0.5 + 1e-7
+
+
+# ---- int8-activation arithmetic (MatMulQ8GemvDot.cu:60-85) on Q8_0 blocks ----------------------------
+
+def q8_blocks(q, d):
+    """Q8_0 blocks from int8 values [N, K] and fp16-exact scales [N, K/32]."""
+    N, K = q.shape
+    blocks = np.zeros((N, K // 32, 34), np.uint8)
+    blocks[:, :, :2] = np.asarray(d, np.float16).reshape(N, K // 32, 1).view(np.uint8)
+    blocks[:, :, 2:] = q.reshape(N, K // 32, 32).view(np.uint8)
+    return blocks.reshape(-1)
+
+
+def test_q8_i8_known_answer():
+    # all-ones activations quantize to 127 with a_scale = fl(1/127); weights 1 / 2 with d = 1: 32 and 64 per block
+    K, N = 64, 2
+    q = np.zeros((N, K), np.int8)
+    q[0], q[1] = 1, 2
+    C = oracle.matmul_q8_i8(q8_blocks(q, np.ones((N, 2))), np.ones((1, K), np.float32), N)
+    np.testing.assert_allclose(C, [[64.0, 128.0]], rtol=3e-7)
+    # scales {0.5, 2} / {1, 0.25} with weight 4 as in q8_withscales (OpRegistry.h:2012-2026): 4*32*(0.5+1), 4*32*(2+0.25)
+    q[:] = 4
+    C = oracle.matmul_q8_i8(q8_blocks(q, np.array([[0.5, 1.0], [2.0, 0.25]])), np.ones((1, K), np.float32), N)
+    np.testing.assert_allclose(C, [[192.0, 288.0]], rtol=3e-7)
+
+
+def test_q8_i8_reduces_to_the_exact_path_on_int8_activations():
+    # integer activations whose every block holds +-127: a_scale = 1, 127/amax = 1, so the quantizer is the
+    # identity and the result must equal the float64 matmul on the dequantized weights
+    rng = np.random.default_rng(3)
+    M, K, N = 3, 256, 40
+    A = rng.integers(-127, 128, (M, K)).astype(np.float32)
+    A.reshape(M, K // 32, 32)[:, :, 5] = 127.0
+    A.reshape(M, K // 32, 32)[:, ::2, 9] = -127.0
+    W = quantized_weights(oracle.Q8_0, N, K, seed=4)
+    q, s = oracle.quantize_act_q8(A)
+    assert np.array_equal(q.astype(np.float32).reshape(A.shape), A) and np.all(s == 1.0)
+    ref = oracle.matmul_gguf(oracle.Q8_0, W, A, N, f64=True)
+    np.testing.assert_allclose(oracle.matmul_q8_i8(W, A, N, f64=True), ref, rtol=1e-12, atol=1e-12)
+    assert normwise_rel_err(oracle.matmul_q8_i8(W, A, N), ref) < 1e-6
+
+
+def test_q8_i8_against_an_integer_numpy_restatement_and_the_fp32_path():
+    rng = np.random.default_rng(5)
+    M, K, N = 4, 512, 64
+    A = rng.standard_normal((M, K), dtype=np.float32)
+    A[1, 32:64] = 0.0                                   # an all-zero block: scale 0, q 0
+    W = quantized_weights(oracle.Q8_0, N, K, seed=6)
+    blocks = W.reshape(N, K // 32, 34)
+    d = blocks[:, :, :2].copy().view(np.float16).astype(np.float64).reshape(N, K // 32)
+    qw = blocks[:, :, 2:].copy().view(np.int8).astype(np.int64)
+    Ab = A.reshape(M, K // 32, 32)
+    amax = np.abs(Ab).max(axis=2)
+    sa = (amax / np.float32(127.0)).astype(np.float32)
+    inv = np.where(amax > 0, np.float32(127.0) / np.where(amax > 0, amax, 1), 0).astype(np.float32)
+    t = Ab * inv[:, :, None]
+    qa = np.clip(np.sign(t) * np.floor(np.abs(t) + np.float32(0.5)), -127, 127).astype(np.int64)
+    dots = np.einsum("mbk,nbk->mnb", qa, qw)
+    want = (dots * sa.astype(np.float64)[:, None, :] * d[None, :, :]).sum(axis=2)
+    np.testing.assert_allclose(oracle.matmul_q8_i8(W, A, N, f64=True), want, rtol=1e-12, atol=1e-12)
+    assert normwise_rel_err(oracle.matmul_q8_i8(W, A, N), want) < 1e-6
+    # what the 8-bit activations cost against the fp32-activation path the other kernels are held to
+    err = normwise_rel_err(want, oracle.matmul_gguf(oracle.Q8_0, W, A, N, f64=True))
+    assert 1e-3 < err < 2e-2
