@@ -113,6 +113,38 @@ def bench_decode_step(torch, np, ops, dev, x_h, steps=5):
             "decode_step_8b_bytes_per_token": int(w_bytes_tok + kv_bytes_tok)}
 
 
+def bench_q8_prefill(torch, ops, dev, shapes=((512, N_FF, N_EMBD), (2048, N_FF, N_EMBD)), reps=10):
+    """Q8_0 prefill GEMM: cuthip_matmul_q8_i8 (int8 activations per 32, int8 MFMA; TOP/s = 2MNK / time including
+    the activation quantizer) and the fp16-activation path of cuthip_matmul_gguf on the same blocks."""
+    res = {}
+    for (M, N, K) in shapes:
+        wq = torch.from_numpy(make_q_weights("Q8_0", 1024, K, 4)).to(dev).repeat(N // 1024)
+        a = torch.randn((M, K), dtype=torch.float16, device=dev)
+        c = torch.empty((M, N), dtype=torch.float16, device=dev)
+        ws8 = torch.empty(lib_q8_ws(ops, M, K), dtype=torch.uint8, device=dev)
+        ws = ops.matmul_gguf_workspace("Q8_0", M, K, N, a.dtype, dev)
+
+        def i8(_s):
+            ops.matmul_q8_i8(a, wq, N, K, out=c, workspace=ws8)
+
+        def f16(_s):
+            ops.matmul_gguf(a, wq, "Q8_0", N, K, out=c, workspace=ws)
+        _, ev, _ = timed_graph(torch, i8, reps, 2)
+        tops = 2.0 * M * N * K * reps / (ev * 1e-3) / 1e12
+        res[f"q8_0_i8_prefill_gemm_M{M}_N{N}_K{K}_TOPs"] = round(tops, 1)
+        res[f"q8_0_i8_prefill_gemm_M{M}_N{N}_K{K}_pct_of_int8_mfma_peak"] = round(tops / 5000.0 * 100, 1)
+        _, ev, _ = timed_graph(torch, f16, reps, 2)
+        res[f"q8_0_f16_prefill_gemm_M{M}_N{N}_K{K}_TFLOPs"] = round(2.0 * M * N * K * reps / (ev * 1e-3) / 1e12, 1)
+        del wq, a, c, ws8, ws
+    torch.cuda.empty_cache()
+    return res
+
+
+def lib_q8_ws(ops, M, K):
+    from cut_amd import lib
+    return max(int(lib.load().cuthip_matmul_q8_i8_workspace_bytes(M, K)), 16)
+
+
 def bench_dequant(torch, ops, dev, reps=20):
     """config 2: dequant of 256 Mi elements to fp16 (a 4 Mi-element tile of quantized N(0, 0.02) weights repeated
     64 times); GB/s = (block bytes in + fp16 bytes out) / kernel time from events."""
@@ -149,6 +181,8 @@ def main():
                     help="only run the Q4_K prefill GEMM (M x 4096) . (14336 x 4096)^T twelve times (target of rocprofv3 runs)")
     ap.add_argument("--dequant-only", action="store_true",
                     help="only run the 256 Mi-element dequant of the four formats (target of rocprofv3 runs)")
+    ap.add_argument("--q8-only", action="store_true",
+                    help="only run the Q8_0 prefill GEMMs at M = 2048 (int8-activation variant and fp16 path)")
     ap.add_argument("--decode-only", action="store_true",
                     help="only run the 8B-shape decode step (target of rocprofv3 runs)")
     args = ap.parse_args()
@@ -173,6 +207,9 @@ def main():
         return
     if args.dequant_only:
         print(json.dumps(bench_dequant(torch, ops, dev, reps=5)))
+        return
+    if args.q8_only:
+        print(json.dumps(bench_q8_prefill(torch, ops, dev, shapes=((2048, N_FF, N_EMBD),), reps=5)))
         return
     if args.decode_only:
         x_h = np.random.default_rng(1).standard_normal((8, N_EMBD), dtype=np.float32).astype(np.float16)
@@ -317,6 +354,9 @@ def main():
             extras[f"q4k_prefill_gemm_M{M}_N{N}_K{K}_single_launch_TFLOPs"] = round(2.0 * M * N * K * 10 / (ev_g * 1e-3) / 1e12, 1)
             del ws
             del wq, a, c
+        # config 5, second half: Q8_0 weights with activations quantized to int8 per 32 on the int8 matrix core
+        # (both launches, quantizer + GEMM, inside the timed region), next to the fp16 path on the same blocks
+        extras.update(bench_q8_prefill(torch, ops, dev))
     result["extras"] = extras
 
     # ---- CPU baseline: the oracle's restatement of the reference path -------------
