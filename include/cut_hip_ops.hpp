@@ -248,5 +248,66 @@ private:
   Tensor output_;
 };
 
+// ---- TransposeQ4NibbleOpNode --------------------------------------------------------------
+// operators/impl/q4transpose/TransposeQ4NibbleOp.cpp:7-23: packed GGML-order nibbles [N, K/2] ->
+// [K, N/2] with the even source row in the low nibble; same checks, messages and padded strides.
+class TransposeQ4NibbleOpNode {
+public:
+  TransposeQ4NibbleOpNode(const Tensor &packedInput, uint32_t N, uint32_t K) : in_(packedInput), N_(N), K_(K) {
+    if (N_ % 2 != 0) throw std::runtime_error("TransposeQ4: N must be even");
+    if (K_ % 32 != 0) throw std::runtime_error("TransposeQ4: K must be a multiple of 32");
+    strideInHalf_ = (K_ / 2 + 3) & ~3u;
+    strideOutHalf_ = (N_ / 2 + 3) & ~3u;
+    if (!packedInput.buffer || packedInput.buffer->bytes() < (size_t)N_ * strideInHalf_)
+      throw std::runtime_error("TransposeQ4: input holds fewer bytes than N rows of the padded stride");
+    storage_ = DeviceBuffer((size_t)K_ * strideOutHalf_);
+    output_ = Tensor{&storage_, {K_, N_ / 2}, DataType::Float16 /* unused: bytes */, strideOutHalf_};
+  }
+  TransposeQ4NibbleOpNode(TransposeQ4NibbleOpNode &&) = delete;
+  std::vector<uint32_t> outputShape() const { return {K_, N_ / 2}; }
+  std::string displayName() const { return "TransposeQ4"; }
+  const Tensor &output() const { return output_; }
+  void dispatch(void *stream = nullptr) const {
+    check(cuthip_transpose_q4_nibble(in_.data(), output_.data(), N_, K_, strideInHalf_, strideOutHalf_, stream),
+          "cuthip_transpose_q4_nibble");
+  }
+
+private:
+  Tensor in_;
+  uint32_t N_, K_, strideInHalf_ = 0, strideOutHalf_ = 0;
+  DeviceBuffer storage_;
+  Tensor output_;
+};
+
+// ---- separated weights from GGUF blocks -----------------------------------------------------
+// What LlamaModel::uploadQ4 / uploadQ8 build per tensor (interface/runner/llama/llama.cpp:940-1000):
+// values [K, N] (int8) or [K, N/2] (nibbles) and fp16 scales [K/32, N] ([2K/32, N] for the affine
+// re-encoding of Q4_K), with the reference's padded strides, produced on the device from the raw blocks.
+struct SeparatedWeights {
+  DeviceBuffer values, scales;
+  uint32_t N = 0, K = 0, strideB = 0, scaleStride = 0;
+  bool q4 = false, affine = false;
+};
+inline void prepareSeparated(SeparatedWeights &out, const Tensor &rawBlocks, GgufFormat format, uint32_t N, uint32_t K,
+                             void *stream = nullptr) {
+  if (format == GgufFormat::Q6_K) throw std::runtime_error("prepareSeparated: Q6_K has no separated layout");
+  if (K == 0 || K % blockElems(format) != 0) throw std::runtime_error("prepareSeparated: K must be a multiple of the block size");
+  out.q4 = format != GgufFormat::Q8_0;
+  out.affine = format == GgufFormat::Q4_K;
+  if (out.q4 && N % 2 != 0) throw std::runtime_error("prepareSeparated: N must be even for packed nibbles");
+  if (!rawBlocks.buffer || rawBlocks.buffer->bytes() < ggufBytes(format, (uint64_t)N * K))
+    throw std::runtime_error("prepareSeparated: raw tensor holds fewer bytes than N x K blocks");
+  out.N = N;
+  out.K = K;
+  out.strideB = ((out.q4 ? N / 2 : N) + 3) & ~3u;
+  out.scaleStride = (N + 3) & ~3u;
+  const uint32_t scaleRows = (out.affine ? 2u : 1u) * (K / 32);
+  out.values = DeviceBuffer((size_t)K * out.strideB);
+  out.scales = DeviceBuffer((size_t)scaleRows * out.scaleStride * 2);
+  check(cuthip_prepare_sep((int)format, rawBlocks.data(), N, K, out.values.data(), out.strideB,
+                           reinterpret_cast<uint16_t *>(out.scales.data()), out.scaleStride, stream),
+        "cuthip_prepare_sep");
+}
+
 }  // namespace hip
 }  // namespace cut

@@ -62,6 +62,13 @@ static void test_validation() {
   EXPECT(throws([&] { MatMulGgufOpNode n(a2, raw, GgufFormat::Q8_0, 8); }));  // K not a multiple of 32
   Tensor a3{&none, {2, 64}, DataType::Float16, 0};
   EXPECT(throws([&] { MatMulGgufOpNode n(a3, raw, GgufFormat::Q8_0, 8); }));  // weights too small
+  EXPECT(throws([&] { TransposeQ4NibbleOpNode n(raw, 3, 64); }));             // odd N (TransposeQ4NibbleOp.cpp:13-15)
+  EXPECT(throws([&] { TransposeQ4NibbleOpNode n(raw, 4, 48); }));             // K not a multiple of 32
+  EXPECT(throws([&] { TransposeQ4NibbleOpNode n(raw, 4, 64); }));             // input too small
+  SeparatedWeights sw;
+  EXPECT(throws([&] { prepareSeparated(sw, raw, GgufFormat::Q6_K, 4, 256); }));
+  EXPECT(throws([&] { prepareSeparated(sw, raw, GgufFormat::Q4_0, 3, 64); }));
+  EXPECT(throws([&] { prepareSeparated(sw, raw, GgufFormat::Q8_0, 4, 64); }));  // raw too small
 }
 
 static double normwise(const std::vector<float> &got, const std::vector<double> &want) {
@@ -97,6 +104,23 @@ static void test_gpu() {
     for (uint32_t r = 0; r < N && same; ++r)
       same = std::memcmp(&got[(size_t)r * dq.outputStride()], &want[(size_t)r * K], K * 4) == 0;
     EXPECT(same);
+
+    // separated [K, N] tensors made on the device, bit for bit against the oracle's host split + transpose
+    if (f == GgufFormat::Q8_0) {
+      SeparatedWeights sw;
+      prepareSeparated(sw, wt, f, N, K);
+      std::vector<int8_t> vals((size_t)K * sw.strideB), v_nk((size_t)N * K);
+      std::vector<uint16_t> sc((size_t)(K / 32) * sw.scaleStride), s_nk((size_t)N * (K / 32));
+      sw.values.download(vals.data(), vals.size());
+      sw.scales.download(sc.data(), sc.size() * 2);
+      orc_split_q8_0(blocks.data(), N, K, v_nk.data(), s_nk.data());
+      bool eq = true;
+      for (uint32_t k = 0; k < K && eq; ++k)
+        for (uint32_t n = 0; n < N && eq; ++n)
+          eq = vals[(size_t)k * sw.strideB + n] == v_nk[(size_t)n * K + k] &&
+               sc[(size_t)(k / 32) * sw.scaleStride + n] == s_nk[(size_t)n * (K / 32) + k / 32];
+      EXPECT(eq);
+    }
 
     // matmul at M = 1 (rank-1 A), 3 and 40 (GEMV, batched GEMV, tiled GEMM), fp32 in / fp32 out
     for (uint32_t M : {1u, 3u, 40u}) {
