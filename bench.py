@@ -175,8 +175,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (reference traffic for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
-    ap.add_argument("--gemm-variant", type=int, default=4, choices=(2, 4),
-                    help="with --gemm-only: 4 = dequantize once + dense GEMM (default), 2 = single-launch GEMM")
+    ap.add_argument("--gemm-variant", type=int, default=4, choices=(2, 4, 5),
+                    help="with --gemm-only: 4 = dequantize once + hand-written dense GEMM (default), 5 = dequantize once + hipBLASLt, 2 = single-launch GEMM")
     ap.add_argument("--gemm-only", type=int, default=0, metavar="M",
                     help="only run the Q4_K prefill GEMM (M x 4096) . (14336 x 4096)^T twelve times (target of rocprofv3 runs)")
     ap.add_argument("--dequant-only", action="store_true",
@@ -221,7 +221,7 @@ def main():
         a = torch.randn((M, N_EMBD), dtype=torch.float16, device=dev)
         c = torch.empty((M, N_FF), dtype=torch.float16, device=dev)
         # variant 4 = dequantize once + dense GEMM (two launches, both inside the timed region); 2 = single launch
-        ws = ops.matmul_gguf_workspace("Q4_K", M, N_EMBD, N_FF, a.dtype, dev) if args.gemm_variant == 4 else None
+        ws = ops.matmul_gguf_workspace("Q4_K", M, N_EMBD, N_FF, a.dtype, dev) if args.gemm_variant >= 4 else None
         for _ in range(2):
             ops.matmul_gguf(a, wq, "Q4_K", N_FF, N_EMBD, out=c, variant=args.gemm_variant, workspace=ws)
         torch.cuda.synchronize()
@@ -333,6 +333,14 @@ def main():
         del head, logits
         torch.cuda.empty_cache()
         # config 5: prefill GEMM, Q4_K weights, fp16 activations, fp16 MFMA with fp32 accumulate
+        try:
+            _a = torch.zeros((1024, 256), dtype=torch.float16, device=dev)
+            _w = torch.from_numpy(make_q_weights("Q4_K", 256, 256, 9)).to(dev)
+            ops.matmul_gguf(_a, _w, "Q4_K", 256, 256, variant=5,
+                            workspace=ops.matmul_gguf_workspace("Q4_K", 1024, 256, 256, _a.dtype, dev))
+            extras["prefill_automatic_choice"] = "MatMulGgufDequantBlasLt (variant 5)"
+        except lib.CutHipError:
+            extras["prefill_automatic_choice"] = "MatMulGgufDequantGemm (variant 4)"
         for (M, N, K) in ((512, N_FF, N_EMBD), (2048, N_FF, N_EMBD), (512, N_EMBD, N_FF), (2048, N_EMBD, N_FF)):
             w_h = w_up_h if N == N_FF else w_down_h
             wq = torch.from_numpy(w_h).to(dev)
@@ -346,10 +354,17 @@ def main():
 
             def gemm1(_s, a=a, wq=wq, c=c, N=N, K=K):  # the single-launch GEMM on the blocks
                 ops.matmul_gguf(a, wq, "Q4_K", N, K, out=c, variant=2)
+
+            def gemm4(_s, a=a, wq=wq, c=c, N=N, K=K, ws=ws):  # dequantize once + the hand-written dense GEMM
+                ops.matmul_gguf(a, wq, "Q4_K", N, K, out=c, variant=4, workspace=ws)
+            # the automatic choice with a workspace: dequantize once, then hipBLASLt's dense GEMM where that library is
+            # present (variant 5), else the hand-written one (variant 4); both launches are inside the timed region
             wall_g, ev_g, _ = timed_graph(torch, gemm, 10, 2)
             tflops = 2.0 * M * N * K * 10 / (ev_g * 1e-3) / 1e12
             extras[f"q4k_prefill_gemm_M{M}_N{N}_K{K}_TFLOPs"] = round(tflops, 1)
             extras[f"q4k_prefill_gemm_M{M}_N{N}_K{K}_pct_of_f16_mfma_peak"] = round(tflops / 2500.0 * 100, 1)
+            wall_g, ev_g, _ = timed_graph(torch, gemm4, 10, 2)
+            extras[f"q4k_prefill_gemm_M{M}_N{N}_K{K}_own_two_pass_TFLOPs"] = round(2.0 * M * N * K * 10 / (ev_g * 1e-3) / 1e12, 1)
             wall_g, ev_g, _ = timed_graph(torch, gemm1, 10, 2)
             extras[f"q4k_prefill_gemm_M{M}_N{N}_K{K}_single_launch_TFLOPs"] = round(2.0 * M * N * K * 10 / (ev_g * 1e-3) / 1e12, 1)
             del ws

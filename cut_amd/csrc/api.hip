@@ -40,6 +40,9 @@ static const cuthip_variant_info_t kMatMulGgufVariants[] = {
     {"MatMulGgufDequantGemm", 256, 1, 256, 256,
      "large-M prefill in two launches: the weights are dequantized once to an fp16 workspace, then a dense fp16 MFMA GEMM "
      "with LDS-direct loads and 128x128 accumulators per wave (needs cuthip_matmul_gguf_ws)"},
+    {"MatMulGgufDequantBlasLt", 256, 1, 256, 256,
+     "large-M prefill in two launches: the weights are dequantized once to an fp16 workspace, then hipBLASLt's dense fp16 "
+     "GEMM (opened at run time; no fused epilogue; needs cuthip_matmul_gguf_ws)"},
 };
 
 static const cuthip_variant_info_t *table(int op, int *count) {

@@ -289,10 +289,17 @@ static DenseShape pick_dense_shape(uint32_t M, uint32_t K, uint32_t N) {
 
 static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
+// scratch the vendor GEMM may use (variant 5) behind the dequantized weights and the converted activations
+constexpr size_t kBlasLtScratch = (size_t)32 << 20;
+
+bool blaslt_available();
+int launch_blaslt_gemm(const void *Wd, const void *A16, void *C, int c_f16, uint32_t M, uint32_t K, uint32_t N, uint32_t strideA,
+                       uint32_t strideC, void *workspace, size_t workspace_bytes, hipStream_t stream);
+
 size_t dense_gemm_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
   DenseShape sh = pick_dense_shape(M, K, N);
-  return align256((size_t)N * K * 2) + align256(a_f16 ? 0 : (size_t)M * K * 2) +
-         (sh.ksplit > 1 ? (size_t)sh.ksplit * M * N * 4 : 0);
+  const size_t partial = sh.ksplit > 1 ? (size_t)sh.ksplit * M * N * 4 : 0;
+  return align256((size_t)N * K * 2) + align256(a_f16 ? 0 : (size_t)M * K * 2) + (partial > kBlasLtScratch ? partial : kBlasLtScratch);
 }
 
 // true where the two-pass path beats the single-launch GEMM: from about a thousand rows; or when the single-launch
@@ -305,8 +312,10 @@ bool dense_gemm_preferred(uint32_t M, uint32_t K, uint32_t N) {
   return M >= 256 || (M > 40 && K >= 8192);
 }
 
+// use_blaslt: the dense GEMM goes to hipBLASLt (no epilogue there: the caller checks)
 int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K,
-                      uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream) {
+                      uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream,
+                      int use_blaslt) {
   uint8_t *w16 = reinterpret_cast<uint8_t *>(workspace);
   if (int rc = launch_dequant_any(fmt, W, w16, CUTHIP_F16, N, K, K, stream)) return rc;
   DenseParams p;
@@ -321,6 +330,13 @@ int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C,
     if (int rc = check_hip(hipGetLastError(), "activation convert launch")) return rc;
     p.A = reinterpret_cast<const uint8_t *>(a16);
     p.strideA = K;
+  }
+  if (use_blaslt) {
+    uint8_t *scratch = w16 + align256((size_t)N * K * 2) + align256(a_f16 ? 0 : (size_t)M * K * 2);
+    const int rc = launch_blaslt_gemm(w16, p.A, C, c_f16, M, K, N, p.strideA, strideC, scratch, kBlasLtScratch, stream);
+    // 1 = asked for by variant index: its errors are the caller's; 2 = automatic choice: a shape the library has no
+    // kernel for goes on to the GEMM below (nothing has been enqueued for it yet)
+    if (rc == CUTHIP_OK || use_blaslt == 1 || rc != CUTHIP_ERR_INVALID) return rc;
   }
   p.C = C;
   p.epi = epi;

@@ -109,7 +109,9 @@ bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a
 size_t dense_gemm_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16);
 bool dense_gemm_preferred(uint32_t M, uint32_t K, uint32_t N);
 int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K,
-                      uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream);
+                      uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream,
+                      int use_blaslt);
+bool blaslt_available();
 
 static int launch_gemv(int fmt, const GemvParams &p, hipStream_t stream) {
   switch (fmt) {
@@ -208,8 +210,8 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
     set_error("cuthip_matmul_gguf: the SwiGLU row-pair epilogue exists in variant 3 only (got variant %d)", variant);
     return CUTHIP_ERR_INVALID;
   }
-  if (variant == 4) {
-    set_error("cuthip_matmul_gguf: variant 4 (dequantize, then dense GEMM) needs a workspace: call cuthip_matmul_gguf_ws");
+  if (variant == 4 || variant == 5) {
+    set_error("cuthip_matmul_gguf: variants 4 and 5 (dequantize, then dense GEMM) need a workspace: call cuthip_matmul_gguf_ws");
     return CUTHIP_ERR_INVALID;
   }
   if (variant == 0 && M > 8) {
@@ -380,7 +382,7 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
                           uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D,
                           int variant, void *workspace, size_t workspace_bytes, void *stream) {
   using namespace cuthip;
-  if ((variant != 4 && variant != -1) || epilogue == CUTHIP_EPI_SWIGLU_PAIRS)
+  if ((variant != 4 && variant != 5 && variant != -1) || epilogue == CUTHIP_EPI_SWIGLU_PAIRS)
     return cuthip_matmul_gguf(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, variant,
                               stream);
   if (int rc = check_matmul_args(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, D))
@@ -423,22 +425,31 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   const bool fits = dense_gemm_fits(M, K, N, strideA, a_f16, A);
   const size_t need = dense_gemm_workspace(M, K, N, a_f16);
   const bool ws_ok = workspace && (uintptr_t)workspace % 256 == 0 && workspace_bytes >= need;
-  if (variant == -1 && !(dense_gemm_preferred(M, K, N) && fits && ws_ok))
+  // with the vendor GEMM behind the dequantization the two-pass path pays earlier: 25 us of dequantization for an FFN
+  // matrix against a single-launch GEMM that decodes the weights once per 128 rows (M = 512, N = 14336: 86 us against 110)
+  const bool lt_ok = variant == -1 && epilogue == CUTHIP_EPI_NONE && fits && ws_ok && blaslt_available();
+  if (variant == -1 && !((dense_gemm_preferred(M, K, N) || (lt_ok && M >= 384)) && fits && ws_ok))
     return cuthip_matmul_gguf(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, -1,
                               stream);
   if (!fits) {
-    set_error("cuthip_matmul_gguf_ws: variant 4 needs K a multiple of 128, 16-byte aligned rows of A and operands below "
-              "4 GiB (M %u, K %u, N %u, strideA %u)", M, K, N, strideA);
+    set_error("cuthip_matmul_gguf_ws: variants 4 and 5 need K a multiple of 128, 16-byte aligned rows of A and operands "
+              "below 4 GiB (M %u, K %u, N %u, strideA %u)", M, K, N, strideA);
     return CUTHIP_ERR_INVALID;
   }
   if (!ws_ok) {
-    set_error("cuthip_matmul_gguf_ws: variant 4 needs a 256-byte aligned workspace of %zu bytes, got %zu", need,
+    set_error("cuthip_matmul_gguf_ws: variants 4 and 5 need a 256-byte aligned workspace of %zu bytes, got %zu", need,
               workspace ? workspace_bytes : (size_t)0);
     return CUTHIP_ERR_INVALID;
   }
+  if (variant == 5 && epilogue != CUTHIP_EPI_NONE) {
+    set_error("cuthip_matmul_gguf_ws: variant 5 (dequantize, then the vendor GEMM) has no fused epilogue: use variant 4");
+    return CUTHIP_ERR_INVALID;
+  }
+  // the dense GEMM of the automatic choice: the vendor library where it is present and nothing is fused
+  const int use_blaslt = variant == 5 ? 1 : lt_ok ? 2 : 0;
   Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
   return launch_dense_gemm(fmt, W, A, a_f16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC, epi, workspace,
-                           reinterpret_cast<hipStream_t>(stream));
+                           reinterpret_cast<hipStream_t>(stream), use_blaslt);
 }
 
 int cuthip_matmul_gguf_pro(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t K, uint32_t N,

@@ -168,11 +168,20 @@ int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void 
  * the weights for every tile of activations.
  * workspace: device, 256-byte aligned, at least
  *            cuthip_matmul_gguf_workspace_bytes(fmt, M, K, N, a_dtype) bytes
- *            (N*K fp16, plus M*K fp16 when A is fp32, plus fp32 partial products
- *            when K is split); contents are scratch.
+ *            (N*K fp16, plus M*K fp16 when A is fp32, plus the larger of the fp32
+ *            partial products of a split K and 32 MiB of scratch for the vendor
+ *            GEMM); contents are scratch.
  * variant  : 4 = the two-pass path (an error if K is not a multiple of 128, the
  *            rows of A are not 16-byte aligned or the workspace is too small);
- *            -1 = choose by shape: variant 4 when it applies and M >= 1024 (or, with so
+ *            5 = MatMulGgufDequantBlasLt: the same dequantization, then hipBLASLt's
+ *            dense fp16 GEMM (the weights are plain fp16 by then, so it is a library
+ *            GEMM; the library is opened with dlopen on first use and its handle is
+ *            created then, the only allocation this library ever causes; an error if
+ *            the library is absent or an epilogue is asked for; CUT_HIP_NO_BLASLT=1 in
+ *            the environment keeps it closed);
+ *            -1 = choose by shape: the two-pass path (variant 5 where hipBLASLt is
+ *            present, has a kernel for the shape and no epilogue is fused, else
+ *            variant 4) when it applies and M >= 1024 (or, with so
  *            few output tiles that the single-launch GEMM would leave most of the chip
  *            idle, from M = 256, and from M = 41 when K >= 8192; K is then split and
  *            the partial products summed), else

@@ -181,7 +181,11 @@ static void test_gpu() {
     m4.dispatch();
     std::vector<float> c4((size_t)M * N);
     m4.output().buffer->download(c4.data(), c4.size() * 4);
-    EXPECT(std::memcmp(c.data(), c4.data(), c.size() * 4) == 0);
+    // the automatic choice may hand the dense GEMM to hipBLASLt (variant 5) where that library is present: same
+    // dequantized weights, fp32 accumulation in another order
+    std::vector<double> c4d(c4.begin(), c4.end());
+    EXPECT(normwise(c, c4d) < 1e-5);
+    EXPECT(normwise(c4, ref) < 1e-3);
   }
   // an explicit variant that cannot take the shape is an error, not a silent fallback
   {

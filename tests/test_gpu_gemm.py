@@ -271,3 +271,61 @@ def test_workspace_paths_under_hip_graph_replay(ops):
     for (M, N, K, w, a, ws, out), e in zip(bufs, eager):
         want = oracle.matmul_gguf(fmt, w.cpu().numpy(), a.float().cpu().numpy(), N, f64=True)
         assert normwise_rel_err(e.cpu().numpy(), want) < TOL_GEMM
+
+
+# ---- variant 5: dequantize once, then the vendor library's dense fp16 GEMM ----------------------------------------
+
+@pytest.mark.parametrize("name", list(oracle.FORMATS))
+@pytest.mark.parametrize("M,N,K", [(70, 136, 256), (300, 520, 1024), (512, 768, 512), (1030, 2056, 256)])
+def test_blaslt_gemm_vs_oracle(ops, name, M, N, K):
+    fmt = oracle.FORMATS[name]
+    W = quantized_weights(fmt, N, K, seed=51)
+    A = gauss_acts((M, K), seed=52, dtype=np.float16)
+    want = oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)
+    got = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=5)
+    assert normwise_rel_err(got, want) < TOL_GEMM
+    got16 = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float16, variant=5)
+    assert normwise_rel_err(got16, want) < TOL
+    # the same dequantized weights through the hand-written GEMM: fp32 accumulation on both sides
+    own = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=4)
+    assert normwise_rel_err(got, own) < 1e-5
+
+
+def test_blaslt_gemm_fp32_activations_and_automatic_choice(ops):
+    fmt = oracle.Q4_K
+    M, N, K = 1100, 520, 512
+    W = quantized_weights(fmt, N, K, seed=53)
+    A = gauss_acts((M, K), seed=54)
+    want = oracle.matmul_gguf(fmt, W, A, N, f64=True)
+    assert normwise_rel_err(gpu_matmul_ws(ops, fmt, W, A, N, K, variant=5), want) < 8e-4
+    # M >= 1024 without an epilogue: the automatic choice takes the same path; with an epilogue the hand-written GEMM
+    auto = gpu_matmul_ws(ops, fmt, W, A, N, K, variant=-1)
+    assert normwise_rel_err(auto, want) < 8e-4
+    D = gauss_acts((M, N), seed=55)
+    add = gpu_matmul_ws(ops, fmt, W, A, N, K, variant=-1, binary="add", d=torch.from_numpy(D).cuda())
+    assert normwise_rel_err(add, want + D) < 8e-4
+    from cut_amd import lib
+    with pytest.raises(lib.CutHipError, match="no fused epilogue"):
+        gpu_matmul_ws(ops, fmt, W, A, N, K, variant=5, unary="silu")
+
+
+def test_blaslt_gemm_under_graph_replay(ops):
+    fmt = oracle.Q4_K
+    M, N, K = 1024, 1024, 512
+    W = torch.from_numpy(quantized_weights(fmt, N, K, seed=56)).cuda()
+    a = torch.from_numpy(gauss_acts((M, K), seed=57, dtype=np.float16)).cuda()
+    ws = ops.matmul_gguf_workspace(fmt, M, K, N, a.dtype, "cuda")
+    c = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    ops.matmul_gguf(a, W, fmt, N, K, out=c, variant=5, workspace=ws)
+    torch.cuda.synchronize()
+    eager = c.clone()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        ops.matmul_gguf(a, W, fmt, N, K, out=c, variant=5, workspace=ws)
+    for _ in range(3):
+        c.zero_()
+        ws.fill_(0xFF)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(c, eager)
