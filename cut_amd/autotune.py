@@ -1,0 +1,88 @@
+"""Autotune sweep for the "hip" section of tuning_data.json (the reference derives its sections with
+scripts/bench/derive_rules.py from an autotune binary's output).
+
+    python -m cut_amd.autotune [--output cut_amd/tuning_data.json] [--reps 20]
+
+For every (format, M, K, N) of the sweep each variant of the MatMulGguf table that accepts the shape is timed through
+the C ABI (HIP events, weights rotated over several copies so that small matrices are not served from cache) and the
+fastest becomes an exact-shape rule `{"variant": v, "conditions": {"shape": [M, K, N]}}` under
+operators.MatMulGguf<fmt>.backends.hip; the entry's default variant is -1 (the library's own choice by shape).
+Needs an MI355X; refuses to run without one."""
+import argparse
+import json
+import os
+import sys
+
+SHAPES_NK = [(14336, 4096), (4096, 14336), (4096, 4096), (1024, 4096), (28672, 4096)]
+BATCHES = [1, 2, 4, 8, 16, 32, 64, 128, 512, 2048]
+FORMATS = ["Q4_K", "Q6_K", "Q8_0"]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--output", default=os.path.join(os.path.dirname(os.path.abspath(__file__)), "tuning_data.json"))
+    ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--formats", default=",".join(FORMATS))
+    args = ap.parse_args()
+    import numpy as np
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("autotune: no GPU")
+    from cut_amd import lib, ops, quantize as Q
+    lib.check(lib.load().cuthip_init(0))
+    dev = torch.device("cuda:0")
+    names = [v["name"] for v in lib.variants(lib.OP_MATMUL_GGUF)]
+    operators = {}
+    for fmt in args.formats.split(","):
+        rules, log = [], []
+        for (N, K) in SHAPES_NK:
+            tile = Q.quantize(fmt, np.random.default_rng(0).standard_normal(1024 * K, dtype=np.float32) * np.float32(0.02))
+            w = torch.from_numpy(tile).to(dev).repeat(N // 1024)
+            copies = [w.clone() for _ in range(max(2, min(8, int(3e8 // w.numel()))))]
+            for M in BATCHES:
+                a = torch.randn((M, K), dtype=torch.float16, device=dev)
+                c = torch.empty((M, N), dtype=torch.float16, device=dev)
+                ws = ops.matmul_gguf_workspace(fmt, M, K, N, a.dtype, dev)
+                best = None
+                for v in [-1] + list(range(len(names))):
+                    try:
+                        for i in range(2):
+                            ops.matmul_gguf(a, copies[i % len(copies)], fmt, N, K, out=c, variant=v, workspace=ws)
+                        torch.cuda.synchronize()
+                    except lib.CutHipError:
+                        continue          # the variant does not take this shape
+                    # the launches are replayed as one HIP graph: timed eagerly, anything under ~10 us would
+                    # measure the host's launch rate instead of the kernel
+                    g = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(g):
+                        for i in range(args.reps):
+                            ops.matmul_gguf(a, copies[i % len(copies)], fmt, N, K, out=c, variant=v, workspace=ws)
+                    g.replay()
+                    torch.cuda.synchronize()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    g.replay()
+                    e1.record()
+                    torch.cuda.synchronize()
+                    del g
+                    us = e0.elapsed_time(e1) * 1e3 / args.reps
+                    log.append({"shape": [M, K, N], "variant": v, "us": round(us, 2)})
+                    if best is None or us < best[1]:
+                        best = (v, us)
+                print(f"{fmt} M={M} K={K} N={N}: variant {best[0]} {best[1]:.1f} us", flush=True)
+                if best[0] >= 0:
+                    rules.append({"variant": best[0], "conditions": {"shape": [M, K, N]}})
+                del ws
+            del copies, w
+            torch.cuda.empty_cache()
+        operators[f"MatMulGguf{fmt}"] = {"backends": {"hip": {"default_variant": -1, "rules": rules, "measurements_us": log}}}
+    info = lib.device_info()
+    out = {"device": info["name"], "arch": info["arch"], "variant_names": names, "operators": operators}
+    with open(args.output, "w") as fh:
+        json.dump(out, fh, separators=(",", ":"))
+        fh.write("\n")
+    print(f"wrote {args.output}")
+
+
+if __name__ == "__main__":
+    main()

@@ -48,7 +48,9 @@ static const cuthip_variant_info_t kMatMulGgufVariants[] = {
 static const cuthip_variant_info_t *table(int op, int *count) {
   switch (op) {
   case CUTHIP_OP_DEQUANT: *count = 1; return kDequantVariants;
-  case CUTHIP_OP_MATMUL_GGUF: *count = 5; return kMatMulGgufVariants;
+  case CUTHIP_OP_MATMUL_GGUF:
+    *count = (int)(sizeof(kMatMulGgufVariants) / sizeof(kMatMulGgufVariants[0]));
+    return kMatMulGgufVariants;
   }
   *count = 0;
   return nullptr;

@@ -388,6 +388,26 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   if (int rc = check_matmul_args(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, D))
     return rc > 0 ? CUTHIP_OK : rc;
   const int a_f16 = a_dtype == CUTHIP_F16;
+  // 9..383 rows with the vendor GEMM at hand: dequantize + hipBLASLt against what the automatic choice would run
+  // otherwise, by a cost model fitted to a sweep over the FFN / attention shapes of an 8B model (microseconds;
+  // Q4_K, graph replay): an 8-row pass 6.5 + weight bytes / 4.3 MB (x 1.45 on rows of K >= 8192), the
+  // single-launch GEMM 62 + weight bytes / 7 MB (K >= 8192: the split two-pass GEMM, 65 + 0.19 M), the vendor path
+  // 14 + N K x 0.65e-6 (0.95e-6 once the fp16 copy outgrows the 256 MB cache) + 2 M N K / 1.6 PFLOP/s.
+  if (variant == -1 && M > 8 && M < 384 && epilogue == CUTHIP_EPI_NONE && workspace && (uintptr_t)workspace % 256 == 0 &&
+      dense_gemm_fits(M, K, N, strideA, a_f16, A) && workspace_bytes >= dense_gemm_workspace(M, K, N, a_f16) &&
+      blaslt_available()) {
+    const double nk = (double)N * K, wb = nk / fmt_elems(fmt) * fmt_bytes(fmt);
+    const double t5 = 14.0 + nk * (nk <= 64e6 ? 0.65e-6 : 0.95e-6) + 2.0 * M * nk / 1.6e9;
+    double other;
+    if (M <= kPassesMaxRows) other = ((M + 7) / 8) * (6.5 + wb / 4.3e6) * (K >= 8192 ? 1.45 : 1.0);
+    else other = K >= 8192 ? 65.0 + 0.19 * M : 62.0 + wb / 7e6;
+    if (t5 < 0.95 * other) {
+      const int rc = launch_dense_gemm(fmt, W, A, a_f16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC,
+                                       Epilogue{CUTHIP_EPI_NONE, 0, nullptr}, workspace,
+                                       reinterpret_cast<hipStream_t>(stream), 2);
+      return rc;
+    }
+  }
   if (variant == -1 && M > 8 && M <= kPassesMaxRows) {   // 8-row passes, each with the workspace (K split on long rows)
     const size_t asz = a_f16 ? 2 : 4, csz = c_dtype == CUTHIP_F16 ? 2 : 4;
     for (uint32_t m0 = 0; m0 < M; m0 += 8) {

@@ -53,6 +53,28 @@ def dequantize(raw: torch.Tensor, fmt, rows: int, cols: int, dtype: torch.dtype 
     return out
 
 
+_FMT_NAMES = {_l.Q8_0: "Q8_0", _l.Q4_0: "Q4_0", _l.Q4_K: "Q4_K", _l.Q6_K: "Q6_K"}
+_tuning = None
+
+
+def enable_tuning(path: str | None = None) -> bool:
+    """Lets matmul_gguf consult shape rules (cut_amd/tuning_data.json by default, the "hip" backend section) when it
+    is called with variant = -1, no epilogue and a workspace: the reference's VariantSelector mechanism
+    (MatMulOp.cpp:242-246).  Returns False, and changes nothing, if the file cannot be loaded."""
+    global _tuning
+    from . import variant_selector as _vs
+    sel = _vs.VariantSelector()
+    if not sel.load(path or _vs.DEFAULT_PATH):
+        return False
+    _tuning = sel
+    return True
+
+
+def disable_tuning() -> None:
+    global _tuning
+    _tuning = None
+
+
 def matmul_gguf(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: int, out_dtype: torch.dtype | None = None,
                 out: torch.Tensor | None = None, unary: str | None = None, binary: str | None = None,
                 d: torch.Tensor | None = None, variant: int = -1, workspace: torch.Tensor | None = None,
@@ -90,6 +112,8 @@ def matmul_gguf(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: int, ou
         epi, op, dptr = _l.EPI_BINARY, _l.BINARY[binary], d.data_ptr()
     adt = _l.F16 if a2.dtype == torch.float16 else _l.F32
     cdt = _l.F16 if out.dtype == torch.float16 else _l.F32
+    if _tuning is not None and variant == -1 and epi == _l.EPI_NONE and workspace is not None:
+        variant = _tuning.select("MatMulGguf" + _FMT_NAMES[f], [M, K, N], -1)
     if workspace is not None:
         _l.check(_l.load().cuthip_matmul_gguf_ws(
             f, w_blocks.data_ptr(), a2.data_ptr(), adt, out.data_ptr(), cdt, M, K, N, a2.stride(0), out.stride(0), epi, op,

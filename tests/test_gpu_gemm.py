@@ -329,3 +329,27 @@ def test_blaslt_gemm_under_graph_replay(ops):
         g.replay()
         torch.cuda.synchronize()
         assert torch.equal(c, eager)
+
+
+def test_tuning_rules_select_the_variant(ops, tmp_path):
+    """ops.enable_tuning: an exact-shape rule of the "hip" section decides the variant of a call with variant = -1."""
+    import json
+    fmt = oracle.Q4_K
+    M, N, K = 48, 512, 512
+    rules = {"operators": {"MatMulGgufQ4_K": {"backends": {"hip": {"default_variant": -1, "rules": [
+        {"variant": 2, "conditions": {"shape": [M, K, N]}}]}}}}}
+    path = tmp_path / "tuning_data.json"
+    path.write_text(json.dumps(rules))
+    W = quantized_weights(fmt, N, K, seed=61)
+    A = gauss_acts((M, K), seed=62, dtype=np.float16)
+    explicit = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=2)
+    assert ops.enable_tuning(str(path))
+    try:
+        tuned = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=-1)
+    finally:
+        ops.disable_tuning()
+    assert np.array_equal(tuned, explicit)
+    assert normwise_rel_err(tuned, oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)) < TOL_GEMM
+    assert not ops.enable_tuning(str(tmp_path / "missing.json"))
+    assert ops.enable_tuning()          # the committed file loads
+    ops.disable_tuning()
