@@ -113,6 +113,36 @@ def bench_decode_step(torch, np, ops, dev, x_h, steps=5):
             "decode_step_8b_bytes_per_token": int(w_bytes_tok + kv_bytes_tok)}
 
 
+def bench_prepare(torch, ops, dev, reps=10):
+    """Load-time preparation of one FFN matrix (14336 x 4096) on the device: GGUF blocks -> separated [K, N] tensors
+    (cuthip_prepare_sep) and fp32 -> Q8_0 blocks (cuthip_quantize_rows_q8_0); GB/s over bytes read + bytes written."""
+    from cut_amd import lib
+    res = {}
+    N, K = N_FF, N_EMBD
+    for name in ("Q8_0", "Q4_0", "Q4_K"):
+        w = torch.from_numpy(make_q_weights(name, 1024, K, 5)).to(dev).repeat(N // 1024)
+        q4 = name != "Q8_0"
+        B = torch.empty((K, N // 2 if q4 else N), dtype=torch.uint8, device=dev)
+        S = torch.empty(((2 if name == "Q4_K" else 1) * K // 32, N), dtype=torch.float16, device=dev)
+        f = lib.FORMATS[name]
+
+        def prep(_s):
+            lib.check(lib.load().cuthip_prepare_sep(f, w.data_ptr(), N, K, B.data_ptr(), B.shape[1], S.data_ptr(), N,
+                                                    torch.cuda.current_stream().cuda_stream))
+        _, ev, _ = timed_graph(torch, prep, reps, 2)
+        res[f"prepare_sep_{name}_14336x4096_GBps"] = round((w.numel() + B.numel() + S.numel() * 2) * reps / (ev * 1e-3) / 1e9, 1)
+        del w, B, S
+    x = torch.randn(N * K, dtype=torch.float32, device=dev) * 0.02
+
+    def quant(_s):
+        ops.quantize_rows_q8_0(x)
+    _, ev, _ = timed_graph(torch, quant, reps, 2)
+    res["quantize_rows_q8_0_14336x4096_GBps"] = round((x.numel() * 4 + x.numel() // 32 * 34) * reps / (ev * 1e-3) / 1e9, 1)
+    del x
+    torch.cuda.empty_cache()
+    return res
+
+
 def bench_q8_prefill(torch, ops, dev, shapes=((512, N_FF, N_EMBD), (2048, N_FF, N_EMBD)), reps=10):
     """Q8_0 prefill GEMM: cuthip_matmul_q8_i8 (int8 activations per 32, int8 MFMA; TOP/s = 2MNK / time including
     the activation quantizer) and the fp16-activation path of cuthip_matmul_gguf on the same blocks."""
@@ -181,6 +211,7 @@ def main():
                     help="only run the Q4_K prefill GEMM (M x 4096) . (14336 x 4096)^T twelve times (target of rocprofv3 runs)")
     ap.add_argument("--dequant-only", action="store_true",
                     help="only run the 256 Mi-element dequant of the four formats (target of rocprofv3 runs)")
+    ap.add_argument("--prepare-only", action="store_true", help="only run the load-time preparation kernels")
     ap.add_argument("--q8-only", action="store_true",
                     help="only run the Q8_0 prefill GEMMs at M = 2048 (int8-activation variant and fp16 path)")
     ap.add_argument("--decode-only", action="store_true",
@@ -207,6 +238,9 @@ def main():
         return
     if args.dequant_only:
         print(json.dumps(bench_dequant(torch, ops, dev, reps=5)))
+        return
+    if args.prepare_only:
+        print(json.dumps(bench_prepare(torch, ops, dev)))
         return
     if args.q8_only:
         print(json.dumps(bench_q8_prefill(torch, ops, dev, shapes=((2048, N_FF, N_EMBD),), reps=5)))
@@ -372,6 +406,7 @@ def main():
         # config 5, second half: Q8_0 weights with activations quantized to int8 per 32 on the int8 matrix core
         # (both launches, quantizer + GEMM, inside the timed region), next to the fp16 path on the same blocks
         extras.update(bench_q8_prefill(torch, ops, dev))
+        extras.update(bench_prepare(torch, ops, dev))
     result["extras"] = extras
 
     # ---- CPU baseline: the oracle's restatement of the reference path -------------
