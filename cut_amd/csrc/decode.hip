@@ -153,10 +153,13 @@ constexpr int kAttnMaxHd = 128;   // head dimension limit (as the reference's sh
 constexpr int kAttnRow = kAttnMaxHd + 8;   // LDS row in halfs: +16 bytes keeps the 64 rows off each other's banks
 
 // partial layout per (query head h, split s): [m, l, o[headDim]] floats at ((h * nsplit + s) * (2 + headDim))
+// HD: the head dimension when it is the common 128 (loops over it unroll and their LDS reads overlap), 0 = any
+template <int HD>
 __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_f16, const half_t *kCache, const half_t *vCache,
                                                            const uint32_t *params, float *partial, uint32_t nHeads,
-                                                           uint32_t nKvHeads, uint32_t headDim, uint32_t alignedKvDim,
+                                                           uint32_t nKvHeads, uint32_t headDimArg, uint32_t alignedKvDim,
                                                            float scale, uint32_t nsplit, uint32_t maxSeqLen) {
+  const uint32_t headDim = HD ? (uint32_t)HD : headDimArg;
   __shared__ __attribute__((aligned(16))) half_t Ks[kAttnChunk * kAttnRow];
   __shared__ __attribute__((aligned(16))) half_t Vs[kAttnChunk * kAttnRow];
   __shared__ __attribute__((aligned(16))) float Qs[4 * kAttnMaxHd];
@@ -210,6 +213,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_
     float sc = 0.0f;
     const half_t *krow = Ks + lane * kAttnRow;
     const f32x4 *qv = reinterpret_cast<const f32x4 *>(Qs + wave * kAttnMaxHd);
+#pragma unroll
     for (uint32_t d = 0; d < headDim; d += 8) {
       half8_t k8 = *reinterpret_cast<const half8_t *>(krow + d);
       f32x4 qa = qv[d / 4], qb = qv[d / 4 + 1];
@@ -231,7 +235,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_
     typedef _Float16 half2v __attribute__((ext_vector_type(2)));
     const f32x4 *pv = reinterpret_cast<const f32x4 *>(Ps + wave * kAttnChunk);
     const uint32_t dcol = min(2 * lane, (uint32_t)kAttnMaxHd - 2);
-#pragma unroll 4
+#pragma unroll
     for (uint32_t t = 0; t < (uint32_t)kAttnChunk; t += 4) {
       f32x4 p4 = pv[t / 4];
       half2v v0 = *reinterpret_cast<const half2v *>(Vs + (t + 0) * kAttnRow + dcol);
@@ -272,6 +276,13 @@ __global__ void __launch_bounds__(128) attn_merge_kernel(const float *partial, c
   const uint32_t used = nsplit;
   const uint32_t rec = 2 + headDim;
   const float *base = partial + (size_t)h * nsplit * rec;
+  // up to 32 splits (a context of 2048): this thread's dimension of every split is requested now, together with the
+  // (max, sum) pairs, so that the whole merge costs one memory round trip instead of three
+  constexpr uint32_t kPre = 32;
+  const bool pre = used <= kPre;
+  float ov[kPre];
+#pragma unroll
+  for (uint32_t s = 0; s < kPre; ++s) ov[s] = (pre && s < used && tid < headDim) ? base[(size_t)s * rec + 2 + tid] : 0.0f;
   float m = -INFINITY;
   for (uint32_t s = tid; s < used; s += 128) m = fmaxf(m, base[(size_t)s * rec]);
   m = wave_max(m);
@@ -291,8 +302,13 @@ __global__ void __launch_bounds__(128) attn_merge_kernel(const float *partial, c
   const float L = red[2] + red[3];
   if (tid < headDim) {
     float o = 0.0f;
+    if (pre) {
+#pragma unroll
+      for (uint32_t s = 0; s < kPre; ++s) o = fmaf(ov[s], s < used ? Ws[s] : 0.0f, o);
+    } else {
 #pragma unroll 8
-    for (uint32_t s = 0; s < used; ++s) o = fmaf(base[(size_t)s * rec + 2 + tid], Ws[s], o);
+      for (uint32_t s = 0; s < used; ++s) o = fmaf(base[(size_t)s * rec + 2 + tid], Ws[s], o);
+    }
     st_act(out, out_f16, (size_t)h * headDim + tid, L > 0.0f ? o / L : 0.0f);
   }
 }
@@ -436,7 +452,8 @@ int cuthip_attn_decode(const void *q, int q_dtype, const void *k_cache, const vo
   }
   uint32_t nsplit = (max_seq_len + kAttnChunk - 1) / kAttnChunk;
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(attn_partial_kernel, dim3(n_kv_heads, nsplit), dim3(256), 0, s, q, q_dtype == CUTHIP_F16,
+  auto partial_kernel = head_dim == 128 ? attn_partial_kernel<128> : attn_partial_kernel<0>;
+  hipLaunchKernelGGL(partial_kernel, dim3(n_kv_heads, nsplit), dim3(256), 0, s, q, q_dtype == CUTHIP_F16,
                      (const half_t *)k_cache, (const half_t *)v_cache, runtime_params, (float *)workspace, n_heads, n_kv_heads,
                      head_dim, aligned_kv_dim, scale, nsplit, max_seq_len);
   if (int rc = check_hip(hipGetLastError(), "attention launch")) return rc;
