@@ -40,7 +40,7 @@ struct BlasLtPlan {
   hipblasLtMatrixLayout_t a = nullptr, b = nullptr, c = nullptr;
   hipblasLtMatmulAlgo_t algo;
   size_t workspace = 0;
-  bool ok = false;
+  bool tried = false, ok = false;
 };
 
 std::mutex g_mu;
@@ -97,7 +97,8 @@ int launch_blaslt_gemm(const void *Wd, const void *A16, void *C, int c_f16, uint
   }
   const PlanKey key{M, K, N, strideA, strideC, c_f16, workspace_bytes};
   BlasLtPlan &plan = g_plans[key];
-  if (!plan.desc) {
+  if (!plan.tried) {
+    plan.tried = true;
     const hipblasOperation_t opT = HIPBLAS_OP_T, opN = HIPBLAS_OP_N;
     const hipDataType ctype = c_f16 ? HIP_R_16F : HIP_R_32F;
     bool ok = lt.desc_create(&plan.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS &&
@@ -123,7 +124,6 @@ int launch_blaslt_gemm(const void *Wd, const void *A16, void *C, int c_f16, uint
       }
     }
     if (pref) lt.pref_destroy(pref);
-    if (!plan.desc) plan.desc = reinterpret_cast<hipblasLtMatmulDesc_t>(&plan);   // marks "tried" when even the descriptor failed
     plan.ok = ok;
   }
   if (!plan.ok) {
