@@ -401,7 +401,19 @@ def main():
             extras[f"q4k_prefill_gemm_M{M}_N{N}_K{K}_own_two_pass_TFLOPs"] = round(2.0 * M * N * K * 10 / (ev_g * 1e-3) / 1e12, 1)
             wall_g, ev_g, _ = timed_graph(torch, gemm1, 10, 2)
             extras[f"q4k_prefill_gemm_M{M}_N{N}_K{K}_single_launch_TFLOPs"] = round(2.0 * M * N * K * 10 / (ev_g * 1e-3) / 1e12, 1)
-            del ws
+            # the same matmul on weights that are kept dequantized (fp16 [N, K], 2 bytes per weight of the 288 GB):
+            # no dequantization inside the call
+            w16 = ops.dequantize(wq, "Q4_K", N, K, torch.float16)
+            ws16 = torch.empty(max(int(lib.load().cuthip_matmul_dense_f16_workspace_bytes(M, K, N, lib.F16)), 256),
+                               dtype=torch.uint8, device=dev)
+
+            def gemm16(_s, a=a, w16=w16, c=c, ws16=ws16):
+                ops.matmul_dense_f16(a, w16, out=c, workspace=ws16)
+            wall_g, ev_g, _ = timed_graph(torch, gemm16, 10, 2)
+            t16 = 2.0 * M * N * K * 10 / (ev_g * 1e-3) / 1e12
+            extras[f"q4k_prefill_gemm_M{M}_N{N}_K{K}_resident_f16_weights_TFLOPs"] = round(t16, 1)
+            extras[f"q4k_prefill_gemm_M{M}_N{N}_K{K}_resident_f16_weights_pct_of_f16_mfma_peak"] = round(t16 / 2500.0 * 100, 1)
+            del ws, w16, ws16
             del wq, a, c
         # config 5, second half: Q8_0 weights with activations quantized to int8 per 32 on the int8 matrix core
         # (both launches, quantizer + GEMM, inside the timed region), next to the fp16 path on the same blocks

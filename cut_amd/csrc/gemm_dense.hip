@@ -302,6 +302,11 @@ size_t dense_gemm_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
   return align256((size_t)N * K * 2) + align256(a_f16 ? 0 : (size_t)M * K * 2) + (partial > kBlasLtScratch ? partial : kBlasLtScratch);
 }
 
+// workspace of the GEMM on resident fp16 weights: converted activations (fp32 input only) + split-K partials / scratch
+size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
+  return dense_gemm_workspace(M, K, N, a_f16) - align256((size_t)N * K * 2);
+}
+
 // true where the two-pass path beats the single-launch GEMM: from about a thousand rows; or when the single-launch
 // kernel's 128 x 128 tiles would leave most of the chip idle, from 256 rows, and already from 41 rows on long K, where
 // that kernel's time is the decode of a whole K-long tile row per workgroup (measured 4096 x 14336: 217-222 us for
@@ -316,14 +321,21 @@ bool dense_gemm_preferred(uint32_t M, uint32_t K, uint32_t N) {
 int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K,
                       uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream,
                       int use_blaslt) {
-  uint8_t *w16 = reinterpret_cast<uint8_t *>(workspace);
-  if (int rc = launch_dequant_any(fmt, W, w16, CUTHIP_F16, N, K, K, stream)) return rc;
+  // fmt < 0: W already holds the dequantized fp16 weights [N][K] (cuthip_matmul_dense_f16); the workspace then starts
+  // with the converted activations.  Otherwise the weights are dequantized to the head of the workspace first.
+  const bool resident = fmt < 0;
+  uint8_t *ws = reinterpret_cast<uint8_t *>(workspace);
+  const uint8_t *w16 = resident ? reinterpret_cast<const uint8_t *>(W) : ws;
+  uint8_t *after_w = resident ? ws : ws + align256((size_t)N * K * 2);
+  if (!resident) {
+    if (int rc = launch_dequant_any(fmt, W, ws, CUTHIP_F16, N, K, K, stream)) return rc;
+  }
   DenseParams p;
   p.W = w16;
   p.A = reinterpret_cast<const uint8_t *>(A);
   p.strideA = strideA;
   if (!a_f16) {
-    half_t *a16 = reinterpret_cast<half_t *>(w16 + align256((size_t)N * K * 2));
+    half_t *a16 = reinterpret_cast<half_t *>(after_w);
     uint32_t chunks = (K / 8 + 255) / 256;
     hipLaunchKernelGGL(cvt_rows_kernel, dim3(M * chunks), dim3(256), 0, stream, reinterpret_cast<const float *>(A), a16, K,
                        strideA, chunks);
@@ -332,7 +344,7 @@ int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C,
     p.strideA = K;
   }
   if (use_blaslt) {
-    uint8_t *scratch = w16 + align256((size_t)N * K * 2) + align256(a_f16 ? 0 : (size_t)M * K * 2);
+    uint8_t *scratch = after_w + align256(a_f16 ? 0 : (size_t)M * K * 2);
     const int rc = launch_blaslt_gemm(w16, p.A, C, c_f16, M, K, N, p.strideA, strideC, scratch, kBlasLtScratch, stream);
     // 1 = asked for by variant index: its errors are the caller's; 2 = automatic choice: a shape the library has no
     // kernel for goes on to the GEMM below (nothing has been enqueued for it yet)
@@ -346,7 +358,7 @@ int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C,
   const DenseShape sh = pick_dense_shape(M, K, N);
   p.ksplit = sh.ksplit;
   p.kper = K / sh.ksplit;
-  p.partial = reinterpret_cast<float *>(w16 + align256((size_t)N * K * 2) + align256(a_f16 ? 0 : (size_t)M * K * 2));
+  p.partial = reinterpret_cast<float *>(after_w + align256(a_f16 ? 0 : (size_t)M * K * 2));
   int rc;
   if (sh.bn == 448) rc = launch_dense_bm<128, 448>(p, stream);
   else if (sh.bm == 256) rc = launch_dense_bm<256, 256>(p, stream);

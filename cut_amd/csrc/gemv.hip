@@ -112,6 +112,7 @@ int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C,
                       uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream,
                       int use_blaslt);
 bool blaslt_available();
+size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16);
 
 static int launch_gemv(int fmt, const GemvParams &p, hipStream_t stream) {
   switch (fmt) {
@@ -469,6 +470,46 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   const int use_blaslt = variant == 5 ? 1 : lt_ok ? 2 : 0;
   Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
   return launch_dense_gemm(fmt, W, A, a_f16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC, epi, workspace,
+                           reinterpret_cast<hipStream_t>(stream), use_blaslt);
+}
+
+size_t cuthip_matmul_dense_f16_workspace_bytes(uint32_t M, uint32_t K, uint32_t N, int a_dtype) {
+  return cuthip::dense_f16_workspace(M, K, N, a_dtype == CUTHIP_F16);
+}
+
+int cuthip_matmul_dense_f16(const void *W16, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M, uint32_t K, uint32_t N,
+                            uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D, void *workspace,
+                            size_t workspace_bytes, void *stream) {
+  using namespace cuthip;
+  if (M == 0 || N == 0) return CUTHIP_OK;
+  if (!W16 || !A || !C || (a_dtype != CUTHIP_F32 && a_dtype != CUTHIP_F16) || (c_dtype != CUTHIP_F32 && c_dtype != CUTHIP_F16) ||
+      strideA < K || strideC < N) {
+    set_error("cuthip_matmul_dense_f16: bad argument (null pointer, dtype, or a stride shorter than its row)");
+    return CUTHIP_ERR_INVALID;
+  }
+  if (epilogue != CUTHIP_EPI_NONE && epilogue != CUTHIP_EPI_UNARY && epilogue != CUTHIP_EPI_BINARY) {
+    set_error("cuthip_matmul_dense_f16: epilogue %d is not supported here", epilogue);
+    return CUTHIP_ERR_INVALID;
+  }
+  if (epilogue == CUTHIP_EPI_BINARY && !D) {
+    set_error("cuthip_matmul_dense_f16: binary epilogue without D");
+    return CUTHIP_ERR_INVALID;
+  }
+  const int a_f16 = a_dtype == CUTHIP_F16;
+  if (!dense_gemm_fits(M, K, N, strideA, a_f16, A) || (uintptr_t)W16 % 256 != 0) {
+    set_error("cuthip_matmul_dense_f16: needs K a multiple of 128, 256-byte aligned weights, 16-byte aligned rows of A and "
+              "operands below 4 GiB (M %u, K %u, N %u, strideA %u)", M, K, N, strideA);
+    return CUTHIP_ERR_INVALID;
+  }
+  const size_t need = dense_f16_workspace(M, K, N, a_f16);
+  if (!workspace || (uintptr_t)workspace % 256 != 0 || workspace_bytes < need) {
+    set_error("cuthip_matmul_dense_f16: needs a 256-byte aligned workspace of %zu bytes, got %zu", need,
+              workspace ? workspace_bytes : (size_t)0);
+    return CUTHIP_ERR_INVALID;
+  }
+  const int use_blaslt = (epilogue == CUTHIP_EPI_NONE && blaslt_available()) ? 2 : 0;
+  Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
+  return launch_dense_gemm(-1, W16, A, a_f16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC, epi, workspace,
                            reinterpret_cast<hipStream_t>(stream), use_blaslt);
 }
 

@@ -36,6 +36,7 @@ EXPORTS = [
     "cuthip_matmul_sep_workspace_bytes", "cuthip_matmul_q8_sep", "cuthip_matmul_q4_sep",
     "cuthip_prepare_sep", "cuthip_transpose_q4_nibble", "cuthip_quantize_rows_q8_0",
     "cuthip_matmul_q8_i8_workspace_bytes", "cuthip_matmul_q8_i8",
+    "cuthip_matmul_dense_f16_workspace_bytes", "cuthip_matmul_dense_f16",
 ]
 
 
@@ -123,10 +124,13 @@ def load() -> C.CDLL:
     lib.cuthip_prepare_sep.argtypes = [i, vp, u32, u32, vp, u32, vp, u32, vp]
     lib.cuthip_transpose_q4_nibble.argtypes = [vp, vp, u32, u32, u32, u32, vp]
     lib.cuthip_quantize_rows_q8_0.argtypes = [vp, C.c_uint64, vp, vp]
+    lib.cuthip_matmul_dense_f16_workspace_bytes.argtypes = [u32, u32, u32, i]
+    lib.cuthip_matmul_dense_f16.argtypes = [vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, vp, C.c_size_t, vp]
     lib.cuthip_matmul_q8_i8_workspace_bytes.argtypes = [u32, u32]
     lib.cuthip_matmul_q8_i8.argtypes = [vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, vp, C.c_size_t, vp]
     sized = ("cuthip_attn_decode_workspace_bytes", "cuthip_matmul_sep_workspace_bytes",
-             "cuthip_matmul_gguf_workspace_bytes", "cuthip_matmul_q8_i8_workspace_bytes")
+             "cuthip_matmul_gguf_workspace_bytes", "cuthip_matmul_q8_i8_workspace_bytes",
+             "cuthip_matmul_dense_f16_workspace_bytes")
     for n in EXPORTS:
         if n != "cuthip_last_error" and n not in sized:
             getattr(lib, n).restype = i

@@ -299,6 +299,37 @@ def matmul_sep(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, N: int, q
     return out
 
 
+def matmul_dense_f16(a: torch.Tensor, w16: torch.Tensor, out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
+                     unary: str | None = None, binary: str | None = None, d: torch.Tensor | None = None,
+                     workspace: torch.Tensor | None = None) -> torch.Tensor:
+    """Prefill matmul on resident dequantized weights: w16 fp16 [N, K] (from dequantize(..., torch.float16)), a [M, K]
+    fp16 or fp32; C = a . w16^T.  The quantized blocks stay the operand of the decode GEMV; this copy serves prefill."""
+    a2 = a if a.dim() == 2 else a.reshape(1, -1)
+    M, K = a2.shape
+    if w16.dtype != torch.float16 or w16.dim() != 2 or w16.shape[1] != K or not w16.is_contiguous():
+        raise _l.CutHipError(f"matmul_dense_f16: w16 must be a contiguous fp16 [N, {K}] tensor")
+    N = w16.shape[0]
+    if a2.dtype not in (torch.float32, torch.float16) or a2.stride(1) != 1:
+        raise _l.CutHipError("matmul_dense_f16: a must be fp32 / fp16 with contiguous rows")
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype or a2.dtype, device=a.device)
+    epi, op, dptr = _l.EPI_NONE, 0, None
+    if unary is not None:
+        epi, op = _l.EPI_UNARY, _l.UNARY[unary]
+    elif binary is not None:
+        if d is None or d.shape != out.shape or d.dtype != out.dtype or d.stride(0) != out.stride(0):
+            raise _l.CutHipError("matmul_dense_f16: binary epilogue needs a D with the dtype, shape and stride of C")
+        epi, op, dptr = _l.EPI_BINARY, _l.BINARY[binary], d.data_ptr()
+    lib = _l.load()
+    if workspace is None:
+        workspace = torch.empty(max(lib.cuthip_matmul_dense_f16_workspace_bytes(M, K, N, _dt(a2)), 256), dtype=torch.uint8,
+                                device=a.device)
+    _l.check(lib.cuthip_matmul_dense_f16(w16.data_ptr(), a2.data_ptr(), _dt(a2), out.data_ptr(), _dt(out), M, K, N,
+                                         a2.stride(0), out.stride(0), epi, op, dptr, workspace.data_ptr(), workspace.numel(),
+                                         _stream_ptr()))
+    return out
+
+
 def matmul_q8_i8(a: torch.Tensor, w_blocks: torch.Tensor, N: int, K: int, out_dtype: torch.dtype | None = None,
                  out: torch.Tensor | None = None, unary: str | None = None, binary: str | None = None,
                  d: torch.Tensor | None = None, workspace: torch.Tensor | None = None) -> torch.Tensor:

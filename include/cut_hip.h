@@ -195,6 +195,21 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
                           uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D,
                           int variant, void *workspace, size_t workspace_bytes, void *stream);
 
+/* Prefill matmul on weights that are kept dequantized: W16 = fp16 [N][K], written once per tensor by
+ * cuthip_dequant(fmt, blocks, W16, CUTHIP_F16, N, K, K, stream) (bit-exact against the reference's CPU dequant +
+ * f32ToF16, gguf_reader.cpp:515-850, llama.cpp:445-482, 805-811).  The reference's runner does the same for its
+ * float path (it uploads dequantized fp16 weights, llama.cpp:800-815); here the GGUF blocks stay resident for the
+ * decode GEMV, which is bound by bytes, and the fp16 copy (2 bytes per weight: 16 GB for an 8B model of the 288 GB)
+ * serves prefill, which is bound by the matrix core, so no prefill call pays for a dequantization.
+ * C[M,N] = A[M,K] . W16^T with fp32 accumulation; the GEMM is hipBLASLt's where that library is present and no
+ * epilogue is fused, else this library's dense fp16 MFMA kernel.  K a multiple of 128; W16 256-byte aligned;
+ * workspace: device, 256-byte aligned, cuthip_matmul_dense_f16_workspace_bytes bytes (converted activations when A is
+ * fp32, split-K partial products, GEMM scratch).  Epilogues: none, unary, binary as in cuthip_matmul_gguf. */
+size_t cuthip_matmul_dense_f16_workspace_bytes(uint32_t M, uint32_t K, uint32_t N, int a_dtype);
+int cuthip_matmul_dense_f16(const void *W16, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M, uint32_t K, uint32_t N,
+                            uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D, void *workspace,
+                            size_t workspace_bytes, void *stream);
+
 /* Fields of an RMSNorm carried across batch-1 matmuls (cuthip_matmul_gguf_carry). */
 typedef struct {
   const float *sumsq_parts;      /* consumer: device [ceil(K/8)], partial sums of squares of the un-normalised activations */

@@ -353,3 +353,43 @@ def test_tuning_rules_select_the_variant(ops, tmp_path):
     assert not ops.enable_tuning(str(tmp_path / "missing.json"))
     assert ops.enable_tuning()          # the committed file loads
     ops.disable_tuning()
+
+
+# ---- prefill on resident dequantized weights (cuthip_matmul_dense_f16) ---------------------------------------------
+
+@pytest.mark.parametrize("name", list(oracle.FORMATS))
+@pytest.mark.parametrize("M,N,K", [(3, 136, 256), (300, 520, 1024), (1030, 264, 512)])
+def test_dense_f16_resident_weights(ops, name, M, N, K):
+    fmt = oracle.FORMATS[name]
+    W = quantized_weights(fmt, N, K, seed=71)
+    w16 = ops.dequantize(torch.from_numpy(W).cuda(), fmt, N, K, torch.float16)
+    # the resident copy is the reference's fp16 weight tensor bit for bit
+    assert np.array_equal(w16.cpu().numpy().reshape(-1).view(np.uint16), oracle.dequant_f16(fmt, W, N * K))
+    A = gauss_acts((M, K), seed=72, dtype=np.float16)
+    want = oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)
+    got = ops.matmul_dense_f16(torch.from_numpy(A).cuda(), w16, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    got = got.cpu().numpy()
+    assert normwise_rel_err(got, want) < (TOL_GEMM if M * N >= 1024 else TOL)
+    # same weights and accumulation as the two-pass path of cuthip_matmul_gguf_ws
+    two_pass = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=4)
+    assert normwise_rel_err(got, two_pass) < 1e-5
+    # fp32 activations and a fused epilogue (the hand-written GEMM)
+    A32 = gauss_acts((M, K), seed=73)
+    D = gauss_acts((M, N), seed=74)
+    add = ops.matmul_dense_f16(torch.from_numpy(A32).cuda(), w16, binary="add", d=torch.from_numpy(D).cuda())
+    torch.cuda.synchronize()
+    want32 = oracle.matmul_gguf(fmt, W, A32, N, f64=True)
+    assert normwise_rel_err(add.cpu().numpy() - D, want32) < 1e-3
+
+
+def test_dense_f16_argument_errors(ops):
+    from cut_amd import lib
+    w16 = torch.zeros((64, 200), dtype=torch.float16, device="cuda")
+    a = torch.zeros((4, 200), dtype=torch.float16, device="cuda")
+    with pytest.raises(lib.CutHipError, match="multiple of 128"):
+        ops.matmul_dense_f16(a, w16)
+    w16 = torch.zeros((64, 256), dtype=torch.float16, device="cuda")
+    a = torch.zeros((4, 256), dtype=torch.float16, device="cuda")
+    with pytest.raises(lib.CutHipError, match="workspace"):
+        ops.matmul_dense_f16(a, w16, workspace=torch.empty(256, dtype=torch.uint8, device="cuda"))
