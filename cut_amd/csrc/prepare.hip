@@ -12,9 +12,11 @@
 //
 // All of it is byte shuffling bound by HBM.  A workgroup copies the block runs
 // of 128 weight rows into LDS with coalesced 2-byte loads (GGUF blocks are only
-// 2-byte aligned), then every thread gathers the bytes of 4 (int8) or 8
-// (nibble) neighbouring rows for one k from LDS and writes one dword, so the
-// transposed rows are written in runs of 128 (64) bytes.
+// 2-byte aligned; the LDS image pads every block so that its quants are dword
+// aligned), then every thread reads one dword (four consecutive k) of 4 (int8)
+// or 8 (nibble) neighbouring rows, transposes the 4 x 4 bytes with v_perm_b32
+// and writes four dwords, so the transposed rows are written in runs of 128
+// (64) bytes.
 #include <cstdint>
 
 #include "common.hpp"
@@ -28,8 +30,8 @@ enum PrepMode { PREP_Q8_0 = 0, PREP_Q4_0 = 1, PREP_Q4_K_AFFINE = 2, PREP_NIBBLES
 
 // k extent of a tile and the bytes one weight row contributes to it
 template <int MODE> struct PrepGeom;
-template <> struct PrepGeom<PREP_Q8_0> { static constexpr int KT = 128, RUN = 4 * 34, PITCH = RUN; };
-template <> struct PrepGeom<PREP_Q4_0> { static constexpr int KT = 256, RUN = 8 * 18, PITCH = RUN; };
+template <> struct PrepGeom<PREP_Q8_0> { static constexpr int KT = 128, RUN = 4 * 34, PITCH = 4 * 36 + 4; };
+template <> struct PrepGeom<PREP_Q4_0> { static constexpr int KT = 256, RUN = 8 * 18, PITCH = 8 * 20 + 4; };
 template <> struct PrepGeom<PREP_Q4_K_AFFINE> { static constexpr int KT = 256, RUN = 144, PITCH = RUN; };
 template <> struct PrepGeom<PREP_NIBBLES> { static constexpr int KT = 256, RUN = 128, PITCH = RUN + 4; };
 
@@ -41,14 +43,17 @@ struct PrepParams {
   uint32_t src_row_bytes;
 };
 
-template <int MODE> __device__ inline uint32_t prep_nibble(const uint8_t *r, uint32_t k) {
-  if (MODE == PREP_Q4_K_AFFINE) {   // piece g = k / 64: low nibbles are its first 32 elements, high nibbles the rest
-    const uint32_t b = r[16 + 32 * (k >> 6) + (k & 31)];
-    return (k & 32) ? b >> 4 : b & 15u;
-  }
-  const uint32_t blk = k >> 5, e = k & 31;   // GGML Q4_0: low nibble of byte j is element j, high nibble element j + 16
-  const uint32_t b = MODE == PREP_Q4_0 ? r[blk * 18 + 2 + (e & 15)] : r[blk * 16 + (e & 15)];
-  return (e & 16) ? b >> 4 : b & 15u;
+// Where the quant byte of element k (a multiple of 4) of a row sits in its LDS image, and the shift that brings its
+// nibble down.  Q4_K: piece g = k / 64, low nibbles are its first 32 elements, high nibbles the rest.  GGML Q4_0 order
+// (also the packed tensor of the separated reader): low nibble of byte j of a block is element j, high nibble element
+// j + 16.  The Q4_0 image keeps each block at 20 bytes ([d][2 bytes unused][qs:16]) so that the quants are dword aligned.
+template <int MODE> __device__ inline uint32_t prep_quant_offset(uint32_t k) {
+  if (MODE == PREP_Q4_K_AFFINE) return 16 + 32 * (k >> 6) + (k & 31);
+  if (MODE == PREP_Q4_0) return (k >> 5) * 20 + 4 + (k & 15);
+  return (k >> 5) * 16 + (k & 15);
+}
+template <int MODE> __device__ inline uint32_t prep_quant_shift(uint32_t k) {
+  return MODE == PREP_Q4_K_AFFINE ? ((k & 32) ? 4u : 0u) : ((k & 16) ? 4u : 0u);
 }
 
 template <int MODE> __global__ void __launch_bounds__(kPrepThreads) prepare_sep_kernel(PrepParams p) {
@@ -63,54 +68,81 @@ template <int MODE> __global__ void __launch_bounds__(kPrepThreads) prepare_sep_
     const uint32_t row = i / W, w = i - row * W, n = n0 + row;
     uint16_t v = 0;
     if (n < p.N && 2 * w < valid) v = (uint16_t)ld_u16(p.src + (size_t)n * p.src_row_bytes + run_off + 2 * w);
-    *reinterpret_cast<uint16_t *>(raw + row * G::PITCH + 2 * w) = v;
+    uint32_t dst = 2 * w;
+    if (MODE == PREP_Q4_0) dst = (w / 9) * 20 + ((w % 9) ? 2 * (w % 9) + 2 : 0);   // scale at 0, quants from byte 4
+    if (MODE == PREP_Q8_0) dst = (w / 17) * 36 + ((w % 17) ? 2 * (w % 17) + 2 : 0);  // [d][2 bytes unused][q:32]
+    *reinterpret_cast<uint16_t *>(raw + row * G::PITCH + dst) = v;
   }
   __syncthreads();
   const uint32_t kt = min((uint32_t)G::KT, p.K - k0);
 
   if constexpr (MODE == PREP_Q8_0) {
-    // item = (k, 4 rows): one dword of B[k, n .. n+3]
+    // item = (4 consecutive k, 4 rows): one dword of LDS per row (the image keeps every block at 36 bytes so that the
+    // quants are dword aligned), a 4 x 4 byte transpose, four dwords B[k + i, n .. n+3]
     const bool words = (p.strideB & 3u) == 0;
-    for (uint32_t i = tid; i < (uint32_t)G::KT * (kPrepRows / 4); i += kPrepThreads) {
-      const uint32_t k = i / (kPrepRows / 4), r4 = (i % (kPrepRows / 4)) * 4, n = n0 + r4;
+    for (uint32_t i = tid; i < (uint32_t)(G::KT / 4) * (kPrepRows / 4); i += kPrepThreads) {
+      const uint32_t k = (i / (kPrepRows / 4)) * 4, r4 = (i % (kPrepRows / 4)) * 4, n = n0 + r4;
       if (k >= kt || n >= p.N) continue;
-      const uint32_t off = (k >> 5) * 34 + 2 + (k & 31);
-      uint32_t b[4];
+      const uint32_t off = (k >> 5) * 36 + 4 + (k & 31);
+      uint32_t pr[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) b[j] = raw[(r4 + j) * G::PITCH + off];
-      uint8_t *dst = p.B + (size_t)(k0 + k) * p.strideB + n;
-      if (words && n + 3 < p.N) {
-        *reinterpret_cast<uint32_t *>(dst) = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
-      } else {
-        for (int j = 0; j < 4 && n + j < p.N; ++j) dst[j] = (uint8_t)b[j];
+      for (int j = 0; j < 4; ++j) pr[j] = *reinterpret_cast<const uint32_t *>(raw + (r4 + j) * G::PITCH + off);
+      const uint32_t t0 = __builtin_amdgcn_perm(pr[1], pr[0], 0x05010400u), t1 = __builtin_amdgcn_perm(pr[3], pr[2], 0x05010400u);
+      const uint32_t t2 = __builtin_amdgcn_perm(pr[1], pr[0], 0x07030602u), t3 = __builtin_amdgcn_perm(pr[3], pr[2], 0x07030602u);
+      const uint32_t out[4] = {__builtin_amdgcn_perm(t1, t0, 0x05040100u), __builtin_amdgcn_perm(t1, t0, 0x07060302u),
+                               __builtin_amdgcn_perm(t3, t2, 0x05040100u), __builtin_amdgcn_perm(t3, t2, 0x07060302u)};
+#pragma unroll
+      for (uint32_t e = 0; e < 4; ++e) {
+        if (k + e >= kt) break;
+        uint8_t *dst = p.B + (size_t)(k0 + k + e) * p.strideB + n;
+        if (words && n + 3 < p.N) {
+          *reinterpret_cast<uint32_t *>(dst) = out[e];
+        } else {
+          for (uint32_t j = 0; j < 4 && n + j < p.N; ++j) dst[j] = (uint8_t)(out[e] >> (8 * j));
+        }
       }
     }
     for (uint32_t i = tid; i < (G::KT / 32) * kPrepRows; i += kPrepThreads) {
       const uint32_t blk = i / kPrepRows, row = i % kPrepRows, n = n0 + row;
       if (n < p.N && blk * 32 < kt)
-        p.S[(size_t)(k0 / 32 + blk) * p.scaleStride + n] = *reinterpret_cast<const uint16_t *>(raw + row * G::PITCH + blk * 34);
+        p.S[(size_t)(k0 / 32 + blk) * p.scaleStride + n] = *reinterpret_cast<const uint16_t *>(raw + row * G::PITCH + blk * 36);
     }
   } else {
-    // item = (k, 8 rows): four bytes of B[k, n/2 .. n/2+3], even row in the low nibble
+    // item = (4 consecutive k, 8 rows): one dword of LDS per row holds the four quants (k .. k+3 share a nibble half
+    // and four neighbouring bytes), row pairs are merged into bytes (even row in the low nibble) and a 4 x 4 byte
+    // transpose (v_perm_b32) turns [row pair][k] into the four output dwords B[k + i, n/2 .. n/2+3]
     const bool words = (p.strideB & 3u) == 0;
-    for (uint32_t i = tid; i < (uint32_t)G::KT * (kPrepRows / 8); i += kPrepThreads) {
-      const uint32_t k = i / (kPrepRows / 8), r8 = (i % (kPrepRows / 8)) * 8, n = n0 + r8;
+    for (uint32_t i = tid; i < (uint32_t)(G::KT / 4) * (kPrepRows / 8); i += kPrepThreads) {
+      const uint32_t k = (i / (kPrepRows / 8)) * 4, r8 = (i % (kPrepRows / 8)) * 8, n = n0 + r8;
       if (k >= kt || n >= p.N) continue;
-      uint32_t word = 0;
+      const uint32_t off = prep_quant_offset<MODE>(k), sh = prep_quant_shift<MODE>(k);
+      uint32_t pr[4];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) word |= prep_nibble<MODE>(raw + (r8 + j) * G::PITCH, k) << (4 * j);   // rows past N are zero
-      uint8_t *dst = p.B + (size_t)(k0 + k) * p.strideB + n / 2;
-      if (words && n + 7 < p.N) {
-        *reinterpret_cast<uint32_t *>(dst) = word;
-      } else {
-        for (uint32_t j = 0; j < 4 && n + 2 * j < p.N; ++j) dst[j] = (uint8_t)(word >> (8 * j));
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = (*reinterpret_cast<const uint32_t *>(raw + (r8 + 2 * j) * G::PITCH + off) >> sh) & 0x0F0F0F0Fu;
+        const uint32_t hi = (*reinterpret_cast<const uint32_t *>(raw + (r8 + 2 * j + 1) * G::PITCH + off) >> sh) & 0x0F0F0F0Fu;
+        pr[j] = lo | (hi << 4);   // byte i: rows (r8 + 2j, r8 + 2j + 1) at k + i; rows past N are zero
+      }
+      const uint32_t t0 = __builtin_amdgcn_perm(pr[1], pr[0], 0x05010400u), t1 = __builtin_amdgcn_perm(pr[3], pr[2], 0x05010400u);
+      const uint32_t t2 = __builtin_amdgcn_perm(pr[1], pr[0], 0x07030602u), t3 = __builtin_amdgcn_perm(pr[3], pr[2], 0x07030602u);
+      const uint32_t out[4] = {__builtin_amdgcn_perm(t1, t0, 0x05040100u), __builtin_amdgcn_perm(t1, t0, 0x07060302u),
+                               __builtin_amdgcn_perm(t3, t2, 0x05040100u), __builtin_amdgcn_perm(t3, t2, 0x07060302u)};
+#pragma unroll
+      for (uint32_t e = 0; e < 4; ++e) {
+        if (k + e >= kt) break;
+        uint8_t *dst = p.B + (size_t)(k0 + k + e) * p.strideB + n / 2;
+        if (words && n + 7 < p.N) {
+          *reinterpret_cast<uint32_t *>(dst) = out[e];
+        } else {
+          for (uint32_t j = 0; j < 4 && n + 2 * j < p.N; ++j) dst[j] = (uint8_t)(out[e] >> (8 * j));
+        }
       }
     }
     if constexpr (MODE == PREP_Q4_0) {
       for (uint32_t i = tid; i < (G::KT / 32) * kPrepRows; i += kPrepThreads) {
         const uint32_t blk = i / kPrepRows, row = i % kPrepRows, n = n0 + row;
         if (n < p.N && blk * 32 < kt)
-          p.S[(size_t)(k0 / 32 + blk) * p.scaleStride + n] = *reinterpret_cast<const uint16_t *>(raw + row * G::PITCH + blk * 18);
+          p.S[(size_t)(k0 / 32 + blk) * p.scaleStride + n] = *reinterpret_cast<const uint16_t *>(raw + row * G::PITCH + blk * 20);
       }
     }
     if constexpr (MODE == PREP_Q4_K_AFFINE) {
