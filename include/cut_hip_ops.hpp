@@ -248,6 +248,46 @@ private:
   Tensor output_;
 };
 
+// ---- MatMulDenseF16OpNode ----------------------------------------------------------------
+// Prefill matmul on weights kept dequantized: w16 is the fp16 [N, K] output of a DequantOpNode (DataType::Float16,
+// row stride K); the float-path matmul of the reference's runner on its fp16 weight tensors (llama.cpp:800-815).
+// The node owns its output and its scratch.
+class MatMulDenseF16OpNode {
+public:
+  MatMulDenseF16OpNode(const Tensor &a, const Tensor &w16, DataType outDtype = DataType::Float16)
+      : a_(a), w_(w16), outDtype_(outDtype) {
+    if (a.shape.empty() || a.shape.size() > 2) throw std::runtime_error("MatMulDenseF16OpNode: A must have rank 1 or 2");
+    if (w16.shape.size() != 2 || w16.dtype != DataType::Float16 || w16.stride() != w16.shape[1])
+      throw std::runtime_error("MatMulDenseF16OpNode: weights must be a dense Float16 [N, K] tensor");
+    M_ = a.shape.size() == 2 ? a.shape[0] : 1u;
+    K_ = a.shape.back();
+    N_ = w16.shape[0];
+    if (M_ == 0 || K_ == 0 || N_ == 0 || w16.shape[1] != K_) throw std::runtime_error("MatMulDenseF16OpNode: A cols must match weight cols");
+    if (K_ % 128 != 0) throw std::runtime_error("MatMulDenseF16OpNode: K must be a multiple of 128");
+    if (!w16.buffer || w16.buffer->bytes() < (size_t)N_ * K_ * 2)
+      throw std::runtime_error("MatMulDenseF16OpNode: weight tensor holds fewer bytes than N x K halfs");
+    storage_ = DeviceBuffer((size_t)M_ * N_ * dtypeBytes(outDtype_));
+    scratch_ = DeviceBuffer(cuthip_matmul_dense_f16_workspace_bytes(M_, K_, N_, (int)a_.dtype));
+    output_ = Tensor{&storage_, a.shape.size() == 2 ? std::vector<uint32_t>{M_, N_} : std::vector<uint32_t>{N_}, outDtype_, N_};
+  }
+  MatMulDenseF16OpNode(MatMulDenseF16OpNode &&) = delete;
+  std::vector<uint32_t> outputShape() const { return output_.shape; }
+  std::string displayName() const { return "MatMulDenseF16"; }
+  const Tensor &output() const { return output_; }
+  void dispatch(void *stream = nullptr) const {
+    check(cuthip_matmul_dense_f16(w_.data(), a_.data(), (int)a_.dtype, output_.data(), (int)outDtype_, M_, K_, N_, a_.stride(), N_,
+                                  CUTHIP_EPI_NONE, 0, nullptr, scratch_.data(), scratch_.bytes(), stream),
+          "cuthip_matmul_dense_f16");
+  }
+
+private:
+  Tensor a_, w_;
+  uint32_t M_ = 0, K_ = 0, N_ = 0;
+  DataType outDtype_;
+  DeviceBuffer storage_, scratch_;
+  Tensor output_;
+};
+
 // ---- TransposeQ4NibbleOpNode --------------------------------------------------------------
 // operators/impl/q4transpose/TransposeQ4NibbleOp.cpp:7-23: packed GGML-order nibbles [N, K/2] ->
 // [K, N/2] with the even source row in the low nibble; same checks, messages and padded strides.

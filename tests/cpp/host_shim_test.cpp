@@ -65,6 +65,13 @@ static void test_validation() {
   EXPECT(throws([&] { TransposeQ4NibbleOpNode n(raw, 3, 64); }));             // odd N (TransposeQ4NibbleOp.cpp:13-15)
   EXPECT(throws([&] { TransposeQ4NibbleOpNode n(raw, 4, 48); }));             // K not a multiple of 32
   EXPECT(throws([&] { TransposeQ4NibbleOpNode n(raw, 4, 64); }));             // input too small
+  Tensor w16bad{&none, {8, 200}, DataType::Float16, 0};
+  Tensor a200{&none, {2, 200}, DataType::Float16, 0};
+  EXPECT(throws([&] { MatMulDenseF16OpNode n(a200, w16bad); }));                // K not a multiple of 128
+  Tensor w16{&none, {8, 256}, DataType::Float16, 0};
+  EXPECT(throws([&] { MatMulDenseF16OpNode n(a200, w16); }));                   // A cols != weight cols
+  Tensor a256{&none, {2, 256}, DataType::Float16, 0};
+  EXPECT(throws([&] { MatMulDenseF16OpNode n(a256, w16); }));                   // weights too small
   SeparatedWeights sw;
   EXPECT(throws([&] { prepareSeparated(sw, raw, GgufFormat::Q6_K, 4, 256); }));
   EXPECT(throws([&] { prepareSeparated(sw, raw, GgufFormat::Q4_0, 3, 64); }));
@@ -186,6 +193,17 @@ static void test_gpu() {
     std::vector<double> c4d(c4.begin(), c4.end());
     EXPECT(normwise(c, c4d) < 1e-5);
     EXPECT(normwise(c4, ref) < 1e-3);
+    // the same product on weights kept dequantized in fp16 (DequantOpNode with a Float16 output feeds the node)
+    if (K % 128 == 0 && ((K + 3) & ~3u) == K) {
+      DequantOpNode dq16(wt, f, N, K, DataType::Float16);
+      dq16.dispatch();
+      MatMulDenseF16OpNode md(at, dq16.output(), DataType::Float32);
+      md.dispatch();
+      std::vector<float> c16((size_t)M * N);
+      md.output().buffer->download(c16.data(), c16.size() * 4);
+      EXPECT(normwise(c16, ref) < 1e-3);
+      EXPECT(normwise(c16, c4d) < 1e-5);
+    }
   }
   // an explicit variant that cannot take the shape is an error, not a silent fallback
   {
