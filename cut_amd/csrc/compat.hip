@@ -185,6 +185,123 @@ template <bool Q4, int MT> static int launch_sep(SepParams p, uint32_t mcount, f
   return CUTHIP_OK;
 }
 
+// ---- prefill on the separated layout: dequantize to fp16 [N][K], then the dense GEMM ------------------------------
+// The GEMV above streams the weights once per 4 rows of A; from kSepDenseRows rows on the tensors are turned into the
+// fp16 [N][K] operand of the dense GEMM first (one launch: value = float(q) * scale (+ min), rounded to nearest even,
+// 64 x 64 tiles transposed through LDS so that both the reads along n and the writes along k are contiguous) and the
+// product goes through the same GEMM as cuthip_matmul_dense_f16 (hipBLASLt without an epilogue, else the hand-written one).
+constexpr uint32_t kSepDenseRows = 32;
+
+bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a_f16, const void *A);
+size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16);
+bool blaslt_available();
+int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K,
+                      uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream,
+                      int use_blaslt);
+
+static size_t sep_w16_bytes(uint32_t K, uint32_t N) { return ((size_t)N * K * 2 + 255) & ~(size_t)255; }
+static bool sep_dense_applies(uint32_t M, uint32_t K, uint32_t N) {
+  return M >= kSepDenseRows && K % 128 == 0 && (uint64_t)N * K * 2 < (1ull << 32) && (uint64_t)M * K * 2 < (1ull << 32);
+}
+
+template <bool Q4>
+__global__ void __launch_bounds__(256) sep_dequant_kernel(const uint8_t *B, const uint16_t *S, half_t *W16, uint32_t K, uint32_t N,
+                                                          uint32_t strideB, uint32_t scaleStride, int affine) {
+  __shared__ half_t tile[64][64 + 2];   // [n][k], rows 33 dwords apart
+  const uint32_t tid = threadIdx.x, n0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
+  {
+    const uint32_t k = k0 + tid / 4, nseg = (tid & 3) * 16;   // 16 columns of one k-row
+    if (k < K) {
+      const uint32_t blk = k / 32, blocksK = K / 32;
+      uint32_t q[4] = {0, 0, 0, 0};
+      const uint32_t n = n0 + nseg;
+      // whole, aligned segments take one vector load for the values and two for the scales
+      const bool fast = n + 16 <= N && (scaleStride & 7u) == 0 && ((uintptr_t)S & 15u) == 0 &&
+                        (strideB & (Q4 ? 7u : 15u)) == 0 && ((uintptr_t)B & (Q4 ? 7u : 15u)) == 0;
+      uint32_t sraw[8], mraw[8];
+      if (fast) {
+        const u32x4 s0 = *reinterpret_cast<const u32x4 *>(S + (size_t)blk * scaleStride + n);
+        const u32x4 s1 = *reinterpret_cast<const u32x4 *>(S + (size_t)blk * scaleStride + n + 8);
+        sraw[0] = s0.x; sraw[1] = s0.y; sraw[2] = s0.z; sraw[3] = s0.w; sraw[4] = s1.x; sraw[5] = s1.y; sraw[6] = s1.z; sraw[7] = s1.w;
+        if (Q4 && affine) {
+          const u32x4 m0 = *reinterpret_cast<const u32x4 *>(S + (size_t)(blocksK + blk) * scaleStride + n);
+          const u32x4 m1 = *reinterpret_cast<const u32x4 *>(S + (size_t)(blocksK + blk) * scaleStride + n + 8);
+          mraw[0] = m0.x; mraw[1] = m0.y; mraw[2] = m0.z; mraw[3] = m0.w; mraw[4] = m1.x; mraw[5] = m1.y; mraw[6] = m1.z; mraw[7] = m1.w;
+        }
+        if (Q4) {
+          const u32x2 b = *reinterpret_cast<const u32x2 *>(B + (size_t)k * strideB + n / 2);
+          const uint32_t w[2] = {b.x, b.y};
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const uint32_t byte = (w[j / 4] >> (8 * (j & 3))) & 0xFFu;
+            q[j / 2] |= ((byte & 15u) | ((byte >> 4) << 8)) << (16 * (j & 1));
+          }
+        } else {
+          const u32x4 b = *reinterpret_cast<const u32x4 *>(B + (size_t)k * strideB + n);
+          q[0] = b.x; q[1] = b.y; q[2] = b.z; q[3] = b.w;
+        }
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const float sc = f16bits_to_f32((sraw[j / 2] >> (16 * (j & 1))) & 0xFFFFu);
+          const uint32_t byte = (q[j / 4] >> (8 * (j & 3))) & 0xFFu;
+          float v;
+          if (Q4) {
+            v = (float)((int)byte - 8) * sc;
+            if (affine) v += f16bits_to_f32((mraw[j / 2] >> (16 * (j & 1))) & 0xFFFFu);
+          } else {
+            v = (float)(int)(int8_t)byte * sc;
+          }
+          tile[nseg + j][tid / 4] = (half_t)v;
+        }
+      } else {
+      if (Q4) {   // 8 bytes = 16 nibbles, even column in the low nibble
+        for (uint32_t j = 0; j < 8 && n + 2 * j < N; ++j) {
+          const uint32_t b = B[(size_t)k * strideB + n / 2 + j];
+          q[j / 2] |= ((b & 15u) | ((b >> 4) << 8)) << (16 * (j & 1));   // two columns per byte -> two bytes
+        }
+      } else {
+        for (uint32_t j = 0; j < 16 && n + j < N; ++j) q[j / 4] |= (uint32_t)B[(size_t)k * strideB + n + j] << (8 * (j & 3));
+      }
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        float v = 0.0f;
+        if (n + j < N) {
+          const float sc = f16bits_to_f32(S[(size_t)blk * scaleStride + n + j]);
+          const uint32_t byte = (q[j / 4] >> (8 * (j & 3))) & 0xFFu;
+          if (Q4) {
+            v = (float)((int)byte - 8) * sc;
+            if (affine) v += f16bits_to_f32(S[(size_t)(blocksK + blk) * scaleStride + n + j]);
+          } else {
+            v = (float)(int)(int8_t)byte * sc;
+          }
+        }
+        tile[nseg + j][tid / 4] = (half_t)v;
+      }
+      }
+    }
+  }
+  __syncthreads();
+  {
+    const uint32_t n = n0 + tid / 4, kseg = (tid & 3) * 16;   // 16 consecutive k of one weight row
+    if (n < N) {
+      half_t *dst = W16 + (size_t)n * K + k0 + kseg;
+      if (k0 + kseg + 16 <= K && (K & 7u) == 0) {   // W16 is 256-byte aligned and K a multiple of 8: 16-byte stores
+        uint32_t w[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const uint16_t lo = __builtin_bit_cast(uint16_t, tile[tid / 4][kseg + 2 * j]);
+          const uint16_t hi = __builtin_bit_cast(uint16_t, tile[tid / 4][kseg + 2 * j + 1]);
+          w[j] = (uint32_t)lo | ((uint32_t)hi << 16);
+        }
+        *reinterpret_cast<u32x4 *>(dst) = u32x4{w[0], w[1], w[2], w[3]};
+        *reinterpret_cast<u32x4 *>(dst + 8) = u32x4{w[4], w[5], w[6], w[7]};
+      } else {
+        for (uint32_t j = 0; j < 16 && k0 + kseg + j < K; ++j) dst[j] = tile[tid / 4][kseg + j];
+      }
+    }
+  }
+}
+
 static int matmul_sep(bool q4, const float *A, const void *B, const void *S, const float *D, float *C, uint32_t M, uint32_t K,
                       uint32_t N, uint32_t strideA, uint32_t strideB, uint32_t strideC, uint32_t scaleStride, int epilogue,
                       int epilogue_op, int affine, void *workspace, size_t workspace_bytes, hipStream_t stream) {
@@ -198,6 +315,22 @@ static int matmul_sep(bool q4, const float *A, const void *B, const void *S, con
   if (epilogue < CUTHIP_EPI_NONE || epilogue > CUTHIP_EPI_BINARY || (epilogue == CUTHIP_EPI_BINARY && !D)) {
     set_error("%s: bad epilogue %d (a binary epilogue needs D)", who, epilogue);
     return CUTHIP_ERR_INVALID;
+  }
+  if (sep_dense_applies(M, K, N) && dense_gemm_fits(M, K, N, strideA, 0, A) && workspace && (uintptr_t)workspace % 256 == 0 &&
+      workspace_bytes >= sep_w16_bytes(K, N) + dense_f16_workspace(M, K, N, 0)) {
+    half_t *w16 = reinterpret_cast<half_t *>(workspace);
+    dim3 grid((N + 63) / 64, (K + 63) / 64);
+    if (q4)
+      hipLaunchKernelGGL(sep_dequant_kernel<true>, grid, dim3(256), 0, stream, reinterpret_cast<const uint8_t *>(B),
+                         reinterpret_cast<const uint16_t *>(S), w16, K, N, strideB, scaleStride, affine);
+    else
+      hipLaunchKernelGGL(sep_dequant_kernel<false>, grid, dim3(256), 0, stream, reinterpret_cast<const uint8_t *>(B),
+                         reinterpret_cast<const uint16_t *>(S), w16, K, N, strideB, scaleStride, 0);
+    if (int rc = check_hip(hipGetLastError(), "separated-layout dequant launch")) return rc;
+    Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
+    return launch_dense_gemm(-1, w16, A, 0, C, 0, M, K, N, strideA, strideC, epi,
+                             reinterpret_cast<uint8_t *>(workspace) + sep_w16_bytes(K, N), stream,
+                             (epilogue == CUTHIP_EPI_NONE && blaslt_available()) ? 2 : 0);
   }
   SepParams p;
   p.A = A;
@@ -236,6 +369,7 @@ using namespace cuthip;
 extern "C" {
 
 size_t cuthip_matmul_sep_workspace_bytes(uint32_t M, uint32_t K, uint32_t N) {
+  if (sep_dense_applies(M, K, N)) return sep_w16_bytes(K, N) + dense_f16_workspace(M, K, N, 0);   // prefill route
   size_t nsplit = (K + kSepWaves * kSepKC - 1) / (kSepWaves * kSepKC);
   return nsplit > 1 ? nsplit * M * N * sizeof(float) : 0;
 }

@@ -293,9 +293,12 @@ int cuthip_matmul_gguf_pro(int fmt, const void *W, const void *A, int a_dtype, v
  * A [M, strideA], C and D [M, strideC] are fp32; K must be a multiple of 32.
  * epilogue / epilogue_op / D as in cuthip_matmul_gguf (MatMulFusion).
  * workspace: device scratch of cuthip_matmul_sep_workspace_bytes(M, K, N)
- * bytes (split-K partial sums; may be NULL when that is 0).  Streams the
- * weights once per 4 rows of A: meant for decode and small batches; prefill
- * belongs on cuthip_matmul_gguf with the native blocks. */
+ * bytes, 256-byte aligned (may be NULL when that is 0).  Below 32 rows of A
+ * (or when K is not a multiple of 128) the weights are streamed once per 4 rows
+ * and the workspace holds split-K partial sums; from 32 rows on the tensors are
+ * first dequantized to fp16 [N][K] in the workspace (one launch) and multiplied
+ * by the dense GEMM of cuthip_matmul_dense_f16 (fp16 operands, fp32 accumulate:
+ * within 1e-3 of the fp32 loop). */
 size_t cuthip_matmul_sep_workspace_bytes(uint32_t M, uint32_t K, uint32_t N);
 int cuthip_matmul_q8_sep(const float *A, const int8_t *B, const uint16_t *scales, const float *D, float *C, uint32_t M,
                          uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideB, uint32_t strideC, uint32_t scaleStride,

@@ -106,3 +106,50 @@ def test_fused_epilogues_and_errors(ops):
     np.testing.assert_array_equal(got.cpu().numpy(), np.maximum(base, 0))
     with pytest.raises(lib.CutHipError):
         ops.matmul_sep(dev(A[:, :100].copy()), dev(B[:100]), dev(S.astype(np.float16)[:3]), N)   # K not a multiple of 32
+
+
+# ---- prefill route: from 32 rows on (K a multiple of 128) the tensors are dequantized to fp16 [N][K] and multiplied by
+# the dense GEMM; fp16 weights and activations, fp32 accumulation: the tolerance of the native prefill path -------------
+
+@pytest.mark.parametrize("M,K,N", [(32, 128, 64), (70, 256, 200), (300, 1024, 520), (1030, 512, 264)])
+def test_prefill_route_q8(ops, M, K, N):
+    rng = np.random.default_rng(M + K + N)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = rng.integers(-127, 128, (K, N)).astype(np.int8)
+    S = rng.uniform(0.001, 0.02, (K // 32, N)).astype(np.float16).astype(np.float32)
+    want = oracle.matmul_sep_q8(A, B, S, f64=True)
+    assert normwise_rel_err(run(ops, A, B, S, N), want) < 1e-3
+    D = rng.standard_normal((M, N)).astype(np.float32)
+    got = ops.matmul_sep(dev(A), dev(B), dev(S.astype(np.float16)), N, binary="add", d=dev(D))   # fused epilogue: own GEMM
+    torch.cuda.synchronize()
+    assert normwise_rel_err(got.cpu().numpy() - D, want) < 1e-3
+
+
+@pytest.mark.parametrize("affine", [False, True])
+@pytest.mark.parametrize("M,K,N", [(32, 128, 66), (300, 1024, 520)])
+def test_prefill_route_q4(ops, affine, M, K, N):
+    rng = np.random.default_rng(M + K + N + affine)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    Bp = rng.integers(0, 256, (K, N // 2)).astype(np.uint8)
+    S = rng.uniform(0.001, 0.02, ((2 if affine else 1) * (K // 32), N)).astype(np.float16).astype(np.float32)
+    if affine:
+        S[K // 32:] = rng.uniform(-0.1, 0.1, (K // 32, N)).astype(np.float16).astype(np.float32)
+    want = oracle.matmul_sep_q4(A[:8], Bp, S, affine=affine).astype(np.float64)   # the CPU loop on the first rows
+    got = run(ops, A, Bp, S, N, q4=True, affine=affine)
+    assert normwise_rel_err(got[:8], want) < 1e-3
+    # rows are independent: the GEMV route on a few rows gives what the prefill route gave for them
+    few = run(ops, A[8:12], Bp, S, N, q4=True, affine=affine)
+    assert normwise_rel_err(got[8:12], few) < 1e-3
+
+
+def test_prefill_route_after_device_preparation(ops):
+    """GGUF Q8_0 blocks -> cuthip_prepare_sep -> separated matmul at prefill size, against the native-block path."""
+    from helpers import quantized_weights
+    M, K, N = 256, 512, 384
+    blocks = quantized_weights(oracle.Q8_0, N, K, seed=9)
+    B, S = ops.prepare_sep(dev(blocks), "Q8_0", N, K)
+    A = np.random.default_rng(10).standard_normal((M, K)).astype(np.float32)
+    got = ops.matmul_sep(dev(A), B, S, N)
+    torch.cuda.synchronize()
+    want = oracle.matmul_gguf(oracle.Q8_0, blocks, A, N, f64=True)
+    assert normwise_rel_err(got.cpu().numpy(), want) < 1e-3
