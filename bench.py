@@ -132,6 +132,17 @@ def bench_prepare(torch, ops, dev, reps=10):
         _, ev, _ = timed_graph(torch, prep, reps, 2)
         res[f"prepare_sep_{name}_14336x4096_GBps"] = round((w.numel() + B.numel() + S.numel() * 2) * reps / (ev * 1e-3) / 1e9, 1)
         del w, B, S
+    # the separated tensors at prefill size (fp32 in / out as the reference): dequantize to fp16 + dense GEMM
+    w = torch.from_numpy(make_q_weights("Q8_0", 1024, K, 5)).to(dev).repeat(N // 1024)
+    Bq, Sq = ops.prepare_sep(w, "Q8_0", N, K)
+    a = torch.randn((2048, K), dtype=torch.float32, device=dev)
+    c = torch.empty((2048, N), dtype=torch.float32, device=dev)
+
+    def sep(_s):
+        ops.matmul_sep(a, Bq, Sq, N, out=c)
+    _, ev, _ = timed_graph(torch, sep, 5, 2)
+    res["separated_q8_prefill_gemm_M2048_N14336_K4096_TFLOPs"] = round(2.0 * 2048 * N * K * 5 / (ev * 1e-3) / 1e12, 1)
+    del w, Bq, Sq, a, c
     x = torch.randn(N * K, dtype=torch.float32, device=dev) * 0.02
 
     def quant(_s):
