@@ -145,7 +145,20 @@ static cuthip::GemvParams gemv_params(int fmt, const void *W, const void *A, int
   return p;
 }
 
-constexpr uint32_t kPassesMaxRows = 40;   // up to here 8-row passes of the decode kernels beat one tiled GEMM launch
+constexpr uint32_t kPassesMaxRows = 40;   // up to here 8-row passes of the decode kernels can beat one tiled GEMM launch
+
+// Costs in microseconds fitted to a sweep over the weight shapes of an 8B model (HIP-graph replay, MI355X): an 8-row
+// pass of the decode kernels 6.5 + weight bytes / 4.3 MB (x 1.45 on rows of K >= 8192, x 1.5 for Q6_K), one launch of
+// the tiled GEMM on the blocks 62 + weight bytes / 7 MB (its cost is the decode of the whole matrix whatever M is; on
+// rows of K >= 8192 it has too few tiles and is never the better one).
+static double weight_bytes(int fmt, uint32_t K, uint32_t N) { return (double)N * K / cuthip::fmt_elems(fmt) * cuthip::fmt_bytes(fmt); }
+static double passes_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
+  return ((M + 7) / 8) * (6.5 + weight_bytes(fmt, K, N) / 4.3e6) * (K >= 8192 ? 1.45 : 1.0) * (fmt == CUTHIP_Q6_K ? 1.5 : 1.0);
+}
+static double single_launch_cost_us(int fmt, uint32_t K, uint32_t N) { return 62.0 + weight_bytes(fmt, K, N) / 7e6; }
+static bool passes_preferred(int fmt, uint32_t M, uint32_t K, uint32_t N) {
+  return M > 8 && M <= kPassesMaxRows && (K >= 8192 || passes_cost_us(fmt, M, K, N) <= single_launch_cost_us(fmt, K, N));
+}
 
 // Argument checks shared by the matmul entry points: 0 = go on, 1 = empty problem (success), < 0 = error.
 static int check_matmul_args(int fmt, const void *W, const void *A, int a_dtype, const void *C, int c_dtype, uint32_t M,
@@ -225,7 +238,7 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
   // 9-40 rows, automatic choice: passes of 8 rows through the decode kernels.  Measured on 14336 x 4096: 14 us per
   // pass, against 69-87 us for the 32-row skinny kernel and 73-80 us for one launch of the tiled GEMM, whose cost
   // is the decode of the whole weight matrix whatever M is.
-  if (variant == -1 && M > 8 && M <= kPassesMaxRows) {
+  if (variant == -1 && passes_preferred(fmt, M, K, N)) {
     const size_t asz = a_dtype == CUTHIP_F16 ? 2 : 4, csz = c_dtype == CUTHIP_F16 ? 2 : 4;
     for (uint32_t m0 = 0; m0 < M; m0 += 8) {
       const uint8_t *a = reinterpret_cast<const uint8_t *>(A) + (size_t)m0 * strideA * asz;
@@ -237,7 +250,7 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
     }
     return CUTHIP_OK;
   }
-  if (variant == 2 || (variant == -1 && M > 32)) {
+  if (variant == 2 || (variant == -1 && M > 8)) {   // 9..40 rows come here when one tiled launch beats the passes
     if ((uint64_t)N * row_bytes > 0xFFFFFFFFFFFFull) {
       set_error("cuthip_matmul_gguf: weight matrix too large");
       return CUTHIP_ERR_INVALID;
@@ -400,11 +413,11 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   if (variant == -1 && M > 8 && M < 384 && epilogue == CUTHIP_EPI_NONE && workspace && (uintptr_t)workspace % 256 == 0 &&
       dense_gemm_fits(M, K, N, strideA, a_f16, A) && workspace_bytes >= dense_gemm_workspace(M, K, N, a_f16) &&
       blaslt_available()) {
-    const double nk = (double)N * K, wb = nk / fmt_elems(fmt) * fmt_bytes(fmt);
+    const double nk = (double)N * K;
     const double t5 = 14.0 + nk * (nk <= 64e6 ? 0.65e-6 : 0.95e-6) + 2.0 * M * nk / 1.6e9;
     double other;
-    if (M <= kPassesMaxRows) other = ((M + 7) / 8) * (6.5 + wb / 4.3e6) * (K >= 8192 ? 1.45 : 1.0);
-    else other = K >= 8192 ? 65.0 + 0.19 * M : 62.0 + wb / 7e6;
+    if (passes_preferred(fmt, M, K, N)) other = passes_cost_us(fmt, M, K, N);
+    else other = K >= 8192 ? 65.0 + 0.19 * M : single_launch_cost_us(fmt, K, N);
     if (t5 < 0.95 * other) {
       const int rc = launch_dense_gemm(fmt, W, A, a_f16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC,
                                        Epilogue{CUTHIP_EPI_NONE, 0, nullptr}, workspace,
@@ -412,7 +425,7 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
       return rc;
     }
   }
-  if (variant == -1 && M > 8 && M <= kPassesMaxRows) {   // 8-row passes, each with the workspace (K split on long rows)
+  if (variant == -1 && passes_preferred(fmt, M, K, N)) {   // 8-row passes, each with the workspace (K split on long rows)
     const size_t asz = a_f16 ? 2 : 4, csz = c_dtype == CUTHIP_F16 ? 2 : 4;
     for (uint32_t m0 = 0; m0 < M; m0 += 8) {
       const uint8_t *a = reinterpret_cast<const uint8_t *>(A) + (size_t)m0 * strideA * asz;
