@@ -58,6 +58,9 @@ static const cuthip_variant_info_t *table(int op, int *count) {
 
 }  // namespace cuthip
 
+namespace cuthip {
+bool blaslt_available();
+}
 using namespace cuthip;
 
 extern "C" {
@@ -82,6 +85,9 @@ int cuthip_init(int device) {
     set_error("cuthip_init: device %d is %s; this library is built for gfx950 only", device, p.gcnArchName);
     return CUTHIP_ERR_NO_DEVICE;
   }
+  // open hipBLASLt (variant 5 of the prefill matmul) now: its handle must not be created inside a stream capture,
+  // where the first matmul of a caller may well run; absence of the library is not an error
+  (void)cuthip::blaslt_available();
   return CUTHIP_OK;
 }
 

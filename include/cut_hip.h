@@ -175,8 +175,10 @@ int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void 
  *            rows of A are not 16-byte aligned or the workspace is too small);
  *            5 = MatMulGgufDequantBlasLt: the same dequantization, then hipBLASLt's
  *            dense fp16 GEMM (the weights are plain fp16 by then, so it is a library
- *            GEMM; the library is opened with dlopen on first use and its handle is
- *            created then, the only allocation this library ever causes; an error if
+ *            GEMM; the library is opened with dlopen by cuthip_init and its handle is
+ *            created then (outside any stream capture), the only allocation this
+ *            library ever causes; the first matmul of a new shape asks the library's
+ *            heuristic for a kernel, on the host; an error if
  *            the library is absent or an epilogue is asked for; CUT_HIP_NO_BLASLT=1 in
  *            the environment keeps it closed);
  *            -1 = choose by shape: the two-pass path (variant 5 where hipBLASLt is
