@@ -60,6 +60,7 @@ static const cuthip_variant_info_t *table(int op, int *count) {
 
 namespace cuthip {
 bool blaslt_available();
+int attn_static_setup();
 }
 using namespace cuthip;
 
@@ -88,7 +89,8 @@ int cuthip_init(int device) {
   // open hipBLASLt (variant 5 of the prefill matmul) now: its handle must not be created inside a stream capture,
   // where the first matmul of a caller may well run; absence of the library is not an error
   (void)cuthip::blaslt_available();
-  return CUTHIP_OK;
+  // device address of the built-in attention scratch on this device (cuthip_attn_decode_static)
+  return cuthip::attn_static_setup();
 }
 
 int cuthip_device_info(cuthip_device_info_t *info) {

@@ -17,6 +17,7 @@
 // split-context decode attention).
 #include <cmath>
 #include <cstdint>
+#include <mutex>
 
 #include "common.hpp"
 
@@ -430,36 +431,111 @@ size_t cuthip_attn_decode_workspace_bytes(uint32_t n_heads, uint32_t head_dim, u
   return (size_t)n_heads * nsplit * (2 + head_dim) * sizeof(float);
 }
 
+// Argument checks shared by the two attention entry points (the workspace is checked by each).
+static int attn_check_args(const char *who, const void *q, int q_dtype, const void *k_cache, const void *v_cache,
+                           const uint32_t *runtime_params, const void *out, int out_dtype, uint32_t n_heads,
+                           uint32_t n_kv_heads, uint32_t head_dim, uint32_t aligned_kv_dim, uint32_t max_seq_len) {
+  if (!q || !k_cache || !v_cache || !runtime_params || !out || n_heads == 0 || n_kv_heads == 0 || n_heads % n_kv_heads ||
+      head_dim == 0 || head_dim > kAttnMaxHd || head_dim % 8 || max_seq_len == 0 || aligned_kv_dim < n_kv_heads * head_dim ||
+      aligned_kv_dim % 8 || bad_dtype(q_dtype) || bad_dtype(out_dtype)) {
+    set_error("%s: bad argument (heads %u/%u, head_dim %u (<= %d, multiple of 8), aligned_kv_dim %u)", who, n_heads, n_kv_heads,
+              head_dim, kAttnMaxHd, aligned_kv_dim);
+    return CUTHIP_ERR_INVALID;
+  }
+  if ((max_seq_len + kAttnChunk - 1) / kAttnChunk > (uint32_t)kAttnMaxSplit) {
+    set_error("%s: max_seq_len %u exceeds %d", who, max_seq_len, kAttnMaxSplit * kAttnChunk);
+    return CUTHIP_ERR_INVALID;
+  }
+  return CUTHIP_OK;
+}
+
+// The two launches of the split-context attention; `partial` holds cuthip_attn_decode_workspace_bytes() bytes.
+static int attn_launch(const void *q, int q_dtype, const void *k_cache, const void *v_cache, const uint32_t *runtime_params,
+                       void *out, int out_dtype, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                       uint32_t aligned_kv_dim, float scale, uint32_t max_seq_len, float *partial, hipStream_t s) {
+  uint32_t nsplit = (max_seq_len + kAttnChunk - 1) / kAttnChunk;
+  auto partial_kernel = head_dim == 128 ? attn_partial_kernel<128> : attn_partial_kernel<0>;
+  hipLaunchKernelGGL(partial_kernel, dim3(n_kv_heads, nsplit), dim3(256), 0, s, q, q_dtype == CUTHIP_F16,
+                     (const half_t *)k_cache, (const half_t *)v_cache, runtime_params, partial, n_heads, n_kv_heads, head_dim,
+                     aligned_kv_dim, scale, nsplit, max_seq_len);
+  if (int rc = check_hip(hipGetLastError(), "attention launch")) return rc;
+  hipLaunchKernelGGL(attn_merge_kernel, dim3(n_heads), dim3(128), 0, s, (const float *)partial, runtime_params, out,
+                     out_dtype == CUTHIP_F16, head_dim, nsplit);
+  return check_hip(hipGetLastError(), "attention merge launch");
+}
+
 int cuthip_attn_decode(const void *q, int q_dtype, const void *k_cache, const void *v_cache, const uint32_t *runtime_params,
                        void *out, int out_dtype, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
                        uint32_t aligned_kv_dim, float scale, uint32_t max_seq_len, void *workspace, size_t workspace_bytes,
                        void *stream) {
-  if (!q || !k_cache || !v_cache || !runtime_params || !out || !workspace || n_heads == 0 || n_kv_heads == 0 ||
-      n_heads % n_kv_heads || head_dim == 0 || head_dim > kAttnMaxHd || head_dim % 8 || max_seq_len == 0 ||
-      aligned_kv_dim < n_kv_heads * head_dim || aligned_kv_dim % 8 || bad_dtype(q_dtype) || bad_dtype(out_dtype)) {
-    set_error("cuthip_attn_decode: bad argument (heads %u/%u, head_dim %u (<= %d, multiple of 8), aligned_kv_dim %u)", n_heads,
-              n_kv_heads, head_dim, kAttnMaxHd, aligned_kv_dim);
-    return CUTHIP_ERR_INVALID;
-  }
-  if ((max_seq_len + kAttnChunk - 1) / kAttnChunk > (uint32_t)kAttnMaxSplit) {
-    set_error("cuthip_attn_decode: max_seq_len %u exceeds %d", max_seq_len, kAttnMaxSplit * kAttnChunk);
-    return CUTHIP_ERR_INVALID;
-  }
-  if (workspace_bytes < cuthip_attn_decode_workspace_bytes(n_heads, head_dim, max_seq_len)) {
-    set_error("cuthip_attn_decode: workspace of %zu bytes, need %zu", workspace_bytes,
+  if (int rc = attn_check_args("cuthip_attn_decode", q, q_dtype, k_cache, v_cache, runtime_params, out, out_dtype, n_heads,
+                               n_kv_heads, head_dim, aligned_kv_dim, max_seq_len))
+    return rc;
+  if (!workspace || workspace_bytes < cuthip_attn_decode_workspace_bytes(n_heads, head_dim, max_seq_len)) {
+    set_error("cuthip_attn_decode: workspace of %zu bytes, need %zu", workspace ? workspace_bytes : (size_t)0,
               cuthip_attn_decode_workspace_bytes(n_heads, head_dim, max_seq_len));
     return CUTHIP_ERR_INVALID;
   }
-  uint32_t nsplit = (max_seq_len + kAttnChunk - 1) / kAttnChunk;
-  hipStream_t s = (hipStream_t)stream;
-  auto partial_kernel = head_dim == 128 ? attn_partial_kernel<128> : attn_partial_kernel<0>;
-  hipLaunchKernelGGL(partial_kernel, dim3(n_kv_heads, nsplit), dim3(256), 0, s, q, q_dtype == CUTHIP_F16,
-                     (const half_t *)k_cache, (const half_t *)v_cache, runtime_params, (float *)workspace, n_heads, n_kv_heads,
-                     head_dim, aligned_kv_dim, scale, nsplit, max_seq_len);
-  if (int rc = check_hip(hipGetLastError(), "attention launch")) return rc;
-  hipLaunchKernelGGL(attn_merge_kernel, dim3(n_heads), dim3(128), 0, s, (const float *)workspace, runtime_params, out,
-                     out_dtype == CUTHIP_F16, head_dim, nsplit);
-  return check_hip(hipGetLastError(), "attention merge launch");
+  return attn_launch(q, q_dtype, k_cache, v_cache, runtime_params, out, out_dtype, n_heads, n_kv_heads, head_dim,
+                     aligned_kv_dim, scale, max_seq_len, (float *)workspace, (hipStream_t)stream);
+}
+
+}  // extern "C"
+
+// ---- the attention without a caller workspace: partial results in a device array of this library ----
+// One copy of the array exists on every GPU the library runs on, at its own address, until the process ends.  The
+// array's name is a host-side stand-in; the device address is taken once per device with hipGetSymbolAddress.
+namespace cuthip {
+constexpr size_t kAttnStaticBytes = 4u << 20;   // 4 MiB: 32 heads of dimension 128 up to a cache capacity of 16,128
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kAttnStaticBytes];
+static void *g_scratch_ptr[kMaxDevices];   // per device; written under g_scratch_mu
+static std::mutex g_scratch_mu;
+
+// Device address of `scratch` on the current device (looked up on first use there); nullptr after set_error.
+static void *attn_static_ptr() {
+  int dev = -1;
+  if (check_hip(hipGetDevice(&dev), "hipGetDevice")) return nullptr;
+  if (dev < 0 || dev >= kMaxDevices) {
+    set_error("attention scratch: device index %d beyond %d", dev, kMaxDevices);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void *ptr = nullptr;
+    if (check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return nullptr;
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+
+// called by cuthip_init with the chosen device current
+int attn_static_setup() { return attn_static_ptr() ? CUTHIP_OK : CUTHIP_ERR_HIP; }
+}  // namespace cuthip
+
+extern "C" {
+
+size_t cuthip_attn_decode_static_max_bytes(void) { return kAttnStaticBytes; }
+
+int cuthip_attn_decode_static(const void *q, int q_dtype, const void *k_cache, const void *v_cache,
+                              const uint32_t *runtime_params, void *out, int out_dtype, uint32_t n_heads, uint32_t n_kv_heads,
+                              uint32_t head_dim, uint32_t aligned_kv_dim, float scale, uint32_t max_seq_len, void *stream) {
+  if (int rc = attn_check_args("cuthip_attn_decode_static", q, q_dtype, k_cache, v_cache, runtime_params, out, out_dtype,
+                               n_heads, n_kv_heads, head_dim, aligned_kv_dim, max_seq_len))
+    return rc;
+  const size_t need = cuthip_attn_decode_workspace_bytes(n_heads, head_dim, max_seq_len);
+  if (need > kAttnStaticBytes) {
+    set_error("cuthip_attn_decode_static: %u heads of dimension %u over a cache of %u positions need %zu bytes of partial "
+              "results, the built-in scratch holds %zu; use cuthip_attn_decode with a workspace", n_heads, head_dim,
+              max_seq_len, need, kAttnStaticBytes);
+    return CUTHIP_ERR_INVALID;
+  }
+  void *ptr = attn_static_ptr();
+  if (!ptr) return CUTHIP_ERR_HIP;
+  // every split record of this call's launch shape is written before the merge reads it, so nothing of an earlier
+  // call's contents is read and nothing needs clearing
+  return attn_launch(q, q_dtype, k_cache, v_cache, runtime_params, out, out_dtype, n_heads, n_kv_heads, head_dim,
+                     aligned_kv_dim, scale, max_seq_len, (float *)ptr, (hipStream_t)stream);
 }
 
 int cuthip_silu_mul(const void *gate_up, int in_dtype, void *out, int out_dtype, uint32_t n, void *stream) {

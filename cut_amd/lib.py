@@ -32,6 +32,7 @@ EXPORTS = [
     "cuthip_dequant", "cuthip_matmul_gguf", "cuthip_matmul_gguf_pro",
     "cuthip_matmul_gguf_workspace_bytes", "cuthip_matmul_gguf_ws", "cuthip_matmul_gguf_pair", "cuthip_matmul_gguf_carry",
     "cuthip_rmsnorm", "cuthip_rope_kv_write", "cuthip_attn_decode_workspace_bytes", "cuthip_attn_decode",
+    "cuthip_attn_decode_static_max_bytes", "cuthip_attn_decode_static",
     "cuthip_silu_mul", "cuthip_argmax",
     "cuthip_matmul_sep_workspace_bytes", "cuthip_matmul_q8_sep", "cuthip_matmul_q4_sep",
     "cuthip_prepare_sep", "cuthip_transpose_q4_nibble", "cuthip_quantize_rows_q8_0",
@@ -116,6 +117,8 @@ def load() -> C.CDLL:
     lib.cuthip_rope_kv_write.argtypes = [vp, vp, vp, i, vp, vp, vp, vp, vp, vp, i, u32, u32, u32, u32, vp]
     lib.cuthip_attn_decode_workspace_bytes.argtypes = [u32, u32, u32]
     lib.cuthip_attn_decode.argtypes = [vp, i, vp, vp, vp, vp, i, u32, u32, u32, u32, f32, u32, vp, C.c_size_t, vp]
+    lib.cuthip_attn_decode_static_max_bytes.argtypes = []
+    lib.cuthip_attn_decode_static.argtypes = [vp, i, vp, vp, vp, vp, i, u32, u32, u32, u32, f32, u32, vp]
     lib.cuthip_silu_mul.argtypes = [vp, i, vp, i, u32, vp]
     lib.cuthip_argmax.argtypes = [vp, i, u32, vp, vp]
     lib.cuthip_matmul_sep_workspace_bytes.argtypes = [u32, u32, u32]
@@ -130,7 +133,7 @@ def load() -> C.CDLL:
     lib.cuthip_matmul_q8_i8.argtypes = [vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, vp, C.c_size_t, vp]
     sized = ("cuthip_attn_decode_workspace_bytes", "cuthip_matmul_sep_workspace_bytes",
              "cuthip_matmul_gguf_workspace_bytes", "cuthip_matmul_q8_i8_workspace_bytes",
-             "cuthip_matmul_dense_f16_workspace_bytes")
+             "cuthip_matmul_dense_f16_workspace_bytes", "cuthip_attn_decode_static_max_bytes")
     for n in EXPORTS:
         if n != "cuthip_last_error" and n not in sized:
             getattr(lib, n).restype = i

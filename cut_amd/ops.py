@@ -255,6 +255,17 @@ def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, r
     return out
 
 
+def attn_decode_static(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, runtime_params: torch.Tensor, n_heads: int,
+                       n_kv_heads: int, head_dim: int, scale: float, out: torch.Tensor,
+                       max_seq_len: int | None = None) -> torch.Tensor:
+    """attn_decode on the library's built-in scratch (no workspace, no allocation; shapes up to 4 MiB of partials)."""
+    _l.check(_l.load().cuthip_attn_decode_static(q.data_ptr(), _dt(q), k_cache.data_ptr(), v_cache.data_ptr(),
+                                                 runtime_params.data_ptr(), out.data_ptr(), _dt(out), n_heads, n_kv_heads,
+                                                 head_dim, k_cache.stride(0), scale, max_seq_len or k_cache.shape[0],
+                                                 _stream_ptr()))
+    return out
+
+
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     _l.check(_l.load().cuthip_silu_mul(gate_up.data_ptr(), _dt(gate_up), out.data_ptr(), _dt(out), out.numel(), _stream_ptr()))
     return out

@@ -392,6 +392,21 @@ int cuthip_attn_decode(const void *q, int q_dtype, const void *k_cache, const vo
                        uint32_t aligned_kv_dim, float scale, uint32_t max_seq_len, void *workspace, size_t workspace_bytes,
                        void *stream);
 
+/* cuthip_attn_decode without a caller workspace.  It has no counterpart in the reference; it exists for callers that
+ * cannot allocate device memory or carry a workspace around (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): the partial results of the context splits live in a device array inside this
+ * library, cuthip_attn_decode_static_max_bytes() = 4 MiB on every GPU the library runs on, held until the process
+ * ends.  The call allocates nothing; its device address is looked up by cuthip_init (or on the first call on a
+ * device).  Shapes whose partial results exceed the array (cuthip_attn_decode_workspace_bytes(n_heads, head_dim,
+ * max_seq_len) > 4 MiB, e.g. 32 heads of dimension 128 beyond a capacity of 16,128) are rejected with
+ * CUTHIP_ERR_INVALID.  All calls on one GPU share the array: calls that overlap on one GPU (two streams, two
+ * threads) race; serialise them or give the others a workspace through cuthip_attn_decode.  Results are identical
+ * to cuthip_attn_decode (same kernels). */
+size_t cuthip_attn_decode_static_max_bytes(void);
+int cuthip_attn_decode_static(const void *q, int q_dtype, const void *k_cache, const void *v_cache,
+                              const uint32_t *runtime_params, void *out, int out_dtype, uint32_t n_heads, uint32_t n_kv_heads,
+                              uint32_t head_dim, uint32_t aligned_kv_dim, float scale, uint32_t max_seq_len, void *stream);
+
 /* out[i] = silu(gate_up[i]) * gate_up[n + i]: the SwiGLU combine after a fused
  * gate+up matmul (llama.cpp:1832-1857: unary SiLU, then BinaryMul). */
 int cuthip_silu_mul(const void *gate_up, int in_dtype, void *out, int out_dtype, uint32_t n, void *stream);
