@@ -23,6 +23,7 @@ def main():
     ap.add_argument("--output", default=os.path.join(os.path.dirname(os.path.abspath(__file__)), "tuning_data.json"))
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--formats", default=",".join(FORMATS))
+    ap.add_argument("--measurements", default=None, help="also write every timing of the sweep to this JSON file")
     args = ap.parse_args()
     import numpy as np
     import torch
@@ -32,7 +33,7 @@ def main():
     lib.check(lib.load().cuthip_init(0))
     dev = torch.device("cuda:0")
     names = [v["name"] for v in lib.variants(lib.OP_MATMUL_GGUF)]
-    operators = {}
+    operators, measurements = {}, {}
     for fmt in args.formats.split(","):
         rules, log = [], []
         for (N, K) in SHAPES_NK:
@@ -75,13 +76,18 @@ def main():
                 del ws
             del copies, w
             torch.cuda.empty_cache()
-        operators[f"MatMulGguf{fmt}"] = {"backends": {"hip": {"default_variant": -1, "rules": rules, "measurements_us": log}}}
+        operators[f"MatMulGguf{fmt}"] = {"backends": {"hip": {"default_variant": -1, "rules": rules}}}
+        measurements[f"MatMulGguf{fmt}"] = log
     info = lib.device_info()
     out = {"device": info["name"], "arch": info["arch"], "variant_names": names, "operators": operators}
     with open(args.output, "w") as fh:
         json.dump(out, fh, separators=(",", ":"))
         fh.write("\n")
     print(f"wrote {args.output}")
+    if args.measurements:
+        with open(args.measurements, "w") as fh:
+            json.dump(measurements, fh, separators=(",", ":"))
+            fh.write("\n")
 
 
 if __name__ == "__main__":

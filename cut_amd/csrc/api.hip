@@ -23,6 +23,42 @@ int check_hip(hipError_t e, const char *what) {
   return CUTHIP_ERR_HIP;
 }
 
+int check_epilogue_op(const char *who, int epilogue, int op) {
+  if (epilogue_op_known(epilogue, op)) return CUTHIP_OK;
+  set_error("%s: operator code %d is not one the %s epilogue implements (the reference's OP_%s_* codes of its "
+            "cut_writeOutput)", who, op, epilogue == CUTHIP_EPI_UNARY ? "unary" : "binary",
+            epilogue == CUTHIP_EPI_UNARY ? "UNARY" : "BINARY");
+  return CUTHIP_ERR_INVALID;
+}
+
+__global__ void __launch_bounds__(256) long_epilogue_kernel(void *C, int c_f16, uint32_t M, uint32_t N, uint32_t strideC,
+                                                            int epilogue, int op, const void *D) {
+  const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (uint64_t)M * N) return;
+  const size_t idx = (size_t)(i / N) * strideC + (size_t)(i % N);
+  float v = c_f16 ? (float)reinterpret_cast<const half_t *>(C)[idx] : reinterpret_cast<const float *>(C)[idx];
+  if (epilogue == CUTHIP_EPI_UNARY) {
+    v = apply_unary_long(op, v);
+  } else {
+    const float d = c_f16 ? (float)reinterpret_cast<const half_t *>(D)[idx] : reinterpret_cast<const float *>(D)[idx];
+    v = apply_binary_long(op, v, d);
+  }
+  store_plain(C, c_f16, idx, v);
+}
+
+int launch_long_epilogue(void *C, int c_f16, uint32_t M, uint32_t N, uint32_t strideC, int epilogue, int op, const void *D,
+                         hipStream_t stream) {
+  const uint64_t total = (uint64_t)M * N;
+  if (total == 0) return CUTHIP_OK;
+  if (epilogue == CUTHIP_EPI_BINARY && D == C) {   // the unfused matmul has already overwritten what D held
+    set_error("binary operator %d is applied after the matmul, in a launch of its own: D must not alias C", op);
+    return CUTHIP_ERR_INVALID;
+  }
+  hipLaunchKernelGGL(long_epilogue_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, stream, C, c_f16, M, N,
+                     strideC, epilogue, op, D);
+  return check_hip(hipGetLastError(), "epilogue launch");
+}
+
 // Variant tables, one per operator family; the index of a row is ABI.
 static const cuthip_variant_info_t kDequantVariants[] = {
     {"DequantGguf8", 256, 1, 1, 2048, "GGUF block dequant, 8 outputs per lane, 16-byte coalesced stores"},
@@ -30,7 +66,7 @@ static const cuthip_variant_info_t kDequantVariants[] = {
 static const cuthip_variant_info_t kMatMulGgufVariants[] = {
     {"MatMulGgufGemvMfma", 64, 4, 8, 32,
      "streaming GEMV / skinny GEMM (M <= 8): 32 weight rows per workgroup, split-K over the waves, "
-     "in-register unpack feeding 32x32x16 f16 MFMA, fp32 per-sub-block scaling"},
+     "in-register unpack feeding 32x32x16 f16 MFMA, fp32 per-sub-block scaling; beyond 8 rows of A the choice by shape"},
     {"MatMulGgufSkinnyMfma", 64, 4, 32, 32, "same pipeline with a 32-row activation tile (8 < M <= 32 per pass)"},
     {"MatMulGgufGemmLds", 256, 1, 128, 128,
      "prefill GEMM: weights dequantized to fp16 tiles in LDS, 32x32x16 f16 MFMA, fp32 accumulate"},
@@ -45,21 +81,68 @@ static const cuthip_variant_info_t kMatMulGgufVariants[] = {
      "GEMM (opened at run time; no fused epilogue; needs cuthip_matmul_gguf_ws)"},
 };
 
+// Separated-layout matmuls: the reference's tables, name for name and index for index
+// (operators/impl/matmul/MatMulQ8Variants.generated.h:20-32, MatMulQ4Variants.generated.h:20-29); the last column
+// says which of this library's two code paths serves the entry.
+static const cuthip_variant_info_t kMatMulQ8Variants[] = {
+    {"MatMulQ8T16R4x4", 16, 16, 64, 64, "Q8 T16 R4x4 -> choice by shape (streaming kernel below 32 rows, dequant + MFMA GEMM from 32)"},
+    {"MatMulQ8Gemv", 256, 1, 1, 256, "Q8 GEMV (M=1 vector) -> column-major streaming kernel"},
+    {"MatMulQ8VecT16R4x4", 16, 16, 64, 64, "Q8 Vec4 T16 R4x4 -> choice by shape"},
+    {"MatMulQ8GemvKPar", 32, 1, 1, 4, "Q8 GEMV K-parallel -> column-major streaming kernel"},
+    {"MatMulQ8GemvKPar8", 32, 8, 1, 8, "Q8 GEMV (M=1, 8 cols/WG, split-K over 8 waves) -> column-major streaming kernel"},
+    {"MatMulQ8GemvDot", 32, 1, 1, 4, "Q8 GEMV dotPacked4x8EXT -> column-major streaming kernel, activations not quantized"},
+    {"MatMulQ8TiledDot", 256, 1, 32, 64, "Q8 TiledDot dotPacked4x8EXT -> choice by shape, activations not quantized"},
+    {"MatMulQ8CoopMatTiled", 128, 1, 32, 32, "Q8 CoopMat 2x2 Tiled -> dequant to fp16, then the dense MFMA GEMM"},
+};
+static const cuthip_variant_info_t kMatMulQ4Variants[] = {
+    {"MatMulQ4T16R4x4", 16, 16, 64, 64, "Q4 T16 R4x4 -> choice by shape (streaming kernel below 32 rows, dequant + MFMA GEMM from 32)"},
+    {"MatMulQ4Gemv", 256, 1, 1, 256, "Q4 GEMV (M=1 vector) -> column-major streaming kernel"},
+    {"MatMulQ4GemvKPar", 32, 1, 1, 4, "Q4 GEMV K-parallel -> column-major streaming kernel"},
+    {"MatMulQ4GemvKPar8", 32, 8, 1, 8, "Q4 GEMV (M=1, 8 cols/WG, split-K over 8 waves) -> column-major streaming kernel"},
+    {"MatMulQ4CoopMatTiled", 128, 1, 32, 32, "Q4 CoopMat 2x2 Tiled -> dequant to fp16, then the dense MFMA GEMM"},
+};
+
 static const cuthip_variant_info_t *table(int op, int *count) {
   switch (op) {
   case CUTHIP_OP_DEQUANT: *count = 1; return kDequantVariants;
   case CUTHIP_OP_MATMUL_GGUF:
     *count = (int)(sizeof(kMatMulGgufVariants) / sizeof(kMatMulGgufVariants[0]));
     return kMatMulGgufVariants;
+  case CUTHIP_OP_MATMUL_Q8:
+    *count = (int)(sizeof(kMatMulQ8Variants) / sizeof(kMatMulQ8Variants[0]));
+    return kMatMulQ8Variants;
+  case CUTHIP_OP_MATMUL_Q4:
+    *count = (int)(sizeof(kMatMulQ4Variants) / sizeof(kMatMulQ4Variants[0]));
+    return kMatMulQ4Variants;
   }
   *count = 0;
   return nullptr;
+}
+
+// A launch that only loads: every thread xors 16-byte loads (four in flight), one dword per workgroup is stored so
+// that the loads cannot be dropped.  The measuring stick for what a launch of a given size can reach when it does
+// nothing but read (cuthip_read_probe).
+__global__ void __launch_bounds__(256) read_probe_kernel(const u32x4 *src, size_t nvec, uint32_t *sink) {
+  const size_t stride = (size_t)gridDim.x * 256 * 4;
+  u32x4 acc{0, 0, 0, 0};
+  for (size_t i = (size_t)blockIdx.x * 1024 + threadIdx.x; i < nvec; i += stride) {
+    u32x4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(src + (i + u * 256 < nvec ? i + u * 256 : i));
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc ^= v[u];
+  }
+  uint32_t r = acc.x ^ acc.y ^ acc.z ^ acc.w;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) r ^= __shfl_xor(r, o);
+  if ((threadIdx.x & 63) == 0) sink[(blockIdx.x * 4 + threadIdx.x / 64) & 0xFFFF] = r;
 }
 
 }  // namespace cuthip
 
 namespace cuthip {
 bool blaslt_available();
+bool blaslt_preferred();
 int attn_static_setup();
 }
 using namespace cuthip;
@@ -86,9 +169,10 @@ int cuthip_init(int device) {
     set_error("cuthip_init: device %d is %s; this library is built for gfx950 only", device, p.gcnArchName);
     return CUTHIP_ERR_NO_DEVICE;
   }
-  // open hipBLASLt (variant 5 of the prefill matmul) now: its handle must not be created inside a stream capture,
-  // where the first matmul of a caller may well run; absence of the library is not an error
-  (void)cuthip::blaslt_available();
+  // hipBLASLt (variant 5 of the prefill matmul) is opt-in: a process that sets CUT_HIP_VENDOR_GEMM opens it now,
+  // because its handle must not be created inside a stream capture, where the first matmul of a caller may well
+  // run; absence of the library is not an error
+  (void)cuthip::blaslt_preferred();
   // device address of the built-in attention scratch on this device (cuthip_attn_decode_static)
   return cuthip::attn_static_setup();
 }
@@ -172,12 +256,96 @@ int cuthip_event_elapsed_ms(void *start, void *stop, float *ms) {
   return check_hip(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop), "hipEventElapsedTime");
 }
 
+int cuthip_read_probe(const void *src, size_t bytes, uint32_t *sink, void *stream) {
+  if (!src || !sink || bytes < 16 || (uintptr_t)src % 16 != 0) {
+    set_error("cuthip_read_probe: needs a 16-byte aligned buffer of at least 16 bytes and a sink of 65,536 dwords");
+    return CUTHIP_ERR_INVALID;
+  }
+  const size_t nvec = bytes / 16;
+  size_t blocks = (nvec + 1023) / 1024;
+  if (blocks > 256 * 16) blocks = 256 * 16;   // 16 workgroups per CU walk the rest
+  hipLaunchKernelGGL(read_probe_kernel, dim3((uint32_t)blocks), dim3(256), 0, (hipStream_t)stream,
+                     reinterpret_cast<const u32x4 *>(src), nvec, sink);
+  return check_hip(hipGetLastError(), "read probe launch");
+}
+
+// ---- capture and replay of a launch sequence (the reusable command buffer of the reference, CudaCommandBuffer.cpp:261-285)
+struct CapturedGraph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+};
+
+int cuthip_graph_begin_capture(void *stream) {
+  if (!stream) {
+    set_error("cuthip_graph_begin_capture: capture needs a stream of its own (not the default stream)");
+    return CUTHIP_ERR_INVALID;
+  }
+  return check_hip(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+}
+
+int cuthip_graph_end_capture(void *stream, void **graph) {
+  if (!stream || !graph) {
+    set_error("cuthip_graph_end_capture: null argument");
+    return CUTHIP_ERR_INVALID;
+  }
+  *graph = nullptr;
+  CapturedGraph g;
+  if (int rc = check_hip(hipStreamEndCapture((hipStream_t)stream, &g.graph), "hipStreamEndCapture")) return rc;
+  if (!g.graph) {
+    set_error("cuthip_graph_end_capture: the capture was invalidated (a call that is not allowed under capture was made)");
+    return CUTHIP_ERR_HIP;
+  }
+  if (int rc = check_hip(hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0), "hipGraphInstantiate")) {
+    (void)hipGraphDestroy(g.graph);
+    return rc;
+  }
+  *graph = new CapturedGraph(g);
+  return CUTHIP_OK;
+}
+
+int cuthip_graph_launch(void *graph, void *stream) {
+  if (!graph) {
+    set_error("cuthip_graph_launch: null graph");
+    return CUTHIP_ERR_INVALID;
+  }
+  return check_hip(hipGraphLaunch(static_cast<CapturedGraph *>(graph)->exec, (hipStream_t)stream), "hipGraphLaunch");
+}
+
+int cuthip_graph_destroy(void *graph) {
+  if (!graph) return CUTHIP_OK;
+  CapturedGraph *g = static_cast<CapturedGraph *>(graph);
+  int rc = check_hip(hipGraphExecDestroy(g->exec), "hipGraphExecDestroy");
+  int rc2 = check_hip(hipGraphDestroy(g->graph), "hipGraphDestroy");
+  delete g;
+  return rc ? rc : rc2;
+}
+
+int cuthip_epilogue_op_supported(int epilogue, int op) {
+  return (epilogue == CUTHIP_EPI_UNARY || epilogue == CUTHIP_EPI_BINARY) && epilogue_op_known(epilogue, op) ? 1 : 0;
+}
+
 int cuthip_variant_count(int op) {
   int n;
   table(op, &n);
   return n;
 }
-int cuthip_variant_default(int op) { return op == CUTHIP_OP_DEQUANT || op == CUTHIP_OP_MATMUL_GGUF ? 0 : CUTHIP_ERR_INVALID; }
+int cuthip_variant_default(int op) {
+  switch (op) {
+  case CUTHIP_OP_DEQUANT: case CUTHIP_OP_MATMUL_GGUF: case CUTHIP_OP_MATMUL_Q4: return 0;   // kMatMulQ4DefaultVariant = 0
+  case CUTHIP_OP_MATMUL_Q8: return 2;                                                         // kMatMulQ8DefaultVariant = 2
+  }
+  set_error("cuthip_variant_default: no operator family %d", op);
+  return CUTHIP_ERR_INVALID;
+}
+int cuthip_variant_available(int op, int index) {
+  int n;
+  if (!table(op, &n) || index < 0 || index >= n) {
+    set_error("cuthip_variant_available: no variant %d in operator family %d", index, op);
+    return CUTHIP_ERR_UNKNOWN_VARIANT;
+  }
+  if (op == CUTHIP_OP_MATMUL_GGUF && index == 5) return blaslt_available() ? 1 : 0;
+  return 1;
+}
 int cuthip_variant_info(int op, int index, cuthip_variant_info_t *info) {
   int n;
   const cuthip_variant_info_t *t = table(op, &n);

@@ -87,31 +87,98 @@ __device__ inline void q4k_scales(uint32_t s0, uint32_t s1, uint32_t s2, uint32_
   m_hi = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
 }
 
-// Unary / binary epilogues of the matmul (MatMulQ8Common.cuh:58-109).
-__device__ inline float apply_unary(int op, float v) {
+// Unary / binary epilogues of the matmul: the operator set and the formulas of cut_writeOutput
+// (operators/impl/matmul/MatMulQ8Common.cuh:58-109), selected by the reference's operator codes.
+// Only six unary (NEG, TANH, RELU, SIGMOID, GELU, SILU) and six binary (ADD, SUB, MUL, DIV, MIN, MAX) operators are part
+// of the matmul kernels' epilogues.  The tiled GEMMs store 128 and more accumulators per lane through fully unrolled
+// loops; with the whole operator set inlined at every store those loops no longer unroll, and the accumulator arrays
+// they index leave the registers (measured: 710 -> 39 TFLOP/s).  The entry points run such a
+// matmul unfused and apply the operator in a second, elementwise launch (launch_long_epilogue).
+__device__ inline float apply_unary_long(int op, float x) {
   switch (op) {
-  case CUTHIP_UNARY_SILU: return v / (1.0f + __expf(-v));
-  case CUTHIP_UNARY_RELU: return v > 0.0f ? v : 0.0f;
-  case CUTHIP_UNARY_GELU_TANH: {
-    float t = 0.7978845608028654f * (v + 0.044715f * v * v * v);
-    return 0.5f * v * (1.0f + tanhf(t));
+  case CUTHIP_UNARY_ABS: return fabsf(x);
+  case CUTHIP_UNARY_SQRT: return sqrtf(x);
+  case CUTHIP_UNARY_SQUARE: return x * x;
+  case CUTHIP_UNARY_RECIPROCAL: return 1.0f / x;
+  case CUTHIP_UNARY_FLOOR: return floorf(x);
+  case CUTHIP_UNARY_CEIL: return ceilf(x);
+  case CUTHIP_UNARY_RELU6: return fminf(fmaxf(x, 0.0f), 6.0f);
+  case CUTHIP_UNARY_EXP: return expf(x);
+  case CUTHIP_UNARY_LOG: return logf(x);
+  case CUTHIP_UNARY_ROUND: return roundf(x);
+  case CUTHIP_UNARY_SOFTPLUS: return logf(1.0f + expf(x));
+  case CUTHIP_UNARY_MISH: return x * tanhf(logf(1.0f + expf(x)));
+  case CUTHIP_UNARY_HARDSWISH: return x * fminf(fmaxf(x / 6.0f + 0.5f, 0.0f), 1.0f);
+  case CUTHIP_UNARY_HARDSIGMOID: return fminf(fmaxf(x / 6.0f + 0.5f, 0.0f), 1.0f);
+  case CUTHIP_UNARY_RSQRT: return 1.0f / sqrtf(x);
   }
-  case CUTHIP_UNARY_SIGMOID: return 1.0f / (1.0f + __expf(-v));
-  case CUTHIP_UNARY_TANH: return tanhf(v);
-  case CUTHIP_UNARY_NEG: return -v;
-  }
-  return v;
+  return x;
 }
-__device__ inline float apply_binary(int op, float v, float d) {
+__device__ inline float apply_binary_long(int op, float a, float b) {
   switch (op) {
-  case CUTHIP_BINARY_ADD: return v + d;
-  case CUTHIP_BINARY_SUB: return v - d;
-  case CUTHIP_BINARY_MUL: return v * d;
-  case CUTHIP_BINARY_DIV: return v / d;
-  case CUTHIP_BINARY_MIN: return fminf(v, d);
-  case CUTHIP_BINARY_MAX: return fmaxf(v, d);
+  case CUTHIP_BINARY_MOD: return a - b * floorf(a / b);
+  case CUTHIP_BINARY_POW: return powf(a, b);
+  case CUTHIP_BINARY_FLOOR_DIV: return floorf(a / b);
   }
-  return v;
+  return a;
+}
+inline bool epilogue_op_long(int epilogue, int op) {
+  if (epilogue == CUTHIP_EPI_UNARY) {
+    switch (op) {
+    case CUTHIP_UNARY_NEG: case CUTHIP_UNARY_TANH: case CUTHIP_UNARY_RELU: case CUTHIP_UNARY_SIGMOID: case CUTHIP_UNARY_GELU:
+    case CUTHIP_UNARY_SILU: return false;   // the six of the kernel epilogues
+    }
+    return true;
+  }
+  if (epilogue == CUTHIP_EPI_BINARY) return op == CUTHIP_BINARY_MOD || op == CUTHIP_BINARY_POW || op == CUTHIP_BINARY_FLOOR_DIV;
+  return false;
+}
+// The operators inside the matmul kernels' epilogues.
+__device__ inline float apply_unary(int op, float x) {
+  switch (op) {
+  case CUTHIP_UNARY_NEG: return -x;
+  case CUTHIP_UNARY_TANH: return tanhf(x);
+  case CUTHIP_UNARY_RELU: return fmaxf(0.0f, x);
+  case CUTHIP_UNARY_SIGMOID: return 1.0f / (1.0f + __expf(-x));
+  case CUTHIP_UNARY_GELU: {
+    float t = 0.7978845608028654f * (x + 0.044715f * x * x * x);   // sqrt(2 / pi)
+    return x * 0.5f * (1.0f + tanhf(t));
+  }
+  case CUTHIP_UNARY_SILU: return x / (1.0f + __expf(-x));
+  }
+  return x;   // the long operators never reach a kernel epilogue (epilogue_op_long)
+}
+__device__ inline float apply_binary(int op, float a, float b) {
+  switch (op) {
+  case CUTHIP_BINARY_ADD: return a + b;
+  case CUTHIP_BINARY_SUB: return a - b;
+  case CUTHIP_BINARY_MUL: return a * b;
+  case CUTHIP_BINARY_DIV: return a / b;
+  case CUTHIP_BINARY_MIN: return fminf(a, b);
+  case CUTHIP_BINARY_MAX: return fmaxf(a, b);
+  }
+  return a;   // the long operators never reach a kernel epilogue (epilogue_op_long)
+}
+inline bool epilogue_op_known(int epilogue, int op) {
+  if (epilogue == CUTHIP_EPI_UNARY) {
+    switch (op) {
+    case CUTHIP_UNARY_NEG: case CUTHIP_UNARY_ABS: case CUTHIP_UNARY_SQRT: case CUTHIP_UNARY_SQUARE:
+    case CUTHIP_UNARY_RECIPROCAL: case CUTHIP_UNARY_EXP: case CUTHIP_UNARY_LOG: case CUTHIP_UNARY_TANH:
+    case CUTHIP_UNARY_FLOOR: case CUTHIP_UNARY_CEIL: case CUTHIP_UNARY_ROUND: case CUTHIP_UNARY_RELU:
+    case CUTHIP_UNARY_SIGMOID: case CUTHIP_UNARY_GELU: case CUTHIP_UNARY_SILU: case CUTHIP_UNARY_SOFTPLUS:
+    case CUTHIP_UNARY_RELU6: case CUTHIP_UNARY_MISH: case CUTHIP_UNARY_HARDSWISH: case CUTHIP_UNARY_HARDSIGMOID:
+    case CUTHIP_UNARY_RSQRT: return true;
+    }
+    return false;
+  }
+  if (epilogue == CUTHIP_EPI_BINARY) {
+    switch (op) {
+    case CUTHIP_BINARY_ADD: case CUTHIP_BINARY_SUB: case CUTHIP_BINARY_MUL: case CUTHIP_BINARY_DIV: case CUTHIP_BINARY_MOD:
+    case CUTHIP_BINARY_POW: case CUTHIP_BINARY_FLOOR_DIV: case CUTHIP_BINARY_MIN: case CUTHIP_BINARY_MAX: return true;
+    }
+    return false;
+  }
+  return true;   // no operator to check
 }
 
 struct Epilogue {
@@ -158,5 +225,11 @@ __device__ inline void store_plain(void *C, int c_f16, size_t idx, float v) {
 
 void set_error(const char *fmt, ...);
 int check_hip(hipError_t e, const char *what);
+// CUTHIP_OK, or CUTHIP_ERR_INVALID with the error set when `op` is not an operator the epilogue kind implements
+int check_epilogue_op(const char *who, int epilogue, int op);
+// C[m, n] = op(C[m, n]) or op(C[m, n], D[m, n]) in place, for the operators of epilogue_op_long: the second launch of a
+// matmul whose fused operator is one of those (C and D are [M, strideC] of fp16 or fp32)
+int launch_long_epilogue(void *C, int c_f16, uint32_t M, uint32_t N, uint32_t strideC, int epilogue, int op, const void *D,
+                         hipStream_t stream);
 
 }  // namespace cuthip

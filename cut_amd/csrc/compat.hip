@@ -194,15 +194,16 @@ constexpr uint32_t kSepDenseRows = 32;
 
 bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a_f16, const void *A);
 size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16);
-bool blaslt_available();
+bool blaslt_preferred();
 int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K,
                       uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream,
                       int use_blaslt);
 
 static size_t sep_w16_bytes(uint32_t K, uint32_t N) { return ((size_t)N * K * 2 + 255) & ~(size_t)255; }
-static bool sep_dense_applies(uint32_t M, uint32_t K, uint32_t N) {
-  return M >= kSepDenseRows && K % 128 == 0 && (uint64_t)N * K * 2 < (1ull << 32) && (uint64_t)M * K * 2 < (1ull << 32);
+static bool sep_dense_fits(uint32_t K, uint32_t N, uint32_t M) {
+  return K % 128 == 0 && (uint64_t)N * K * 2 < (1ull << 32) && (uint64_t)M * K * 2 < (1ull << 32);
 }
+static bool sep_dense_applies(uint32_t M, uint32_t K, uint32_t N) { return M >= kSepDenseRows && sep_dense_fits(K, N, M); }
 
 template <bool Q4>
 __global__ void __launch_bounds__(256) sep_dequant_kernel(const uint8_t *B, const uint16_t *S, half_t *W16, uint32_t K, uint32_t N,
@@ -302,10 +303,47 @@ __global__ void __launch_bounds__(256) sep_dequant_kernel(const uint8_t *B, cons
   }
 }
 
+// Which of the two code paths a variant index of the reference's tables asks for.  The tables hold the reference's
+// names at the reference's indices (MatMulQ8Variants.generated.h:20-32, MatMulQ4Variants.generated.h:20-29); its
+// eight / five shaders collapse onto the two kernels here:
+//   tiled shaders (Q8 0, 2, 6; Q4 0) and -1            -> the choice by shape the reference's own default makes
+//   GEMV shaders (Q8 1, 3, 4, 5; Q4 1, 2, 3)            -> the streaming kernel, whatever M is
+//   cooperative-matrix shaders (Q8 7; Q4 4)            -> dequantize to fp16, then the dense MFMA GEMM
+// The reference's int8-activation shaders (Q8 5 GemvDot, 6 TiledDot) run here with fp32 / fp16 activations, i.e.
+// closer to the fp32 loop than the reference's own result for those indices.
+enum SepRoute { kSepAuto = 0, kSepStream = 1, kSepDense = 2 };
+static int sep_route(bool q4, int variant) {
+  if (variant == -1) return kSepAuto;
+  if (q4) {
+    switch (variant) {
+    case 0: return kSepAuto;
+    case 1: case 2: case 3: return kSepStream;
+    case 4: return kSepDense;
+    }
+  } else {
+    switch (variant) {
+    case 0: case 2: case 6: return kSepAuto;
+    case 1: case 3: case 4: case 5: return kSepStream;
+    case 7: return kSepDense;
+    }
+  }
+  return -1;
+}
+static size_t sep_stream_bytes(uint32_t M, uint32_t K, uint32_t N) {
+  size_t nsplit = (K + kSepWaves * kSepKC - 1) / (kSepWaves * kSepKC);
+  return nsplit > 1 ? nsplit * M * N * sizeof(float) : 0;
+}
+
 static int matmul_sep(bool q4, const float *A, const void *B, const void *S, const float *D, float *C, uint32_t M, uint32_t K,
                       uint32_t N, uint32_t strideA, uint32_t strideB, uint32_t strideC, uint32_t scaleStride, int epilogue,
-                      int epilogue_op, int affine, void *workspace, size_t workspace_bytes, hipStream_t stream) {
+                      int epilogue_op, int affine, int variant, void *workspace, size_t workspace_bytes, hipStream_t stream) {
   const char *who = q4 ? "cuthip_matmul_q4_sep" : "cuthip_matmul_q8_sep";
+  const int route = sep_route(q4, variant);
+  if (route < 0) {
+    set_error("%s: unknown variant index %d (table has %d)", who, variant,
+              cuthip_variant_count(q4 ? CUTHIP_OP_MATMUL_Q4 : CUTHIP_OP_MATMUL_Q8));
+    return CUTHIP_ERR_UNKNOWN_VARIANT;
+  }
   if (!A || !B || !S || !C || M == 0 || K == 0 || N == 0 || K % 32 || strideA < K || strideC < N || scaleStride < N ||
       strideB < (q4 ? (N + 1) / 2 : N) || (q4 && (N & 1))) {
     set_error("%s: bad argument (M %u, K %u (multiple of 32), N %u%s, strides %u %u %u %u)", who, M, K, N,
@@ -316,8 +354,22 @@ static int matmul_sep(bool q4, const float *A, const void *B, const void *S, con
     set_error("%s: bad epilogue %d (a binary epilogue needs D)", who, epilogue);
     return CUTHIP_ERR_INVALID;
   }
-  if (sep_dense_applies(M, K, N) && dense_gemm_fits(M, K, N, strideA, 0, A) && workspace && (uintptr_t)workspace % 256 == 0 &&
-      workspace_bytes >= sep_w16_bytes(K, N) + dense_f16_workspace(M, K, N, 0)) {
+  if (int rc = check_epilogue_op(who, epilogue, epilogue_op)) return rc;
+  if (epilogue_op_long(epilogue, epilogue_op)) {   // unfused matmul, then the operator as an elementwise launch
+    if (int rc = matmul_sep(q4, A, B, S, nullptr, C, M, K, N, strideA, strideB, strideC, scaleStride, CUTHIP_EPI_NONE, 0, affine,
+                            variant, workspace, workspace_bytes, stream))
+      return rc;
+    return launch_long_epilogue(C, 0, M, N, strideC, epilogue, epilogue_op, D, stream);
+  }
+  const bool dense_ok = sep_dense_fits(K, N, M) && dense_gemm_fits(M, K, N, strideA, 0, A) && workspace &&
+                        (uintptr_t)workspace % 256 == 0 && workspace_bytes >= sep_w16_bytes(K, N) + dense_f16_workspace(M, K, N, 0);
+  if (route == kSepDense && !dense_ok) {
+    set_error("%s: variant %d (dequantize, then the MFMA GEMM) needs K a multiple of 128, 16-byte aligned rows of A and a "
+              "256-byte aligned workspace of %zu bytes (K %u, strideA %u, workspace %zu)", who, variant,
+              sep_w16_bytes(K, N) + dense_f16_workspace(M, K, N, 0), K, strideA, workspace ? workspace_bytes : (size_t)0);
+    return CUTHIP_ERR_INVALID;
+  }
+  if (dense_ok && (route == kSepDense || (route == kSepAuto && M >= kSepDenseRows))) {
     half_t *w16 = reinterpret_cast<half_t *>(workspace);
     dim3 grid((N + 63) / 64, (K + 63) / 64);
     if (q4)
@@ -330,7 +382,7 @@ static int matmul_sep(bool q4, const float *A, const void *B, const void *S, con
     Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
     return launch_dense_gemm(-1, w16, A, 0, C, 0, M, K, N, strideA, strideC, epi,
                              reinterpret_cast<uint8_t *>(workspace) + sep_w16_bytes(K, N), stream,
-                             (epilogue == CUTHIP_EPI_NONE && blaslt_available()) ? 2 : 0);
+                             (epilogue == CUTHIP_EPI_NONE && blaslt_preferred()) ? 2 : 0);
   }
   SepParams p;
   p.A = A;
@@ -370,23 +422,29 @@ extern "C" {
 
 size_t cuthip_matmul_sep_workspace_bytes(uint32_t M, uint32_t K, uint32_t N) {
   if (sep_dense_applies(M, K, N)) return sep_w16_bytes(K, N) + dense_f16_workspace(M, K, N, 0);   // prefill route
-  size_t nsplit = (K + kSepWaves * kSepKC - 1) / (kSepWaves * kSepKC);
-  return nsplit > 1 ? nsplit * M * N * sizeof(float) : 0;
+  return sep_stream_bytes(M, K, N);
+}
+
+size_t cuthip_matmul_sep_workspace_bytes_for(int op, int variant, uint32_t M, uint32_t K, uint32_t N) {
+  const int route = sep_route(op == CUTHIP_OP_MATMUL_Q4, variant);
+  if (route == kSepStream) return sep_stream_bytes(M, K, N);
+  if (route == kSepDense) return sep_w16_bytes(K, N) + dense_f16_workspace(M, K, N, 0);
+  return cuthip_matmul_sep_workspace_bytes(M, K, N);
 }
 
 int cuthip_matmul_q8_sep(const float *A, const int8_t *B, const uint16_t *scales, const float *D, float *C, uint32_t M,
                          uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideB, uint32_t strideC, uint32_t scaleStride,
-                         int epilogue, int epilogue_op, void *workspace, size_t workspace_bytes, void *stream) {
+                         int epilogue, int epilogue_op, int variant, void *workspace, size_t workspace_bytes, void *stream) {
   return matmul_sep(false, A, B, scales, D, C, M, K, N, strideA, strideB, strideC, scaleStride, epilogue, epilogue_op, 0,
-                    workspace, workspace_bytes, (hipStream_t)stream);
+                    variant, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 int cuthip_matmul_q4_sep(const float *A, const uint8_t *packedB, const uint16_t *scales, const float *D, float *C, uint32_t M,
                          uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideBNpacked, uint32_t strideC,
-                         uint32_t scaleStride, int epilogue, int epilogue_op, int affine, void *workspace,
+                         uint32_t scaleStride, int epilogue, int epilogue_op, int affine, int variant, void *workspace,
                          size_t workspace_bytes, void *stream) {
   return matmul_sep(true, A, packedB, scales, D, C, M, K, N, strideA, strideBNpacked, strideC, scaleStride, epilogue,
-                    epilogue_op, affine, workspace, workspace_bytes, (hipStream_t)stream);
+                    epilogue_op, affine, variant, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -13,13 +13,21 @@
 // a workgroup owns one KV head and a chunk of 64 positions; its four waves
 // are the (up to four at a time) query heads sharing that KV head, so K and V
 // are read from HBM once, staged in LDS, and the softmax is carried as
-// (max, sum, weighted V) partials that a second kernel merges (the usual
-// split-context decode attention).
+// (max, sum, weighted V) partials (the usual split-context decode attention).
+// A second, small kernel merges the partials.  Merging inside the first kernel
+// (the workgroup that draws the last ticket of a KV head's counter reads the
+// records back; all workgroups of a head placed on one XCD so that records
+// and tickets stay in that XCD's L2; no fences) was built and measured: the
+// three dependent hops (stores acknowledged, ticket, records read back) cost
+// 5.5 us against the 4.5 us of the merge launch (12.8 us against 11.4 us per
+// layer), because every dependent memory access costs about a microsecond
+// here, in the XCD's own L2 as well.
 #include <cmath>
 #include <cstdint>
+#include <cstdlib>
 #include <mutex>
 
-#include "common.hpp"
+#include "gemv_formats.hpp"
 
 namespace cuthip {
 
@@ -48,8 +56,9 @@ __device__ inline float wave_max(float v) {
 // passes and all their loads are issued before the first use (a decode row is a few KB: one memory round trip).
 constexpr int kNormGroups = 4;   // 256 threads x 8 elements x 4 = rows of up to 8192 elements without a re-read
 
-template <bool F16> __device__ inline void ld8(const void *p, size_t i, uint32_t n_left, float (&v)[8]) {
-  if (n_left >= 8) {
+// vec_ok: the row allows 16-byte loads; otherwise (or in the last, short group) the up to 8 elements are loaded singly
+template <bool F16> __device__ inline void ld8(const void *p, size_t i, uint32_t n_left, bool vec_ok, float (&v)[8]) {
+  if (vec_ok && n_left >= 8) {
     if (F16) {
       half8_t h = *reinterpret_cast<const half8_t *>(reinterpret_cast<const half_t *>(p) + i);
 #pragma unroll
@@ -76,7 +85,7 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const void *x, const float
 #pragma unroll
   for (int g = 0; g < kNormGroups; ++g) {
     uint32_t i = (g * 256 + tid) * 8;
-    if (i < dim) ld8<XF16>(x, off + i, aligned ? dim - i : min(dim - i, 7u), v[g]);   // unaligned rows: element loads
+    if (i < dim) ld8<XF16>(x, off + i, dim - i, aligned != 0, v[g]);   // unaligned rows: element loads
   }
 #pragma unroll
   for (int g = 0; g < kNormGroups; ++g) {
@@ -127,10 +136,12 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const void *x, const float
 __global__ void __launch_bounds__(256) rope_kv_kernel(const void *q, const void *k, const void *v, int in_f16,
                                                       const uint32_t *params, const float *cosT, const float *sinT,
                                                       half_t *kCache, half_t *vCache, void *qOut, int qout_f16, uint32_t qDim,
-                                                      uint32_t kvDim, uint32_t headDim, uint32_t alignedKvDim) {
+                                                      uint32_t kvDim, uint32_t headDim, uint32_t alignedKvDim,
+                                                      uint32_t maxPositions) {
   const uint32_t gid = blockIdx.x * 256 + threadIdx.x, halfDim = headDim / 2;
   if (gid >= qDim + 2 * kvDim) return;
   const uint32_t pos = params[0];
+  if (pos >= maxPositions) return;   // past the caches and the tables: nothing is read or written
   const float *c = cosT + (size_t)pos * halfDim, *s = sinT + (size_t)pos * halfDim;
   auto rot = [&](const void *src, uint32_t i) {
     uint32_t d = i % headDim;
@@ -386,6 +397,128 @@ __global__ void __launch_bounds__(1024) argmax_kernel(const void *x, int x_f16, 
   }
 }
 
+// ---- greedy sampling after the matmul that produced the logits ----
+// One workgroup.  The matmul left, per group of 8 vocabulary rows, the largest logit and its row (ArgmaxPart); this
+// kernel applies the repetition penalty to the listed tokens (RepetitionPenalty.cu:19-41: logit > 0 ? logit / f :
+// logit * f, written back to the logits), re-derives the groups whose winner was one of them, and reduces.  Without
+// parts (parts == nullptr) it scans the logits themselves.  List semantics are those of the dense factor vector the
+// runner fills (llama.cpp:2566-2592): a token listed several times is penalised once, with the factor of its last entry.
+constexpr uint32_t kMaxPenalized = 1024;
+
+__device__ inline void better(float v, uint32_t i, float &best, uint32_t &idx) {
+  if (v > best || (v == best && i < idx)) {
+    best = v;
+    idx = i;
+  }
+}
+
+__global__ void __launch_bounds__(1024) argmax_finish_kernel(const ArgmaxPart *parts, void *logits, int x_f16, uint32_t n,
+                                                             const int32_t *pen_tokens, const float *pen_factors,
+                                                             uint32_t n_pen, uint32_t *out) {
+  __shared__ int32_t ptok[kMaxPenalized];
+  __shared__ float pval[kMaxPenalized];   // the penalised logit of an effective entry
+  __shared__ float bv[16];
+  __shared__ uint32_t bi[16];
+  const uint32_t tid = threadIdx.x;
+  float best = -INFINITY;
+  uint32_t idx = 0xFFFFFFFFu;
+  if (tid < n_pen) ptok[tid] = pen_tokens[tid];
+  __syncthreads();
+  if (tid < n_pen) {
+    const int32_t t = ptok[tid];
+    bool effective = t >= 0 && (uint32_t)t < n;
+    for (uint32_t k = tid + 1; effective && k < n_pen; ++k) effective = ptok[k] != t;   // a later entry of the same token wins
+    float v = 0.0f;
+    if (effective) {
+      const float l = ld_act(logits, x_f16, (size_t)t), f = pen_factors[tid];
+      v = l > 0.0f ? l / f : l * f;
+      st_act(logits, x_f16, (size_t)t, v);
+      if (x_f16) v = (float)(half_t)v;   // as stored
+    }
+    __syncthreads();            // every entry has read its token before any is marked
+    if (!effective) ptok[tid] = -1;
+    pval[tid] = v;
+  } else {
+    __syncthreads();
+  }
+  __syncthreads();
+  // value of row r as the penalised logits hold it: listed rows from the table above (their stores may not be
+  // visible to the other waves yet), all others from memory
+  auto row_value = [&](uint32_t r) {
+    for (uint32_t k = 0; k < n_pen; ++k)
+      if (ptok[k] == (int32_t)r) return pval[k];
+    return ld_act(logits, x_f16, (size_t)r);
+  };
+  if (parts) {
+    const uint32_t ngroups = (n + 7) / 8;
+    constexpr int kInFlight = 8;   // pairs requested together: one memory round trip per 8192 groups instead of one per 1024
+    for (uint32_t g0 = tid; g0 < ngroups; g0 += 1024 * kInFlight) {
+      ArgmaxPart p[kInFlight];
+#pragma unroll
+      for (int u = 0; u < kInFlight; ++u) p[u] = parts[min(g0 + u * 1024, ngroups - 1)];
+#pragma unroll
+      for (int u = 0; u < kInFlight; ++u) {
+        const uint32_t g = g0 + u * 1024;
+        if (g >= ngroups) break;
+        bool listed = false;
+        for (uint32_t k = 0; k < n_pen; ++k) listed |= ptok[k] >= 0 && ((uint32_t)ptok[k] >> 3) == g;
+        if (!listed) {
+          better(p[u].value, p[u].index, best, idx);
+        } else {
+          for (uint32_t r = g * 8; r < min(n, g * 8 + 8); ++r) better(row_value(r), r, best, idx);
+        }
+      }
+    }
+  } else {
+    for (uint32_t r = tid; r < n; r += 1024) better(n_pen ? row_value(r) : ld_act(logits, x_f16, (size_t)r), r, best, idx);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    float ov = __shfl_xor(best, o);
+    uint32_t oi = __shfl_xor(idx, o);
+    better(ov, oi, best, idx);
+  }
+  if ((tid & 63) == 0) {
+    bv[tid >> 6] = best;
+    bi[tid >> 6] = idx;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < 16; ++w) better(bv[w], bi[w], best, idx);
+    out[0] = idx;
+  }
+}
+
+// ---- RepetitionPenaltyOpNode on a dense factor vector (RepetitionPenalty.cu:19-41) ----
+__global__ void __launch_bounds__(256) repetition_penalty_kernel(const float *logits, const float *factors, float *out, uint32_t n) {
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const float l = logits[i], f = factors[i];
+  out[i] = l > 0.0f ? l / f : l * f;
+}
+
+// ---- EmbeddingCol (operators/impl/memory/EmbeddingCol.cu:16-44): gather from a table kept column-wise ----
+// format 0: fp16 table; 1: int8 table with fp16 scales per 32 dims (the loader's separated Q8_0 tensors)
+__global__ void __launch_bounds__(256) embedding_col_kernel(const uint32_t *indices, const void *matrix, const uint16_t *scales,
+                                                            float *out, uint32_t numIndices, uint32_t embDim,
+                                                            uint32_t vocabStride, uint32_t scaleStride, uint32_t outStride,
+                                                            uint32_t vocab, int format) {
+  const uint32_t gid = blockIdx.x * 256 + threadIdx.x;
+  if (gid >= numIndices * embDim) return;
+  const uint32_t i = gid / embDim, d = gid % embDim, t = indices[i];
+  float v = 0.0f;
+  if (t < vocab) {   // an index past the table reads nothing and yields zero
+    const size_t idx = (size_t)d * vocabStride + t;
+    if (format == 0) {
+      v = f16bits_to_f32(reinterpret_cast<const uint16_t *>(matrix)[idx]);
+    } else {
+      const int b = reinterpret_cast<const int8_t *>(matrix)[idx];
+      v = (float)b * f16bits_to_f32(scales[(size_t)(d >> 5) * scaleStride + t]);
+    }
+  }
+  out[(size_t)i * outStride + d] = v;
+}
+
 static bool bad_dtype(int d) { return d != CUTHIP_F32 && d != CUTHIP_F16; }
 
 }  // namespace cuthip
@@ -412,7 +545,7 @@ int cuthip_rmsnorm(const void *x, int x_dtype, const float *weight, void *out, i
 int cuthip_rope_kv_write(const void *q, const void *k, const void *v, int in_dtype, const uint32_t *runtime_params,
                          const float *cos_table, const float *sin_table, void *k_cache, void *v_cache, void *q_out,
                          int q_out_dtype, uint32_t q_dim, uint32_t kv_dim, uint32_t head_dim, uint32_t aligned_kv_dim,
-                         void *stream) {
+                         uint32_t max_positions, void *stream) {
   if (!q || !k || !v || !runtime_params || !cos_table || !sin_table || !k_cache || !v_cache || !q_out || head_dim == 0 ||
       head_dim % 2 || q_dim % head_dim || kv_dim % head_dim || aligned_kv_dim < kv_dim || bad_dtype(in_dtype) ||
       bad_dtype(q_out_dtype)) {
@@ -422,7 +555,7 @@ int cuthip_rope_kv_write(const void *q, const void *k, const void *v, int in_dty
   uint32_t total = q_dim + 2 * kv_dim;
   hipLaunchKernelGGL(rope_kv_kernel, dim3((total + 255) / 256), dim3(256), 0, (hipStream_t)stream, q, k, v,
                      in_dtype == CUTHIP_F16, runtime_params, cos_table, sin_table, (half_t *)k_cache, (half_t *)v_cache, q_out,
-                     q_out_dtype == CUTHIP_F16, q_dim, kv_dim, head_dim, aligned_kv_dim);
+                     q_out_dtype == CUTHIP_F16, q_dim, kv_dim, head_dim, aligned_kv_dim, max_positions);
   return check_hip(hipGetLastError(), "rope launch");
 }
 
@@ -452,12 +585,12 @@ static int attn_check_args(const char *who, const void *q, int q_dtype, const vo
 // The two launches of the split-context attention; `partial` holds cuthip_attn_decode_workspace_bytes() bytes.
 static int attn_launch(const void *q, int q_dtype, const void *k_cache, const void *v_cache, const uint32_t *runtime_params,
                        void *out, int out_dtype, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
-                       uint32_t aligned_kv_dim, float scale, uint32_t max_seq_len, float *partial, hipStream_t s) {
+                       uint32_t aligned_kv_dim, float scale, uint32_t max_seq_len, void *partial, hipStream_t s) {
   uint32_t nsplit = (max_seq_len + kAttnChunk - 1) / kAttnChunk;
   auto partial_kernel = head_dim == 128 ? attn_partial_kernel<128> : attn_partial_kernel<0>;
   hipLaunchKernelGGL(partial_kernel, dim3(n_kv_heads, nsplit), dim3(256), 0, s, q, q_dtype == CUTHIP_F16,
-                     (const half_t *)k_cache, (const half_t *)v_cache, runtime_params, partial, n_heads, n_kv_heads, head_dim,
-                     aligned_kv_dim, scale, nsplit, max_seq_len);
+                     (const half_t *)k_cache, (const half_t *)v_cache, runtime_params, (float *)partial, n_heads, n_kv_heads,
+                     head_dim, aligned_kv_dim, scale, nsplit, max_seq_len);
   if (int rc = check_hip(hipGetLastError(), "attention launch")) return rc;
   hipLaunchKernelGGL(attn_merge_kernel, dim3(n_heads), dim3(128), 0, s, (const float *)partial, runtime_params, out,
                      out_dtype == CUTHIP_F16, head_dim, nsplit);
@@ -471,13 +604,14 @@ int cuthip_attn_decode(const void *q, int q_dtype, const void *k_cache, const vo
   if (int rc = attn_check_args("cuthip_attn_decode", q, q_dtype, k_cache, v_cache, runtime_params, out, out_dtype, n_heads,
                                n_kv_heads, head_dim, aligned_kv_dim, max_seq_len))
     return rc;
-  if (!workspace || workspace_bytes < cuthip_attn_decode_workspace_bytes(n_heads, head_dim, max_seq_len)) {
+  if (!workspace || (uintptr_t)workspace % 4 != 0 ||
+      workspace_bytes < cuthip_attn_decode_workspace_bytes(n_heads, head_dim, max_seq_len)) {
     set_error("cuthip_attn_decode: workspace of %zu bytes, need %zu", workspace ? workspace_bytes : (size_t)0,
               cuthip_attn_decode_workspace_bytes(n_heads, head_dim, max_seq_len));
     return CUTHIP_ERR_INVALID;
   }
   return attn_launch(q, q_dtype, k_cache, v_cache, runtime_params, out, out_dtype, n_heads, n_kv_heads, head_dim,
-                     aligned_kv_dim, scale, max_seq_len, (float *)workspace, (hipStream_t)stream);
+                     aligned_kv_dim, scale, max_seq_len, workspace, (hipStream_t)stream);
 }
 
 }  // extern "C"
@@ -517,6 +651,7 @@ extern "C" {
 
 size_t cuthip_attn_decode_static_max_bytes(void) { return kAttnStaticBytes; }
 
+
 int cuthip_attn_decode_static(const void *q, int q_dtype, const void *k_cache, const void *v_cache,
                               const uint32_t *runtime_params, void *out, int out_dtype, uint32_t n_heads, uint32_t n_kv_heads,
                               uint32_t head_dim, uint32_t aligned_kv_dim, float scale, uint32_t max_seq_len, void *stream) {
@@ -535,7 +670,7 @@ int cuthip_attn_decode_static(const void *q, int q_dtype, const void *k_cache, c
   // every split record of this call's launch shape is written before the merge reads it, so nothing of an earlier
   // call's contents is read and nothing needs clearing
   return attn_launch(q, q_dtype, k_cache, v_cache, runtime_params, out, out_dtype, n_heads, n_kv_heads, head_dim,
-                     aligned_kv_dim, scale, max_seq_len, (float *)ptr, (hipStream_t)stream);
+                     aligned_kv_dim, scale, max_seq_len, ptr, (hipStream_t)stream);
 }
 
 int cuthip_silu_mul(const void *gate_up, int in_dtype, void *out, int out_dtype, uint32_t n, void *stream) {
@@ -558,3 +693,55 @@ int cuthip_argmax(const void *x, int x_dtype, uint32_t n, uint32_t *out_index, v
 }
 
 }  // extern "C"
+
+extern "C" {
+
+int cuthip_argmax_penalized(void *logits, int x_dtype, uint32_t n, const int32_t *pen_tokens, const float *pen_factors,
+                            uint32_t n_pen, uint32_t *out_index, void *stream) {
+  if (!logits || !out_index || n == 0 || bad_dtype(x_dtype) || n_pen > kMaxPenalized || (n_pen && (!pen_tokens || !pen_factors))) {
+    set_error("cuthip_argmax_penalized: bad argument (n %u, %u penalised tokens, at most %u)", n, n_pen, kMaxPenalized);
+    return CUTHIP_ERR_INVALID;
+  }
+  hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const ArgmaxPart *)nullptr, logits,
+                     x_dtype == CUTHIP_F16, n, pen_tokens, pen_factors, n_pen, out_index);
+  return check_hip(hipGetLastError(), "argmax launch");
+}
+
+int cuthip_repetition_penalty(const float *logits, const float *factors, float *out, uint32_t n, void *stream) {
+  if (!logits || !factors || !out) {
+    set_error("cuthip_repetition_penalty: null argument");
+    return CUTHIP_ERR_INVALID;
+  }
+  if (n == 0) return CUTHIP_OK;
+  hipLaunchKernelGGL(repetition_penalty_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, logits, factors, out, n);
+  return check_hip(hipGetLastError(), "repetition penalty launch");
+}
+
+int cuthip_embedding_col(const uint32_t *indices, const void *matrix, const uint16_t *scales, float *out, uint32_t num_indices,
+                         uint32_t emb_dim, uint32_t vocab_stride, uint32_t scale_stride, uint32_t out_stride, uint32_t vocab,
+                         int format, void *stream) {
+  if (!indices || !matrix || !out || (format != 0 && format != 1) || (format == 1 && !scales) || out_stride < emb_dim ||
+      vocab > vocab_stride || (format == 1 && vocab > scale_stride) || (uint64_t)num_indices * emb_dim > 0xFFFFFFFFull) {
+    set_error("cuthip_embedding_col: bad argument (format %d, emb_dim %u, vocab %u, strides %u %u %u)", format, emb_dim, vocab,
+              vocab_stride, scale_stride, out_stride);
+    return CUTHIP_ERR_INVALID;
+  }
+  const uint32_t total = num_indices * emb_dim;
+  if (total == 0) return CUTHIP_OK;
+  hipLaunchKernelGGL(embedding_col_kernel, dim3((total + 255) / 256), dim3(256), 0, (hipStream_t)stream, indices, matrix, scales,
+                     out, num_indices, emb_dim, vocab_stride, scale_stride, out_stride, vocab, format);
+  return check_hip(hipGetLastError(), "embedding launch");
+}
+
+}  // extern "C"
+
+namespace cuthip {
+// second launch of cuthip_matmul_gguf_argmax (gemv.hip): arguments validated there
+int launch_argmax_finish(const ArgmaxPart *parts, void *logits, int x_f16, uint32_t n, const int32_t *pen_tokens,
+                         const float *pen_factors, uint32_t n_pen, uint32_t *out_index, hipStream_t stream) {
+  hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(1024), 0, stream, parts, logits, x_f16, n, pen_tokens, pen_factors,
+                     n_pen, out_index);
+  return check_hip(hipGetLastError(), "argmax launch");
+}
+uint32_t max_penalized() { return kMaxPenalized; }
+}  // namespace cuthip

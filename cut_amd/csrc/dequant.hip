@@ -175,6 +175,52 @@ __device__ __forceinline__ void dequant_slot(const uint8_t *__restrict__ blocks,
   }
 }
 
+// Embedding gather on GGUF blocks: out[i, :] = dequant(row token_ids[i]); a workgroup covers 2048 elements of one
+// gathered row.  A token id past the table yields a zero row.
+template <int FMT, bool F16OUT, bool VEC>
+__global__ void __launch_bounds__(256)
+embedding_rows_kernel(const uint8_t *__restrict__ blocks, const uint32_t *__restrict__ token_ids, void *__restrict__ out,
+                      uint32_t n_rows, uint32_t cols, uint32_t out_stride, uint32_t chunks_per_row, size_t row_bytes) {
+  const uint32_t i = blockIdx.x / chunks_per_row, chunk = blockIdx.x - i * chunks_per_row;
+  const uint32_t col = (chunk * 256u + threadIdx.x) * 8u;
+  if (col >= cols) return;
+  const uint32_t tok = token_ids[i];
+  uint8_t *dst_row = reinterpret_cast<uint8_t *>(out) + (size_t)i * out_stride * (F16OUT ? 2 : 4);
+  if (tok >= n_rows) {
+    for (int e = 0; e < 8; ++e) {
+      if (F16OUT) reinterpret_cast<uint16_t *>(dst_row)[col + e] = 0;
+      else reinterpret_cast<float *>(dst_row)[col + e] = 0.0f;
+    }
+    return;
+  }
+  dequant_slot<FMT, F16OUT, VEC, true>(blocks + (size_t)tok * row_bytes, dst_row, 0, col, out_stride, row_bytes);
+}
+
+template <int FMT>
+static int launch_embedding(const void *blocks, const uint32_t *token_ids, void *out, int out_dtype, uint32_t n_ids,
+                            uint32_t n_rows, uint32_t cols, uint32_t out_stride, hipStream_t stream) {
+  const size_t row_bytes = (size_t)(cols / Fmt<FMT>::elems) * Fmt<FMT>::bytes;
+  const uint32_t chunks = (cols / 8 + 255) / 256;
+  const uint64_t grid = (uint64_t)n_ids * chunks;
+  if (grid > 0x7FFFFFFFull) {
+    set_error("cuthip_embedding_rows: too many rows for one launch");
+    return CUTHIP_ERR_INVALID;
+  }
+  const bool f16 = out_dtype == CUTHIP_F16;
+  const bool vec = ((uintptr_t)out % 16 == 0) && ((out_stride * (f16 ? 2 : 4)) % 16 == 0);
+  const uint8_t *src = reinterpret_cast<const uint8_t *>(blocks);
+  dim3 g((uint32_t)grid), b(256);
+#define CUTHIP_LAUNCH(F16, VEC) \
+  hipLaunchKernelGGL((embedding_rows_kernel<FMT, F16, VEC>), g, b, 0, stream, src, token_ids, out, n_rows, cols, out_stride, chunks, row_bytes)
+  if (f16) {
+    if (vec) CUTHIP_LAUNCH(true, true); else CUTHIP_LAUNCH(true, false);
+  } else {
+    if (vec) CUTHIP_LAUNCH(false, true); else CUTHIP_LAUNCH(false, false);
+  }
+#undef CUTHIP_LAUNCH
+  return check_hip(hipGetLastError(), "embedding launch");
+}
+
 template <int FMT>
 static int launch_dequant(const void *blocks, void *out, int out_dtype, uint32_t rows, uint32_t cols,
                           uint32_t out_stride, hipStream_t stream, int keep_cached = 0) {
@@ -258,5 +304,27 @@ extern "C" int cuthip_dequant(int fmt, const void *blocks, void *out, int out_dt
   case CUTHIP_Q4_0: return launch_dequant<CUTHIP_Q4_0>(blocks, out, out_dtype, rows, cols, out_stride, s);
   case CUTHIP_Q4_K: return launch_dequant<CUTHIP_Q4_K>(blocks, out, out_dtype, rows, cols, out_stride, s);
   default: return launch_dequant<CUTHIP_Q6_K>(blocks, out, out_dtype, rows, cols, out_stride, s);
+  }
+}
+
+extern "C" int cuthip_embedding_rows(int fmt, const void *blocks, const uint32_t *token_ids, uint32_t n_ids, uint32_t n_rows,
+                                     uint32_t dim, void *out, int out_dtype, uint32_t out_stride, void *stream) {
+  using namespace cuthip;
+  if (fmt < CUTHIP_Q8_0 || fmt > CUTHIP_Q6_K || (out_dtype != CUTHIP_F32 && out_dtype != CUTHIP_F16)) {
+    set_error("cuthip_embedding_rows: unknown format %d or output dtype %d", fmt, out_dtype);
+    return CUTHIP_ERR_INVALID;
+  }
+  if (n_ids == 0 || dim == 0) return CUTHIP_OK;
+  if (!blocks || !token_ids || !out || dim % fmt_elems(fmt) != 0 || out_stride < dim || (uintptr_t)blocks % 2 != 0) {
+    set_error("cuthip_embedding_rows: bad argument (dim %u must be a multiple of the block size %d, out_stride %u >= dim)", dim,
+              fmt_elems(fmt), out_stride);
+    return CUTHIP_ERR_INVALID;
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  switch (fmt) {
+  case CUTHIP_Q8_0: return launch_embedding<CUTHIP_Q8_0>(blocks, token_ids, out, out_dtype, n_ids, n_rows, dim, out_stride, s);
+  case CUTHIP_Q4_0: return launch_embedding<CUTHIP_Q4_0>(blocks, token_ids, out, out_dtype, n_ids, n_rows, dim, out_stride, s);
+  case CUTHIP_Q4_K: return launch_embedding<CUTHIP_Q4_K>(blocks, token_ids, out, out_dtype, n_ids, n_rows, dim, out_stride, s);
+  default: return launch_embedding<CUTHIP_Q6_K>(blocks, token_ids, out, out_dtype, n_ids, n_rows, dim, out_stride, s);
   }
 }

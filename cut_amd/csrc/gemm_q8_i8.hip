@@ -259,6 +259,13 @@ int cuthip_matmul_q8_i8(const void *W, const void *A, int a_dtype, void *C, int 
     set_error("cuthip_matmul_q8_i8: binary epilogue without D");
     return CUTHIP_ERR_INVALID;
   }
+  if (int rc = check_epilogue_op("cuthip_matmul_q8_i8", epilogue, epilogue_op)) return rc;
+  if (epilogue_op_long(epilogue, epilogue_op)) {
+    if (int rc = cuthip_matmul_q8_i8(W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, CUTHIP_EPI_NONE, 0, nullptr, workspace,
+                                     workspace_bytes, stream))
+      return rc;
+    return launch_long_epilogue(C, c_dtype == CUTHIP_F16, M, N, strideC, epilogue, epilogue_op, D, (hipStream_t)stream);
+  }
   const size_t need = cuthip_matmul_q8_i8_workspace_bytes(M, K);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15u)) {
     set_error("cuthip_matmul_q8_i8: workspace of %zu bytes (16-byte aligned) needed, got %zu", need, workspace_bytes);

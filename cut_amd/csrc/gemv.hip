@@ -115,6 +115,7 @@ int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C,
                       uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream,
                       int use_blaslt);
 bool blaslt_available();
+bool blaslt_preferred();
 size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16);
 
 static int launch_gemv(int fmt, const GemvParams &p, hipStream_t stream) {
@@ -211,6 +212,14 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
   using namespace cuthip;
   if (int rc = check_matmul_args(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, D))
     return rc > 0 ? CUTHIP_OK : rc;
+  if (int rc = check_epilogue_op("cuthip_matmul_gguf", epilogue, epilogue_op)) return rc;
+  if (epilogue_op_long(epilogue, epilogue_op)) {   // unfused matmul, then the operator as an elementwise launch
+    if (int rc = cuthip_matmul_gguf(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, CUTHIP_EPI_NONE, 0, nullptr,
+                                    variant, stream))
+      return rc;
+    return launch_long_epilogue(C, c_dtype == CUTHIP_F16, M, N, strideC, epilogue, epilogue_op, D,
+                                reinterpret_cast<hipStream_t>(stream));
+  }
   int nvar = cuthip_variant_count(CUTHIP_OP_MATMUL_GGUF);
   if (variant < -1 || variant >= nvar) {
     set_error("cuthip_matmul_gguf: unknown variant index %d (table has %d)", variant, nvar);
@@ -221,7 +230,8 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
     set_error("cuthip_matmul_gguf: K too large");
     return CUTHIP_ERR_INVALID;
   }
-  // variant table: 0 streaming GEMV (M <= 8), 1 skinny passes of 32 rows, 2 LDS-tiled GEMM
+  // variant table: 0 streaming GEMV (M <= 8; beyond, as -1), 1 skinny passes of 32 rows, 2 LDS-tiled GEMM,
+  // 3 the 8-row GEMV, 4 / 5 dequantize + dense GEMM (workspace entry point only)
   Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
   if (epilogue == CUTHIP_EPI_SWIGLU_PAIRS && variant != -1 && variant != 3) {
     set_error("cuthip_matmul_gguf: the SwiGLU row-pair epilogue exists in variant 3 only (got variant %d)", variant);
@@ -231,10 +241,8 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
     set_error("cuthip_matmul_gguf: variants 4 and 5 (dequantize, then dense GEMM) need a workspace: call cuthip_matmul_gguf_ws");
     return CUTHIP_ERR_INVALID;
   }
-  if (variant == 0 && M > 8) {
-    set_error("cuthip_matmul_gguf: variant 0 (GEMV) handles M <= 8, got M = %u", M);
-    return CUTHIP_ERR_INVALID;
-  }
+  // the table's default entry is valid for every M: beyond the 8 rows its GEMV takes it is the choice by shape
+  if (variant == 0 && M > 8) variant = -1;
   // 9-40 rows, automatic choice: passes of 8 rows through the decode kernels.  Measured on 14336 x 4096: 14 us per
   // pass, against 69-87 us for the 32-row skinny kernel and 73-80 us for one launch of the tiled GEMM, whose cost
   // is the decode of the whole weight matrix whatever M is.
@@ -296,6 +304,17 @@ int cuthip_matmul_gguf_carry(int fmt, const void *W, const void *A, int a_dtype,
   using namespace cuthip;
   const uint32_t n_out = epilogue == CUTHIP_EPI_SWIGLU_PAIRS ? N / 2 : N;
   if (int rc = check_matmul_args(fmt, W, A, a_dtype, C, c_dtype, 1, K, N, K, n_out, epilogue, D)) return rc > 0 ? CUTHIP_OK : rc;
+  if (int rc = check_epilogue_op("cuthip_matmul_gguf_carry", epilogue, epilogue_op)) return rc;
+  if (epilogue_op_long(epilogue, epilogue_op)) {
+    if (carry && (carry->next_norm_weight || carry->next_x16 || carry->next_sumsq_parts)) {
+      set_error("cuthip_matmul_gguf_carry: operator %d runs as a launch of its own after the matmul and cannot feed the "
+                "producer side of a carried RMSNorm", epilogue_op);
+      return CUTHIP_ERR_INVALID;
+    }
+    if (int rc = cuthip_matmul_gguf_carry(fmt, W, A, a_dtype, C, c_dtype, K, N, CUTHIP_EPI_NONE, 0, nullptr, carry, stream))
+      return rc;
+    return launch_long_epilogue(C, c_dtype == CUTHIP_F16, 1, N, N, epilogue, epilogue_op, D, reinterpret_cast<hipStream_t>(stream));
+  }
   GemvParams p = gemv_params(fmt, W, A, a_dtype, C, c_dtype, 1, K, N, K, n_out,
                              Epilogue{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr});
   if (!apply_carry(p, carry, epilogue != CUTHIP_EPI_SWIGLU_PAIRS)) {
@@ -310,6 +329,60 @@ int cuthip_matmul_gguf_carry(int fmt, const void *W, const void *A, int a_dtype,
     return CUTHIP_ERR_INVALID;
   }
   return rc;
+}
+
+}  // extern "C"
+
+namespace cuthip {
+int launch_argmax_finish(const ArgmaxPart *parts, void *logits, int x_f16, uint32_t n, const int32_t *pen_tokens,
+                         const float *pen_factors, uint32_t n_pen, uint32_t *out_index, hipStream_t stream);
+uint32_t max_penalized();
+}
+
+extern "C" {
+
+size_t cuthip_matmul_gguf_argmax_workspace_bytes(uint32_t N) { return (size_t)((N + 7) / 8) * sizeof(cuthip::ArgmaxPart); }
+
+int cuthip_matmul_gguf_argmax(int fmt, const void *W, const void *A, int a_dtype, void *logits, int c_dtype, uint32_t K, uint32_t N,
+                              const cuthip_norm_carry_t *carry, const int32_t *pen_tokens, const float *pen_factors,
+                              uint32_t n_pen, void *workspace, size_t workspace_bytes, uint32_t *out_index, void *stream) {
+  using namespace cuthip;
+  if (int rc = check_matmul_args(fmt, W, A, a_dtype, logits, c_dtype, 1, K, N, K, N, CUTHIP_EPI_NONE, nullptr)) {
+    if (rc > 0) {
+      set_error("cuthip_matmul_gguf_argmax: empty vocabulary");
+      return CUTHIP_ERR_INVALID;
+    }
+    return rc;
+  }
+  if (!out_index || n_pen > max_penalized() || (n_pen && (!pen_tokens || !pen_factors))) {
+    set_error("cuthip_matmul_gguf_argmax: out_index missing, or %u penalised tokens without their arrays / beyond %u", n_pen,
+              max_penalized());
+    return CUTHIP_ERR_INVALID;
+  }
+  if (carry && (carry->next_norm_weight || carry->next_x16 || carry->next_sumsq_parts)) {
+    set_error("cuthip_matmul_gguf_argmax: only the consumer fields of the carried RMSNorm apply here");
+    return CUTHIP_ERR_INVALID;
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  GemvParams p = gemv_params(fmt, W, A, a_dtype, logits, c_dtype, 1, K, N, K, N, Epilogue{CUTHIP_EPI_NONE, 0, nullptr});
+  apply_carry(p, carry, false);
+  // the arg-max rides in the matmul's epilogue where the 8-row GEMV runs one K range per wave (any vocabulary-sized N)
+  // and the caller brought room for the per-group winners; otherwise the logits are scanned by the second launch
+  const bool fused = pick_rows8_shape(N, p.nsteps).kw == 1 && workspace && (uintptr_t)workspace % 8 == 0 &&
+                     workspace_bytes >= cuthip_matmul_gguf_argmax_workspace_bytes(N);
+  if (fused) p.argmax_parts = reinterpret_cast<ArgmaxPart *>(workspace);
+  bool taken = false;
+  int rc = launch_rows8_any(fmt, p, s, &taken);
+  if (rc) return rc;
+  if (!taken) {   // activations beyond the LDS budget of the 8-row GEMV: the fallback kernel, no carried norm
+    if (carry && carry->sumsq_parts) {
+      set_error("cuthip_matmul_gguf_argmax: K = %u does not fit the LDS budget of the 8-row GEMV (needed for the carried norm)", K);
+      return CUTHIP_ERR_INVALID;
+    }
+    p.argmax_parts = nullptr;
+    if (int rc2 = launch_gemv(fmt, p, s)) return rc2;
+  }
+  return launch_argmax_finish(p.argmax_parts, logits, c_dtype == CUTHIP_F16, N, pen_tokens, pen_factors, n_pen, out_index, s);
 }
 
 int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, int fmt_b, const void *Wb, uint32_t Nb,
@@ -338,6 +411,7 @@ int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, in
     ra.q_dim = rope->q_dim;
     ra.head_dim = hd;
     ra.kv_stride = rope->aligned_kv_dim;
+    ra.max_pos = rope->max_positions;
     rb = ra;
     rb.mode = 2;
     if (!Ca) Ca = rope->q_out;   // the plain outputs are not written in this mode
@@ -404,6 +478,14 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
                               stream);
   if (int rc = check_matmul_args(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, D))
     return rc > 0 ? CUTHIP_OK : rc;
+  if (int rc = check_epilogue_op("cuthip_matmul_gguf_ws", epilogue, epilogue_op)) return rc;
+  if (epilogue_op_long(epilogue, epilogue_op)) {
+    if (int rc = cuthip_matmul_gguf_ws(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, CUTHIP_EPI_NONE, 0, nullptr,
+                                       variant, workspace, workspace_bytes, stream))
+      return rc;
+    return launch_long_epilogue(C, c_dtype == CUTHIP_F16, M, N, strideC, epilogue, epilogue_op, D,
+                                reinterpret_cast<hipStream_t>(stream));
+  }
   const int a_f16 = a_dtype == CUTHIP_F16;
   // 9..383 rows with the vendor GEMM at hand: dequantize + hipBLASLt against what the automatic choice would run
   // otherwise, by a cost model fitted to a sweep over the FFN / attention shapes of an 8B model (microseconds;
@@ -412,7 +494,7 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   // 14 + N K x 0.65e-6 (0.95e-6 once the fp16 copy outgrows the 256 MB cache) + 2 M N K / 1.6 PFLOP/s.
   if (variant == -1 && M > 8 && M < 384 && epilogue == CUTHIP_EPI_NONE && workspace && (uintptr_t)workspace % 256 == 0 &&
       dense_gemm_fits(M, K, N, strideA, a_f16, A) && workspace_bytes >= dense_gemm_workspace(M, K, N, a_f16) &&
-      blaslt_available()) {
+      blaslt_preferred()) {
     const double nk = (double)N * K;
     const double t5 = 14.0 + nk * (nk <= 64e6 ? 0.65e-6 : 0.95e-6) + 2.0 * M * nk / 1.6e9;
     double other;
@@ -464,7 +546,7 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   const bool ws_ok = workspace && (uintptr_t)workspace % 256 == 0 && workspace_bytes >= need;
   // with the vendor GEMM behind the dequantization the two-pass path pays earlier: 25 us of dequantization for an FFN
   // matrix against a single-launch GEMM that decodes the weights once per 128 rows (M = 512, N = 14336: 86 us against 110)
-  const bool lt_ok = variant == -1 && epilogue == CUTHIP_EPI_NONE && fits && ws_ok && blaslt_available();
+  const bool lt_ok = variant == -1 && epilogue == CUTHIP_EPI_NONE && fits && ws_ok && blaslt_preferred();
   if (variant == -1 && !((dense_gemm_preferred(M, K, N) || (lt_ok && M >= 384)) && fits && ws_ok))
     return cuthip_matmul_gguf(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, -1,
                               stream);
@@ -511,6 +593,14 @@ int cuthip_matmul_dense_f16(const void *W16, const void *A, int a_dtype, void *C
     set_error("cuthip_matmul_dense_f16: binary epilogue without D");
     return CUTHIP_ERR_INVALID;
   }
+  if (int rc = check_epilogue_op("cuthip_matmul_dense_f16", epilogue, epilogue_op)) return rc;
+  if (epilogue_op_long(epilogue, epilogue_op)) {
+    if (int rc = cuthip_matmul_dense_f16(W16, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, CUTHIP_EPI_NONE, 0, nullptr,
+                                         workspace, workspace_bytes, stream))
+      return rc;
+    return launch_long_epilogue(C, c_dtype == CUTHIP_F16, M, N, strideC, epilogue, epilogue_op, D,
+                                reinterpret_cast<hipStream_t>(stream));
+  }
   const int a_f16 = a_dtype == CUTHIP_F16;
   if (!dense_gemm_fits(M, K, N, strideA, a_f16, A) || (uintptr_t)W16 % 256 != 0) {
     set_error("cuthip_matmul_dense_f16: needs K a multiple of 128, 256-byte aligned weights, 16-byte aligned rows of A and "
@@ -523,7 +613,7 @@ int cuthip_matmul_dense_f16(const void *W16, const void *A, int a_dtype, void *C
               workspace ? workspace_bytes : (size_t)0);
     return CUTHIP_ERR_INVALID;
   }
-  const int use_blaslt = (epilogue == CUTHIP_EPI_NONE && blaslt_available()) ? 2 : 0;
+  const int use_blaslt = (epilogue == CUTHIP_EPI_NONE && blaslt_preferred()) ? 2 : 0;
   Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
   return launch_dense_gemm(-1, W16, A, a_f16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC, epi, workspace,
                            reinterpret_cast<hipStream_t>(stream), use_blaslt);
@@ -540,6 +630,13 @@ int cuthip_matmul_gguf_pro(int fmt, const void *W, const void *A, int a_dtype, v
       epilogue < CUTHIP_EPI_NONE || epilogue > CUTHIP_EPI_BINARY || (epilogue == CUTHIP_EPI_BINARY && !D)) {
     set_error("cuthip_matmul_gguf_pro: bad argument (format %d, K %u, N %u, epilogue %d)", fmt, K, N, epilogue);
     return CUTHIP_ERR_INVALID;
+  }
+  if (int rc = check_epilogue_op("cuthip_matmul_gguf_pro", epilogue, epilogue_op)) return rc;
+  if (epilogue_op_long(epilogue, epilogue_op)) {
+    if (int rc = cuthip_matmul_gguf_pro(fmt, W, A, a_dtype, C, c_dtype, K, N, CUTHIP_EPI_NONE, 0, nullptr, prologue, norm_weight,
+                                        eps, stream))
+      return rc;
+    return launch_long_epilogue(C, c_dtype == CUTHIP_F16, 1, N, N, epilogue, epilogue_op, D, reinterpret_cast<hipStream_t>(stream));
   }
   if (prologue == CUTHIP_PRO_RMSNORM) {
     if (!norm_weight || (uintptr_t)norm_weight % 16 != 0 || K % 8 != 0 || (uintptr_t)A % 16 != 0) {

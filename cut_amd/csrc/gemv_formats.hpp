@@ -18,6 +18,12 @@ struct RopeAppend {
   int q_out_f16 = 0;
   half_t *k_cache = nullptr, *v_cache = nullptr;
   uint32_t q_dim = 0, head_dim = 0, kv_stride = 0;
+  uint32_t max_pos = 0;   // rows of the caches and tables; a position at or beyond it writes nothing
+};
+
+struct ArgmaxPart {
+  float value;      // -inf if the group holds no row
+  uint32_t index;   // row of the first maximum of the group
 };
 
 struct GemvParams {
@@ -43,6 +49,10 @@ struct GemvParams {
   const float *next_norm_w = nullptr;
   half_t *next_x16 = nullptr;
   float *next_sumsq_parts = nullptr;
+  // Greedy sampling folded into the matmul that produces the logits (8-row GEMV, batch 1, one K range per wave):
+  // every wave also stores the largest of its 8 outputs (as stored in C) and its row index to argmax_parts[n / 8];
+  // a one-workgroup kernel finishes the reduction.
+  ArgmaxPart *argmax_parts = nullptr;
 };
 
 // ---- per-tile configuration -------------------------------------------------

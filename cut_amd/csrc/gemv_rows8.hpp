@@ -79,6 +79,7 @@ __device__ inline float wave_sum_all(float v) {
 // One output row of a matmul with the RoPE / cache-append epilogue: v = this row's product, partner = the
 // neighbouring row's (row ^ 1), cs / sn = the table entries of the pair at the current position.
 __device__ inline void rope_store(const RopeAppend &r, uint32_t row, float v, float partner, float cs, float sn, uint32_t pos) {
+  if (pos >= r.max_pos) return;
   if (r.mode == 2) {
     r.v_cache[(size_t)pos * r.kv_stride + row] = (half_t)v;
     return;
@@ -568,7 +569,7 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
   }
   float pre_cs = 0.0f, pre_sn = 0.0f;
   const uint32_t rope_pos = p.rope.mode ? p.rope.params[0] : 0u;
-  if (pre_ok && p.rope.mode == 1) {
+  if (pre_ok && p.rope.mode == 1 && rope_pos < p.rope.max_pos) {
     const size_t ti = (size_t)rope_pos * (p.rope.head_dim / 2) + ((prow % p.rope.head_dim) >> 1);
     pre_cs = p.rope.cosT[ti];
     pre_sn = p.rope.sinT[ti];
@@ -712,6 +713,8 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
     writer = c.g == 0;
   }
   float carry_sq = 0.0f;
+  float am_v = -INFINITY;          // this lane's candidate for the arg-max of the wave's 8 rows (writer lanes only)
+  uint32_t am_i = 0xFFFFFFFFu;
   // SwiGLU over row pairs: weight rows 2i / 2i+1 are gate_i / up_i, C[m, i] = silu(gate) * up.  The partner row
   // sits four lanes up (same piece, same K half); in the folded path it is the next thread.
   const bool swiglu = p.epi.kind == CUTHIP_EPI_SWIGLU_PAIRS;
@@ -745,9 +748,25 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
               p.next_x16[n0 + r8] = (half_t)(v * p.next_norm_w[n0 + r8]);
               carry_sq = v * v;
             }
+            if (MT == 1) {
+              am_v = p.c_f16 ? (float)(half_t)v : v;   // the value as C holds it
+              am_i = n0 + r8;
+            }
           }
         }
       }
+    }
+    if (MT == 1 && p.argmax_parts) {   // (uniform) largest of the wave's rows, the first one on a tie
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(am_v, o);
+        const uint32_t oi = __shfl_xor(am_i, o);
+        if (ov > am_v || (ov == am_v && oi < am_i)) {
+          am_v = ov;
+          am_i = oi;
+        }
+      }
+      if (lane == 0 && n0 < p.N) p.argmax_parts[n0 / 8] = ArgmaxPart{am_v, am_i};
     }
   } else {
     __syncthreads();   // all waves are done with the staged activations

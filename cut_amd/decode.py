@@ -35,6 +35,7 @@ class DecodeConfig:
     fmt_v: str = "Q6_K"
     fmt_ffn: str = "Q4_K"
     fmt_head: str = "Q6_K"
+    fmt_embd: str = "Q4_K"
 
     @property
     def q_dim(self) -> int:
@@ -59,8 +60,12 @@ class DecodeStep:
     plus 'out_norm' (fp32) and 'head' at the top level."""
 
     def __init__(self, cfg: DecodeConfig, layers: list[dict], out_norm: torch.Tensor, head: torch.Tensor, device="cuda:0",
-                 fuse: int = 4):
-        """fuse: 4 (default) = 3 plus RMSNorm carried across the matmuls (see _step_carry): the producer of the
+                 fuse: int = 4, embedding: torch.Tensor | None = None, penalty_window: int = 0):
+        """embedding: the token-embedding table as GGUF blocks [vocab, hidden] (cfg.fmt_embd); with it a step starts from
+        self.token (the id the previous step sampled, on the device) instead of a caller-filled self.x, so a replayed
+        graph feeds itself.  penalty_window: entries of the repetition-penalty list (self.pen_tokens / self.pen_factors,
+        set by set_penalties; unused entries hold token -1); 0 = plain greedy sampling.
+        fuse: 4 (default) = 3 plus RMSNorm carried across the matmuls (see _step_carry): the producer of the
         residual stream stores x * norm_weight and partial sums of x^2, the consumer scales its result, so neither
         repeats the norm per workgroup and the RMSNorm launches disappear; 3 = SiLU(gate) * up runs in the epilogue of the gate+up matmul (the producer), whose rows
         are interleaved gate_0, up_0, gate_1, ... for it: 'gate_up' is re-laid out once, here, and the layer dicts are
@@ -100,14 +105,40 @@ class DecodeStep:
         self.sin_t = torch.sin(ang).to(f32).to(dev).contiguous()
         self.ws = ops.attn_decode_workspace(c.n_heads, c.head_dim, c.max_ctx, dev)
         self.scale = 1.0 / math.sqrt(c.head_dim)
+        self.embedding = embedding
+        self.head_ws = ops.lm_head_workspace(c.vocab, dev)
+        self.pen_tokens = torch.full((penalty_window,), -1, dtype=torch.int32, device=dev) if penalty_window else None
+        self.pen_factors = torch.ones(penalty_window, dtype=f32, device=dev) if penalty_window else None
+
+    def set_penalties(self, tokens: list[int], penalty: float, suppressed: list[int] = ()) -> None:
+        """Host-side update between graph replays: the recent window at `penalty`, then `suppressed` tokens (end of
+        sequence while a minimum length is enforced) at 1e9, the non-unit entries of the dense factor vector the
+        reference's runner uploads (interface/runner/llama/llama.cpp:2566-2592).  The most recent entries are kept
+        when the list is longer than the window."""
+        cap = self.pen_tokens.numel()
+        pairs = ([(t, penalty) for t in tokens] + [(t, 1e9) for t in suppressed])[-cap:]
+        toks = [t for t, _ in pairs] + [-1] * (cap - len(pairs))
+        facs = [f for _, f in pairs] + [1.0] * (cap - len(pairs))
+        self.pen_tokens.copy_(torch.tensor(toks, dtype=torch.int32))
+        self.pen_factors.copy_(torch.tensor(facs, dtype=torch.float32))
 
     def set_position(self, pos: int) -> None:
         """Host-side update between graph replays (a 8-byte copy; the kernels read it on the device)."""
         self.params.copy_(torch.tensor([pos, pos + 1], dtype=torch.int32))
 
+    def _sample(self) -> None:
+        """Penalty on the listed tokens (if a window was asked for) and the arg-max of the logits."""
+        if self.pen_tokens is not None:
+            ops.argmax_penalized(self.logits, self.token, self.pen_tokens, self.pen_factors)
+        else:
+            ops.argmax(self.logits, self.token)
+
     def step(self) -> None:
-        """Consumes self.x (the embedding of the current token), leaves logits and the arg-max token."""
+        """Consumes self.token through the embedding table (or, without a table, a caller-filled self.x), leaves the
+        logits and the sampled token."""
         c = self.cfg
+        if self.embedding is not None:
+            ops.embedding_rows(self.embedding, c.fmt_embd, self.token, c.vocab, c.hidden, self.x.view(1, -1))
         if self.fuse == 2:
             return self._step_fused()
         if self.fuse == 4:
@@ -141,11 +172,11 @@ class DecodeStep:
                                 d=self.x.view(1, -1))
         ops.rmsnorm(self.x, self.out_norm, c.eps, out=self.xn.view(1, -1))
         ops.matmul_gguf(self.xn, self.head, c.fmt_head, c.vocab, c.hidden, out=self.logits.view(1, -1))
-        ops.argmax(self.logits, self.token)
+        self._sample()
 
     def _step_carry(self) -> None:
         """Six launches per layer (q|k|v with RoPE and cache append, attention, merge, wo, gate+up with SwiGLU, down);
-        only the first RMSNorm of the step is a kernel.  Every matmul that forms the
+        only the first RMSNorm of the step is a kernel, and the arg-max rides in the epilogue of the head matmul.  Every matmul that forms the
         residual stream (wo, w_down) also stores x * next_norm_weight as fp16 and the sum of x^2 over each group of 8
         outputs; the matmul that consumes it adds those partial sums (fixed order) and scales its result by
         rsqrt(sum / hidden + eps).  Producers and consumers alternate, so one array of partial sums serves all."""
@@ -169,8 +200,8 @@ class DecodeStep:
             nxt = self.layers[i + 1]["attn_norm"] if i + 1 < n_layers else self.out_norm
             ops.matmul_gguf_carry(self.act, L["down"], c.fmt_ffn, c.hidden, c.ffn, self.x, binary="add", d=self.x,
                                   carry=ops.norm_carry(next_norm_weight=nxt, next_x16=self.xn, next_sumsq_parts=self.sumsq_parts))
-        ops.matmul_gguf_carry(self.xn, self.head, c.fmt_head, c.vocab, c.hidden, self.logits, carry=consume)
-        ops.argmax(self.logits, self.token)
+        ops.matmul_gguf_argmax(self.xn, self.head, c.fmt_head, c.vocab, c.hidden, self.logits, self.token, carry=consume,
+                               pen_tokens=self.pen_tokens, pen_factors=self.pen_factors, workspace=self.head_ws)
 
     def _step_fused(self) -> None:
         c = self.cfg
@@ -186,4 +217,4 @@ class DecodeStep:
             ops.matmul_gguf_pro(self.x, L["gate_up"], c.fmt_ffn, 2 * c.ffn, c.hidden, self.gu, "rmsnorm", L["ffn_norm"], c.eps)
             ops.matmul_gguf_pro(self.gu, L["down"], c.fmt_ffn, c.hidden, c.ffn, self.x, "swiglu", binary="add", d=self.x)
         ops.matmul_gguf_pro(self.x, self.head, c.fmt_head, c.vocab, c.hidden, self.logits, "rmsnorm", self.out_norm, c.eps)
-        ops.argmax(self.logits, self.token)
+        self._sample()

@@ -16,8 +16,12 @@ Q8_0, Q4_0, Q4_K, Q6_K = 0, 1, 2, 3
 F32, F16 = 0, 1
 OP_DEQUANT, OP_MATMUL_GGUF, OP_MATMUL_Q8, OP_MATMUL_Q4 = 0, 1, 2, 3
 EPI_NONE, EPI_UNARY, EPI_BINARY, EPI_SWIGLU_PAIRS = 0, 1, 2, 3
-UNARY = {"silu": 0, "relu": 1, "gelu_tanh": 2, "sigmoid": 3, "tanh": 4, "neg": 5}
-BINARY = {"add": 0, "sub": 1, "mul": 2, "div": 3, "min": 4, "max": 5}
+# epilogue operators: the reference's OP_UNARY_* / OP_BINARY_* codes (operators/runtime/ComputeOpsShared.h), the set of
+# cut_writeOutput (operators/impl/matmul/MatMulQ8Common.cuh:58-109)
+UNARY = {"neg": 100, "abs": 101, "sqrt": 102, "square": 103, "reciprocal": 104, "exp": 106, "log": 109, "tanh": 121,
+         "floor": 122, "ceil": 123, "round": 124, "relu": 130, "sigmoid": 131, "gelu": 132, "gelu_tanh": 132, "silu": 133,
+         "softplus": 134, "relu6": 137, "mish": 141, "hardswish": 142, "hardsigmoid": 143, "rsqrt": 148}
+BINARY = {"add": 0, "sub": 1, "mul": 2, "div": 3, "mod": 4, "pow": 5, "floor_div": 6, "min": 13, "max": 14}
 FORMATS = {"Q8_0": Q8_0, "Q4_0": Q4_0, "Q4_K": Q4_K, "Q6_K": Q6_K}
 BLOCK_ELEMS = {Q8_0: 32, Q4_0: 32, Q4_K: 256, Q6_K: 256}
 BLOCK_BYTES = {Q8_0: 34, Q4_0: 18, Q4_K: 144, Q6_K: 210}
@@ -28,13 +32,16 @@ EXPORTS = [
     "cuthip_malloc", "cuthip_free", "cuthip_memcpy_h2d", "cuthip_memcpy_d2h", "cuthip_memcpy_d2d", "cuthip_memset",
     "cuthip_stream_create", "cuthip_stream_destroy", "cuthip_stream_sync",
     "cuthip_event_create", "cuthip_event_destroy", "cuthip_event_record", "cuthip_event_sync", "cuthip_event_elapsed_ms",
-    "cuthip_variant_count", "cuthip_variant_default", "cuthip_variant_info", "cuthip_variant_lookup",
+    "cuthip_read_probe", "cuthip_epilogue_op_supported",
+    "cuthip_graph_begin_capture", "cuthip_graph_end_capture", "cuthip_graph_launch", "cuthip_graph_destroy",
+    "cuthip_variant_count", "cuthip_variant_default", "cuthip_variant_available", "cuthip_variant_info", "cuthip_variant_lookup",
     "cuthip_dequant", "cuthip_matmul_gguf", "cuthip_matmul_gguf_pro",
     "cuthip_matmul_gguf_workspace_bytes", "cuthip_matmul_gguf_ws", "cuthip_matmul_gguf_pair", "cuthip_matmul_gguf_carry",
     "cuthip_rmsnorm", "cuthip_rope_kv_write", "cuthip_attn_decode_workspace_bytes", "cuthip_attn_decode",
     "cuthip_attn_decode_static_max_bytes", "cuthip_attn_decode_static",
-    "cuthip_silu_mul", "cuthip_argmax",
-    "cuthip_matmul_sep_workspace_bytes", "cuthip_matmul_q8_sep", "cuthip_matmul_q4_sep",
+    "cuthip_silu_mul", "cuthip_argmax", "cuthip_repetition_penalty", "cuthip_argmax_penalized",
+    "cuthip_matmul_gguf_argmax_workspace_bytes", "cuthip_matmul_gguf_argmax", "cuthip_embedding_rows", "cuthip_embedding_col",
+    "cuthip_matmul_sep_workspace_bytes", "cuthip_matmul_sep_workspace_bytes_for", "cuthip_matmul_q8_sep", "cuthip_matmul_q4_sep",
     "cuthip_prepare_sep", "cuthip_transpose_q4_nibble", "cuthip_quantize_rows_q8_0",
     "cuthip_matmul_q8_i8_workspace_bytes", "cuthip_matmul_q8_i8",
     "cuthip_matmul_dense_f16_workspace_bytes", "cuthip_matmul_dense_f16",
@@ -51,7 +58,7 @@ class RopeAppend(C.Structure):
     """cuthip_rope_append_t: device pointers as integers."""
     _fields_ = [("runtime_params", C.c_void_p), ("cos_table", C.c_void_p), ("sin_table", C.c_void_p), ("q_out", C.c_void_p),
                 ("q_out_dtype", C.c_int), ("k_cache", C.c_void_p), ("v_cache", C.c_void_p), ("q_dim", C.c_uint32),
-                ("head_dim", C.c_uint32), ("aligned_kv_dim", C.c_uint32)]
+                ("head_dim", C.c_uint32), ("aligned_kv_dim", C.c_uint32), ("max_positions", C.c_uint32)]
 
 
 class CutHipError(RuntimeError):
@@ -100,8 +107,15 @@ def load() -> C.CDLL:
     lib.cuthip_event_record.argtypes = [vp, vp]
     lib.cuthip_event_sync.argtypes = [vp]
     lib.cuthip_event_elapsed_ms.argtypes = [vp, vp, C.POINTER(C.c_float)]
+    lib.cuthip_read_probe.argtypes = [vp, C.c_size_t, vp, vp]
+    lib.cuthip_epilogue_op_supported.argtypes = [i, i]
+    lib.cuthip_graph_begin_capture.argtypes = [vp]
+    lib.cuthip_graph_end_capture.argtypes = [vp, C.POINTER(vp)]
+    lib.cuthip_graph_launch.argtypes = [vp, vp]
+    lib.cuthip_graph_destroy.argtypes = [vp]
     lib.cuthip_variant_count.argtypes = [i]
     lib.cuthip_variant_default.argtypes = [i]
+    lib.cuthip_variant_available.argtypes = [i, i]
     lib.cuthip_variant_info.argtypes = [i, i, C.POINTER(VariantInfo)]
     lib.cuthip_variant_lookup.argtypes = [i, C.c_char_p]
     lib.cuthip_dequant.argtypes = [i, vp, vp, i, u32, u32, u32, vp]
@@ -114,16 +128,24 @@ def load() -> C.CDLL:
     f32 = C.c_float
     lib.cuthip_matmul_gguf_pro.argtypes = [i, vp, vp, i, vp, i, u32, u32, i, i, vp, i, vp, f32, vp]
     lib.cuthip_rmsnorm.argtypes = [vp, i, vp, vp, i, u32, u32, u32, f32, vp]
-    lib.cuthip_rope_kv_write.argtypes = [vp, vp, vp, i, vp, vp, vp, vp, vp, vp, i, u32, u32, u32, u32, vp]
+    lib.cuthip_rope_kv_write.argtypes = [vp, vp, vp, i, vp, vp, vp, vp, vp, vp, i, u32, u32, u32, u32, u32, vp]
     lib.cuthip_attn_decode_workspace_bytes.argtypes = [u32, u32, u32]
     lib.cuthip_attn_decode.argtypes = [vp, i, vp, vp, vp, vp, i, u32, u32, u32, u32, f32, u32, vp, C.c_size_t, vp]
     lib.cuthip_attn_decode_static_max_bytes.argtypes = []
     lib.cuthip_attn_decode_static.argtypes = [vp, i, vp, vp, vp, vp, i, u32, u32, u32, u32, f32, u32, vp]
     lib.cuthip_silu_mul.argtypes = [vp, i, vp, i, u32, vp]
     lib.cuthip_argmax.argtypes = [vp, i, u32, vp, vp]
+    lib.cuthip_repetition_penalty.argtypes = [vp, vp, vp, u32, vp]
+    lib.cuthip_argmax_penalized.argtypes = [vp, i, u32, vp, vp, u32, vp, vp]
+    lib.cuthip_matmul_gguf_argmax_workspace_bytes.argtypes = [u32]
+    lib.cuthip_matmul_gguf_argmax.argtypes = [i, vp, vp, i, vp, i, u32, u32, C.POINTER(NormCarry), vp, vp, u32, vp, C.c_size_t,
+                                              vp, vp]
+    lib.cuthip_embedding_rows.argtypes = [i, vp, vp, u32, u32, u32, vp, i, u32, vp]
+    lib.cuthip_embedding_col.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, i, vp]
     lib.cuthip_matmul_sep_workspace_bytes.argtypes = [u32, u32, u32]
-    lib.cuthip_matmul_q8_sep.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, u32, i, i, vp, C.c_size_t, vp]
-    lib.cuthip_matmul_q4_sep.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, u32, i, i, i, vp, C.c_size_t, vp]
+    lib.cuthip_matmul_sep_workspace_bytes_for.argtypes = [i, i, u32, u32, u32]
+    lib.cuthip_matmul_q8_sep.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, u32, i, i, i, vp, C.c_size_t, vp]
+    lib.cuthip_matmul_q4_sep.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, u32, i, i, i, i, vp, C.c_size_t, vp]
     lib.cuthip_prepare_sep.argtypes = [i, vp, u32, u32, vp, u32, vp, u32, vp]
     lib.cuthip_transpose_q4_nibble.argtypes = [vp, vp, u32, u32, u32, u32, vp]
     lib.cuthip_quantize_rows_q8_0.argtypes = [vp, C.c_uint64, vp, vp]
@@ -131,9 +153,10 @@ def load() -> C.CDLL:
     lib.cuthip_matmul_dense_f16.argtypes = [vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, vp, C.c_size_t, vp]
     lib.cuthip_matmul_q8_i8_workspace_bytes.argtypes = [u32, u32]
     lib.cuthip_matmul_q8_i8.argtypes = [vp, vp, i, vp, i, u32, u32, u32, u32, u32, i, i, vp, vp, C.c_size_t, vp]
-    sized = ("cuthip_attn_decode_workspace_bytes", "cuthip_matmul_sep_workspace_bytes",
+    sized = ("cuthip_attn_decode_workspace_bytes", "cuthip_matmul_sep_workspace_bytes", "cuthip_matmul_sep_workspace_bytes_for",
              "cuthip_matmul_gguf_workspace_bytes", "cuthip_matmul_q8_i8_workspace_bytes",
-             "cuthip_matmul_dense_f16_workspace_bytes", "cuthip_attn_decode_static_max_bytes")
+             "cuthip_matmul_dense_f16_workspace_bytes", "cuthip_attn_decode_static_max_bytes",
+             "cuthip_matmul_gguf_argmax_workspace_bytes")
     for n in EXPORTS:
         if n != "cuthip_last_error" and n not in sized:
             getattr(lib, n).restype = i

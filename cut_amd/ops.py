@@ -10,6 +10,8 @@ reference's constructors do (MatMulOp.cpp:288-329).
 """
 from __future__ import annotations
 
+import ctypes as C
+
 import torch
 
 from . import lib as _l
@@ -114,6 +116,10 @@ def matmul_gguf(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: int, ou
     cdt = _l.F16 if out.dtype == torch.float16 else _l.F32
     if _tuning is not None and variant == -1 and epi == _l.EPI_NONE and workspace is not None:
         variant = _tuning.select("MatMulGguf" + _FMT_NAMES[f], [M, K, N], -1)
+        # a rule may name a variant this process cannot run (the vendor-GEMM variant without its library): the
+        # hand-written two-pass GEMM takes its place
+        if variant >= 0 and _l.load().cuthip_variant_available(_l.OP_MATMUL_GGUF, variant) != 1:
+            variant = 4 if variant == 5 else -1
     if workspace is not None:
         _l.check(_l.load().cuthip_matmul_gguf_ws(
             f, w_blocks.data_ptr(), a2.data_ptr(), adt, out.data_ptr(), cdt, M, K, N, a2.stride(0), out.stride(0), epi, op,
@@ -165,7 +171,8 @@ def rope_append(runtime_params: torch.Tensor, cos_t: torch.Tensor, sin_t: torch.
     if k_cache.dtype != torch.float16 or v_cache.dtype != torch.float16 or k_cache.stride(0) != v_cache.stride(0):
         raise _l.CutHipError("rope_append: caches must be fp16 with one row stride")
     return _l.RopeAppend(runtime_params.data_ptr(), cos_t.data_ptr(), sin_t.data_ptr(), q_out.data_ptr(), _dt(q_out),
-                         k_cache.data_ptr(), v_cache.data_ptr(), q_dim, head_dim, k_cache.stride(0))
+                         k_cache.data_ptr(), v_cache.data_ptr(), q_dim, head_dim, k_cache.stride(0),
+                         min(k_cache.shape[0], cos_t.shape[0]))
 
 
 def interleave_rope_rows(w_blocks: torch.Tensor, n_rows: int, head_dim: int) -> torch.Tensor:
@@ -236,7 +243,7 @@ def rope_kv_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, runtime_par
     _l.check(_l.load().cuthip_rope_kv_write(q.data_ptr(), k.data_ptr(), v.data_ptr(), _dt(q), runtime_params.data_ptr(),
                                             cos_t.data_ptr(), sin_t.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                             q_out.data_ptr(), _dt(q_out), q.numel(), k.numel(), head_dim, k_cache.stride(0),
-                                            _stream_ptr()))
+                                            min(k_cache.shape[0], cos_t.shape[0]), _stream_ptr()))
     return q_out
 
 
@@ -276,12 +283,84 @@ def argmax(x: torch.Tensor, out_index: torch.Tensor) -> torch.Tensor:
     return out_index
 
 
+def repetition_penalty(logits: torch.Tensor, factors: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """RepetitionPenaltyOpNode on the dense fp32 factor vector (1 for tokens that are not penalised)."""
+    if logits.dtype != torch.float32 or factors.dtype != torch.float32 or logits.numel() != factors.numel():
+        raise _l.CutHipError("RepetitionPenalty: logits and penaltyFactors must be fp32 tensors of the same shape")
+    out = torch.empty_like(logits) if out is None else out
+    _l.check(_l.load().cuthip_repetition_penalty(logits.data_ptr(), factors.data_ptr(), out.data_ptr(), logits.numel(), _stream_ptr()))
+    return out
+
+
+def _pen_args(pen_tokens, pen_factors):
+    if pen_tokens is None:
+        return None, None, 0
+    if pen_tokens.dtype != torch.int32 or pen_factors.dtype != torch.float32 or pen_tokens.numel() != pen_factors.numel():
+        raise _l.CutHipError("penalised tokens are int32 ids with one fp32 factor each")
+    return pen_tokens.data_ptr(), pen_factors.data_ptr(), pen_tokens.numel()
+
+
+def argmax_penalized(logits: torch.Tensor, out_index: torch.Tensor, pen_tokens: torch.Tensor | None = None,
+                     pen_factors: torch.Tensor | None = None) -> torch.Tensor:
+    """Repetition penalty on the listed tokens (in place), then the arg-max (cuthip_argmax_penalized)."""
+    pt, pf, n = _pen_args(pen_tokens, pen_factors)
+    _l.check(_l.load().cuthip_argmax_penalized(logits.data_ptr(), _dt(logits), logits.numel(), pt, pf, n, out_index.data_ptr(),
+                                               _stream_ptr()))
+    return out_index
+
+
+def lm_head_workspace(N: int, device) -> torch.Tensor:
+    return torch.empty(max(int(_l.load().cuthip_matmul_gguf_argmax_workspace_bytes(N)), 8), dtype=torch.uint8, device=device)
+
+
+def matmul_gguf_argmax(a: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, K: int, logits: torch.Tensor, out_index: torch.Tensor,
+                       carry=None, pen_tokens: torch.Tensor | None = None, pen_factors: torch.Tensor | None = None,
+                       workspace: torch.Tensor | None = None) -> torch.Tensor:
+    """The output head with the sampling folded in: logits = a . dequant(W)^T, penalty on the listed tokens, arg-max."""
+    f = _fmt(fmt)
+    if a.numel() != K or not a.is_contiguous() or logits.numel() != N or not logits.is_contiguous():
+        raise _l.CutHipError("matmul_gguf_argmax: a is a contiguous vector of K elements, logits one of N")
+    pt, pf, n = _pen_args(pen_tokens, pen_factors)
+    _l.check(_l.load().cuthip_matmul_gguf_argmax(f, w_blocks.data_ptr(), a.data_ptr(), _dt(a), logits.data_ptr(), _dt(logits), K, N,
+                                                 C.byref(carry) if carry is not None else None, pt, pf, n,
+                                                 workspace.data_ptr() if workspace is not None else None,
+                                                 workspace.numel() if workspace is not None else 0, out_index.data_ptr(),
+                                                 _stream_ptr()))
+    return out_index
+
+
+def embedding_rows(w_blocks: torch.Tensor, fmt, token_ids: torch.Tensor, n_rows: int, dim: int, out: torch.Tensor) -> torch.Tensor:
+    """out[i] = dequant(row token_ids[i]) of a GGUF table [n_rows, dim]; token_ids int32/uint32 on the device."""
+    if token_ids.dtype not in (torch.int32, torch.uint32) or out.stride(-1) != 1 or out.numel() < token_ids.numel() * dim:
+        raise _l.CutHipError("embedding_rows: token ids are 32-bit integers, out holds one row of dim per id")
+    out2 = out if out.dim() == 2 else out.view(token_ids.numel(), -1)
+    _l.check(_l.load().cuthip_embedding_rows(_fmt(fmt), w_blocks.data_ptr(), token_ids.data_ptr(), token_ids.numel(), n_rows, dim,
+                                             out2.data_ptr(), _dt(out2), out2.stride(0), _stream_ptr()))
+    return out
+
+
+def embedding_col(indices: torch.Tensor, matrix: torch.Tensor, scales: torch.Tensor | None, emb_dim: int, vocab: int,
+                  out: torch.Tensor | None = None) -> torch.Tensor:
+    """EmbeddingColOpNode: matrix [emb_dim, vocab_stride] column-wise, fp16 (scales None) or int8 with fp16 scales
+    [emb_dim / 32, scale_stride]; returns fp32 [len(indices), emb_dim]."""
+    fmt = 0 if scales is None else 1
+    if matrix.dim() != 2 or matrix.dtype != (torch.float16 if fmt == 0 else torch.int8) or indices.dtype not in (torch.int32, torch.uint32):
+        raise _l.CutHipError("embedding_col: matrix is 2-D fp16 (no scales) or int8 (fp16 scales), indices 32-bit integers")
+    if out is None:
+        out = torch.empty((indices.numel(), emb_dim), dtype=torch.float32, device=matrix.device)
+    _l.check(_l.load().cuthip_embedding_col(indices.data_ptr(), matrix.data_ptr(), scales.data_ptr() if fmt else None, out.data_ptr(),
+                                            indices.numel(), emb_dim, matrix.stride(0), scales.stride(0) if fmt else 0, out.stride(0),
+                                            vocab, fmt, _stream_ptr()))
+    return out
+
+
 # ---- the reference's separated weight layout ----------------------------------------------------------
 def matmul_sep(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, N: int, q4: bool = False, affine: bool = False,
                out: torch.Tensor | None = None, unary: str | None = None, binary: str | None = None,
-               d: torch.Tensor | None = None) -> torch.Tensor:
+               d: torch.Tensor | None = None, variant: int = -1) -> torch.Tensor:
     """Operations::matmul(a, packedB, scalesB) of the reference on its own layout: a fp32 [M, K]; b int8 [K, N]
-    (q4: uint8 [K, N/2], even column in the low nibble); scales fp16 [K/32, N] ([2K/32, N] when affine)."""
+    (q4: uint8 [K, N/2], even column in the low nibble); scales fp16 [K/32, N] ([2K/32, N] when affine).
+    variant: the reference's `spec` (an index of its MatMulQ8 / MatMulQ4 variant tables), -1 = by shape."""
     a2 = a if a.dim() == 2 else a.reshape(1, -1)
     M, K = a2.shape
     if a2.dtype != torch.float32 or scales.dtype != torch.float16 or b.element_size() != 1 or b.dim() != 2 or scales.dim() != 2:
@@ -299,14 +378,14 @@ def matmul_sep(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, N: int, q
             raise _l.CutHipError("matmul_sep: binary epilogue needs an fp32 D with the shape and stride of C")
         epi, op, dptr = _l.EPI_BINARY, _l.BINARY[binary], d.data_ptr()
     lib = _l.load()
-    ws_bytes = lib.cuthip_matmul_sep_workspace_bytes(M, K, N)
+    ws_bytes = lib.cuthip_matmul_sep_workspace_bytes_for(_l.OP_MATMUL_Q4 if q4 else _l.OP_MATMUL_Q8, variant, M, K, N)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=a.device)
     common = (a2.data_ptr(), b.data_ptr(), scales.data_ptr(), dptr, out.data_ptr(), M, K, N, a2.stride(0), b.stride(0),
               out.stride(0), scales.stride(0), epi, op)
     if q4:
-        _l.check(lib.cuthip_matmul_q4_sep(*common, int(affine), ws.data_ptr(), ws_bytes, _stream_ptr()))
+        _l.check(lib.cuthip_matmul_q4_sep(*common, int(affine), variant, ws.data_ptr(), ws_bytes, _stream_ptr()))
     else:
-        _l.check(lib.cuthip_matmul_q8_sep(*common, ws.data_ptr(), ws_bytes, _stream_ptr()))
+        _l.check(lib.cuthip_matmul_q8_sep(*common, variant, ws.data_ptr(), ws_bytes, _stream_ptr()))
     return out
 
 

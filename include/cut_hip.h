@@ -52,8 +52,29 @@ typedef enum {
    * strideC counts the N/2 outputs; epilogue_op and D unused. */
   CUTHIP_EPI_SWIGLU_PAIRS = 3
 } cuthip_epilogue;
-typedef enum { CUTHIP_UNARY_SILU = 0, CUTHIP_UNARY_RELU = 1, CUTHIP_UNARY_GELU_TANH = 2, CUTHIP_UNARY_SIGMOID = 3, CUTHIP_UNARY_TANH = 4, CUTHIP_UNARY_NEG = 5 } cuthip_unary_op;
-typedef enum { CUTHIP_BINARY_ADD = 0, CUTHIP_BINARY_SUB = 1, CUTHIP_BINARY_MUL = 2, CUTHIP_BINARY_DIV = 3, CUTHIP_BINARY_MIN = 4, CUTHIP_BINARY_MAX = 5 } cuthip_binary_op;
+/* epilogue_op of a fused epilogue: the reference's operator codes themselves (OP_UNARY_* / OP_BINARY_* of
+ * operators/runtime/ComputeOpsShared.h:22-40, 118-167, the value of its FUSION_OP specialization constant), so a
+ * caller passes what MatMulOpNode::setFusion received.  The set is what cut_writeOutput implements
+ * (operators/impl/matmul/MatMulQ8Common.cuh:58-109: 21 unary and 9 binary operators) with the same formulas; any
+ * other code is refused with CUTHIP_ERR_INVALID (the reference's shader would silently store the unfused value).
+ * NEG, TANH, RELU, SIGMOID, GELU, SILU and ADD, SUB, MUL, DIV, MIN, MAX (what the runner's graphs fuse) run inside the
+ * matmul kernels; the others are applied by a second, elementwise launch on the same stream (inlined at every store
+ * of the tiled GEMMs the whole set costs those kernels their register allocation): same
+ * result up to the rounding of C to its dtype in between, and for MOD, POW, FLOOR_DIV D must not alias C. */
+typedef enum {
+  CUTHIP_UNARY_NEG = 100, CUTHIP_UNARY_ABS = 101, CUTHIP_UNARY_SQRT = 102, CUTHIP_UNARY_SQUARE = 103,
+  CUTHIP_UNARY_RECIPROCAL = 104, CUTHIP_UNARY_EXP = 106, CUTHIP_UNARY_LOG = 109, CUTHIP_UNARY_TANH = 121,
+  CUTHIP_UNARY_FLOOR = 122, CUTHIP_UNARY_CEIL = 123, CUTHIP_UNARY_ROUND = 124, CUTHIP_UNARY_RELU = 130,
+  CUTHIP_UNARY_SIGMOID = 131, CUTHIP_UNARY_GELU = 132, CUTHIP_UNARY_GELU_TANH = 132, CUTHIP_UNARY_SILU = 133,
+  CUTHIP_UNARY_SOFTPLUS = 134, CUTHIP_UNARY_RELU6 = 137, CUTHIP_UNARY_MISH = 141, CUTHIP_UNARY_HARDSWISH = 142,
+  CUTHIP_UNARY_HARDSIGMOID = 143, CUTHIP_UNARY_RSQRT = 148
+} cuthip_unary_op;
+typedef enum {
+  CUTHIP_BINARY_ADD = 0, CUTHIP_BINARY_SUB = 1, CUTHIP_BINARY_MUL = 2, CUTHIP_BINARY_DIV = 3, CUTHIP_BINARY_MOD = 4,
+  CUTHIP_BINARY_POW = 5, CUTHIP_BINARY_FLOOR_DIV = 6, CUTHIP_BINARY_MIN = 13, CUTHIP_BINARY_MAX = 14
+} cuthip_binary_op;
+/* 1 if `op` is an operator the given epilogue kind implements, else 0. */
+int cuthip_epilogue_op_supported(int epilogue, int op);
 
 /* Prologues on the activations of cuthip_matmul_gguf_pro. */
 typedef enum { CUTHIP_PRO_NONE = 0, CUTHIP_PRO_RMSNORM = 1, CUTHIP_PRO_SWIGLU = 2 } cuthip_prologue;
@@ -109,9 +130,35 @@ int cuthip_event_record(void *event, void *stream);
 int cuthip_event_sync(void *event);
 int cuthip_event_elapsed_ms(void *start, void *stop, float *ms);
 
+/* Capture and replay of a launch sequence: what the reference's reusable command buffers do on its CUDA backend
+ * (core/backends/cuda/CudaCommandBuffer.cpp:261-285: cuStreamBeginCapture, the dispatches, cuStreamEndCapture,
+ * cuGraphInstantiate once, then cuGraphLaunch per token).  Between begin and end every cuthip_* launch on `stream`
+ * (a stream from cuthip_stream_create, not the default one) is recorded instead of run; no entry point of this
+ * library allocates, so all of them may be captured (cuthip_memset is the exception: clear memory before the capture
+ * or with a kernel of the sequence).  Values that change between replays (position, sequence length, token ids,
+ * penalty lists) are read from device memory by the kernels, so the host updates those buffers and launches the same
+ * graph again.  The handle owns both the graph and its executable form. */
+int cuthip_graph_begin_capture(void *stream);
+int cuthip_graph_end_capture(void *stream, void **graph);
+int cuthip_graph_launch(void *graph, void *stream);
+int cuthip_graph_destroy(void *graph);
+
+/* Measurement aid (no counterpart in the reference): one launch that only reads `bytes` of device memory with
+ * 16-byte loads (the tail below 16 bytes is ignored) and stores one dword per wave into sink (65,536 dwords).  Its
+ * duration is what a launch of that size can reach on the part when it does nothing but load, the yardstick the
+ * streaming kernels are held against (bench.py --calibrate-read). */
+int cuthip_read_probe(const void *src, size_t bytes, uint32_t *sink, void *stream);
+
 /* ---- variant tables ---------------------------------------------------- */
 int cuthip_variant_count(int op);
+/* Default index of a table: the reference's kMatMulQ8DefaultVariant = 2 / kMatMulQ4DefaultVariant = 0 for the
+ * separated-layout tables; 0 for CUTHIP_OP_MATMUL_GGUF, whose entry 0 is valid for every M (it is the streaming GEMV
+ * up to 8 rows of A and the library's choice by shape beyond), so that the reference's idiom
+ * `spec ? *spec : kDefaultVariant` (MatMulOp.cpp:244-246) never yields an index the shape rejects. */
 int cuthip_variant_default(int op);
+/* 1 if the variant can run in this process, 0 if not (MatMulGgufDequantBlasLt without hipBLASLt), < 0 = no such
+ * variant.  A tuning rule that names an unavailable variant is to be skipped by the caller. */
+int cuthip_variant_available(int op, int index);
 int cuthip_variant_info(int op, int index, cuthip_variant_info_t *info);
 /* Index of a variant by name, or CUTHIP_ERR_UNKNOWN_VARIANT: an unknown name is
  * a hard error, never a silently skipped dispatch (the hazard described in
@@ -232,8 +279,9 @@ typedef struct {
   const float *cos_table, *sin_table; /* [position][head_dim / 2] */
   void *q_out;
   int q_out_dtype;
-  void *k_cache, *v_cache;          /* fp16 [max_ctx][aligned_kv_dim] */
+  void *k_cache, *v_cache;          /* fp16 [max_positions][aligned_kv_dim] */
   uint32_t q_dim, head_dim, aligned_kv_dim;
+  uint32_t max_positions;           /* rows of the caches and of the tables: a position at or beyond it writes nothing */
 } cuthip_rope_append_t;
 
 /* Two batch-1 matmuls on the same activations in one launch:
@@ -300,14 +348,25 @@ int cuthip_matmul_gguf_pro(int fmt, const void *W, const void *A, int a_dtype, v
  * and the workspace holds split-K partial sums; from 32 rows on the tensors are
  * first dequantized to fp16 [N][K] in the workspace (one launch) and multiplied
  * by the dense GEMM of cuthip_matmul_dense_f16 (fp16 operands, fp32 accumulate:
- * within 1e-3 of the fp32 loop). */
+ * within 1e-3 of the fp32 loop).
+ * variant: the MatMulOpNode `spec` argument, an index into the CUTHIP_OP_MATMUL_Q8 / CUTHIP_OP_MATMUL_Q4 tables,
+ * which hold the reference's variant names at the reference's indices (MatMulQ8Variants.generated.h:20-32, default 2;
+ * MatMulQ4Variants.generated.h:20-29, default 0; "indices are ABI", MatMulOp.cpp:353-356), or -1 = choose by shape.
+ * The reference's shaders collapse onto two kernels here: its tiled shaders (Q8 0, 2, 6; Q4 0) choose by shape as -1
+ * does; its GEMV shaders (Q8 1, 3, 4, 5; Q4 1, 2, 3) stream the weights once per 4 rows whatever M is; its
+ * cooperative-matrix shaders (Q8 7; Q4 4) dequantize to fp16 and run the dense MFMA GEMM whatever M is (an error if
+ * K is not a multiple of 128 or the workspace is too small).  The int8-activation shaders of the reference (Q8 5, 6)
+ * run with unquantized activations here.  Any other index: CUTHIP_ERR_UNKNOWN_VARIANT.
+ * cuthip_matmul_sep_workspace_bytes sizes the workspace for variant -1 and the table defaults,
+ * cuthip_matmul_sep_workspace_bytes_for(op, variant, ...) for an explicit index. */
 size_t cuthip_matmul_sep_workspace_bytes(uint32_t M, uint32_t K, uint32_t N);
+size_t cuthip_matmul_sep_workspace_bytes_for(int op, int variant, uint32_t M, uint32_t K, uint32_t N);
 int cuthip_matmul_q8_sep(const float *A, const int8_t *B, const uint16_t *scales, const float *D, float *C, uint32_t M,
                          uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideB, uint32_t strideC, uint32_t scaleStride,
-                         int epilogue, int epilogue_op, void *workspace, size_t workspace_bytes, void *stream);
+                         int epilogue, int epilogue_op, int variant, void *workspace, size_t workspace_bytes, void *stream);
 int cuthip_matmul_q4_sep(const float *A, const uint8_t *packedB, const uint16_t *scales, const float *D, float *C, uint32_t M,
                          uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideBNpacked, uint32_t strideC,
-                         uint32_t scaleStride, int epilogue, int epilogue_op, int affine, void *workspace,
+                         uint32_t scaleStride, int epilogue, int epilogue_op, int affine, int variant, void *workspace,
                          size_t workspace_bytes, void *stream);
 
 /* ---- Q8_0 weights x int8 activations on the int8 matrix core -----------------
@@ -375,17 +434,23 @@ int cuthip_rmsnorm(const void *x, int x_dtype, const float *weight, void *out, i
 /* Half-split RoPE on q [q_dim] and k [kv_dim] with tables [pos][head_dim/2];
  * k (rotated) and v are stored as fp16 to cache row `position`
  * (rows of aligned_kv_dim elements); q (rotated) goes to q_out
- * (operators/impl/attention/FusedRoPEKVWrite.cu:12-81). */
+ * (operators/impl/attention/FusedRoPEKVWrite.cu:12-81).  max_positions: rows of the caches and of the tables; the
+ * position is read on the device, so it cannot be refused here: a position at or beyond max_positions writes
+ * nothing at all (the reference would write past the cache). */
 int cuthip_rope_kv_write(const void *q, const void *k, const void *v, int in_dtype, const uint32_t *runtime_params,
                          const float *cos_table, const float *sin_table, void *k_cache, void *v_cache, void *q_out,
                          int q_out_dtype, uint32_t q_dim, uint32_t kv_dim, uint32_t head_dim, uint32_t aligned_kv_dim,
-                         void *stream);
+                         uint32_t max_positions, void *stream);
 
 /* Scaled dot-product attention of one token over an fp16 KV cache with GQA:
  * out[h,:] = softmax(scale * q[h,:] . K[0:seq, h/nRep, :]) . V[0:seq, h/nRep, :]
  * (operators/impl/attention/Attention.cu:35-106; head_dim <= 128 as there).
- * workspace: device scratch of cuthip_attn_decode_workspace_bytes(); the
- * call allocates nothing.  max_seq_len sizes the launch (cache capacity). */
+ * workspace: device scratch of cuthip_attn_decode_workspace_bytes(); the call allocates nothing.
+ * max_seq_len bounds the launch: any value from the current sequence length up to the cache capacity (at most
+ *   65,536).  The call reads max_seq_len positions of K and V whatever runtime_params[1] says (its loads do not wait
+ *   for that value: waiting puts a second memory round trip in front of every workgroup, measured + 1.7 us per
+ *   launch), so a caller that knows the length on the host passes it rounded up, and a caller that replays a captured
+ *   graph captures one per context bucket; a sequence length beyond max_seq_len is attended up to max_seq_len only. */
 size_t cuthip_attn_decode_workspace_bytes(uint32_t n_heads, uint32_t head_dim, uint32_t max_seq_len);
 int cuthip_attn_decode(const void *q, int q_dtype, const void *k_cache, const void *v_cache, const uint32_t *runtime_params,
                        void *out, int out_dtype, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
@@ -413,6 +478,48 @@ int cuthip_silu_mul(const void *gate_up, int in_dtype, void *out, int out_dtype,
 
 /* Index of the first maximum of x[0:n] (greedy sampling), written to device memory. */
 int cuthip_argmax(const void *x, int x_dtype, uint32_t n, uint32_t *out_index, void *stream);
+
+/* RepetitionPenaltyOpNode (operators/impl/sampling/RepetitionPenaltyOp.cpp:9-66, RepetitionPenalty.cu:19-41) on the
+ * dense factor vector the runner uploads per token: out[i] = logits[i] > 0 ? logits[i] / factors[i] : logits[i] *
+ * factors[i]; all fp32 [n]; out may be logits. */
+int cuthip_repetition_penalty(const float *logits, const float *factors, float *out, uint32_t n, void *stream);
+
+/* The runner's "penalty, then arg-max" (interface/runner/llama/llama.cpp:2145-2152) without the dense factor vector:
+ * pen_tokens / pen_factors (device, n_pen <= 1024 entries) list the penalised tokens, i.e. the entries of the runner's
+ * factor vector that are not 1 (llama.cpp:2566-2592: the recent window at `repeat_penalty`, then end-of-sequence
+ * tokens at 1e9); as there, a token listed several times is penalised once, with the factor of its last entry, and
+ * ids outside [0, n) are ignored.  The listed logits are rewritten in place (the penalised logits), the index of the
+ * first maximum of the result goes to out_index (device).  One workgroup; n_pen = 0 is a plain arg-max. */
+int cuthip_argmax_penalized(void *logits, int x_dtype, uint32_t n, const int32_t *pen_tokens, const float *pen_factors,
+                            uint32_t n_pen, uint32_t *out_index, void *stream);
+
+/* The output head of a decode step with the sampling folded in: logits[N] = A[K] . dequant(W)^T (batch 1; carry: the
+ * consumer side of a carried RMSNorm or NULL), then the penalty and arg-max of cuthip_argmax_penalized.  The matmul's
+ * epilogue leaves the winner of every 8 vocabulary rows in the workspace, so the second launch reduces N / 8 pairs
+ * instead of scanning N logits (the reference runs LM head, RepetitionPenalty and ReduceArgmax as three dispatches,
+ * llama.cpp:2145-2152).  workspace: device, 8-byte aligned, cuthip_matmul_gguf_argmax_workspace_bytes(N) bytes, scratch
+ * (without it, or where the matmul's shape does not allow the epilogue, the logits are scanned instead: same result). */
+size_t cuthip_matmul_gguf_argmax_workspace_bytes(uint32_t N);
+int cuthip_matmul_gguf_argmax(int fmt, const void *W, const void *A, int a_dtype, void *logits, int c_dtype, uint32_t K, uint32_t N,
+                              const cuthip_norm_carry_t *carry, const int32_t *pen_tokens, const float *pen_factors,
+                              uint32_t n_pen, void *workspace, size_t workspace_bytes, uint32_t *out_index, void *stream);
+
+/* Embedding lookup on a table kept as GGUF blocks (row t = the embedding of token t, as in the file):
+ * out[i, 0:dim] = dequant(row token_ids[i]), i < n_ids; token_ids on the device, so a captured graph follows the
+ * token it sampled itself.  Bit-identical to cuthip_dequant of that row (fp32, or fp16 with the reference's
+ * narrowing); an id >= n_rows yields a zero row.  Replaces Operations::embedding on the dequantized table
+ * (interface/runner/llama/llama.cpp:1037-1046) without ever materialising that table. */
+int cuthip_embedding_rows(int fmt, const void *blocks, const uint32_t *token_ids, uint32_t n_ids, uint32_t n_rows,
+                          uint32_t dim, void *out, int out_dtype, uint32_t out_stride, void *stream);
+
+/* EmbeddingColOpNode (operators/impl/memory/EmbeddingCol.cu:16-44) on the loader's column-wise tables, arguments
+ * are its push constants: value of (token t, dim d) at matrix[d * vocab_stride + t]; format 0: fp16 table, format 1:
+ * int8 table with fp16 scales[(d >> 5) * scale_stride + t] (the separated Q8_0 tensors of cuthip_prepare_sep).  out
+ * fp32 [num_indices, out_stride].  vocab bounds the indices (an index >= vocab yields zeros; the reference reads
+ * out of bounds). */
+int cuthip_embedding_col(const uint32_t *indices, const void *matrix, const uint16_t *scales, float *out, uint32_t num_indices,
+                         uint32_t emb_dim, uint32_t vocab_stride, uint32_t scale_stride, uint32_t out_stride, uint32_t vocab,
+                         int format, void *stream);
 
 #ifdef __cplusplus
 }

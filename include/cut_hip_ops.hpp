@@ -51,6 +51,51 @@ inline size_t ggufBytes(GgufFormat f, uint64_t elems) { return (size_t)(elems / 
 // Selects the device once; throws if it is not a gfx950.
 inline void init(int device = 0) { check(cuthip_init(device), "cuthip_init"); }
 
+// A stream of the backend (the reference keeps 16 of them, core/backends/cuda/CudaStructs.h:20).
+class Stream {
+public:
+  Stream() { check(cuthip_stream_create(&s_), "cuthip_stream_create"); }
+  ~Stream() {
+    if (s_) cuthip_stream_destroy(s_);
+  }
+  Stream(const Stream &) = delete;
+  Stream &operator=(const Stream &) = delete;
+  void *get() const { return s_; }
+  void sync() const { check(cuthip_stream_sync(s_), "cuthip_stream_sync"); }
+
+private:
+  void *s_ = nullptr;
+};
+
+// The reusable command buffer of the reference on its CUDA backend (CommandBuffer begin / encode / end / resubmit,
+// core/backends/cuda/CudaCommandBuffer.cpp:261-285): the dispatches between begin() and end() are captured once and
+// replay() launches them again with one call.  Buffers the kernels read on the device (activations, runtime
+// parameters) may be rewritten between replays.
+class CommandGraph {
+public:
+  CommandGraph() = default;
+  ~CommandGraph() {
+    if (graph_) cuthip_graph_destroy(graph_);
+  }
+  CommandGraph(const CommandGraph &) = delete;
+  CommandGraph &operator=(const CommandGraph &) = delete;
+  void begin(const Stream &s) { check(cuthip_graph_begin_capture(s.get()), "cuthip_graph_begin_capture"); }
+  void end(const Stream &s) {
+    if (graph_) {
+      cuthip_graph_destroy(graph_);
+      graph_ = nullptr;
+    }
+    check(cuthip_graph_end_capture(s.get(), &graph_), "cuthip_graph_end_capture");
+  }
+  void replay(const Stream &s) const {
+    if (!graph_) throw std::runtime_error("CommandGraph::replay: nothing captured");
+    check(cuthip_graph_launch(graph_, s.get()), "cuthip_graph_launch");
+  }
+
+private:
+  void *graph_ = nullptr;
+};
+
 // Owning device allocation (the role of a ref-counted ComputeHandle buffer,
 // core/backends/cuda/CudaContainers.cpp:354-384, without the pooling).
 class DeviceBuffer {

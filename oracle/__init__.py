@@ -32,6 +32,31 @@ def build(force: bool = False) -> None:
         subprocess.check_call(args + ["ref"], stdout=subprocess.DEVNULL)
 
 
+def embedding_col(indices, matrix, scales, emb_dim: int, fmt: int) -> np.ndarray:
+    """EmbeddingCol: matrix [emb_dim, vocab] column-wise (fmt 0: fp16 bits as uint16; fmt 1: int8 with fp16 scales
+    [emb_dim / 32, vocab]); returns fp32 [len(indices), emb_dim]."""
+    idx = _c(indices, np.uint32).reshape(-1)
+    m = _c(matrix, np.uint16 if fmt == 0 else np.int8)
+    sc = _c(scales, np.uint16) if fmt == 1 else np.zeros((1, 1), np.uint16)
+    out = np.empty((idx.size, emb_dim), np.float32)
+    _lib.orc_embedding_col(_p(idx), _p(m), _p(sc), idx.size, emb_dim, m.shape[1], sc.shape[1], emb_dim, fmt, _p(out))
+    return out
+
+
+def repetition_penalty(logits, factors) -> np.ndarray:
+    lg, f = _c(logits, np.float32).reshape(-1), _c(factors, np.float32).reshape(-1)
+    out = np.empty_like(lg)
+    _lib.orc_repetition_penalty(_p(lg), _p(f), lg.size, _p(out))
+    return out
+
+
+def penalty_factors(recent, penalty: float, vocab: int) -> np.ndarray:
+    r = _c(recent, np.int32).reshape(-1)
+    out = np.empty(vocab, np.float32)
+    _lib.orc_penalty_factors(_p(r), r.size, penalty, vocab, _p(out))
+    return out
+
+
 def _load():
     if not os.path.exists(_LIB_PATH):
         build()
@@ -69,6 +94,9 @@ def _load():
         "orc_rope_kv_write": (None, [f32p, f32p, f32p, u32, f32p, f32p, u32, u32, u32, u32, f32p, u16p, u16p]),
         "orc_attention_decode": (None, [f32p, u16p, u16p, u32, u32, u32, u32, u32, C.c_float, f32p]),
         "orc_silu_mul": (None, [f32p, u32, f32p]),
+        "orc_embedding_col": (None, [u8p, u8p, u16p, u32, u32, u32, u32, u32, C.c_int, f32p]),
+        "orc_repetition_penalty": (None, [f32p, f32p, u32, f32p]),
+        "orc_penalty_factors": (None, [u8p, u32, C.c_float, u32, f32p]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)

@@ -885,3 +885,43 @@ void orc_silu_mul(const float *gate_up, uint32_t n, float *out) {
     out[i] = (float)(g / (1.0 + exp(-(double)g))) * gate_up[(size_t)n + i];
   }
 }
+
+/* operators/impl/memory/EmbeddingCol.cu:16-44: gather of embedding rows from a table kept column-wise,
+ * value of (token t, dim d) at index d * vocabStride + t.  format 0: fp16 table; format 1: int8 table with fp16
+ * scales per 32 dims, scale of (d, t) at (d >> 5) * scaleStride + t (the separated Q8_0 layout of the loader). */
+void orc_embedding_col(const uint32_t *indices, const void *matrix, const uint16_t *scales,
+                       uint32_t num_indices, uint32_t emb_dim, uint32_t vocab_stride,
+                       uint32_t scale_stride, uint32_t out_stride, int format, float *out) {
+  for (uint32_t i = 0; i < num_indices; ++i) {
+    uint32_t t = indices[i];
+    for (uint32_t d = 0; d < emb_dim; ++d) {
+      size_t idx = (size_t)d * vocab_stride + t;
+      float v;
+      if (format == 0) {
+        v = orc_runner_f16_to_f32(((const uint16_t *)matrix)[idx]); /* __half2float: IEEE, NaN payload kept */
+      } else {
+        int b = ((const int8_t *)matrix)[idx];
+        float sc = orc_runner_f16_to_f32(scales[(size_t)(d >> 5) * scale_stride + t]);
+        v = (float)b * sc;
+      }
+      out[(size_t)i * out_stride + d] = v;
+    }
+  }
+}
+
+/* operators/impl/sampling/RepetitionPenalty.cu:19-41: logit > 0 ? logit / factor : logit * factor
+ * (factor 1 for tokens that are not penalised). */
+void orc_repetition_penalty(const float *logits, const float *factors, uint32_t n, float *out) {
+  for (uint32_t i = 0; i < n; ++i)
+    out[i] = logits[i] > 0.0f ? logits[i] / factors[i] : logits[i] * factors[i];
+}
+
+/* The dense factor vector the runner builds before every token (interface/runner/llama/llama.cpp:2566-2592):
+ * factor[token] = penalty for every token of the recent window (once, however often it occurs), 1 elsewhere. */
+void orc_penalty_factors(const int32_t *recent, uint32_t n_recent, float penalty, uint32_t vocab, float *factors) {
+  for (uint32_t i = 0; i < vocab; ++i)
+    factors[i] = 1.0f;
+  for (uint32_t i = 0; i < n_recent; ++i)
+    if (recent[i] >= 0 && (uint32_t)recent[i] < vocab)
+      factors[recent[i]] = penalty;
+}

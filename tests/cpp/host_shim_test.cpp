@@ -205,6 +205,56 @@ static void test_gpu() {
       EXPECT(normwise(c16, c4d) < 1e-5);
     }
   }
+  // a chain of two matmuls (up projection with SiLU, then down projection with a residual add) captured once and
+  // replayed on new activations: what a cached decode segment of the reference's runner does per token
+  {
+    const uint32_t K = 512, H = 768;
+    std::mt19937 rng(7);
+    std::normal_distribution<float> gw(0.0f, 0.05f), ga(0.0f, 1.0f);
+    std::vector<float> w1((size_t)H * K), w2((size_t)K * H);
+    for (auto &v : w1) v = gw(rng);
+    for (auto &v : w2) v = gw(rng);
+    std::vector<uint8_t> b1(ggufBytes(GgufFormat::Q4_K, (uint64_t)H * K)), b2(ggufBytes(GgufFormat::Q6_K, (uint64_t)K * H));
+    EXPECT(orc_quantize(CUTHIP_Q4_K, w1.data(), w1.size(), b1.data()) == 0);
+    EXPECT(orc_quantize(CUTHIP_Q6_K, w2.data(), w2.size(), b2.data()) == 0);
+    DeviceBuffer w1dev(b1.data(), b1.size()), w2dev(b2.data(), b2.size());
+    Tensor w1t{&w1dev, {(uint32_t)b1.size()}, DataType::Float32, 0}, w2t{&w2dev, {(uint32_t)b2.size()}, DataType::Float32, 0};
+    std::vector<float> x(K);
+    DeviceBuffer xdev(x.data(), x.size() * 4);
+    Tensor xt{&xdev, {K}, DataType::Float32, 0};
+    MatMulGgufOpNode up(xt, w1t, GgufFormat::Q4_K, H);
+    up.setFusion(MatMulFusion::Unary, CUTHIP_UNARY_SILU);
+    MatMulGgufOpNode down(up.output(), w2t, GgufFormat::Q6_K, K);
+    Tensor res{&xdev, {1, K}, DataType::Float32, K};
+    down.setFusion(MatMulFusion::Binary, CUTHIP_BINARY_ADD, res);
+    Stream stream;
+    CommandGraph graph;
+    up.dispatch(stream.get());      // one eager pass first (nothing of it is needed later)
+    down.dispatch(stream.get());
+    stream.sync();
+    graph.begin(stream);
+    up.dispatch(stream.get());
+    down.dispatch(stream.get());
+    graph.end(stream);
+    for (int rep = 0; rep < 3; ++rep) {
+      for (auto &v : x) v = ga(rng);
+      xdev.upload(x.data(), x.size() * 4);
+      graph.replay(stream);
+      stream.sync();
+      std::vector<float> got(K);
+      down.output().buffer->download(got.data(), got.size() * 4);
+      // the same chain on the CPU: fp64 products, SiLU in between, residual at the end
+      std::vector<double> h(H), y(K);
+      EXPECT(orc_matmul_gguf_f64(CUTHIP_Q4_K, b1.data(), x.data(), 1, K, H, h.data()) == 0);
+      std::vector<float> hf(H);
+      for (uint32_t i = 0; i < H; ++i) hf[i] = (float)(h[i] / (1.0 + std::exp(-h[i])));
+      EXPECT(orc_matmul_gguf_f64(CUTHIP_Q6_K, b2.data(), hf.data(), 1, H, K, y.data()) == 0);
+      for (uint32_t i = 0; i < K; ++i) y[i] += x[i];
+      double err = normwise(got, y);
+      if (!(err < 1e-3)) std::printf("graph replay %d err %g\n", rep, err);
+      EXPECT(err < 1e-3);
+    }
+  }
   // an explicit variant that cannot take the shape is an error, not a silent fallback
   {
     std::vector<uint8_t> blocks(ggufBytes(GgufFormat::Q8_0, 64 * 64), 0);
@@ -213,8 +263,11 @@ static void test_gpu() {
     std::vector<float> a(16 * 64, 1.0f);
     DeviceBuffer adev(a.data(), a.size() * 4);
     Tensor at{&adev, {16, 64}, DataType::Float32, 0};
-    MatMulGgufOpNode mm(at, wt, GgufFormat::Q8_0, 64, DataType::Float32, 0u);   // variant 0 handles M <= 8
+    MatMulGgufOpNode mm(at, wt, GgufFormat::Q8_0, 64, DataType::Float32, 3u);   // variant 3 (8-row GEMV) handles M <= 8
     EXPECT(throws([&] { mm.dispatch(); }));
+    // the table's default entry (0) takes every M: beyond 8 rows it is the library's choice by shape
+    MatMulGgufOpNode md(at, wt, GgufFormat::Q8_0, 64, DataType::Float32, 0u);
+    EXPECT(!throws([&] { md.dispatch(); }));
   }
 }
 

@@ -40,6 +40,74 @@ def test_variant_tables():
     assert L.variants(L.OP_DEQUANT)[0]["name"] == "DequantGguf8"
 
 
+# The reference's tables (operators/impl/matmul/MatMulQ8Variants.generated.h:20-32, MatMulQ4Variants.generated.h:20-29):
+# name, wgX, wgY, effTileM, effTileN at each index, and the defaults kMatMulQ8DefaultVariant / kMatMulQ4DefaultVariant.
+REF_Q8 = [("MatMulQ8T16R4x4", 16, 16, 64, 64), ("MatMulQ8Gemv", 256, 1, 1, 256), ("MatMulQ8VecT16R4x4", 16, 16, 64, 64),
+          ("MatMulQ8GemvKPar", 32, 1, 1, 4), ("MatMulQ8GemvKPar8", 32, 8, 1, 8), ("MatMulQ8GemvDot", 32, 1, 1, 4),
+          ("MatMulQ8TiledDot", 256, 1, 32, 64), ("MatMulQ8CoopMatTiled", 128, 1, 32, 32)]
+REF_Q4 = [("MatMulQ4T16R4x4", 16, 16, 64, 64), ("MatMulQ4Gemv", 256, 1, 1, 256), ("MatMulQ4GemvKPar", 32, 1, 1, 4),
+          ("MatMulQ4GemvKPar8", 32, 8, 1, 8), ("MatMulQ4CoopMatTiled", 128, 1, 32, 32)]
+
+
+@pytest.mark.parametrize("op,ref,default", [(L.OP_MATMUL_Q8, REF_Q8, 2), (L.OP_MATMUL_Q4, REF_Q4, 0)])
+def test_separated_layout_tables_hold_the_reference_names_at_the_reference_indices(op, ref, default):
+    lib = L.load()
+    v = L.variants(op)
+    assert [(x["name"], x["wgX"], x["wgY"], x["effTileM"], x["effTileN"]) for x in v] == ref
+    assert lib.cuthip_variant_count(op) == len(ref)
+    assert lib.cuthip_variant_default(op) == default
+    for i, row in enumerate(ref):
+        assert lib.cuthip_variant_lookup(op, row[0].encode()) == i
+        assert lib.cuthip_variant_available(op, i) == 1
+    assert lib.cuthip_variant_available(op, len(ref)) == -4
+
+
+def test_separated_layout_entry_points_take_the_variant_index():
+    """Unknown indices are refused before anything touches the GPU (no device is needed to see that)."""
+    lib = L.load()
+    one = C.c_void_p(256)
+    common = (one, one, one, None, one, 1, 64, 4, 64, 4, 4, 4, 0, 0)
+    assert lib.cuthip_matmul_q8_sep(*common, 8, None, 0, None) == -4
+    assert b"unknown variant index 8" in lib.cuthip_last_error()
+    assert lib.cuthip_matmul_q8_sep(*common, -2, None, 0, None) == -4
+    assert lib.cuthip_matmul_q4_sep(*common, 0, 5, None, 0, None) == -4
+    # the cooperative-matrix indices need K a multiple of 128 and a workspace: refused with a message, not skipped
+    assert lib.cuthip_matmul_q8_sep(*common, 7, None, 0, None) == -1
+    assert b"multiple of 128" in lib.cuthip_last_error()
+    assert lib.cuthip_matmul_q4_sep(*common, 0, 4, None, 0, None) == -1
+    # sizing follows the route of the index: a GEMV index never asks for the fp16 copy of the weights
+    small = lib.cuthip_matmul_sep_workspace_bytes_for(L.OP_MATMUL_Q8, 4, 32, 4096, 4096)
+    big = lib.cuthip_matmul_sep_workspace_bytes_for(L.OP_MATMUL_Q8, 7, 32, 4096, 4096)
+    auto = lib.cuthip_matmul_sep_workspace_bytes_for(L.OP_MATMUL_Q8, -1, 32, 4096, 4096)
+    assert big >= 4096 * 4096 * 2 > small and auto == lib.cuthip_matmul_sep_workspace_bytes(32, 4096, 4096) == big
+    assert lib.cuthip_matmul_sep_workspace_bytes_for(L.OP_MATMUL_Q4, 4, 1, 4096, 4096) >= 4096 * 4096 * 2
+
+
+def test_default_variant_of_the_gguf_table_is_valid_for_every_m():
+    lib = L.load()
+    assert lib.cuthip_variant_default(L.OP_MATMUL_GGUF) == 0
+    assert lib.cuthip_variant_default(77) == -1
+    assert lib.cuthip_variant_available(L.OP_MATMUL_GGUF, 4) == 1
+    assert lib.cuthip_variant_available(L.OP_MATMUL_GGUF, 5) in (0, 1)
+
+
+def test_fusion_operator_codes_are_the_reference_codes():
+    """OP_UNARY_* / OP_BINARY_* of operators/runtime/ComputeOpsShared.h:22-40, 118-167 for the operators that
+    cut_writeOutput implements (MatMulQ8Common.cuh:58-109)."""
+    assert L.UNARY == {"neg": 100, "abs": 101, "sqrt": 102, "square": 103, "reciprocal": 104, "exp": 106, "log": 109,
+                       "tanh": 121, "floor": 122, "ceil": 123, "round": 124, "relu": 130, "sigmoid": 131, "gelu": 132,
+                       "gelu_tanh": 132, "silu": 133, "softplus": 134, "relu6": 137, "mish": 141, "hardswish": 142,
+                       "hardsigmoid": 143, "rsqrt": 148}
+    assert L.BINARY == {"add": 0, "sub": 1, "mul": 2, "div": 3, "mod": 4, "pow": 5, "floor_div": 6, "min": 13, "max": 14}
+    lib = L.load()
+    assert sum(lib.cuthip_epilogue_op_supported(L.EPI_UNARY, c) for c in range(0, 200)) == 21
+    assert sum(lib.cuthip_epilogue_op_supported(L.EPI_BINARY, c) for c in range(0, 200)) == 9
+    header = open(os.path.join(ROOT, "include", "cut_hip.h")).read()
+    for name, code in list(L.UNARY.items()) + list(L.BINARY.items()):
+        kind = "UNARY" if name in L.UNARY and code >= 100 else "BINARY"
+        assert re.search(rf"CUTHIP_{kind}_{name.upper()} = {code}\b", header), (name, code)
+
+
 def test_argument_validation_without_a_device():
     lib = L.load()
     one = C.c_void_p(16)

@@ -72,8 +72,35 @@ def test_rope_kv_write(ops, n_heads, n_kv, hd, pos):
     assert not got_k[:pos].any() and not got_k[pos + 1:].any()
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("rows,dim,stride,offset", [(1, 1001, 1001, 0), (3, 1001, 1001, 0), (2, 1000, 1003, 0), (2, 4096, 4096, 1),
+                                                    (3, 5, 5, 0), (2, 7, 9, 3), (1, 8, 8, 1), (2, 9000, 9001, 0)])
+def test_rmsnorm_unaligned_rows(ops, dtype, rows, dim, stride, offset):
+    """Rows that do not start on a 16-byte boundary (odd dim or stride, a view that starts one element in), rows
+    shorter than one 8-element group and rows longer than the register window: every element must be read (the sum of
+    squares and every output), checked against the oracle."""
+    rng = np.random.default_rng(rows * dim + stride + offset)
+    buf = rng.standard_normal(offset + rows * stride).astype(dtype)
+    x = np.stack([buf[offset + r * stride: offset + r * stride + dim] for r in range(rows)])
+    w = rng.uniform(0.5, 1.5, dim).astype(np.float32)
+    want = oracle.rmsnorm(x.astype(np.float32), w, 1e-5)
+    xd = dev(buf)[offset:].as_strided((rows, dim), (stride, 1))
+    assert xd.data_ptr() % 16 != 0 or stride % 8 != 0 or dim < 8
+    for out_dtype, tol in ((torch.float32, 2e-6), (torch.float16, 1e-3)):
+        out = torch.full((rows, stride), -7.0, dtype=out_dtype, device="cuda")
+        ops.rmsnorm(xd, dev(w), 1e-5, out=out[:, :dim] if stride != dim else out)
+        torch.cuda.synchronize()
+        got = out.float().cpu().numpy()
+        np.testing.assert_allclose(got[:, :dim], want, rtol=tol, atol=tol * 1e-1)
+        assert np.all(got[:, dim:] == -7.0)   # the padding between rows is not written
+
+
 @pytest.mark.parametrize("n_heads,n_kv,hd,seq,max_ctx", [(32, 8, 128, 2048, 2048), (32, 8, 128, 1, 2048), (8, 2, 64, 77, 128),
-                                                       (6, 1, 128, 130, 256), (4, 4, 16, 64, 64)])
+                                                       (6, 1, 128, 130, 256), (4, 4, 16, 64, 64),
+                                                       # most splits empty; 128 splits (beyond the merge's register window);
+                                                       # 64 full splits; 8 query heads per KV head (two passes over the waves)
+                                                       (32, 8, 128, 5, 2048), (16, 4, 128, 4100, 8192), (8, 2, 64, 4096, 4096),
+                                                       (8, 1, 32, 200, 512)])
 def test_attention_decode(ops, n_heads, n_kv, hd, seq, max_ctx):
     rng = np.random.default_rng(seq)
     q = rng.standard_normal(n_heads * hd).astype(np.float32)
@@ -94,6 +121,13 @@ def test_attention_decode(ops, n_heads, n_kv, hd, seq, max_ctx):
     V2[seq:] = np.float16(np.nan)
     out = torch.empty(n_heads * hd, dtype=torch.float32, device="cuda")
     ops.attn_decode(dev(q), dev(K2), dev(V2), params, n_heads, n_kv, hd, scale, ws, out)
+    torch.cuda.synchronize()
+    assert normwise_rel_err(out.cpu().numpy(), want) < 2e-6
+    # an empty sequence: every split is empty and the output is zero, not NaN
+    ops.attn_decode(dev(q), dev(K2), dev(V2), dev(np.array([0, 0], np.int32)), n_heads, n_kv, hd, scale, ws, out)
+    torch.cuda.synchronize()
+    assert torch.all(out == 0)
+    ops.attn_decode(dev(q), dev(K), dev(V), params, n_heads, n_kv, hd, scale, ws, out)
     torch.cuda.synchronize()
     assert normwise_rel_err(out.cpu().numpy(), want) < 2e-6
 
@@ -125,6 +159,119 @@ def test_silu_mul_and_argmax(ops):
             torch.cuda.synchronize()
             assert int(idx.item()) == hot, (dt, n, off)
     del big
+
+
+@pytest.mark.parametrize("name", list(oracle.FORMATS))
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+def test_embedding_rows_from_gguf_blocks(ops, name, out_dtype):
+    """Gathered rows are bit-identical to the dequantized rows of the table (fp32: the CPU dequant; fp16: followed by the
+    reference's narrowing); ids on the device, repeated ids, an id past the table (zero row), a padded output stride."""
+    fmt = oracle.FORMATS[name]
+    vocab, dim = 300, 1024
+    table = quantized_weights(fmt, vocab, dim, seed=40)
+    ids = np.array([0, 299, 17, 17, 123, 300, 4000000000], np.uint32)
+    out = torch.full((len(ids), dim + 8), -3.0, dtype=out_dtype, device="cuda")
+    ops.embedding_rows(dev(table), fmt, dev(ids.view(np.int32)), vocab, dim, out[:, :dim])
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.all(got[:, dim:] == -3.0)
+    if out_dtype == torch.float32:
+        full = oracle.dequant(fmt, table, vocab * dim).reshape(vocab, dim)
+        want = np.stack([full[i] if i < vocab else np.zeros(dim, np.float32) for i in ids])
+        assert np.array_equal(got[:, :dim].view(np.uint32), want.view(np.uint32))
+    else:
+        full = oracle.dequant_f16(fmt, table, vocab * dim).reshape(vocab, dim)
+        want = np.stack([full[i] if i < vocab else np.zeros(dim, np.uint16) for i in ids])
+        assert np.array_equal(got[:, :dim].view(np.uint16), want)
+
+
+def test_embedding_col_against_oracle(ops):
+    """EmbeddingColOpNode on the tensors cuthip_prepare_sep writes (int8 [K, N] + fp16 scales [K/32, N]) and on an fp16
+    table, bit-exact against the oracle's restatement; the same rows as the GGUF gather."""
+    vocab, dim = 200, 256
+    table = quantized_weights(oracle.Q8_0, vocab, dim, seed=41)
+    B, S = ops.prepare_sep(dev(table), "Q8_0", vocab, dim)       # the loader's separated tensors, produced on the GPU
+    ids = np.array([5, 199, 0, 5], np.uint32)
+    got = ops.embedding_col(dev(ids.view(np.int32)), B.view(torch.int8), S, dim, vocab)
+    torch.cuda.synchronize()
+    want = oracle.embedding_col(ids, B.cpu().numpy().view(np.int8), S.cpu().numpy().view(np.uint16), dim, 1)
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    rows = oracle.dequant(oracle.Q8_0, table, vocab * dim).reshape(vocab, dim)[ids]
+    assert np.array_equal(want.view(np.uint32), rows.view(np.uint32))
+    t16 = np.random.default_rng(42).standard_normal((dim, vocab + 4)).astype(np.float16)
+    got16 = ops.embedding_col(dev(np.array([1, 198, 250], np.int32)), dev(t16), None, dim, vocab)
+    torch.cuda.synchronize()
+    w16 = oracle.embedding_col(np.array([1, 198], np.uint32), np.ascontiguousarray(t16).view(np.uint16), None, dim, 0)
+    assert np.array_equal(got16.cpu().numpy()[:2], w16) and not got16.cpu().numpy()[2].any()   # index past the vocabulary: zeros
+
+
+def test_repetition_penalty_and_penalized_argmax(ops):
+    """The dense operator against the oracle; the sparse list + arg-max against `dense penalty, then arg-max` with the
+    factor vector the runner would have built (repeated tokens penalised once, later entries override, ids out of
+    range ignored), for fp32 and fp16 logits; the logits are rewritten in place."""
+    rng = np.random.default_rng(50)
+    n = 128256
+    lg = (rng.standard_normal(n) * 3).astype(np.float32)
+    hot = int(np.argmax(lg))
+    second = int(np.argsort(lg)[-2])
+    fac = oracle.penalty_factors([hot, 12, 12, n + 5, -7, 99], 1.3, n)
+    out = ops.repetition_penalty(dev(lg), dev(fac))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), oracle.repetition_penalty(lg, fac))
+    idx = torch.zeros(1, dtype=torch.int32, device="cuda")
+    for dt in (np.float32, np.float16):
+        l_h = lg.astype(dt)
+        cases = [([], []), ([hot, 12, 12, n + 5, -7, 99], [100.0] * 6), ([hot, second, hot], [50.0, 60.0, 1.0]),
+                 ([hot] + [-1] * 63, [1e9] + [1.0] * 63)]
+        for toks, facs in cases:
+            dense = np.ones(n, np.float32)
+            for t, f in zip(toks, facs):
+                if 0 <= t < n:
+                    dense[t] = f                       # later entries override, as successive writes to factors[t] do
+            want_l = oracle.repetition_penalty(l_h.astype(np.float32), dense).astype(dt)
+            d = dev(l_h.copy())
+            pt = dev(np.array(toks, np.int32)) if toks else None
+            pf = dev(np.array(facs, np.float32)) if toks else None
+            ops.argmax_penalized(d, idx, pt, pf)
+            torch.cuda.synchronize()
+            assert int(idx.item()) == int(np.argmax(want_l)), (dt, toks)
+            assert np.array_equal(d.cpu().numpy(), want_l)
+
+
+@pytest.mark.parametrize("name,N,K", [("Q6_K", 128256, 4096), ("Q4_K", 14336, 4096), ("Q8_0", 12296, 512), ("Q6_K", 1000, 512)])
+def test_head_matmul_with_argmax_in_the_epilogue(ops, name, N, K):
+    """cuthip_matmul_gguf_argmax against the plain matmul followed by `penalty, then arg-max`: same logits bit for bit,
+    same token, with and without a penalty list that hits the unpenalised winner; N = 1000 takes the path without the
+    epilogue (K split inside the workgroup), the others the per-wave winners."""
+    fmt = oracle.FORMATS[name]
+    tile = quantized_weights(fmt, min(N, 1002), K, seed=60)
+    rb = oracle.n_bytes(fmt, K)
+    reps = -(-N // 1002)
+    W = dev(np.concatenate([np.roll(tile.reshape(-1, rb), 13 * t, axis=0) for t in range(reps)])[:N].reshape(-1))
+    a = dev(gauss_acts((1, K), seed=61, dtype=np.float16)).view(-1)
+    plain = ops.matmul_gguf(a, W, fmt, N, K, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    ref = plain.cpu().numpy()[0]
+    order = np.argsort(ref)
+    top, runner_up = int(order[-1]), int(order[-2])
+    ws = ops.lm_head_workspace(N, "cuda")
+    idx = torch.full((1,), -1, dtype=torch.int32, device="cuda")
+    for toks, facs in (([], []), ([top, 3, top], [1000.0, 2.0, 1000.0]), ([top, runner_up, 7], [1e9, 1e9, 1.5])):
+        logits = torch.empty(N, dtype=torch.float32, device="cuda")
+        dense = np.ones(N, np.float32)
+        for t, f in zip(toks, facs):
+            dense[t] = f
+        want_l = oracle.repetition_penalty(ref, dense)
+        pt = dev(np.array(toks, np.int32)) if toks else None
+        pf = dev(np.array(facs, np.float32)) if toks else None
+        ops.matmul_gguf_argmax(a, W, fmt, N, K, logits, idx, pen_tokens=pt, pen_factors=pf, workspace=ws)
+        torch.cuda.synchronize()
+        assert np.array_equal(logits.cpu().numpy(), want_l)
+        assert int(idx.item()) == int(np.argmax(want_l)), toks
+    # without a workspace: the logits are scanned instead, same answer
+    ops.matmul_gguf_argmax(a, W, fmt, N, K, logits, idx)
+    torch.cuda.synchronize()
+    assert int(idx.item()) == int(np.argmax(ref))   # the tile repeats, so the maximum does too: the first row wins
 
 
 def _oracle_step(cfg, layers_h, out_norm, head, x, pos, kc, vc, cos_t, sin_t):
@@ -223,6 +370,145 @@ def test_small_decode_step_against_oracle_chain(ops, fuse):
         g.replay()
         torch.cuda.synchronize()
         assert np.array_equal(step.logits.cpu().numpy(), got)
+
+
+@pytest.mark.parametrize("fuse", [4, 0])
+def test_decode_steps_feed_themselves_through_embedding_and_penalty(ops, fuse):
+    """Three consecutive tokens of a small model: every step gathers the embedding of the token the previous step
+    sampled (on the device), and samples with a repetition-penalty window; the logits of every step are checked
+    against the oracle chain fed with the same token, the sampled token against `penalty, then arg-max` of the step's
+    own logits (so a near-tie cannot make the two chains drift apart), eagerly and under replay of one captured graph."""
+    from cut_amd.decode import DecodeConfig, DecodeStep
+    cfg = DecodeConfig(hidden=512, n_layers=2, n_heads=8, n_kv_heads=2, head_dim=64, ffn=1024, vocab=2048, max_ctx=64)
+    rng = np.random.default_rng(21)
+
+    def qw(fmt, n, k):
+        return oracle.quantize(fmt, (rng.standard_normal(n * k) * 0.05).astype(np.float32))
+    layers_h = [{"qk": qw(oracle.Q4_K, cfg.q_dim + cfg.kv_dim, cfg.hidden), "v": qw(oracle.Q6_K, cfg.kv_dim, cfg.hidden),
+                 "o": qw(oracle.Q4_K, cfg.hidden, cfg.q_dim), "gate_up": qw(oracle.Q4_K, 2 * cfg.ffn, cfg.hidden),
+                 "down": qw(oracle.Q4_K, cfg.hidden, cfg.ffn),
+                 "attn_norm": rng.uniform(0.5, 1.5, cfg.hidden).astype(np.float32),
+                 "ffn_norm": rng.uniform(0.5, 1.5, cfg.hidden).astype(np.float32)} for _ in range(cfg.n_layers)]
+    out_norm = rng.uniform(0.5, 1.5, cfg.hidden).astype(np.float32)
+    head = qw(oracle.Q6_K, cfg.vocab, cfg.hidden)
+    embd = oracle.quantize(oracle.Q4_K, rng.standard_normal(cfg.vocab * cfg.hidden).astype(np.float32))
+    embd_f = oracle.dequant(oracle.Q4_K, embd, cfg.vocab * cfg.hidden).reshape(cfg.vocab, cfg.hidden)
+
+    def run(replay):
+        step = DecodeStep(cfg, [{k: dev(v) for k, v in L.items()} for L in layers_h], dev(out_norm), dev(head), fuse=fuse,
+                          embedding=dev(embd), penalty_window=8)
+        kc = [np.zeros((cfg.max_ctx, cfg.kv_dim), np.uint16) for _ in range(cfg.n_layers)]
+        vc = [np.zeros((cfg.max_ctx, cfg.kv_dim), np.uint16) for _ in range(cfg.n_layers)]
+        cos_t, sin_t = step.cos_t.cpu().numpy(), step.sin_t.cpu().numpy()
+        token, history, graph = 77, [77], None
+        step.token.fill_(token)
+        for pos in range(3):
+            step.set_position(pos)
+            step.set_penalties(history, 1.5, suppressed=[5])
+            torch.cuda.synchronize()
+            if replay:
+                if graph is None:
+                    step.step()                      # warm-up outside the capture (same inputs: the caches are rewritten)
+                    step.token.fill_(token)
+                    torch.cuda.synchronize()
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph):
+                        step.step()
+                    step.token.fill_(token)
+                graph.replay()
+            else:
+                step.step()
+            torch.cuda.synchronize()
+            got = step.logits.cpu().numpy()
+            want = _oracle_step(cfg, layers_h, out_norm, head, embd_f[token].copy(), pos, kc, vc, cos_t, sin_t)
+            fac = oracle.penalty_factors(history, 1.5, cfg.vocab)
+            fac[5] = 1e9
+            assert normwise_rel_err(got, oracle.repetition_penalty(want, fac)) < 1e-3, pos   # the step leaves the penalised logits
+            new = int(step.token.item())
+            assert new == int(np.argmax(got)), pos
+            assert new != 5
+            token = new
+            history.append(token)
+            # the next step of the oracle chain attends over the rows the GPU stored (its own differ from them by an
+            # fp16 ulp here and there, which a two-position softmax would amplify beyond the per-step bound)
+            for i in range(cfg.n_layers):
+                gk = step.k_cache[i].cpu().numpy().view(np.uint16)
+                gv = step.v_cache[i].cpu().numpy().view(np.uint16)
+                assert normwise_rel_err(gk[pos].view(np.float16).astype(np.float32), kc[i][pos].view(np.float16).astype(np.float32)) < 5e-3
+                kc[i][:pos + 1], vc[i][:pos + 1] = gk[:pos + 1], gv[:pos + 1]
+        return history
+    assert run(False) == run(True)
+
+
+def test_full_size_layer_and_head_against_oracle_chain(ops):
+    """BASELINE config 4 at its real geometry, one layer deep: hidden 4096, 32 query / 8 KV heads of 128, FFN 14336,
+    KV context 2048 (2047 cached positions + the current token), Q4_K projections, Q6_K w_v and the Q6_K
+    128256 x 4096 output head (16,032 row groups, the largest launch of the step).  The logits are compared with the
+    same chain composed from oracle calls on 512 sampled vocabulary rows (the head is sliced for the oracle; the GPU
+    runs it whole), normwise <= 1e-3.  The head's rows are a 2004-row quantized tile, rolled by a different amount
+    in each of its 64 repeats, so that sampled rows differ while the host encoder stays within seconds."""
+    from cut_amd.decode import DecodeConfig, DecodeStep
+    cfg = DecodeConfig(n_layers=1)
+    assert (cfg.hidden, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, cfg.ffn, cfg.vocab, cfg.max_ctx) == \
+        (4096, 32, 8, 128, 14336, 128256, 2048)
+    rng = np.random.default_rng(2048)
+    L = {"qk": quantized_weights(oracle.Q4_K, cfg.q_dim + cfg.kv_dim, cfg.hidden, seed=1),
+         "v": quantized_weights(oracle.Q6_K, cfg.kv_dim, cfg.hidden, seed=2),
+         "o": quantized_weights(oracle.Q4_K, cfg.hidden, cfg.q_dim, seed=3),
+         "gate_up": quantized_weights(oracle.Q4_K, 2 * cfg.ffn, cfg.hidden, seed=4),
+         "down": quantized_weights(oracle.Q4_K, cfg.hidden, cfg.ffn, seed=5),
+         "attn_norm": rng.uniform(0.5, 1.5, cfg.hidden).astype(np.float32),
+         "ffn_norm": rng.uniform(0.5, 1.5, cfg.hidden).astype(np.float32)}
+    out_norm = rng.uniform(0.5, 1.5, cfg.hidden).astype(np.float32)
+    tile_rows, reps = 2004, 64
+    rb = oracle.n_bytes(oracle.Q6_K, cfg.hidden)
+    tile = quantized_weights(oracle.Q6_K, tile_rows, cfg.hidden, seed=6).reshape(tile_rows, rb)
+    head = np.concatenate([np.roll(tile, 37 * t, axis=0) for t in range(reps)]).reshape(-1)
+    assert head.size == cfg.vocab * rb
+    pos = cfg.max_ctx - 1
+    kc = np.zeros((cfg.max_ctx, cfg.kv_dim), np.uint16)
+    vc = np.zeros((cfg.max_ctx, cfg.kv_dim), np.uint16)
+    kc[:pos] = (rng.standard_normal((pos, cfg.kv_dim)) * 0.5).astype(np.float16).view(np.uint16)
+    vc[:pos] = rng.standard_normal((pos, cfg.kv_dim)).astype(np.float16).view(np.uint16)
+    x = rng.standard_normal(cfg.hidden).astype(np.float32)
+    sample = np.unique(np.concatenate([np.arange(0, 16), np.arange(cfg.vocab - 16, cfg.vocab),
+                                       rng.choice(cfg.vocab, 480, replace=False)]))
+    head_rows = head.reshape(cfg.vocab, rb)[sample].reshape(-1)
+
+    for fuse in (4, 0):
+        step = DecodeStep(cfg, [{k: dev(v) for k, v in L.items()}], dev(out_norm), dev(head), fuse=fuse)
+        step.k_cache[0].copy_(dev(kc.view(np.float16)))
+        step.v_cache[0].copy_(dev(vc.view(np.float16)))
+        step.x.copy_(dev(x))
+        step.set_position(pos)
+        step.step()
+        torch.cuda.synchronize()
+        got = step.logits.cpu().numpy()
+        if fuse == 4:
+            cos_t, sin_t = step.cos_t.cpu().numpy(), step.sin_t.cpu().numpy()
+            sub = dataclasses_replace_vocab(cfg, len(sample))
+            want = _oracle_step(sub, [L], out_norm, head_rows, x.copy(), pos, [kc.copy()], [vc.copy()], cos_t, sin_t)
+        assert np.all(np.isfinite(got))
+        assert normwise_rel_err(got[sample], want) < 1e-3, fuse
+        assert int(step.token.item()) == int(np.argmax(got))
+        # the cache row of the current token was appended, the cached context left as it was
+        v_new = step.v_cache[0][pos].float().cpu().numpy()
+        assert normwise_rel_err(v_new, _v_row(L, cfg, x)) < 1e-3
+        assert np.array_equal(step.v_cache[0][:pos].cpu().numpy().view(np.uint16), vc[:pos])
+        assert np.array_equal(step.k_cache[0][:pos].cpu().numpy().view(np.uint16), kc[:pos])
+        del step
+        torch.cuda.empty_cache()
+
+
+def dataclasses_replace_vocab(cfg, vocab):
+    import dataclasses
+    return dataclasses.replace(cfg, vocab=vocab)
+
+
+def _v_row(L, cfg, x):
+    """The v projection of the current token by the oracle chain."""
+    xn = oracle.rmsnorm(x, L["attn_norm"], cfg.eps).astype(np.float16).astype(np.float32)
+    return oracle.matmul_gguf(oracle.Q6_K, L["v"], xn[None], cfg.kv_dim, f64=True)[0].astype(np.float32)
 
 
 @pytest.mark.parametrize("name", ["Q4_K", "Q6_K", "Q8_0", "Q4_0"])

@@ -123,11 +123,12 @@ def test_nonfinite_scales_keep_their_class(ops):
         assert np.array_equal(got[fin].view(np.uint32), want[fin].view(np.uint32)), name
 
 
-def test_full_size_properties(ops):
-    """256 Mi elements (BASELINE config 2) -> fp16: tiled weights, so every
+@pytest.mark.parametrize("name", list(oracle.FORMATS))
+def test_full_size_properties(ops, name):
+    """256 Mi elements (BASELINE config 2) -> fp16, every format: tiled weights, so every
     repeat of the tile must dequantize to the same bits as the first, which is
     checked against the oracle; plus a checksum over the whole output."""
-    fmt = oracle.Q4_K
+    fmt = oracle.FORMATS[name]
     tile_rows, cols, reps = 1024, 4096, 64  # 64 x 4 Mi = 256 Mi elements
     tile = quantized_weights(fmt, tile_rows, cols, seed=0)
     raw = torch.from_numpy(tile).cuda().repeat(reps)

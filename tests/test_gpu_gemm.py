@@ -298,9 +298,10 @@ def test_blaslt_gemm_fp32_activations_and_automatic_choice(ops):
     A = gauss_acts((M, K), seed=54)
     want = oracle.matmul_gguf(fmt, W, A, N, f64=True)
     assert normwise_rel_err(gpu_matmul_ws(ops, fmt, W, A, N, K, variant=5), want) < 8e-4
-    # M >= 1024 without an epilogue: the automatic choice takes the same path; with an epilogue the hand-written GEMM
+    # the automatic choice never takes the vendor library (that is opt-in): it is the hand-written two-pass GEMM, bit for bit
     auto = gpu_matmul_ws(ops, fmt, W, A, N, K, variant=-1)
     assert normwise_rel_err(auto, want) < 8e-4
+    assert np.array_equal(auto, gpu_matmul_ws(ops, fmt, W, A, N, K, variant=4))
     D = gauss_acts((M, N), seed=55)
     add = gpu_matmul_ws(ops, fmt, W, A, N, K, variant=-1, binary="add", d=torch.from_numpy(D).cuda())
     assert normwise_rel_err(add, want + D) < 8e-4

@@ -157,6 +157,89 @@ def test_fused_epilogues(ops):
     assert np.array_equal(add, plain + D)
 
 
+# cut_writeOutput's operator set (operators/impl/matmul/MatMulQ8Common.cuh:58-109) restated in float64 numpy
+UNARY_F64 = {
+    "neg": lambda x: -x, "abs": np.abs, "sqrt": np.sqrt, "square": lambda x: x * x, "reciprocal": lambda x: 1.0 / x,
+    "exp": np.exp, "log": np.log, "tanh": np.tanh, "floor": np.floor, "ceil": np.ceil,
+    "round": lambda x: np.sign(x) * np.floor(np.abs(x) + 0.5),   # half away from zero, as roundf
+    "relu": lambda x: np.maximum(0.0, x), "sigmoid": lambda x: 1.0 / (1.0 + np.exp(-x)),
+    "gelu": lambda x: x * 0.5 * (1.0 + np.tanh(np.sqrt(2.0 / 3.14159265) * (x + 0.044715 * x * x * x))),
+    "silu": lambda x: x / (1.0 + np.exp(-x)), "softplus": lambda x: np.log(1.0 + np.exp(x)),
+    "relu6": lambda x: np.clip(x, 0.0, 6.0), "mish": lambda x: x * np.tanh(np.log(1.0 + np.exp(x))),
+    "hardswish": lambda x: x * np.clip(x / 6.0 + 0.5, 0.0, 1.0), "hardsigmoid": lambda x: np.clip(x / 6.0 + 0.5, 0.0, 1.0),
+    "rsqrt": lambda x: 1.0 / np.sqrt(x),
+}
+BINARY_F64 = {
+    "add": lambda a, b: a + b, "sub": lambda a, b: a - b, "mul": lambda a, b: a * b, "div": lambda a, b: a / b,
+    "mod": lambda a, b: a - b * np.floor(a / b), "pow": lambda a, b: np.power(a, b), "floor_div": lambda a, b: np.floor(a / b),
+    "min": np.minimum, "max": np.maximum,
+}
+
+
+@pytest.mark.parametrize("M", [1, 3, 64])   # the 8-row GEMV (direct epilogue), the same kernel's batch path, the tiled GEMM
+@pytest.mark.parametrize("op", sorted(UNARY_F64))
+def test_every_unary_fusion_op(ops, op, M):
+    """All 21 unary operators of the reference's fused epilogue, applied to the matmul result, against the float64
+    formula on the unfused GPU result (so the comparison isolates the operator; the matmul itself is checked
+    elsewhere).  Inputs are scaled so that sqrt / log / rsqrt see both signs (NaN where the reference gives NaN)."""
+    fmt = oracle.Q4_K
+    N, K = 264, 512
+    W = quantized_weights(fmt, N, K, seed=30)
+    A = (gauss_acts((M, K), seed=31) * 4.0).astype(np.float16)
+    plain = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32)
+    got = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32, unary=op)
+    with np.errstate(all="ignore"):
+        want = UNARY_F64[op](plain.astype(np.float64))
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    if op in ("floor", "ceil", "round", "neg", "abs", "relu", "relu6", "square"):
+        assert np.array_equal(got[ok], want[ok].astype(np.float32))   # exact in fp32
+    else:
+        # the formulas are evaluated in fp32 on the device, as the reference does: log(1 + exp(x)) loses up to 2^-24
+        # absolute in the sum, hence the absolute term
+        np.testing.assert_allclose(got[ok], want[ok], rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("M", [1, 3, 64])
+@pytest.mark.parametrize("op", sorted(BINARY_F64))
+def test_every_binary_fusion_op(ops, op, M):
+    """All 9 binary operators (matmul result op D) against float64."""
+    fmt = oracle.Q4_K
+    N, K = 264, 512
+    W = quantized_weights(fmt, N, K, seed=32)
+    A = (gauss_acts((M, K), seed=33) * 4.0).astype(np.float16)
+    D = gauss_acts((M, N), seed=34) * np.float32(1.5)
+    if op == "pow":
+        D = np.round(D * 2.0).astype(np.float32)   # integer exponents: defined for negative bases too
+    plain = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32)
+    got = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32, binary=op, d=torch.from_numpy(D).cuda())
+    with np.errstate(all="ignore"):
+        want = BINARY_F64[op](plain.astype(np.float64), D.astype(np.float64))
+    if op in ("add", "sub", "mul", "div", "min", "max"):
+        assert np.array_equal(got, want.astype(np.float32))   # one correctly rounded fp32 operation
+    elif op in ("mod", "floor_div"):
+        # a / b is rounded to fp32 before floor: where the float64 quotient sits within an ulp of an integer the two may
+        # legitimately differ by one step of b; everywhere else they agree
+        q = plain.astype(np.float64) / D.astype(np.float64)
+        safe = np.abs(q - np.round(q)) > 1e-5 * np.maximum(1.0, np.abs(q))
+        np.testing.assert_allclose(got[safe], want[safe], rtol=2e-6, atol=2e-6)
+        assert safe.mean() > 0.99
+    else:
+        fin = np.isfinite(want) & (np.abs(want) < 1e30)
+        np.testing.assert_allclose(got[fin], want[fin], rtol=3e-6, atol=1e-30)
+
+
+def test_unknown_fusion_operator_is_refused(ops):
+    from cut_amd import lib
+    L = lib.load()
+    assert L.cuthip_epilogue_op_supported(lib.EPI_UNARY, 133) == 1 and L.cuthip_epilogue_op_supported(lib.EPI_UNARY, 105) == 0
+    assert L.cuthip_epilogue_op_supported(lib.EPI_BINARY, 14) == 1 and L.cuthip_epilogue_op_supported(lib.EPI_BINARY, 7) == 0
+    t = torch.zeros(1024, dtype=torch.float32, device="cuda")
+    rc = L.cuthip_matmul_gguf(lib.Q4_K, t.data_ptr(), t.data_ptr(), lib.F32, t.data_ptr(), lib.F32, 1, 256, 4, 256, 4,
+                              lib.EPI_UNARY, 105, None, -1, None)   # OP_UNARY_SIGN: not in cut_writeOutput
+    assert rc == -1 and b"operator code 105" in L.cuthip_last_error()
+
+
 def test_strided_a_and_c(ops):
     fmt = oracle.Q6_K
     N, K, M = 64, 512, 2

@@ -89,16 +89,17 @@ def test_distance_from_the_fp32_path_and_epilogues(ops):
     np.testing.assert_allclose(host(ops.matmul_q8_i8(dev(A), dev(W), N, K, unary="relu")), np.maximum(ref, 0), rtol=0, atol=1e-4)
 
 
-def test_full_shape_sampled(ops):
-    # BASELINE configs[4] shape at M = 512: sampled rows and columns against the oracle, linearity in the scale of A
-    M, K, N = 512, 4096, 14336
+@pytest.mark.parametrize("M", [512, 2048])
+def test_full_shape_sampled(ops, M):
+    # BASELINE configs[4] shapes (M = 512 and 2048): sampled rows and columns against the oracle, linearity in the scale of A
+    K, N = 4096, 14336
     rng = np.random.default_rng(11)
     A = rng.standard_normal((M, K), dtype=np.float32).astype(np.float16)
     tile = quantized_weights(oracle.Q8_0, 512, K, seed=12)
     W = np.tile(tile, N // 512)
     Wd, Ad = dev(W), dev(A)
     got = host(ops.matmul_q8_i8(Ad, Wd, N, K, out_dtype=torch.float32))
-    rows = [0, 1, 255, 256, 511]
+    rows = [0, 1, 255, 256, 511, M - 129, M - 1]
     ref = oracle.matmul_q8_i8(tile, A[rows].astype(np.float32), 512, f64=True)
     for c0 in (0, 512 * 13, N - 512):
         assert normwise_rel_err(got[rows][:, c0:c0 + 512], ref) < 1e-5

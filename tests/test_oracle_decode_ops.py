@@ -115,3 +115,43 @@ def test_silu_mul():
     want = g.astype(np.float64) / (1 + np.exp(-g.astype(np.float64))) * u
     np.testing.assert_allclose(got, want, rtol=2e-7, atol=1e-12)
     assert got[0] == 0.0 and abs(got[3] - 10.0) < 1e-6
+
+
+# ---- embedding gather and repetition penalty ---------------------------------------------------------------
+
+def test_embedding_col_int8_equals_dequant_of_the_gguf_row():
+    """EmbeddingCol on the loader's separated Q8_0 tensors (values [N, K] and scales [N, K/32] transposed to the
+    column-wise [K, N] / [K/32, N] form the GPU upload produces) gathers exactly the dequantized GGUF row: the
+    pinned dequantizer fixes every index of the column-wise addressing (d * vocabStride + t, (d >> 5) * scaleStride + t)."""
+    vocab, dim = 40, 96
+    rng = np.random.default_rng(5)
+    blocks = oracle.quantize(oracle.Q8_0, (rng.standard_normal(vocab * dim) * 0.05).astype(np.float32))
+    vals, scales = oracle.split_q8_0(blocks, vocab, dim)           # [vocab, dim] int8, [vocab, dim/32] fp16 bits
+    matrix = np.ascontiguousarray(vals.reshape(vocab, dim).T)       # [dim, vocab]
+    sc = np.ascontiguousarray(scales.reshape(vocab, dim // 32).T)   # [dim/32, vocab]
+    idx = np.array([0, 39, 7, 7, 21], np.uint32)
+    got = oracle.embedding_col(idx, matrix, sc, dim, 1)
+    want = oracle.dequant(oracle.Q8_0, blocks, vocab * dim).reshape(vocab, dim)[idx]
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_embedding_col_fp16_is_the_table_column():
+    vocab, dim = 17, 24
+    rng = np.random.default_rng(6)
+    table = rng.standard_normal((dim, vocab)).astype(np.float16)
+    got = oracle.embedding_col(np.array([3, 16, 0], np.uint32), table.view(np.uint16), None, dim, 0)
+    assert np.array_equal(got, table.astype(np.float32).T[[3, 16, 0]])
+
+
+def test_repetition_penalty_closed_forms():
+    """factor 1 is the identity; a positive logit is divided, a negative one multiplied, zero stays zero (the sign
+    test is `> 0`); the factor vector built from a token window marks each token once."""
+    lg = np.array([2.0, -2.0, 0.0, 5.0, -0.5, 3.0], np.float32)
+    assert np.array_equal(oracle.repetition_penalty(lg, np.ones(6, np.float32)), lg)
+    f = np.array([1.0, 1.0, 4.0, 2.0, 2.0, 1.0], np.float32)
+    assert np.array_equal(oracle.repetition_penalty(lg, f), np.array([2.0, -2.0, 0.0, 2.5, -1.0, 3.0], np.float32))
+    fac = oracle.penalty_factors([3, 4, 3, 3, -1, 99], 2.0, 6)
+    assert np.array_equal(fac, np.array([1, 1, 1, 2, 2, 1], np.float32))
+    # penalising twice is not what a repeated token gets
+    once = oracle.repetition_penalty(lg, fac)
+    assert once[3] == 2.5 and once[4] == -1.0
