@@ -33,10 +33,8 @@
 #include <stdio.h>
 #include <stdlib.h>
 
-#include <type_traits>
-#include <utility>
-
 #include "common.hpp"
+#include "gemm_store.hpp"
 
 namespace cuthip {
 
@@ -46,13 +44,6 @@ int launch_dequant_any(int fmt, const void *blocks, void *out, int out_dtype, ui
 typedef _Float16 half8v __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) uint8_t lds_u8;
 
-template <int... Is, class F> __device__ inline void static_for_impl(std::integer_sequence<int, Is...>, F &&f) {
-  (f(std::integral_constant<int, Is>{}), ...);
-}
-template <int N, class F> __device__ inline void static_for(F &&f) {
-  static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F &&>(f));
-}
-
 struct DenseParams {
   const uint8_t *A, *W;  // fp16 [M, strideA], fp16 [N, K]
   void *C;
@@ -61,6 +52,11 @@ struct DenseParams {
   int c_f16;
   uint32_t ksplit, kper;  // K is cut into ksplit ranges of kper (a multiple of 128); a workgroup multiplies one range
   float *partial;         // ksplit > 1: fp32 [ksplit][M][N] partial products instead of C
+  // L2 warm-up: in every slice a workgroup touches, pf_dist slices ahead, every pf_wsplit-th row of its weight panel
+  // and every pf_asplit-th row of its activation tile; the workgroups that run beside it on the same XCD and share the
+  // panel (the tile) touch the other rows.
+  uint32_t pf_dist, pf_wsplit, pf_asplit;
+  int vec_store;          // C (and a binary epilogue's operand) allow 16-byte accesses
 };
 
 constexpr int kDBN = 256, kDBK = 64;
@@ -75,19 +71,21 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
   static_assert((NJ == 4 && (MI == 4 || MI == 2)) || (NJ == 7 && MI == 2), "tile shape");
   static_assert((BM + BN) * 128 * 2 <= 160 * 1024, "two LDS stages");
   static_assert((NL - 1) * LSTEP < 3 * NM, "the last load must be issued before the last k-step of the slice");
-  __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * 128];
-  __shared__ __attribute__((aligned(1024))) uint8_t sA1[BM * 128];
-  __shared__ __attribute__((aligned(1024))) uint8_t sB0[BN * 128];
-  __shared__ __attribute__((aligned(1024))) uint8_t sB1[BN * 128];
+  static_assert(4 * stripe_floats<NJ>() * 4 <= (BM + BN) * 128 * 2, "the output staging reuses the operand stages");
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[(BM + BN) * 128 * 2];
+  uint8_t *const sA0 = lds, *const sA1 = lds + BM * 128, *const sB0 = lds + BM * 256, *const sB1 = lds + BM * 256 + BN * 128;
+  constexpr int NPF = 2;                     // L2 warm-up loads per wave per slice: 4 waves x 64 lanes x NPF lines
+  __shared__ uint32_t pf_sink[4 * 64];       // where they land; never read
 
   // XCD-aware tile order: ids id, id+8, id+16, ... share an XCD and its L2; give
   // them the M-tiles of the same weight panels.
   const uint32_t tiles = p.mtiles * p.ntiles, split = blockIdx.x / tiles;
-  uint32_t id = blockIdx.x - split * tiles, mt, nt;
+  uint32_t id = blockIdx.x - split * tiles, mt, nt, aphase = 0;
   if (p.ntiles % 8 == 0) {
     uint32_t xcd = id & 7, slot = id >> 3;
     nt = (slot / p.mtiles) * 8 + xcd;
     mt = slot % p.mtiles;
+    aphase = (slot / p.mtiles) % p.pf_asplit;
   } else {
     nt = id / p.mtiles;
     mt = id % p.mtiles;
@@ -112,12 +110,34 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
     uint32_t r = min(n0 + 8 * (4 * v + wave) + (lane >> 3), p.N - 1);
     boff[v] = r * p.K * 2 + chunk;
   }
+  // the lambdas below capture plain locals, never a field of p: a captured parameter block is copied to scratch memory
+  const uint8_t *const gA = p.A, *const gW = p.W;
+  const uint32_t pf_dist = p.pf_dist, Mrows = p.M, Ncols = p.N;
   auto load_one = [&](int l, uint8_t *na, uint8_t *nb, uint32_t k0) {
-    const uint8_t *ga = p.A + (size_t)k0 * 2, *gb = p.W + (size_t)k0 * 2;
+    const uint8_t *ga = gA + (size_t)k0 * 2, *gb = gW + (size_t)k0 * 2;
     if (l < NLA)
       __builtin_amdgcn_global_load_lds(ga + aoff[l], na + (4 * l + wave) * 1024, 16, 0, 0);
     else
       __builtin_amdgcn_global_load_lds(gb + boff[l - NLA], nb + (4 * (l - NLA) + wave) * 1024, 16, 0, 0);
+  };
+
+  // Line q = 256 i + tid of the warm-up: the first ceil(BN / wsplit) are rows of the weight panel, the next
+  // ceil(BM / asplit) rows of the activation tile; what is left over repeats the first line of the panel.
+  const uint8_t *pfp[NPF];
+  {
+    const uint32_t nw = (BN + p.pf_wsplit - 1) / p.pf_wsplit, na = (BM + p.pf_asplit - 1) / p.pf_asplit;
+#pragma unroll
+    for (int i = 0; i < NPF; ++i) {
+      const uint32_t q = 256 * i + tid;
+      uint32_t wr = mt % p.pf_wsplit + (q < nw ? q : 0) * p.pf_wsplit, ar = aphase + (q - nw) * p.pf_asplit;
+      const bool is_a = q >= nw && q - nw < na && ar < BM;
+      wr = min(n0 + min(wr, (uint32_t)BN - 1), p.N - 1);
+      ar = min(m0 + ar, p.M - 1);
+      pfp[i] = is_a ? p.A + (size_t)ar * p.strideA * 2 : p.W + (size_t)wr * p.K * 2;
+    }
+  }
+  auto warm_one = [&](int i, uint32_t k0) {
+    __builtin_amdgcn_global_load_lds(pfp[i] + (size_t)k0 * 2, pf_sink + wave * 64, 4, 0, 0);
   };
 
   f32x16 acc[MI][NJ];
@@ -143,7 +163,8 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
   // The NM MFMAs of one k-step on fragment set f.  After MFMA idx: the idx-th fragment read of k-step s of
   // (sa, sb) into the other set, and, in every LSTEP-th slot of the slice (g = position of the group in the
   // slice), one load of the next slice (k0) into (na, nb).
-  auto group = [&](int g, int f, const uint8_t *sa, const uint8_t *sb, int s, uint8_t *na, uint8_t *nb, uint32_t k0) {
+  auto group = [&](int g, int f, const uint8_t *sa, const uint8_t *sb, int s, uint8_t *na, uint8_t *nb, uint32_t k0,
+                   uint32_t kpf) {
     const uint32_t pa = (uint32_t)(uintptr_t)(lds_u8 *)(sa) + arow + xs[s];
     const uint32_t pb = (uint32_t)(uintptr_t)(lds_u8 *)(sb) + brow + xs[s];
 #pragma unroll
@@ -156,6 +177,7 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
         asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[f ^ 1][idx - MI]) : "v"(pb), "n"((idx - MI) * 4096) : "memory");
       const int q = g * NM + idx;
       if (q % LSTEP == 0 && q / LSTEP < NL) load_one(q / LSTEP, na, nb, k0);
+      if (g == 3 && idx % 4 == 0 && idx / 4 < NPF) warm_one(idx / 4, kpf);   // younger than every load of the slice
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -165,19 +187,26 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
   // slice's last k-step; its MFMAs run under the first fragment reads of this slice.  The loads of the slice
   // after the last one re-read the last slice (never used) instead of branching around the MFMAs.
   auto slice = [&](uint8_t *sa, uint8_t *sb, uint8_t *na, uint8_t *nb, uint32_t t) {
-    const uint32_t k0 = min(kbeg + (t + 1) * kDBK, klast);
-    group(0, 1, sa, sb, 0, na, nb, k0);
+    const uint32_t k0 = min(kbeg + (t + 1) * kDBK, klast), kpf = min(kbeg + (t + pf_dist) * kDBK, klast);
+    group(0, 1, sa, sb, 0, na, nb, k0, kpf);
     CUTHIP_WAIT_FRAGS(0, 0);
-    group(1, 0, sa, sb, 1, na, nb, k0);
+    group(1, 0, sa, sb, 1, na, nb, k0, kpf);
     CUTHIP_WAIT_FRAGS(1, 0);
-    group(2, 1, sa, sb, 2, na, nb, k0);
+    group(2, 1, sa, sb, 2, na, nb, k0, kpf);
     CUTHIP_WAIT_FRAGS(0, 0);
-    group(3, 0, sa, sb, 3, na, nb, k0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next slice has landed in (na, nb)
+    group(3, 0, sa, sb, 3, na, nb, k0, kpf);
+    // The next slice has landed in (na, nb).  The warm-up loads of this slice stay in flight (memory returns in order
+    // and they are the youngest); those of the slice before had this whole slice to come back.
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NPF) : "memory");
     CUTHIP_WAIT_FRAGS(1, 0);                           // and this wave is done reading (sa, sb)
-    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_barrier" ::: "memory");   // as text: before __syncthreads() or the builtin the compiler waits for every load in flight
+    __builtin_amdgcn_sched_barrier(0);
   };
 
+  for (uint32_t d = 1; d < p.pf_dist; ++d)
+#pragma unroll
+    for (int i = 0; i < NPF; ++i) warm_one(i, min(kbeg + d * kDBK, klast));
 #pragma unroll
   for (int l = 0; l < NL; ++l) load_one(l, sA0, sB0, kbeg);
 #pragma unroll
@@ -195,24 +224,31 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[1][i], fb[1][j], acc[i][j], 0, 0, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last warm-up loads: nothing may land after the exit
 #undef CUTHIP_WAIT_FRAGS
 
-  // C tile: register r of lane l holds row 8*(r/4) + 4*(l>>5) + r%4, column l & 31 of its 32x32 block.
-  // Compile-time tile indices: a rolled loop would index the accumulators dynamically and copy them to scratch.
-  static_for<MI * NJ>([&](auto ij) {
-    constexpr int i = decltype(ij)::value / NJ, j = decltype(ij)::value % NJ;
-    const uint32_t col = n0 + wn * (BN / 2) + 32 * j + (lane & 31);
-    const uint32_t row0 = m0 + wm * (BM / 2) + 32 * i + 4 * (lane >> 5);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const uint32_t row = row0 + 8 * (r >> 2) + (r & 3);
-      if (row < p.M && col < p.N) {
-        if (p.ksplit > 1)
-          p.partial[((size_t)split * p.M + row) * p.N + col] = acc[i][j][r];
-        else
-          store_out(p.C, p.epi, p.c_f16, (size_t)row * p.strideC + col, acc[i][j][r]);
-      }
-    }
+  // C tile through LDS, a 32-row stripe of the wave's sub-tile at a time.  The operand stages are free once every
+  // wave has its last loads back and has read its last fragments.
+  __syncthreads();
+  lds_f32 *stage = (lds_f32 *)(lds_u8 *)(lds) + wave * stripe_floats<NJ>();
+  void *cbase = p.C;
+  uint32_t ldc = p.strideC;
+  int c_f16 = p.c_f16;
+  Epilogue epi = p.epi;
+  if (p.ksplit > 1) {   // fp32 partial products [ksplit][M][N]; the reduce kernel applies the epilogue
+    cbase = p.partial + (size_t)split * p.M * p.N;
+    ldc = p.N;
+    c_f16 = 0;
+    epi.kind = CUTHIP_EPI_NONE;
+  }
+  const bool vec = p.ksplit > 1 ? p.N % 4 == 0 : p.vec_store != 0;
+  static_for<MI>([&](auto ii) __attribute__((always_inline)) {
+    constexpr int i = decltype(ii)::value;
+    static_for<NJ>([&](auto jj) __attribute__((always_inline)) {
+      constexpr int j = decltype(jj)::value;
+      stage_tile32<NJ>(stage, j, acc[i][j], lane);
+    });
+    store_staged32<NJ>(stage, m0 + wm * (BM / 2) + 32 * i, n0 + wn * (BN / 2), Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
   });
 #endif
 }
@@ -242,6 +278,17 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *partial
 template <int BM, int BN> static int launch_dense_bm(DenseParams p, hipStream_t stream) {
   p.mtiles = (p.M + BM - 1) / BM;
   p.ntiles = (p.N + BN - 1) / BN;
+  // Who runs beside whom: with the XCD-aware order an XCD's 32 CUs hold 32 consecutive slots = the M-tiles of
+  // 32 / mtiles weight panels.  Otherwise every workgroup warms all its own lines.
+  p.pf_dist = 3;
+  p.pf_wsplit = p.pf_asplit = 1;
+  if (p.ntiles % 8 == 0) {
+    p.pf_wsplit = p.mtiles < 32 ? p.mtiles : 32;
+    const uint32_t panels = 32 / p.pf_wsplit, per_xcd = p.ntiles / 8;
+    p.pf_asplit = panels < per_xcd ? panels : per_xcd;
+    if (p.pf_asplit == 0) p.pf_asplit = 1;
+  }
+  if (const char *env = getenv("CUT_HIP_DENSE_PF")) p.pf_dist = (uint32_t)atoi(env);
   uint64_t grid = (uint64_t)p.mtiles * p.ntiles * p.ksplit;
   if (grid > 0x7FFFFFFFull) {
     set_error("cuthip_matmul_gguf_ws: problem too large for one launch");
@@ -355,6 +402,7 @@ int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C,
   p.M = M; p.N = N; p.K = K; p.strideC = strideC;
   p.mtiles = p.ntiles = 0;
   p.c_f16 = c_f16;
+  p.vec_store = store8_aligned(C, strideC, c_f16, epi) ? 1 : 0;
   const DenseShape sh = pick_dense_shape(M, K, N);
   p.ksplit = sh.ksplit;
   p.kper = K / sh.ksplit;
