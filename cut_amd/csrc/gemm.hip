@@ -27,6 +27,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "gemm_store.hpp"
 
 namespace cuthip {
 
@@ -39,6 +40,7 @@ struct GemmParams {
   uint32_t row_bytes;
   uint32_t mtiles, ntiles;
   int a_f16, c_f16;
+  int vec_store;   // C (and a binary epilogue's operand) allow 16-byte accesses
 };
 
 constexpr int kBN = 128, kBK = 64, kLdsRow = kBK + 8;  // halfs per LDS row
@@ -155,6 +157,7 @@ template <> struct Sub<CUTHIP_Q4_0> {
 };
 
 typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) uint8_t lds_u8g;
 
 // ---- the kernel -----------------------------------------------------------------
 template <int FMT, int BM, bool AF16>
@@ -277,18 +280,22 @@ __global__ void __launch_bounds__(256, 2) gemm_kernel(GemmParams p) {
     mma_slice();
   }
 
-  // C tile: register r of lane l holds row 8*(r/4) + 4*(l>>5) + r%4, column l & 31 of its 32x32 block
-#pragma unroll
-  for (int i = 0; i < MI; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      uint32_t col = n0 + wn * 64 + 32 * j + (lane & 31);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        uint32_t row = m0 + wm * (BM / 2) + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (row < p.M && col < p.N) store_out(p.C, p.epi, p.c_f16, (size_t)row * p.strideC + col, acc[i][j][r]);
-      }
-    }
+  // C tile through LDS, a 32-row stripe of the wave's sub-tile at a time (gemm_store.hpp); the operand tiles are free
+  // once every wave has multiplied the last slice
+  static_assert(4 * stripe_floats<2>() * 4 <= (BM + kBN) * kLdsRow * 2, "the output staging reuses the operand tiles");
+  __syncthreads();
+  lds_f32 *stage = (lds_f32 *)(lds_u8g *)(lds) + wave * stripe_floats<2>();
+  const Epilogue epi = p.epi;
+  const uint32_t Mrows = p.M, Ncols = p.N, ldc = p.strideC;
+  void *const cbase = p.C;
+  const int c_f16 = p.c_f16;
+  const bool vec = p.vec_store != 0;
+  static_for<MI>([&](auto ii) __attribute__((always_inline)) {
+    constexpr int i = decltype(ii)::value;
+    stage_tile32<2>(stage, 0, acc[i][0], lane);
+    stage_tile32<2>(stage, 1, acc[i][1], lane);
+    store_staged32<2>(stage, m0 + wm * (BM / 2) + 32 * i, n0 + wn * 64, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+  });
 }
 
 template <int FMT, int BM, bool AF16> static int launch_gemm_bm(GemmParams p, hipStream_t stream) {
@@ -333,6 +340,7 @@ int launch_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c
   p.row_bytes = (uint32_t)((uint64_t)(K / fmt_elems(fmt)) * fmt_bytes(fmt));
   p.mtiles = p.ntiles = 0;
   p.a_f16 = a_f16; p.c_f16 = c_f16;
+  p.vec_store = store8_aligned(C, strideC, c_f16, epi) ? 1 : 0;
   switch (fmt) {
   case CUTHIP_Q8_0: return launch_gemm_fmt<CUTHIP_Q8_0>(p, stream);
   case CUTHIP_Q4_0: return launch_gemm_fmt<CUTHIP_Q4_0>(p, stream);

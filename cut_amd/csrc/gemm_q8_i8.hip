@@ -26,11 +26,13 @@
 #include <cstdint>
 
 #include "common.hpp"
+#include "gemm_store.hpp"
 
 namespace cuthip {
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) uint8_t lds_u8i;
 
 constexpr int kI8BM = 128, kI8BN = 128, kI8BK = 128, kI8Blocks = kI8BK / 32;
 constexpr int kI8Pitch = kI8BK + 16;   // bytes per LDS row: 16-byte aligned, rows 36 dwords apart
@@ -44,6 +46,7 @@ struct I8Params {
   uint32_t M, K, N, strideC, row_bytes, nblk;
   uint32_t mtiles, ntiles;
   int c_f16;
+  int vec_store;   // C (and a binary epilogue's operand) allow 16-byte accesses
 };
 
 // 8 lanes per block of 32 activations (MatMulQ8GemvDot.cu:60-64)
@@ -87,8 +90,8 @@ __global__ void __launch_bounds__(256) quantize_act_kernel(const void *A, uint32
 }
 
 __global__ void __launch_bounds__(256, 2) gemm_q8_i8_kernel(I8Params p) {
-  __shared__ __attribute__((aligned(16))) uint8_t As[kI8BM * kI8Pitch];
-  __shared__ __attribute__((aligned(16))) uint8_t Bs[kI8BN * kI8Pitch];
+  __shared__ __attribute__((aligned(16))) uint8_t ab_s[(kI8BM + kI8BN) * kI8Pitch];   // the operand tiles, then the output staging
+  uint8_t *const As = ab_s, *const Bs = ab_s + kI8BM * kI8Pitch;
   __shared__ __attribute__((aligned(16))) float sa_s[kI8Blocks][kI8BM];
   __shared__ __attribute__((aligned(16))) float sw_s[kI8Blocks][kI8BN];
 
@@ -210,17 +213,26 @@ __global__ void __launch_bounds__(256, 2) gemm_q8_i8_kernel(I8Params p) {
     mma_slice();
   }
 
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const uint32_t col = n0 + wn * 64 + 32 * j + (lane & 31);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const uint32_t row = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (row < p.M && col < p.N) store_out(p.C, p.epi, p.c_f16, (size_t)row * p.strideC + col, acc[i][j][r]);
-      }
-    }
+  // C tile through LDS, a 32-row stripe of the wave's sub-tile at a time (gemm_store.hpp); the operand tiles are free
+  // once every wave has multiplied the last slice
+  static_assert(4 * stripe_floats<2>() * 4 <= (kI8BM + kI8BN) * kI8Pitch, "the output staging reuses the operand tiles");
+  __syncthreads();
+  lds_f32 *stage = (lds_f32 *)(lds_u8i *)(ab_s) + wave * stripe_floats<2>();
+  const Epilogue epi = p.epi;
+  const uint32_t Mrows = p.M, Ncols = p.N, ldc = p.strideC;
+  void *const cbase = p.C;
+  const int c_f16 = p.c_f16;
+  const bool vec = p.vec_store != 0;
+  static_for<2>([&](auto ii) __attribute__((always_inline)) {
+    constexpr int i = decltype(ii)::value;
+    static_for<2>([&](auto jj) __attribute__((always_inline)) {
+      constexpr int j = decltype(jj)::value;
+      f32x16 t;
+      static_for<16>([&](auto rr) __attribute__((always_inline)) { t[decltype(rr)::value] = acc[i][j][decltype(rr)::value]; });
+      stage_tile32<2>(stage, j, t, lane);
+    });
+    store_staged32<2>(stage, m0 + wm * 64 + 32 * i, n0 + wn * 64, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+  });
 }
 
 static size_t q8_i8_qa_bytes(uint32_t M, uint32_t K) { return ((size_t)M * K + 255) & ~(size_t)255; }
@@ -302,6 +314,7 @@ int cuthip_matmul_q8_i8(const void *W, const void *A, int a_dtype, void *C, int 
   p.mtiles = (M + kI8BM - 1) / kI8BM;
   p.ntiles = (N + kI8BN - 1) / kI8BN;
   p.c_f16 = c_dtype == CUTHIP_F16;
+  p.vec_store = store8_aligned(C, strideC, p.c_f16, p.epi) ? 1 : 0;
   hipLaunchKernelGGL(gemm_q8_i8_kernel, dim3((uint32_t)tiles), dim3(256), 0, s, p);
   return check_hip(hipGetLastError(), "int8 gemm launch");
 }
