@@ -79,7 +79,9 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
 
   // XCD-aware tile order: ids id, id+8, id+16, ... share an XCD and its L2; give
   // them the M-tiles of the same weight panels.
-  const uint32_t tiles = p.mtiles * p.ntiles, split = blockIdx.x / tiles;
+  // (the quotients come out of the vector ALU: readfirstlane moves what depends on them back to SGPRs, where the
+  // scalar-base loads below need their addresses)
+  const uint32_t tiles = p.mtiles * p.ntiles, split = __builtin_amdgcn_readfirstlane(blockIdx.x / tiles);
   uint32_t id = blockIdx.x - split * tiles, mt, nt, aphase = 0;
   if (p.ntiles % 8 == 0) {
     uint32_t xcd = id & 7, slot = id >> 3;
@@ -90,8 +92,11 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
     nt = id / p.mtiles;
     mt = id % p.mtiles;
   }
+  mt = __builtin_amdgcn_readfirstlane(mt);
+  nt = __builtin_amdgcn_readfirstlane(nt);
+  aphase = __builtin_amdgcn_readfirstlane(aphase);
   const uint32_t m0 = mt * BM, n0 = nt * BN;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave: in an SGPR
   const int wm = wave >> 1, wn = wave & 1;
 
   // copy assignment: load v of wave w fills the 8-row group 4 v + w of its tile
@@ -114,11 +119,14 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
   const uint8_t *const gA = p.A, *const gW = p.W;
   const uint32_t pf_dist = p.pf_dist, Mrows = p.M, Ncols = p.N;
   auto load_one = [&](int l, uint8_t *na, uint8_t *nb, uint32_t k0) {
-    const uint8_t *ga = gA + (size_t)k0 * 2, *gb = gW + (size_t)k0 * 2;
-    if (l < NLA)
-      __builtin_amdgcn_global_load_lds(ga + aoff[l], na + (4 * l + wave) * 1024, 16, 0, 0);
-    else
-      __builtin_amdgcn_global_load_lds(gb + boff[l - NLA], nb + (4 * (l - NLA) + wave) * 1024, 16, 0, 0);
+    // As text, in the form scalar base + 32-bit lane offset with the LDS address moved to M0 from an SGPR: through
+    // the builtin every load costs a 64-bit vector add and a v_readfirstlane between the MFMAs.  M0 is not on the
+    // clobber list (the compiler reserves it and says so); every instruction of this kernel that reads M0 sits in a
+    // statement like this one, behind its own s_mov.
+    const uint8_t *g = (l < NLA ? gA : gW) + (size_t)k0 * 2;
+    const uint32_t voff = l < NLA ? aoff[l] : boff[l - NLA];
+    const uint32_t dst = (uint32_t)(uintptr_t)(lds_u8 *)(l < NLA ? na : nb) + (4 * (l < NLA ? l : l - NLA) + wave) * 1024;
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(g), "s"(dst) : "memory");
   };
 
   // Line q = 256 i + tid of the warm-up: the first ceil(BN / wsplit) are rows of the weight panel, the next
@@ -137,7 +145,9 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
     }
   }
   auto warm_one = [&](int i, uint32_t k0) {
-    __builtin_amdgcn_global_load_lds(pfp[i] + (size_t)k0 * 2, pf_sink + wave * 64, 4, 0, 0);
+    const uint8_t *g = pfp[i] + (size_t)k0 * 2;
+    const uint32_t dst = (uint32_t)(uintptr_t)(lds_u8 *)(reinterpret_cast<uint8_t *>(pf_sink)) + wave * 256;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(dst) : "memory");
   };
 
   f32x16 acc[MI][NJ];
@@ -152,10 +162,14 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
   for (int s = 0; s < 4; ++s) xs[s] = ((2 * s + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
 
   half8v fa[2][MI], fb[2][NJ];
-  // Waits until at most n of this wave's LDS reads are outstanding; the fragment registers pass through the
-  // statement so that no MFMA that uses them can be scheduled above it.
+  // Waits until at most n of this wave's LDS reads are outstanding.  The fragment registers then pass through an
+  // empty statement, so that no MFMA that uses them can be scheduled above the wait, and so that any register copy the
+  // allocator makes for them is placed behind the wait too: the fragment reads are text the compiler cannot see into,
+  // and a copy in front of the wait would read registers the LDS has not written yet.
 #define CUTHIP_WAIT_FRAGS(f, n)                                                                                  \
-  asm volatile("s_waitcnt lgkmcnt(" #n ")"                                                                         \
+  asm volatile("s_waitcnt lgkmcnt(" #n ")" ::: "memory");                                                          \
+  __builtin_amdgcn_sched_barrier(0);                                                                               \
+  asm volatile(""                                                                                                  \
                : "+v"(fa[f][0]), "+v"(fa[f][1]), "+v"(fa[f][MI - 2]), "+v"(fa[f][MI - 1]), "+v"(fb[f][0]),         \
                  "+v"(fb[f][1]), "+v"(fb[f][2]), "+v"(fb[f][3]), "+v"(fb[f][NJ - 3]), "+v"(fb[f][NJ - 2]),           \
                  "+v"(fb[f][NJ - 1]))
@@ -182,7 +196,7 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
     }
   };
 
-  const uint32_t kbeg = split * p.kper, nsl = p.kper / kDBK, klast = kbeg + p.kper - kDBK;
+  const uint32_t kbeg = __builtin_amdgcn_readfirstlane(split * p.kper), nsl = p.kper / kDBK, klast = kbeg + p.kper - kDBK;
   // One slice, entered right after a barrier with nothing in flight.  Set 1 holds the fragments of the previous
   // slice's last k-step; its MFMAs run under the first fragment reads of this slice.  The loads of the slice
   // after the last one re-read the last slice (never used) instead of branching around the MFMAs.
