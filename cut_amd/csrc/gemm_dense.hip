@@ -59,22 +59,28 @@ struct DenseParams {
   int vec_store;          // C (and a binary epilogue's operand) allow 16-byte accesses
 };
 
-constexpr int kDBN = 256, kDBK = 64;
+[[maybe_unused]] constexpr int kDBK = 64;   // K elements per LDS stage
 
-template <int BM, int BN>
+// WM: waves along M (4 / WM along N); a wave owns a (BM / WM) x (BN / WN) sub-tile
+template <int BM, int BN, int WM = 2>
 __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // LDS address-space casts and AMDGPU inline asm: the host pass only needs the stub
-  constexpr int MI = BM / 64, NJ = BN / 64;  // 32 x 32 MFMA tiles per wave: MI x NJ
+  constexpr int WN = 4 / WM;
+  constexpr int MI = BM / (32 * WM), NJ = BN / (32 * WN);  // 32 x 32 MFMA tiles per wave: MI x NJ
   constexpr int NM = MI * NJ;                  // MFMAs per k-step of 16
   constexpr int NLA = BM / 32, NL = (BM + BN) / 32;  // LDS-direct loads per wave per slice (A, total)
-  constexpr int LSTEP = (NL - 1) * 3 < 3 * NM ? 3 : 2;   // one load every LSTEP-th MFMA slot
+  constexpr int NPF = 2;                     // L2 warm-up loads per wave per slice: 4 waves x 64 lanes x NPF lines
+  // one load every LSTEP-th MFMA slot of the slice, the warm-up loads in its last NPF slots
+#ifndef CUTHIP_LSTEP_CAP
+#define CUTHIP_LSTEP_CAP 3
+#endif
+  constexpr int LSTEP = (4 * NM - NPF - 1) / (NL - 1) < CUTHIP_LSTEP_CAP ? (4 * NM - NPF - 1) / (NL - 1) : CUTHIP_LSTEP_CAP;
   static_assert((NJ == 4 && (MI == 4 || MI == 2)) || (NJ == 7 && MI == 2), "tile shape");
   static_assert((BM + BN) * 128 * 2 <= 160 * 1024, "two LDS stages");
-  static_assert((NL - 1) * LSTEP < 3 * NM, "the last load must be issued before the last k-step of the slice");
+  static_assert(LSTEP >= 1 && (NL - 1) * LSTEP < 4 * NM - NPF, "the loads of a slice precede its warm-up loads");
   static_assert(4 * stripe_floats<NJ>() * 4 <= (BM + BN) * 128 * 2, "the output staging reuses the operand stages");
   __shared__ __attribute__((aligned(1024))) uint8_t lds[(BM + BN) * 128 * 2];
   uint8_t *const sA0 = lds, *const sA1 = lds + BM * 128, *const sB0 = lds + BM * 256, *const sB1 = lds + BM * 256 + BN * 128;
-  constexpr int NPF = 2;                     // L2 warm-up loads per wave per slice: 4 waves x 64 lanes x NPF lines
   __shared__ uint32_t pf_sink[4 * 64];       // where they land; never read
 
   // XCD-aware tile order: ids id, id+8, id+16, ... share an XCD and its L2; give
@@ -97,7 +103,7 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
   aphase = __builtin_amdgcn_readfirstlane(aphase);
   const uint32_t m0 = mt * BM, n0 = nt * BN;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave: in an SGPR
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WN, wn = wave % WN;
 
   // copy assignment: load v of wave w fills the 8-row group 4 v + w of its tile
   uint32_t aoff[NLA], boff[BN / 32];
@@ -156,7 +162,7 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
 #pragma unroll
     for (int j = 0; j < NJ; ++j) acc[i][j] = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
-  const uint32_t arow = (wm * (BM / 2) + (lane & 31)) * 128, brow = (wn * (BN / 2) + (lane & 31)) * 128;
+  const uint32_t arow = (wm * (BM / WM) + (lane & 31)) * 128, brow = (wn * (BN / WN) + (lane & 31)) * 128;
   uint32_t xs[4];
 #pragma unroll
   for (int s = 0; s < 4; ++s) xs[s] = ((2 * s + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
@@ -191,7 +197,7 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
         asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[f ^ 1][idx - MI]) : "v"(pb), "n"((idx - MI) * 4096) : "memory");
       const int q = g * NM + idx;
       if (q % LSTEP == 0 && q / LSTEP < NL) load_one(q / LSTEP, na, nb, k0);
-      if (g == 3 && idx % 4 == 0 && idx / 4 < NPF) warm_one(idx / 4, kpf);   // younger than every load of the slice
+      if (g == 3 && idx >= NM - NPF) warm_one(idx - (NM - NPF), kpf);   // younger than every load of the slice
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -262,7 +268,7 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
       constexpr int j = decltype(jj)::value;
       stage_tile32<NJ>(stage, j, acc[i][j], lane);
     });
-    store_staged32<NJ>(stage, m0 + wm * (BM / 2) + 32 * i, n0 + wn * (BN / 2), Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    store_staged32<NJ>(stage, m0 + wm * (BM / WM) + 32 * i, n0 + wn * (BN / WN), Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
   });
 #endif
 }
@@ -289,7 +295,7 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *partial
   store_out(C, epi, c_f16, (size_t)row * strideC + col, v);
 }
 
-template <int BM, int BN> static int launch_dense_bm(DenseParams p, hipStream_t stream) {
+template <int BM, int BN, int WM = 2> static int launch_dense_bm(DenseParams p, hipStream_t stream) {
   p.mtiles = (p.M + BM - 1) / BM;
   p.ntiles = (p.N + BN - 1) / BN;
   // Who runs beside whom: with the XCD-aware order an XCD's 32 CUs hold 32 consecutive slots = the M-tiles of
@@ -308,7 +314,7 @@ template <int BM, int BN> static int launch_dense_bm(DenseParams p, hipStream_t 
     set_error("cuthip_matmul_gguf_ws: problem too large for one launch");
     return CUTHIP_ERR_INVALID;
   }
-  auto kern = gemm_dense_kernel<BM, BN>;
+  auto kern = gemm_dense_kernel<BM, BN, WM>;
   hipLaunchKernelGGL(kern, dim3((uint32_t)grid), dim3(256), 0, stream, p);
   return check_hip(hipGetLastError(), "dense gemm launch");
 }
@@ -326,26 +332,38 @@ bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a
   return true;
 }
 
-// Tile height and number of K ranges: 256-row tiles when they give every CU a workgroup, else 128-row tiles if
-// those do, else 256-row tiles with K split (partials in the workspace, summed by a second kernel).
+// Tile shape and number of K ranges.  Candidates in the order of their measured cost per multiply-add on whole rounds
+// (2048 x 14336 x 4096 and 512 x 14336 x 4096, same box): 256 x 224 (four waves along M) 0.95, 128 x 448 1.00,
+// 128 x 256 1.04, 256 x 256 1.15.  A shape costs rounds over the 256 CUs x tile area x that factor; tiles that hang
+// over the edge of C count in full.  When the best shape leaves most of the chip idle, K is split over 128 x 256
+// tiles instead (partials in the workspace, summed by a second kernel).
 struct DenseShape { int bm, bn; uint32_t ksplit; };
 static DenseShape pick_dense_shape(uint32_t M, uint32_t K, uint32_t N) {
-  const uint64_t nt = (N + kDBN - 1) / kDBN, tiles256 = (uint64_t)((M + 255) / 256) * nt, tiles128 = (uint64_t)((M + 127) / 128) * nt;
-  // 128 x 448 tiles when they come out as whole rounds over the 256 CUs where 256 x 256 tiles would leave a partial
-  // round (N = 14336 = 32 x 448 at M = 2048: 512 tiles = 2 rounds, against 448 tiles = 1.75 rounds)
-  if (const char *env = getenv("CUT_HIP_DENSE_TILE")) {   // "bm,bn" tuning aid: 256,256 / 128,256 / 128,448
+  if (const char *env = getenv("CUT_HIP_DENSE_TILE")) {   // "bm,bn" tuning aid: 256,224 / 128,448 / 128,256 / 256,256
     int bm = 0, bn = 0;
-    if (sscanf(env, "%d,%d", &bm, &bn) == 2 && ((bn == 256 && (bm == 256 || bm == 128)) || (bn == 448 && bm == 128)))
+    if (sscanf(env, "%d,%d", &bm, &bn) == 2 &&
+        ((bn == 256 && (bm == 256 || bm == 128)) || (bn == 448 && bm == 128) || (bn == 224 && bm == 256)))
       return DenseShape{bm, bn, 1};
   }
-  const uint64_t t448 = (uint64_t)((M + 127) / 128) * ((N + 447) / 448);
-  if (N % 448 == 0 && t448 >= 256 && t448 % 256 == 0 && tiles256 % 256 != 0) return DenseShape{128, 448, 1};
-  if (tiles256 >= 256) return DenseShape{256, 256, 1};
-  if (tiles128 >= 224) return DenseShape{128, 256, 1};
+  static const struct { int bm, bn; double cost; } cands[] = {{256, 224, 0.95}, {128, 448, 1.00}, {128, 256, 1.04}, {256, 256, 1.15}};
+  int best = 0;
+  double best_t = 0.0;
+  uint64_t best_tiles = 0;
+  for (int c = 0; c < 4; ++c) {
+    const uint64_t tiles = (uint64_t)((M + cands[c].bm - 1) / cands[c].bm) * ((N + cands[c].bn - 1) / cands[c].bn);
+    const double t = (double)((tiles + 255) / 256) * cands[c].bm * cands[c].bn * cands[c].cost;
+    if (c == 0 || t < best_t) {
+      best = c;
+      best_t = t;
+      best_tiles = tiles;
+    }
+  }
+  if (best_tiles >= 192) return DenseShape{cands[best].bm, cands[best].bn, 1};
+  const uint64_t tiles128 = (uint64_t)((M + 127) / 128) * ((N + 255) / 256);
   uint32_t s = 1;
-  while (s < 8 && tiles256 * s < 192 && K % (2 * s * 128) == 0) s *= 2;
-  if (s == 1) return DenseShape{tiles128 > tiles256 ? 128 : 256, 256, 1};
-  return DenseShape{256, 256, s};
+  while (s < 8 && tiles128 * s < 192 && K % (2 * s * 128) == 0) s *= 2;
+  if (s == 1) return DenseShape{cands[best].bm, cands[best].bn, 1};
+  return DenseShape{128, 256, s};
 }
 
 static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
@@ -423,6 +441,7 @@ int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C,
   p.partial = reinterpret_cast<float *>(after_w + align256(a_f16 ? 0 : (size_t)M * K * 2));
   int rc;
   if (sh.bn == 448) rc = launch_dense_bm<128, 448>(p, stream);
+  else if (sh.bn == 224) rc = launch_dense_bm<256, 224, 4>(p, stream);
   else if (sh.bm == 256) rc = launch_dense_bm<256, 256>(p, stream);
   else rc = launch_dense_bm<128, 256>(p, stream);
   if (rc) return rc;
