@@ -5,8 +5,9 @@ scripts/bench/derive_rules.py from an autotune binary's output).
 
 For every (format, M, K, N) of the sweep each variant of the MatMulGguf table that accepts the shape is timed through
 the C ABI (HIP events, weights rotated over several copies so that small matrices are not served from cache) and the
-fastest becomes an exact-shape rule `{"variant": v, "conditions": {"shape": [M, K, N]}}` under
-operators.MatMulGguf<fmt>.backends.hip; the entry's default variant is -1 (the library's own choice by shape).
+fastest hand-written one (with --with-vendor: fastest of all) becomes an exact-shape rule
+`{"variant": v, "conditions": {"shape": [M, K, N]}}` under operators.MatMulGguf<fmt>.backends.hip where it beats the
+library's own choice by more than 3 %; the entry's default variant is -1 (the library's own choice by shape).
 Needs an MI355X; refuses to run without one."""
 import argparse
 import json
@@ -14,7 +15,7 @@ import os
 import sys
 
 SHAPES_NK = [(14336, 4096), (4096, 14336), (4096, 4096), (1024, 4096), (28672, 4096)]
-BATCHES = [1, 2, 4, 8, 16, 32, 64, 128, 512, 2048]
+BATCHES = [1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048]
 FORMATS = ["Q4_K", "Q6_K", "Q8_0"]
 
 
@@ -24,6 +25,8 @@ def main():
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--formats", default=",".join(FORMATS))
     ap.add_argument("--measurements", default=None, help="also write every timing of the sweep to this JSON file")
+    ap.add_argument("--with-vendor", action="store_true",
+                    help="let rules name the dequantize + hipBLASLt variant too (it is timed and logged either way)")
     args = ap.parse_args()
     import numpy as np
     import torch
@@ -44,7 +47,7 @@ def main():
                 a = torch.randn((M, K), dtype=torch.float16, device=dev)
                 c = torch.empty((M, N), dtype=torch.float16, device=dev)
                 ws = ops.matmul_gguf_workspace(fmt, M, K, N, a.dtype, dev)
-                best = None
+                best, auto_us = None, None
                 for v in [-1] + list(range(len(names))):
                     try:
                         for i in range(2):
@@ -68,10 +71,15 @@ def main():
                     del g
                     us = e0.elapsed_time(e1) * 1e3 / args.reps
                     log.append({"shape": [M, K, N], "variant": v, "us": round(us, 2)})
+                    if v == -1:
+                        auto_us = us
+                    if names[v] == "MatMulGgufDequantBlasLt" and v >= 0 and not args.with_vendor:
+                        continue
                     if best is None or us < best[1]:
                         best = (v, us)
-                print(f"{fmt} M={M} K={K} N={N}: variant {best[0]} {best[1]:.1f} us", flush=True)
-                if best[0] >= 0:
+                print(f"{fmt} M={M} K={K} N={N}: variant {best[0]} {best[1]:.1f} us (library's choice {auto_us:.1f})", flush=True)
+                # a rule only where a named variant beats the library's own choice by more than the noise of the timing
+                if best[0] >= 0 and best[1] < 0.97 * auto_us:
                     rules.append({"variant": best[0], "conditions": {"shape": [M, K, N]}})
                 del ws
             del copies, w

@@ -386,14 +386,23 @@ size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
   return dense_gemm_workspace(M, K, N, a_f16) - align256((size_t)N * K * 2);
 }
 
-// true where the two-pass path beats the single-launch GEMM: from about a thousand rows; or when the single-launch
-// kernel's 128 x 128 tiles would leave most of the chip idle, from 256 rows, and already from 41 rows on long K, where
-// that kernel's time is the decode of a whole K-long tile row per workgroup (measured 4096 x 14336: 217-222 us for
-// any M up to 512, against 91-131 us for dequantize + dense GEMM with K split)
-bool dense_gemm_preferred(uint32_t M, uint32_t K, uint32_t N) {
-  if (M >= 1024) return true;
-  if ((uint64_t)((M + 127) / 128) * ((N + 127) / 128) >= 200) return false;
-  return M >= 256 || (M > 40 && K >= 8192);
+// Cost models in microseconds for the automatic choice between the two-pass path and the single-launch GEMM, fitted to
+// a sweep over the weight shapes of an 8B model (all formats, M = 16 .. 2048, HIP-graph replay, MI355X):
+//   two-pass      3 + N K (bytes per weight + 2) / 6.0 MB   the dequantization (reads the blocks, writes fp16)
+//                 + 20 + 2 ceil128(M) N K / 1.05 PFLOP/s     the dense GEMM (tiles are at least 128 rows high)
+//   single launch K x c_fmt x max(1, tiles / 256)            c = 14.7 ns (Q4_K, Q4_0), 19.6 ns (Q8_0), 23.5 ns (Q6_K):
+//                 a workgroup decodes its K-long strip of weights once per 128 rows of A, and nothing overlaps that
+//                 walk until every CU holds more than one 128 x 128 tile.
+// Measured against them (Q4_K, M x N x K): 64 x 4096 x 4096 38 / 62 us, 512 x 14336 x 4096 99 / 105, 512 x 28672 x 4096
+// 173 / 203, 256 x 28672 x 4096 147 / 107; Q6_K 64 x 14336 x 4096 79 / 104.
+double dense_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
+  const double nk = (double)N * K, bpw = (double)fmt_bytes(fmt) / fmt_elems(fmt);
+  return 3.0 + nk * (bpw + 2.0) / 6.0e6 + 20.0 + 2.0 * (double)((M + 127) / 128 * 128) * nk / 1.05e9;
+}
+double single_launch_rows_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
+  const double c = fmt == CUTHIP_Q6_K ? 23.5e-3 : fmt == CUTHIP_Q8_0 ? 19.6e-3 : 14.7e-3;
+  const double tiles = (double)((M + 127) / 128) * ((N + 127) / 128);
+  return K * c * (tiles > 256.0 ? tiles / 256.0 : 1.0);
 }
 
 // use_blaslt: the dense GEMM goes to hipBLASLt (no epilogue there: the caller checks)

@@ -110,7 +110,8 @@ int launch_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c
 
 bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a_f16, const void *A);
 size_t dense_gemm_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16);
-bool dense_gemm_preferred(uint32_t M, uint32_t K, uint32_t N);
+double dense_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N);
+double single_launch_rows_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N);
 int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K,
                       uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream,
                       int use_blaslt);
@@ -149,12 +150,13 @@ static cuthip::GemvParams gemv_params(int fmt, const void *W, const void *A, int
 constexpr uint32_t kPassesMaxRows = 40;   // up to here 8-row passes of the decode kernels can beat one tiled GEMM launch
 
 // Costs in microseconds fitted to a sweep over the weight shapes of an 8B model (HIP-graph replay, MI355X): an 8-row
-// pass of the decode kernels 6.5 + weight bytes / 4.3 MB (x 1.45 on rows of K >= 8192, x 1.5 for Q6_K), one launch of
+// pass of the decode kernels 6.5 + weight bytes / 4.3 MB (x 1.45 on rows of K >= 8192, x 1.5 for Q6_K, x 1.55 for both), one launch of
 // the tiled GEMM on the blocks 62 + weight bytes / 7 MB (its cost is the decode of the whole matrix whatever M is; on
 // rows of K >= 8192 it has too few tiles and is never the better one).
 static double weight_bytes(int fmt, uint32_t K, uint32_t N) { return (double)N * K / cuthip::fmt_elems(fmt) * cuthip::fmt_bytes(fmt); }
 static double passes_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
-  return ((M + 7) / 8) * (6.5 + weight_bytes(fmt, K, N) / 4.3e6) * (K >= 8192 ? 1.45 : 1.0) * (fmt == CUTHIP_Q6_K ? 1.5 : 1.0);
+  const double f = K >= 8192 ? (fmt == CUTHIP_Q6_K ? 1.55 : 1.45) : (fmt == CUTHIP_Q6_K ? 1.5 : 1.0);
+  return ((M + 7) / 8) * (6.5 + weight_bytes(fmt, K, N) / 4.3e6) * f;
 }
 static double single_launch_cost_us(int fmt, uint32_t K, uint32_t N) { return 62.0 + weight_bytes(fmt, K, N) / 7e6; }
 static bool passes_preferred(int fmt, uint32_t M, uint32_t K, uint32_t N) {
@@ -507,7 +509,19 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
       return rc;
     }
   }
-  if (variant == -1 && passes_preferred(fmt, M, K, N)) {   // 8-row passes, each with the workspace (K split on long rows)
+  // Beyond 8 rows, with a workspace at hand: dequantize + dense GEMM where its modelled cost is below that of what
+  // would run otherwise (8-row passes up to 40 rows where those beat the single-launch GEMM, else that GEMM); against
+  // either only by a margin (a tenth, a twentieth): the models are rough.  From 1024 rows always.
+  const bool fits = dense_gemm_fits(M, K, N, strideA, a_f16, A);
+  const size_t need = dense_gemm_workspace(M, K, N, a_f16);
+  const bool ws_ok = workspace && (uintptr_t)workspace % 256 == 0 && workspace_bytes >= need;
+  bool dense_first = false;
+  if (variant == -1 && M > 8 && fits && ws_ok) {
+    const double t4 = dense_cost_us(fmt, M, K, N);
+    dense_first = M >= 1024 || (passes_preferred(fmt, M, K, N) ? t4 < 0.9 * passes_cost_us(fmt, M, K, N)
+                                                               : t4 < 0.95 * single_launch_rows_cost_us(fmt, M, K, N));
+  }
+  if (variant == -1 && !dense_first && passes_preferred(fmt, M, K, N)) {   // 8-row passes, each with the workspace (K split on long rows)
     const size_t asz = a_f16 ? 2 : 4, csz = c_dtype == CUTHIP_F16 ? 2 : 4;
     for (uint32_t m0 = 0; m0 < M; m0 += 8) {
       const uint8_t *a = reinterpret_cast<const uint8_t *>(A) + (size_t)m0 * strideA * asz;
@@ -520,7 +534,7 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
     return CUTHIP_OK;
   }
   // batch 3-8 on long rows: the 8-row GEMV with K split across workgroups, partial products in the workspace
-  if (variant == -1 && ksplit_gemv_preferred(M, K, N) && workspace && (uintptr_t)workspace % 16 == 0 &&
+  if (variant == -1 && !dense_first && ksplit_gemv_preferred(M, K, N) && workspace && (uintptr_t)workspace % 16 == 0 &&
       workspace_bytes >= ksplit_gemv_workspace(M, K, N) && (uintptr_t)A % 16 == 0 && (strideA * (a_f16 ? 2 : 4)) % 16 == 0) {
     const GemvParams p = gemv_params(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC,
                                      Epilogue{CUTHIP_EPI_NONE, 0, nullptr});
@@ -541,13 +555,10 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
                        strideC, epi, c_dtype == CUTHIP_F16);
     return check_hip(hipGetLastError(), "split-K reduce launch");
   }
-  const bool fits = dense_gemm_fits(M, K, N, strideA, a_f16, A);
-  const size_t need = dense_gemm_workspace(M, K, N, a_f16);
-  const bool ws_ok = workspace && (uintptr_t)workspace % 256 == 0 && workspace_bytes >= need;
   // with the vendor GEMM behind the dequantization the two-pass path pays earlier: 25 us of dequantization for an FFN
   // matrix against a single-launch GEMM that decodes the weights once per 128 rows (M = 512, N = 14336: 86 us against 110)
   const bool lt_ok = variant == -1 && epilogue == CUTHIP_EPI_NONE && fits && ws_ok && blaslt_preferred();
-  if (variant == -1 && !((dense_gemm_preferred(M, K, N) || (lt_ok && M >= 384)) && fits && ws_ok))
+  if (variant == -1 && !((dense_first || (lt_ok && M >= 384)) && fits && ws_ok))
     return cuthip_matmul_gguf(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, -1,
                               stream);
   if (!fits) {
