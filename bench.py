@@ -106,7 +106,21 @@ def bench_decode_step(torch, np, ops, dev, x_h, steps=5):
     wall_c, ev_c, _ = timed_graph(torch, decode_step, steps, 1)
     w_bytes_tok = cfg.n_layers * sum(v.numel() for v in base.values()) + head.numel()
     kv_bytes_tok = cfg.n_layers * 2 * cfg.max_ctx * cfg.kv_dim * 2
-    return {"decode_step_8b_ctx2048_ms_per_token": round(ev_c / steps, 3),
+    # What the launch bound of the attention costs: 256 cached positions, once in the 2048-position cache (the attention
+    # launches, and reads, for 2048) and once with a cache and a launch bound of 256 (same weights).
+    dstep.set_position(255)
+    _, ev_short, _ = timed_graph(torch, decode_step, steps, 1)
+    import dataclasses
+    cfg256 = dataclasses.replace(cfg, max_ctx=256)
+    dstep256 = DecodeStep(cfg256, layers, ones, head, dev, fuse=int(os.environ.get("CUT_DECODE_FUSE", "4")), embedding=embd)
+    for kc, vc in zip(dstep256.k_cache, dstep256.v_cache):
+        kc.normal_(0.0, 0.5)
+        vc.normal_(0.0, 1.0)
+    dstep256.set_position(255)
+    _, ev_256, _ = timed_graph(torch, lambda _s: dstep256.step(), steps, 1)
+    return {"decode_step_8b_ctx256_in_cache2048_ms_per_token": round(ev_short / steps, 3),
+            "decode_step_8b_ctx256_in_cache256_ms_per_token": round(ev_256 / steps, 3),
+            "decode_step_8b_ctx2048_ms_per_token": round(ev_c / steps, 3),
             "decode_step_8b_ctx2048_tok_per_s": round(steps * 1e3 / ev_c, 1),
             "decode_step_8b_ctx2048_GBps": round((w_bytes_tok + kv_bytes_tok) * steps / (ev_c * 1e-3) / 1e9, 1),
             "decode_step_8b_bytes_per_token": int(w_bytes_tok + kv_bytes_tok)}

@@ -86,6 +86,8 @@ class GGUFFile:
             t = self._read("I")
             self.tensors[name] = TensorInfo(name, dims, t, self._read("Q"))
         align = int(self.metadata.get("general.alignment", DEFAULT_ALIGNMENT))
+        if align <= 0:
+            raise GGUFError(f"general.alignment must be positive, got {align}")
         self.data_offset = (self._pos + align - 1) // align * align
         for info in self.tensors.values():
             if self.data_offset + info.offset + info.nbytes > self._buf.size:
@@ -124,6 +126,8 @@ class GGUFFile:
                 arr = np.frombuffer(self._buf[self._pos:self._pos + nbytes].tobytes(), dtype=dt)
                 self._pos += nbytes
                 return arr
+            if n > self._buf.size - self._pos:   # every element takes at least one byte
+                raise GGUFError("unexpected end of file in an array")
             return [self._value(et) for _ in range(n)]
         raise GGUFError(f"Unsupported metadata value type {t}")
 

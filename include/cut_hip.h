@@ -310,7 +310,9 @@ int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, in
  *     before the epilogue, i.e. computes RMSNorm(x) . W^T with the rounding to fp16
  *     taken before the scaling.
  * The partial sums are added in a fixed order (no atomics): results are
- * reproducible from run to run.
+ * reproducible from run to run.  next_x16 holds the un-normalised C[n] * weight[n]:
+ * the carry is exact to fp16 rounding while |C[n] * weight[n]| <= 65504 (larger
+ * products store as infinity; the plain RMSNorm kernel has no such limit).
  * Any field group may be NULL.  M = 1, the 8-row GEMV only; other arguments as
  * cuthip_matmul_gguf (strideA = K, strideC = N, or N/2 with CUTHIP_EPI_SWIGLU_PAIRS). */
 int cuthip_matmul_gguf_carry(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t K, uint32_t N,
@@ -348,7 +350,10 @@ int cuthip_matmul_gguf_pro(int fmt, const void *W, const void *A, int a_dtype, v
  * and the workspace holds split-K partial sums; from 32 rows on the tensors are
  * first dequantized to fp16 [N][K] in the workspace (one launch) and multiplied
  * by the dense GEMM of cuthip_matmul_dense_f16 (fp16 operands, fp32 accumulate:
- * within 1e-3 of the fp32 loop).
+ * within 1e-3 of the fp32 loop, normwise).  That path rounds the fp32 activations
+ * and the products q * scale to fp16 once each, where the reference's kernels
+ * keep fmaf(a, q * scale, acc) in fp32: activations beyond the fp16 range
+ * (|a| > 65504) become infinite there; the GEMV variants (Q8 1, Q4 1) take any fp32.
  * variant: the MatMulOpNode `spec` argument, an index into the CUTHIP_OP_MATMUL_Q8 / CUTHIP_OP_MATMUL_Q4 tables,
  * which hold the reference's variant names at the reference's indices (MatMulQ8Variants.generated.h:20-32, default 2;
  * MatMulQ4Variants.generated.h:20-29, default 0; "indices are ABI", MatMulOp.cpp:353-356), or -1 = choose by shape.

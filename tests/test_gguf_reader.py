@@ -77,6 +77,19 @@ def test_errors(tmp_path):
     v9.write_bytes(data[:4] + (9).to_bytes(4, "little") + data[8:])
     with pytest.raises(gguf.GGUFError, match="version"):
         gguf.GGUFFile(str(v9))
+    # general.alignment = 0 and an array that claims more elements than the file has bytes: errors, not crashes
+    import struct
+
+    def kv_file(name, key, type_code, payload):
+        k = key.encode()
+        blob = struct.pack("<IIQQ", 0x46554747, 3, 0, 1) + struct.pack("<Q", len(k)) + k + struct.pack("<I", type_code) + payload
+        f = tmp_path / name
+        f.write_bytes(blob + b"\0" * 64)
+        return str(f)
+    with pytest.raises(gguf.GGUFError, match="alignment"):
+        gguf.GGUFFile(kv_file("align0.gguf", "general.alignment", 4, struct.pack("<I", 0)))
+    with pytest.raises(gguf.GGUFError, match="array"):    # array of strings (type 8), count 2^40
+        gguf.GGUFFile(kv_file("count.gguf", "tokenizer.tokens", 9, struct.pack("<IQ", 8, 1 << 40)))
 
 
 @pytest.mark.skipif(not oracle.have_ref(), reason="oracle/_ref (compiled reference reader) is not built")

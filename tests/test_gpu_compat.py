@@ -125,6 +125,23 @@ def test_prefill_route_q8(ops, M, K, N):
     assert normwise_rel_err(got.cpu().numpy() - D, want) < 1e-3
 
 
+def test_prefill_route_rounds_activations_to_fp16(ops):
+    """The contract of the prefill route in cut_hip.h: fp32 activations are rounded to fp16 once.  Large magnitudes
+    inside the fp16 range keep the 1e-3 normwise bound; beyond 65504 the result is not finite there, while the GEMV
+    variant (reference index 1) computes in fp32 and stays within 1e-5."""
+    M, K, N = 64, 512, 136
+    rng = np.random.default_rng(77)
+    A = (rng.standard_normal((M, K)) * 1.0e3).astype(np.float32)
+    B = rng.integers(-127, 128, (K, N)).astype(np.int8)
+    S = rng.uniform(0.001, 0.02, (K // 32, N)).astype(np.float16).astype(np.float32)
+    want = oracle.matmul_sep_q8(A, B, S, f64=True)
+    assert normwise_rel_err(run(ops, A, B, S, N), want) < 1e-3
+    A[3, 17] = 1.0e5
+    want = oracle.matmul_sep_q8(A, B, S, f64=True)
+    assert not np.isfinite(run(ops, A, B, S, N)[3]).all()
+    assert normwise_rel_err(run(ops, A, B, S, N, variant=1), want) < 1e-5
+
+
 @pytest.mark.parametrize("affine", [False, True])
 @pytest.mark.parametrize("M,K,N", [(32, 128, 66), (300, 1024, 520)])
 def test_prefill_route_q4(ops, affine, M, K, N):

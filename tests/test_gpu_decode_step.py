@@ -615,6 +615,36 @@ def test_carried_rmsnorm_equals_rmsnorm_then_matmul(ops):
     assert normwise_rel_err(got.cpu().numpy()[None, :], want.cpu().numpy()) < 5e-4
 
 
+@pytest.mark.parametrize("outlier", [1.0e3, 3.0e4])
+def test_carried_rmsnorm_with_residual_outliers(ops, outlier):
+    """The carried norm keeps x * norm_weight in fp16 between the producer and the consumer: a residual stream with a
+    few very large entries (as real models have) must still give RMSNorm -> matmul of the float64 oracle, as long as
+    |x * w| stays below the fp16 maximum (65504; the documented limit of the carry)."""
+    fmt = oracle.Q4_K
+    hidden, N = 4096, 256
+    rng = np.random.default_rng(190)
+    x = rng.standard_normal(hidden).astype(np.float32)
+    x[[5, 1234, 4000]] = [outlier, -outlier, 0.7 * outlier]
+    g = rng.uniform(0.5, 1.5, hidden).astype(np.float32)
+    Wp = dev(quantized_weights(fmt, hidden, hidden, seed=191))
+    Wc_h = quantized_weights(fmt, N, hidden, seed=192)
+    a = np.zeros((1, hidden), dtype=np.float16)                 # the producer adds nothing: its output is the residual x
+    xs = torch.from_numpy(x).cuda()
+    x16 = torch.empty(hidden, dtype=torch.float16, device="cuda")
+    parts = torch.zeros(hidden // 8, dtype=torch.float32, device="cuda")
+    ops.matmul_gguf_carry(dev(a).view(-1), Wp, fmt, hidden, hidden, xs, binary="add", d=xs,
+                          carry=ops.norm_carry(next_norm_weight=dev(g), next_x16=x16, next_sumsq_parts=parts))
+    got = torch.empty(N, dtype=torch.float32, device="cuda")
+    ops.matmul_gguf_carry(x16, dev(Wc_h), fmt, N, hidden, got, carry=ops.norm_carry(sumsq_parts=parts, eps=1e-5))
+    torch.cuda.synchronize()
+    assert np.array_equal(xs.cpu().numpy(), x)
+    assert np.isfinite(x16.cpu().numpy().astype(np.float32)).all()
+    x64 = x.astype(np.float64)
+    xn = x64 / np.sqrt(np.mean(x64 * x64) + 1e-5) * g.astype(np.float64)
+    want = oracle.dequant(fmt, Wc_h, N * hidden).astype(np.float64).reshape(N, hidden) @ xn
+    assert normwise_rel_err(got.cpu().numpy()[None, :].astype(np.float64), want[None, :]) < 1e-3
+
+
 @pytest.mark.parametrize("fa,fb", [("Q4_K", "Q6_K"), ("Q4_K", "Q4_K"), ("Q8_0", "Q8_0")])
 @pytest.mark.parametrize("n_heads,n_kv,hd,K,pos", [(32, 8, 128, 4096, 2047), (4, 2, 64, 256, 0), (8, 2, 64, 1024, 17),
                                                    (2, 1, 16, 512, 3)])
