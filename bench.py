@@ -270,6 +270,8 @@ def main():
     ap.add_argument("--prepare-only", action="store_true", help="only run the load-time preparation kernels")
     ap.add_argument("--q8-only", action="store_true",
                     help="only run the Q8_0 prefill GEMMs at M = 2048 (int8-activation variant and fp16 path)")
+    ap.add_argument("--gemv-batch-only", type=int, default=0, metavar="B",
+                    help="only run the FFN GEMV step at batch B (2..8), for profiling")
     ap.add_argument("--decode-only", action="store_true",
                     help="only run the 8B-shape decode step (target of rocprofv3 runs)")
     args = ap.parse_args()
@@ -363,6 +365,12 @@ def main():
     def ffn_bytes(b):
         return 3 * w_bytes + b * 2 * (2 * (N_EMBD + N_FF) + (N_FF + N_EMBD))
 
+    if args.gemv_batch_only:
+        b = args.gemv_batch_only
+        wall_b, ev_b, _ = timed_graph(torch, ffn_step(b), 120, 12)
+        print(json.dumps({f"q4k_ffn_gemv_batch{b}_GBps": round(ffn_bytes(b) * 120 / wall_b / 1e9, 1),
+                          "us_per_launch": round(ev_b * 1e3 / 360, 2)}))
+        return
     # ---- headline: batch 1 --------------------------------------------------
     wall, ev_ms, used_graph = timed_graph(torch, ffn_step(1), args.steps, args.warmup)
     step_bytes = ffn_bytes(1)
