@@ -262,13 +262,16 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
     epi.kind = CUTHIP_EPI_NONE;
   }
   const bool vec = p.ksplit > 1 ? p.N % 4 == 0 : p.vec_store != 0;
+  const bool plain16 = vec && c_f16 && epi.kind == CUTHIP_EPI_NONE;   // the common case gets the short store loop
   static_for<MI>([&](auto ii) __attribute__((always_inline)) {
     constexpr int i = decltype(ii)::value;
     static_for<NJ>([&](auto jj) __attribute__((always_inline)) {
       constexpr int j = decltype(jj)::value;
       stage_tile32<NJ>(stage, j, acc[i][j], lane);
     });
-    store_staged32<NJ>(stage, m0 + wm * (BM / WM) + 32 * i, n0 + wn * (BN / WN), Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    const uint32_t r0 = m0 + wm * (BM / WM) + 32 * i, c0 = n0 + wn * (BN / WN);
+    if (plain16) store_staged32<NJ, true>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    else store_staged32<NJ, false>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
   });
 #endif
 }

@@ -99,7 +99,10 @@ template <int NJ> __device__ __forceinline__ void stage_tile32(lds_f32 *stage, i
     wr[(8 * (r >> 2) + (r & 3)) * stripe_ld<NJ>()] = a[r];
   });
 }
-template <int NJ>
+// PLAIN16: the caller has checked that there is no epilogue operator, C is fp16 and 16-byte stores are allowed; the loop
+// is then a read, a conversion and a store (the general form carries every operator of the epilogue in each of its
+// unrolled iterations).
+template <int NJ, bool PLAIN16 = false>
 __device__ __forceinline__ void store_staged32(const lds_f32 *stage, uint32_t row0, uint32_t col0, uint32_t M, uint32_t N, void *C,
                                                uint32_t strideC, int c_f16, const Epilogue &e, bool vec, int lane) {
   constexpr int LD = stripe_ld<NJ>(), CH = 4 * NJ;   // CH chunks of 8 columns per row
@@ -109,7 +112,17 @@ __device__ __forceinline__ void store_staged32(const lds_f32 *stage, uint32_t ro
     const lds_f32x4 *src = reinterpret_cast<const lds_f32x4 *>(stage + row * LD + 8 * c8);
     const f32x4 lo = src[0], hi = src[1];
     const uint32_t grow = row0 + row, gcol = col0 + 8 * c8;
-    if (grow < M && gcol < N) store_out8(C, e, c_f16, (size_t)grow * strideC + gcol, lo, hi, gcol, N, vec);
+    if constexpr (PLAIN16) {
+      if (grow < M && gcol + 8 <= N) {
+        const half8_t o{(half_t)lo[0], (half_t)lo[1], (half_t)lo[2], (half_t)lo[3],
+                        (half_t)hi[0], (half_t)hi[1], (half_t)hi[2], (half_t)hi[3]};
+        *reinterpret_cast<half8_t *>(reinterpret_cast<half_t *>(C) + (size_t)grow * strideC + gcol) = o;
+      } else if (grow < M && gcol < N) {
+        store_out8(C, e, c_f16, (size_t)grow * strideC + gcol, lo, hi, gcol, N, false);
+      }
+    } else {
+      if (grow < M && gcol < N) store_out8(C, e, c_f16, (size_t)grow * strideC + gcol, lo, hi, gcol, N, vec);
+    }
   }
 }
 
