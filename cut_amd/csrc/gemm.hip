@@ -290,11 +290,16 @@ __global__ void __launch_bounds__(256, 2) gemm_kernel(GemmParams p) {
   void *const cbase = p.C;
   const int c_f16 = p.c_f16;
   const bool vec = p.vec_store != 0;
+  // the common cases get the short store loops: no operator, or the residual add
+  const int fast = !(vec && c_f16) ? 0 : epi.kind == CUTHIP_EPI_NONE ? 1
+                   : (epi.kind == CUTHIP_EPI_BINARY && epi.op == CUTHIP_BINARY_ADD) ? 2 : 0;
   static_for<MI>([&](auto ii) __attribute__((always_inline)) {
     constexpr int i = decltype(ii)::value;
     stage_tile32<2>(stage, 0, acc[i][0], lane);
     stage_tile32<2>(stage, 1, acc[i][1], lane);
-    store_staged32<2>(stage, m0 + wm * (BM / 2) + 32 * i, n0 + wn * 64, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    if (fast == 1) store_staged32<2, 1>(stage, m0 + wm * (BM / 2) + 32 * i, n0 + wn * 64, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    else if (fast == 2) store_staged32<2, 2>(stage, m0 + wm * (BM / 2) + 32 * i, n0 + wn * 64, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    else store_staged32<2, 0>(stage, m0 + wm * (BM / 2) + 32 * i, n0 + wn * 64, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
   });
 }
 

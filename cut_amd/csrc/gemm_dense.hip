@@ -262,7 +262,9 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
     epi.kind = CUTHIP_EPI_NONE;
   }
   const bool vec = p.ksplit > 1 ? p.N % 4 == 0 : p.vec_store != 0;
-  const bool plain16 = vec && c_f16 && epi.kind == CUTHIP_EPI_NONE;   // the common case gets the short store loop
+  // the common cases get the short store loops: no operator, or the residual add
+  const int fast = !(vec && c_f16) ? 0 : epi.kind == CUTHIP_EPI_NONE ? 1
+                   : (epi.kind == CUTHIP_EPI_BINARY && epi.op == CUTHIP_BINARY_ADD) ? 2 : 0;
   static_for<MI>([&](auto ii) __attribute__((always_inline)) {
     constexpr int i = decltype(ii)::value;
     static_for<NJ>([&](auto jj) __attribute__((always_inline)) {
@@ -270,8 +272,9 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
       stage_tile32<NJ>(stage, j, acc[i][j], lane);
     });
     const uint32_t r0 = m0 + wm * (BM / WM) + 32 * i, c0 = n0 + wn * (BN / WN);
-    if (plain16) store_staged32<NJ, true>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
-    else store_staged32<NJ, false>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    if (fast == 1) store_staged32<NJ, 1>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    else if (fast == 2) store_staged32<NJ, 2>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    else store_staged32<NJ, 0>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
   });
 #endif
 }

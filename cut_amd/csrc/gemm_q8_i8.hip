@@ -223,6 +223,9 @@ __global__ void __launch_bounds__(256, 2) gemm_q8_i8_kernel(I8Params p) {
   void *const cbase = p.C;
   const int c_f16 = p.c_f16;
   const bool vec = p.vec_store != 0;
+  // the common cases get the short store loops: no operator, or the residual add
+  const int fast = !(vec && c_f16) ? 0 : epi.kind == CUTHIP_EPI_NONE ? 1
+                   : (epi.kind == CUTHIP_EPI_BINARY && epi.op == CUTHIP_BINARY_ADD) ? 2 : 0;
   static_for<2>([&](auto ii) __attribute__((always_inline)) {
     constexpr int i = decltype(ii)::value;
     static_for<2>([&](auto jj) __attribute__((always_inline)) {
@@ -231,7 +234,9 @@ __global__ void __launch_bounds__(256, 2) gemm_q8_i8_kernel(I8Params p) {
       static_for<16>([&](auto rr) __attribute__((always_inline)) { t[decltype(rr)::value] = acc[i][j][decltype(rr)::value]; });
       stage_tile32<2>(stage, j, t, lane);
     });
-    store_staged32<2>(stage, m0 + wm * 64 + 32 * i, n0 + wn * 64, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    if (fast == 1) store_staged32<2, 1>(stage, m0 + wm * 64 + 32 * i, n0 + wn * 64, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    else if (fast == 2) store_staged32<2, 2>(stage, m0 + wm * 64 + 32 * i, n0 + wn * 64, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    else store_staged32<2, 0>(stage, m0 + wm * 64 + 32 * i, n0 + wn * 64, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
   });
 }
 

@@ -99,26 +99,46 @@ template <int NJ> __device__ __forceinline__ void stage_tile32(lds_f32 *stage, i
     wr[(8 * (r >> 2) + (r & 3)) * stripe_ld<NJ>()] = a[r];
   });
 }
-// PLAIN16: the caller has checked that there is no epilogue operator, C is fp16 and 16-byte stores are allowed; the loop
-// is then a read, a conversion and a store (the general form carries every operator of the epilogue in each of its
-// unrolled iterations).
-template <int NJ, bool PLAIN16 = false>
+// FAST: 0 = any epilogue and output type; 1 = the caller has checked that there is no epilogue operator, C is fp16 and
+// 16-byte stores are allowed; 2 = the same with the binary operator ADD (the residual of a transformer block, D fp16).
+// The fast loops are a read, a conversion (an add) and a store; the general form carries every operator of the epilogue
+// in each iteration and waits for its loads of D and its stores one iteration at a time.
+template <int NJ, int FAST = 0>
 __device__ __forceinline__ void store_staged32(const lds_f32 *stage, uint32_t row0, uint32_t col0, uint32_t M, uint32_t N, void *C,
                                                uint32_t strideC, int c_f16, const Epilogue &e, bool vec, int lane) {
   constexpr int LD = stripe_ld<NJ>(), CH = 4 * NJ;   // CH chunks of 8 columns per row
-#pragma unroll
+  // the fast loops are unrolled (a dozen instructions per iteration); the general one stays a loop: unrolled, its
+  // operator switches made the kernels several times larger for nothing
+#pragma unroll FAST != 0 ? 32 * CH / 64 : 1
   for (int it = 0; it < 32 * CH / 64; ++it) {
     const int c = it * 64 + lane, row = c / CH, c8 = c % CH;
     const lds_f32x4 *src = reinterpret_cast<const lds_f32x4 *>(stage + row * LD + 8 * c8);
     const f32x4 lo = src[0], hi = src[1];
     const uint32_t grow = row0 + row, gcol = col0 + 8 * c8;
-    if constexpr (PLAIN16) {
+    if constexpr (FAST != 0) {
       if (grow < M && gcol + 8 <= N) {
-        const half8_t o{(half_t)lo[0], (half_t)lo[1], (half_t)lo[2], (half_t)lo[3],
-                        (half_t)hi[0], (half_t)hi[1], (half_t)hi[2], (half_t)hi[3]};
-        *reinterpret_cast<half8_t *>(reinterpret_cast<half_t *>(C) + (size_t)grow * strideC + gcol) = o;
-      } else if (grow < M && gcol < N) {
-        store_out8(C, e, c_f16, (size_t)grow * strideC + gcol, lo, hi, gcol, N, false);
+        const size_t idx = (size_t)grow * strideC + gcol;
+        f32x4 a = lo, b = hi;
+        if constexpr (FAST == 2) {
+          const half8_t d = *reinterpret_cast<const half8_t *>(reinterpret_cast<const half_t *>(e.D) + idx);
+          a += f32x4{(float)d[0], (float)d[1], (float)d[2], (float)d[3]};
+          b += f32x4{(float)d[4], (float)d[5], (float)d[6], (float)d[7]};
+        }
+        const half8_t o{(half_t)a[0], (half_t)a[1], (half_t)a[2], (half_t)a[3],
+                        (half_t)b[0], (half_t)b[1], (half_t)b[2], (half_t)b[3]};
+        *reinterpret_cast<half8_t *>(reinterpret_cast<half_t *>(C) + idx) = o;
+      } else if (grow < M && gcol < N) {   // the ragged right edge, element by element
+        const size_t idx = (size_t)grow * strideC + gcol;
+        half_t *cp = reinterpret_cast<half_t *>(C) + idx;
+        const half_t *dp = reinterpret_cast<const half_t *>(e.D) + idx;
+        static_for<8>([&](auto kk) __attribute__((always_inline)) {
+          constexpr int k = decltype(kk)::value;
+          if (gcol + k < N) {
+            float v = k < 4 ? lo[k & 3] : hi[k & 3];
+            if constexpr (FAST == 2) v += (float)dp[k];
+            cp[k] = (half_t)v;
+          }
+        });
       }
     } else {
       if (grow < M && gcol < N) store_out8(C, e, c_f16, (size_t)grow * strideC + gcol, lo, hi, gcol, N, vec);
