@@ -263,8 +263,9 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
   }
   const bool vec = p.ksplit > 1 ? p.N % 4 == 0 : p.vec_store != 0;
   // the common cases get the short store loops: no operator, or the residual add
-  const int fast = !(vec && c_f16) ? 0 : epi.kind == CUTHIP_EPI_NONE ? 1
-                   : (epi.kind == CUTHIP_EPI_BINARY && epi.op == CUTHIP_BINARY_ADD) ? 2 : 0;
+  const int fast = !vec ? 0 : (!c_f16 ? (epi.kind == CUTHIP_EPI_NONE ? 3 : 0)
+                               : epi.kind == CUTHIP_EPI_NONE ? 1
+                               : (epi.kind == CUTHIP_EPI_BINARY && epi.op == CUTHIP_BINARY_ADD) ? 2 : 0);
   static_for<MI>([&](auto ii) __attribute__((always_inline)) {
     constexpr int i = decltype(ii)::value;
     static_for<NJ>([&](auto jj) __attribute__((always_inline)) {
@@ -274,6 +275,7 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
     const uint32_t r0 = m0 + wm * (BM / WM) + 32 * i, c0 = n0 + wn * (BN / WN);
     if (fast == 1) store_staged32<NJ, 1>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
     else if (fast == 2) store_staged32<NJ, 2>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    else if (fast == 3) store_staged32<NJ, 3>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
     else store_staged32<NJ, 0>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
   });
 #endif
@@ -299,6 +301,62 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *partial
   for (uint32_t s = 0; s < ksplit; ++s) v += partial[s * mn + i];
   const uint32_t row = (uint32_t)(i / N), col = (uint32_t)(i - (size_t)row * N);
   store_out(C, epi, c_f16, (size_t)row * strideC + col, v);
+}
+
+// The same for eight consecutive outputs per thread when there is no operator and rows allow 16-byte accesses: every
+// load of every K range is requested before the first add, the sum leaves in one store (two for fp32 C).
+template <bool F16OUT>
+__global__ void __launch_bounds__(256) splitk_reduce8_kernel(const float *partial, uint32_t ksplit, uint32_t M, uint32_t N, void *C,
+                                                             uint32_t strideC) {
+  const size_t mn = (size_t)M * N, i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (i >= mn) return;
+  f32x4 lo = {0.0f, 0.0f, 0.0f, 0.0f}, hi = lo;
+  uint32_t s = 0;
+  for (; s + 4 <= ksplit; s += 4) {   // four K ranges in flight at a time
+    f32x4 a[4], b[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const f32x4 *src = reinterpret_cast<const f32x4 *>(partial + (s + u) * mn + i);
+      a[u] = src[0];
+      b[u] = src[1];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      lo += a[u];
+      hi += b[u];
+    }
+  }
+  for (; s < ksplit; ++s) {
+    const f32x4 *src = reinterpret_cast<const f32x4 *>(partial + s * mn + i);
+    lo += src[0];
+    hi += src[1];
+  }
+  const uint32_t row = (uint32_t)(i / N), col = (uint32_t)(i - (size_t)row * N);
+  const size_t idx = (size_t)row * strideC + col;
+  if constexpr (F16OUT) {
+    const half8_t o{(half_t)lo[0], (half_t)lo[1], (half_t)lo[2], (half_t)lo[3], (half_t)hi[0], (half_t)hi[1], (half_t)hi[2], (half_t)hi[3]};
+    *reinterpret_cast<half8_t *>(reinterpret_cast<half_t *>(C) + idx) = o;
+  } else {
+    f32x4 *cp = reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(C) + idx);
+    cp[0] = lo;
+    cp[1] = hi;
+  }
+}
+
+// sums the fp32 partial products [ksplit][M][N] of a K split into C through the epilogue (same order of additions in
+// both kernels: K range 0 first)
+int launch_splitk_reduce(const float *partial, uint32_t ksplit, uint32_t M, uint32_t N, void *C, uint32_t strideC, Epilogue epi,
+                         int c_f16, hipStream_t stream) {
+  const uint64_t mn = (uint64_t)M * N;
+  if (epi.kind == CUTHIP_EPI_NONE && N % 8 == 0 && (uintptr_t)partial % 16 == 0 && store8_aligned(C, strideC, c_f16, epi)) {
+    const dim3 grid((uint32_t)((mn / 8 + 255) / 256));
+    if (c_f16) hipLaunchKernelGGL(splitk_reduce8_kernel<true>, grid, dim3(256), 0, stream, partial, ksplit, M, N, C, strideC);
+    else hipLaunchKernelGGL(splitk_reduce8_kernel<false>, grid, dim3(256), 0, stream, partial, ksplit, M, N, C, strideC);
+  } else {
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((uint32_t)((mn + 255) / 256)), dim3(256), 0, stream, partial, ksplit, M, N, C,
+                       strideC, epi, c_f16);
+  }
+  return check_hip(hipGetLastError(), "split-K reduce launch");
 }
 
 template <int BM, int BN, int WM = 2> static int launch_dense_bm(DenseParams p, hipStream_t stream) {
@@ -461,10 +519,7 @@ int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C,
   else rc = launch_dense_bm<128, 256>(p, stream);
   if (rc) return rc;
   if (sh.ksplit > 1) {
-    const uint64_t mn = (uint64_t)M * N;
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((uint32_t)((mn + 255) / 256)), dim3(256), 0, stream, p.partial, sh.ksplit, M,
-                       N, C, strideC, epi, c_f16);
-    return check_hip(hipGetLastError(), "split-K reduce launch");
+    return launch_splitk_reduce(p.partial, sh.ksplit, M, N, C, strideC, epi, c_f16, stream);
   }
   return CUTHIP_OK;
 }

@@ -100,7 +100,8 @@ template <int NJ> __device__ __forceinline__ void stage_tile32(lds_f32 *stage, i
   });
 }
 // FAST: 0 = any epilogue and output type; 1 = the caller has checked that there is no epilogue operator, C is fp16 and
-// 16-byte stores are allowed; 2 = the same with the binary operator ADD (the residual of a transformer block, D fp16).
+// 16-byte stores are allowed; 2 = the same with the binary operator ADD (the residual of a transformer block, D fp16);
+// 3 = no operator, fp32 C (the partial products of a K split).
 // The fast loops are a read, a conversion (an add) and a store; the general form carries every operator of the epilogue
 // in each iteration and waits for its loads of D and its stores one iteration at a time.
 template <int NJ, int FAST = 0>
@@ -115,7 +116,19 @@ __device__ __forceinline__ void store_staged32(const lds_f32 *stage, uint32_t ro
     const lds_f32x4 *src = reinterpret_cast<const lds_f32x4 *>(stage + row * LD + 8 * c8);
     const f32x4 lo = src[0], hi = src[1];
     const uint32_t grow = row0 + row, gcol = col0 + 8 * c8;
-    if constexpr (FAST != 0) {
+    if constexpr (FAST == 3) {
+      if (grow < M && gcol + 8 <= N) {
+        f32x4 *cp = reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(C) + (size_t)grow * strideC + gcol);
+        cp[0] = lo;
+        cp[1] = hi;
+      } else if (grow < M && gcol < N) {
+        float *cp = reinterpret_cast<float *>(C) + (size_t)grow * strideC + gcol;
+        static_for<8>([&](auto kk) __attribute__((always_inline)) {
+          constexpr int k = decltype(kk)::value;
+          if (gcol + k < N) cp[k] = k < 4 ? lo[k & 3] : hi[k & 3];
+        });
+      }
+    } else if constexpr (FAST != 0) {
       if (grow < M && gcol + 8 <= N) {
         const size_t idx = (size_t)grow * strideC + gcol;
         f32x4 a = lo, b = hi;

@@ -51,8 +51,8 @@ CUTHIP_EXTERN_KSPLIT(CUTHIP_Q6_K)
 #undef CUTHIP_EXTERN_KSPLIT
 
 // defined with the two-pass GEMM: C = epilogue(sum of the fp32 partial products)
-__global__ void splitk_reduce_kernel(const float *partial, uint32_t ksplit, uint32_t M, uint32_t N, void *C, uint32_t strideC,
-                                     Epilogue epi, int c_f16);
+int launch_splitk_reduce(const float *partial, uint32_t ksplit, uint32_t M, uint32_t N, void *C, uint32_t strideC, Epilogue epi,
+                         int c_f16, hipStream_t stream);
 
 // The split across workgroups pays where one row group per workgroup would re-stage long activations for few rows:
 // batch 2-8, rows of at least 32 steps, and not enough row groups to fill the chip without splitting K.
@@ -550,10 +550,7 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
     }
     if (rc) return rc;
     Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
-    const uint64_t mn = (uint64_t)M * N;
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((uint32_t)((mn + 255) / 256)), dim3(256), 0, s, partial, parts, M, N, C,
-                       strideC, epi, c_dtype == CUTHIP_F16);
-    return check_hip(hipGetLastError(), "split-K reduce launch");
+    return launch_splitk_reduce(partial, parts, M, N, C, strideC, epi, c_dtype == CUTHIP_F16, s);
   }
   // with the vendor GEMM behind the dequantization the two-pass path pays earlier: 25 us of dequantization for an FFN
   // matrix against a single-launch GEMM that decodes the weights once per 128 rows (M = 512, N = 14336: 86 us against 110)
