@@ -397,8 +397,8 @@ bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a
 }
 
 // Tile shape and number of K ranges.  Candidates in the order of their measured cost per multiply-add on whole rounds
-// (2048 x 14336 x 4096 and 512 x 14336 x 4096, same box): 256 x 224 (four waves along M) 0.95, 128 x 448 1.00,
-// 128 x 256 1.04, 256 x 256 1.15.  A shape costs rounds over the 256 CUs x tile area x that factor; tiles that hang
+// (2048 x 14336 x 4096, every shape forced in turn on one box): 256 x 224 (four waves along M) 0.96, 128 x 448 1.00,
+// 256 x 256 1.03, 128 x 256 1.24.  A shape costs rounds over the 256 CUs x tile area x that factor; tiles that hang
 // over the edge of C count in full.  When the best shape leaves most of the chip idle, K is split over 128 x 256
 // tiles instead (partials in the workspace, summed by a second kernel).
 struct DenseShape { int bm, bn; uint32_t ksplit; };
@@ -409,7 +409,7 @@ static DenseShape pick_dense_shape(uint32_t M, uint32_t K, uint32_t N) {
         ((bn == 256 && (bm == 256 || bm == 128)) || (bn == 448 && bm == 128) || (bn == 224 && bm == 256)))
       return DenseShape{bm, bn, 1};
   }
-  static const struct { int bm, bn; double cost; } cands[] = {{256, 224, 0.95}, {128, 448, 1.00}, {128, 256, 1.04}, {256, 256, 1.15}};
+  static const struct { int bm, bn; double cost; } cands[] = {{256, 224, 0.96}, {128, 448, 1.00}, {256, 256, 1.03}, {128, 256, 1.24}};
   int best = 0;
   double best_t = 0.0;
   uint64_t best_tiles = 0;
@@ -453,7 +453,7 @@ size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
 // Cost models in microseconds for the automatic choice between the two-pass path and the single-launch GEMM, fitted to
 // a sweep over the weight shapes of an 8B model (all formats, M = 16 .. 2048, HIP-graph replay, MI355X):
 //   two-pass      3 + N K (bytes per weight + 2) / 6.0 MB   the dequantization (reads the blocks, writes fp16)
-//                 + 20 + 2 ceil128(M) N K / 1.05 PFLOP/s     the dense GEMM (tiles are at least 128 rows high)
+//                 + 17 + 2 ceil128(M) N K / 1.15 PFLOP/s     the dense GEMM (tiles are at least 128 rows high)
 //   single launch K x c_fmt x max(1, tiles / 256)            c = 14.7 ns (Q4_K, Q4_0), 19.6 ns (Q8_0), 23.5 ns (Q6_K):
 //                 a workgroup decodes its K-long strip of weights once per 128 rows of A, and nothing overlaps that
 //                 walk until every CU holds more than one 128 x 128 tile.
@@ -461,7 +461,7 @@ size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
 // 173 / 203, 256 x 28672 x 4096 147 / 107; Q6_K 64 x 14336 x 4096 79 / 104.
 double dense_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
   const double nk = (double)N * K, bpw = (double)fmt_bytes(fmt) / fmt_elems(fmt);
-  return 3.0 + nk * (bpw + 2.0) / 6.0e6 + 20.0 + 2.0 * (double)((M + 127) / 128 * 128) * nk / 1.05e9;
+  return 3.0 + nk * (bpw + 2.0) / 6.0e6 + 17.0 + 2.0 * (double)((M + 127) / 128 * 128) * nk / 1.15e9;
 }
 double single_launch_rows_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
   const double c = fmt == CUTHIP_Q6_K ? 23.5e-3 : fmt == CUTHIP_Q8_0 ? 19.6e-3 : 14.7e-3;
