@@ -263,6 +263,7 @@ def main():
                          "1 GiB: what a launch of the headline GEMV's size can reach on this part when it only loads")
     ap.add_argument("--gemm-variant", type=int, default=4, choices=(2, 4, 5),
                     help="with --gemm-only: 4 = dequantize once + hand-written dense GEMM (default), 5 = dequantize once + hipBLASLt, 2 = single-launch GEMM")
+    ap.add_argument("--gemm-down", action="store_true", help="with --gemm-only: the down-projection shape (N = 4096, K = 14336)")
     ap.add_argument("--gemm-only", type=int, default=0, metavar="M",
                     help="only run the Q4_K prefill GEMM (M x 4096) . (14336 x 4096)^T twelve times (target of rocprofv3 runs)")
     ap.add_argument("--dequant-only", action="store_true",
@@ -312,23 +313,24 @@ def main():
         return
     if args.gemm_only:
         M = args.gemm_only
-        wq = torch.from_numpy(make_q_weights("Q4_K", N_FF, N_EMBD, 0)).to(dev)
-        a = torch.randn((M, N_EMBD), dtype=torch.float16, device=dev)
-        c = torch.empty((M, N_FF), dtype=torch.float16, device=dev)
+        GN, GK = (N_EMBD, N_FF) if args.gemm_down else (N_FF, N_EMBD)
+        wq = torch.from_numpy(make_q_weights("Q4_K", GN, GK, 0)).to(dev)
+        a = torch.randn((M, GK), dtype=torch.float16, device=dev)
+        c = torch.empty((M, GN), dtype=torch.float16, device=dev)
         # variant 4 = dequantize once + dense GEMM (two launches, both inside the timed region); 2 = single launch
-        ws = ops.matmul_gguf_workspace("Q4_K", M, N_EMBD, N_FF, a.dtype, dev) if args.gemm_variant >= 4 else None
+        ws = ops.matmul_gguf_workspace("Q4_K", M, GK, GN, a.dtype, dev) if args.gemm_variant >= 4 else None
         for _ in range(2):
-            ops.matmul_gguf(a, wq, "Q4_K", N_FF, N_EMBD, out=c, variant=args.gemm_variant, workspace=ws)
+            ops.matmul_gguf(a, wq, "Q4_K", GN, GK, out=c, variant=args.gemm_variant, workspace=ws)
         torch.cuda.synchronize()
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         ev0.record()
         for _ in range(10):
-            ops.matmul_gguf(a, wq, "Q4_K", N_FF, N_EMBD, out=c, variant=args.gemm_variant, workspace=ws)
+            ops.matmul_gguf(a, wq, "Q4_K", GN, GK, out=c, variant=args.gemm_variant, workspace=ws)
         ev1.record()
         torch.cuda.synchronize()
         us = ev0.elapsed_time(ev1) * 1e3 / 10
-        print(json.dumps({"gemm": f"Q4_K M={M} N={N_FF} K={N_EMBD}", "variant": args.gemm_variant,
-                          "us_per_matmul": round(us, 1), "TFLOPs": round(2.0 * M * N_FF * N_EMBD / us / 1e6, 1)}))
+        print(json.dumps({"gemm": f"Q4_K M={M} N={GN} K={GK}", "variant": args.gemm_variant,
+                          "us_per_matmul": round(us, 1), "TFLOPs": round(2.0 * M * GN * GK / us / 1e6, 1)}))
         return
     log(f"[bench] {info['name']} {info['arch']} CUs={info['compute_units']}")
 

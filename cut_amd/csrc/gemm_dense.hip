@@ -403,11 +403,12 @@ bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a
 // tiles instead (partials in the workspace, summed by a second kernel).
 struct DenseShape { int bm, bn; uint32_t ksplit; };
 static DenseShape pick_dense_shape(uint32_t M, uint32_t K, uint32_t N) {
-  if (const char *env = getenv("CUT_HIP_DENSE_TILE")) {   // "bm,bn" tuning aid: 256,224 / 128,448 / 128,256 / 256,256
-    int bm = 0, bn = 0;
-    if (sscanf(env, "%d,%d", &bm, &bn) == 2 &&
-        ((bn == 256 && (bm == 256 || bm == 128)) || (bn == 448 && bm == 128) || (bn == 224 && bm == 256)))
-      return DenseShape{bm, bn, 1};
+  if (const char *env = getenv("CUT_HIP_DENSE_TILE")) {   // "bm,bn[,ksplit]" tuning aid: 256,224 / 128,448 / 128,256 / 256,256
+    int bm = 0, bn = 0, ks = 1;
+    const int got = sscanf(env, "%d,%d,%d", &bm, &bn, &ks);   // optional third field: K ranges (1, 2, 4, 8)
+    if (got >= 2 && ((bn == 256 && (bm == 256 || bm == 128)) || (bn == 448 && bm == 128) || (bn == 224 && bm == 256)) &&
+        (ks == 1 || ks == 2 || ks == 4 || ks == 8) && K % (ks * 128) == 0)
+      return DenseShape{bm, bn, (uint32_t)ks};
   }
   static const struct { int bm, bn; double cost; } cands[] = {{256, 224, 0.96}, {128, 448, 1.00}, {256, 256, 1.03}, {128, 256, 1.24}};
   int best = 0;
