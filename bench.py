@@ -155,7 +155,28 @@ def bench_prepare(torch, ops, dev, reps=10):
         ops.matmul_sep(a, Bq, Sq, N, out=c)
     _, ev, _ = timed_graph(torch, sep, 5, 2)
     res["separated_q8_prefill_gemm_M2048_N14336_K4096_TFLOPs"] = round(2.0 * 2048 * N * K * 5 / (ev * 1e-3) / 1e12, 1)
-    del w, Bq, Sq, a, c
+    # the same tensors at decode size (one row of fp32 activations): bytes of values + scales over the launch time, the
+    # weights rotated over four copies; then the affine Q4 tensors the reference makes of Q4_K
+    a1 = torch.randn((1, K), dtype=torch.float32, device=dev)
+    c1 = torch.empty((1, N), dtype=torch.float32, device=dev)
+    copies8 = [(Bq.clone(), Sq.clone()) for _ in range(4)]
+
+    def sep1(s_):
+        b_, s2_ = copies8[s_ % 4]
+        ops.matmul_sep(a1, b_, s2_, N, out=c1)
+    _, ev, _ = timed_graph(torch, sep1, 40, 4)
+    res["separated_q8_gemv_14336x4096_GBps"] = round((Bq.numel() + Sq.numel() * 2) * 40 / (ev * 1e-3) / 1e9, 1)
+    del copies8
+    w4 = torch.from_numpy(make_q_weights("Q4_K", 1024, K, 6)).to(dev).repeat(N // 1024)
+    B4, S4 = ops.prepare_sep(w4, "Q4_K", N, K)
+    copies4 = [(B4.clone(), S4.clone()) for _ in range(4)]
+
+    def sep4(s_):
+        b_, s2_ = copies4[s_ % 4]
+        ops.matmul_sep(a1, b_, s2_, N, q4=True, affine=True, out=c1)
+    _, ev, _ = timed_graph(torch, sep4, 40, 4)
+    res["separated_q4_affine_gemv_14336x4096_GBps"] = round((B4.numel() + S4.numel() * 2) * 40 / (ev * 1e-3) / 1e9, 1)
+    del w, Bq, Sq, a, c, w4, B4, S4, copies4, a1, c1
     x = torch.randn(N * K, dtype=torch.float32, device=dev) * 0.02
 
     def quant(_s):

@@ -69,55 +69,89 @@ __global__ void __launch_bounds__(64 * kSepWaves, 2) sep_gemv_kernel(SepParams p
   const uint32_t ncols = c0 < p.N ? min((uint32_t)kSepCols, p.N - c0) : 0u;
   if (k0 < p.K && ncols) {
     const float *xw = &xs[0][wave * kSepKC];
-    for (int kk = 0; kk < kSepKC; ++kk) {
-      float q[kSepCols];
+    // One k-row of this lane's 16 columns: 16 bytes of int8 or 8 bytes of nibbles (as the low half of a u32x4).
+    auto load_row = [&](uint32_t k) -> u32x4 {
+      u32x4 w = u32x4{0, 0, 0, 0};
       if (Q4) {
-        const uint8_t *src = p.B + (size_t)(k0 + kk) * p.strideB + c0 / 2;
-        uint32_t w0, w1;
+        const uint8_t *src = p.B + (size_t)k * p.strideB + c0 / 2;
         if (ncols == kSepCols) {
-          u32x2 w = ld_u32x2(src);
-          w0 = w.x;
-          w1 = w.y;
+          const u32x2 v = ld_u32x2(src);
+          w.x = v.x;
+          w.y = v.y;
         } else {   // last lane of a ragged row: byte loads inside the row
-          w0 = w1 = 0;
-          for (uint32_t b = 0; b < (ncols + 1) / 2; ++b) {
-            uint32_t v = src[b];
-            if (b < 4) w0 |= v << (8 * b);
-            else w1 |= v << (8 * (b - 4));
-          }
-        }
-#pragma unroll
-        for (int c = 0; c < 8; ++c) {
-          q[c] = (float)((w0 >> (4 * c)) & 0xF);
-          q[8 + c] = (float)((w1 >> (4 * c)) & 0xF);
+          for (uint32_t b = 0; b < (ncols + 1) / 2; ++b) w[b >> 2] |= (uint32_t)src[b] << (8 * (b & 3));
         }
       } else {
-        const uint8_t *src = p.B + (size_t)(k0 + kk) * p.strideB + c0;
-        u32x4 w;
+        const uint8_t *src = p.B + (size_t)k * p.strideB + c0;
         if (ncols == kSepCols) {
           w = ld_u32x4(src);
         } else {
-          w = u32x4{0, 0, 0, 0};
           for (uint32_t b = 0; b < ncols; ++b) w[b >> 2] |= (uint32_t)src[b] << (8 * (b & 3));
         }
-#pragma unroll
-        for (int c = 0; c < kSepCols; ++c) q[c] = (float)(int)(int8_t)((w[c >> 2] >> (8 * (c & 3))) & 0xFF);
       }
-#pragma unroll
-      for (int m = 0; m < MT; ++m) {
-        float x = xw[m * (kSepWaves * kSepKC) + kk];
-        sx[m] += x;
-#pragma unroll
-        for (int c = 0; c < kSepCols; ++c) bs[m][c] = fmaf(x, q[c], bs[m][c]);
+      return w;
+    };
+    // the block's scales (and minima), fp16 [k/32][scaleStride]: requested before the rows, used after them
+    const uint32_t blk = k0 / 32;
+    const uint16_t *srow = p.S + (size_t)blk * p.scaleStride + c0;
+    const uint16_t *mrow = p.S + (size_t)(blocksK + blk) * p.scaleStride + c0;
+    const bool svec = ncols == kSepCols && ((uintptr_t)srow & 15u) == 0 && ((uintptr_t)mrow & 15u) == 0;
+    u32x4 sraw[2] = {u32x4{0, 0, 0, 0}, u32x4{0, 0, 0, 0}}, mraw[2] = {u32x4{0, 0, 0, 0}, u32x4{0, 0, 0, 0}};
+    if (svec) {
+      sraw[0] = ld_u32x4(reinterpret_cast<const uint8_t *>(srow));
+      sraw[1] = ld_u32x4(reinterpret_cast<const uint8_t *>(srow) + 16);
+      if (Q4 && p.affine) {
+        mraw[0] = ld_u32x4(reinterpret_cast<const uint8_t *>(mrow));
+        mraw[1] = ld_u32x4(reinterpret_cast<const uint8_t *>(mrow) + 16);
       }
     }
-    // the block's scales (and minima): fp16 [k/32][scaleStride]
-    const uint32_t blk = k0 / 32;
+    // The 32 rows in four groups of eight: the loads of a group are in flight while the group before it is multiplied
+    // (one load per iteration with its use right behind it left every load's latency exposed: 1.7 TB/s).
+    constexpr int G = 8;
+    u32x4 wbuf[2][G];
+#pragma unroll
+    for (int j = 0; j < G; ++j) wbuf[0][j] = load_row(k0 + j);
+#pragma unroll
+    for (int g = 0; g < kSepKC / G; ++g) {
+      if (g + 1 < kSepKC / G) {
+#pragma unroll
+        for (int j = 0; j < G; ++j) wbuf[(g + 1) & 1][j] = load_row(k0 + (g + 1) * G + j);
+      }
+#pragma unroll
+      for (int j = 0; j < G; ++j) {
+        const u32x4 w = wbuf[g & 1][j];
+        const int kk = g * G + j;
+        float q[kSepCols];
+        if (Q4) {
+#pragma unroll
+          for (int c = 0; c < 8; ++c) {
+            q[c] = (float)((w.x >> (4 * c)) & 0xF);
+            q[8 + c] = (float)((w.y >> (4 * c)) & 0xF);
+          }
+        } else {
+#pragma unroll
+          for (int c = 0; c < kSepCols; ++c) q[c] = (float)(int)(int8_t)((w[c >> 2] >> (8 * (c & 3))) & 0xFF);
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          float x = xw[m * (kSepWaves * kSepKC) + kk];
+          sx[m] += x;
+#pragma unroll
+          for (int c = 0; c < kSepCols; ++c) bs[m][c] = fmaf(x, q[c], bs[m][c]);
+        }
+      }
+    }
 #pragma unroll
     for (int c = 0; c < kSepCols; ++c) {
       if ((uint32_t)c < ncols) {
-        float s = f16bits_to_f32(p.S[(size_t)blk * p.scaleStride + c0 + c]);
-        float mn = (Q4 && p.affine) ? f16bits_to_f32(p.S[(size_t)(blocksK + blk) * p.scaleStride + c0 + c]) : 0.0f;
+        float s, mn = 0.0f;
+        if (svec) {
+          s = f16bits_to_f32((sraw[c >> 3][(c >> 1) & 3] >> (16 * (c & 1))) & 0xFFFFu);
+          if (Q4 && p.affine) mn = f16bits_to_f32((mraw[c >> 3][(c >> 1) & 3] >> (16 * (c & 1))) & 0xFFFFu);
+        } else {
+          s = f16bits_to_f32(srow[c]);
+          if (Q4 && p.affine) mn = f16bits_to_f32(mrow[c]);
+        }
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
           float v = Q4 ? fmaf(-8.0f, sx[m], bs[m][c]) : bs[m][c];
@@ -167,6 +201,7 @@ __global__ void __launch_bounds__(256) sep_reduce_kernel(const float *ws, float 
   if (i >= mcount * N) return;
   uint32_t row = m0 + i / N, n = i % N;
   float v = 0.0f;
+#pragma unroll 8
   for (uint32_t s = 0; s < nsplit; ++s) v += ws[((size_t)s * M + row) * N + n];
   store_out(C, epi, 0, (size_t)row * strideC + n, v);
 }
