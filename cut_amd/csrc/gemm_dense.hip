@@ -281,6 +281,223 @@ __global__ void __launch_bounds__(256, 1) gemm_dense_kernel(DenseParams p) {
 #endif
 }
 
+// ---- the same GEMM on v_mfma_f32_16x16x32_f16 ------------------------------------------------------------------------
+// Same tiles, loads, LDS image and stages as gemm_dense_kernel; the products are 16 x 16 x 32 MFMAs (4 passes) instead
+// of 32 x 32 x 16 (8 passes).  The part throttles its clock under matrix-core load, less so under this instruction (a
+// loop of nothing but MFMAs on random fp16 data: 1.55-1.71 PFLOP/s against 1.47-1.60), and the vendor's kernel, which
+// uses it, runs at 1.83 GHz where gemm_dense_kernel runs at 1.5-1.6.
+// A wave's sub-tile is MI x NJ tiles of 16 x 16.  Per 32-wide k-step it walks the B fragments j = 0 .. NJ-1 and
+// multiplies each with the MI A fragments of the step; B fragments are read kAhead fragments ahead into a ring of
+// eight, A fragments a step ahead into the other half of a double buffer.  The fragment reads are ordinary LDS loads
+// (the compiler places the exact s_waitcnt lgkmcnt before each first use; it knows nothing of the LDS-direct loads,
+// which are text, so it adds no wait for them).  All reads of a slice have been issued kTail + 2 groups before its end;
+// the wave then waits for them, for its loads of the next slice and for the barrier, and multiplies the last kTail
+// groups from registers behind the barrier, under the first reads of the next slice.
+typedef __attribute__((address_space(3))) half8v lds_half8v;
+
+template <int BM, int BN, int WM = 2>
+__global__ void __launch_bounds__(256, 1) gemm_dense16_kernel(DenseParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int WN = 4 / WM;
+  constexpr int MI = BM / (16 * WM), NJ = BN / (16 * WN);   // 16 x 16 MFMA tiles per wave
+  constexpr int NB = 2 * NJ;                                 // B fragments per slice (two k-steps of 32)
+  constexpr int kAhead = 6, kTail = 3;                       // B fragments read ahead; groups multiplied behind the barrier
+  constexpr int NLA = BM / 32, NL = (BM + BN) / 32;          // LDS-direct loads per wave per slice (A, total)
+  constexpr int NPF = 2;
+  constexpr int LFIRST = 0, LLAST = (NB - kTail - 1) * MI;   // MFMA slots of a slice that carry a load
+  constexpr int LSTEP = (LLAST - LFIRST) / NL;
+  static_assert(NB % 8 == 0 || (2 * NB) % 8 == 0, "the B ring of eight must close over the two slices of a loop trip");
+  static_assert(NJ >= kAhead + 2 && LSTEP >= 1 && MI >= 2, "tile shape");
+  static_assert((BM + BN) * 128 * 2 <= 160 * 1024, "two LDS stages");
+  static_assert(4 * stripe_floats<NJ / 2>() * 4 <= (BM + BN) * 128 * 2, "the output staging reuses the operand stages");
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[(BM + BN) * 128 * 2];
+  uint8_t *const sA0 = lds, *const sA1 = lds + BM * 128, *const sB0 = lds + BM * 256, *const sB1 = lds + BM * 256 + BN * 128;
+  __shared__ uint32_t pf_sink[4 * 64];
+
+  const uint32_t tiles = p.mtiles * p.ntiles, split = __builtin_amdgcn_readfirstlane(blockIdx.x / tiles);
+  uint32_t id = blockIdx.x - split * tiles, mt, nt, aphase = 0;
+  if (p.ntiles % 8 == 0) {
+    uint32_t xcd = id & 7, slot = id >> 3;
+    nt = (slot / p.mtiles) * 8 + xcd;
+    mt = slot % p.mtiles;
+    aphase = (slot / p.mtiles) % p.pf_asplit;
+  } else {
+    nt = id / p.mtiles;
+    mt = id % p.mtiles;
+  }
+  mt = __builtin_amdgcn_readfirstlane(mt);
+  nt = __builtin_amdgcn_readfirstlane(nt);
+  aphase = __builtin_amdgcn_readfirstlane(aphase);
+  const uint32_t m0 = mt * BM, n0 = nt * BN;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+
+  uint32_t aoff[NLA], boff[BN / 32];
+  const uint32_t chunk = ((lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7)) * 16;
+#pragma unroll
+  for (int v = 0; v < NLA; ++v) {
+    uint32_t r = min(m0 + 8 * (4 * v + wave) + (lane >> 3), p.M - 1);
+    aoff[v] = r * p.strideA * 2 + chunk;
+  }
+#pragma unroll
+  for (int v = 0; v < BN / 32; ++v) {
+    uint32_t r = min(n0 + 8 * (4 * v + wave) + (lane >> 3), p.N - 1);
+    boff[v] = r * p.K * 2 + chunk;
+  }
+  const uint8_t *const gA = p.A, *const gW = p.W;
+  const uint32_t pf_dist = p.pf_dist, Mrows = p.M, Ncols = p.N;
+  auto load_one = [&](int l, uint8_t *na, uint8_t *nb, uint32_t k0) {
+    const uint8_t *g = (l < NLA ? gA : gW) + (size_t)k0 * 2;
+    const uint32_t voff = l < NLA ? aoff[l] : boff[l - NLA];
+    const uint32_t dst = (uint32_t)(uintptr_t)(lds_u8 *)(l < NLA ? na : nb) + (4 * (l < NLA ? l : l - NLA) + wave) * 1024;
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(g), "s"(dst) : "memory");
+  };
+  const uint8_t *pfp[NPF];
+  {
+    const uint32_t nw = (BN + p.pf_wsplit - 1) / p.pf_wsplit, na = (BM + p.pf_asplit - 1) / p.pf_asplit;
+#pragma unroll
+    for (int i = 0; i < NPF; ++i) {
+      const uint32_t q = 256 * i + tid;
+      uint32_t wr = mt % p.pf_wsplit + (q < nw ? q : 0) * p.pf_wsplit, ar = aphase + (q - nw) * p.pf_asplit;
+      const bool is_a = q >= nw && q - nw < na && ar < BM;
+      wr = min(n0 + min(wr, (uint32_t)BN - 1), p.N - 1);
+      ar = min(m0 + ar, p.M - 1);
+      pfp[i] = is_a ? p.A + (size_t)ar * p.strideA * 2 : p.W + (size_t)wr * p.K * 2;
+    }
+  }
+  auto warm_one = [&](int i, uint32_t k0) {
+    const uint8_t *g = pfp[i] + (size_t)k0 * 2;
+    const uint32_t dst = (uint32_t)(uintptr_t)(lds_u8 *)(reinterpret_cast<uint8_t *>(pf_sink)) + wave * 256;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(dst) : "memory");
+  };
+
+  f32x4 acc[MI][NJ];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) acc[i][j] = f32x4{0, 0, 0, 0};
+
+  // fragment of 16 rows x 32 k: lane l holds row l & 15, the 8 halfs of chunk 4 s + (l >> 4) of k-step s; rows of a
+  // fragment start at a multiple of 16, so the swizzle key (row >> 1) & 7 is ((l & 15) >> 1)
+  const uint32_t arow = (wm * (BM / WM) + (lane & 15)) * 128, brow = (wn * (BN / WN) + (lane & 15)) * 128;
+  uint32_t xs[2];
+#pragma unroll
+  for (int s2 = 0; s2 < 2; ++s2) xs[s2] = ((4 * s2 + (lane >> 4)) ^ ((lane & 15) >> 1)) * 16;
+  auto read_a = [&](const uint8_t *sa, int s2, int i) -> half8v {
+    return *reinterpret_cast<const lds_half8v *>((const lds_u8 *)(sa) + arow + xs[s2] + i * 2048);
+  };
+  auto read_b = [&](const uint8_t *sb, int t) -> half8v {   // t: fragment of the slice, k-step t / NJ, tile t % NJ
+    return *reinterpret_cast<const lds_half8v *>((const lds_u8 *)(sb) + brow + xs[t / NJ] + (t % NJ) * 2048);
+  };
+
+  half8v fa[2][MI], fb[8];
+  const uint32_t kbeg = __builtin_amdgcn_readfirstlane(split * p.kper), nsl = p.kper / kDBK, klast = kbeg + p.kper - kDBK;
+
+  // MFMA group g of a slice: B fragment g (ring slot (ring0 + g) & 7) against the MI A fragments of its k-step.
+  // With each MFMA at most one LDS read and one load: the reads of this slice's own fragments while they are still
+  // ahead (rd_b, rd_a), or - in the tail, behind the barrier - the first reads of the next slice (next_*).
+  // cur_*: the stage this group's fragments came from and later reads of this slice go to; nxt_*: the other stage.
+  auto group = [&](auto gg, auto ring0c, const uint8_t *ca, const uint8_t *cb, uint8_t *na, uint8_t *nb, uint32_t k0, uint32_t kpf,
+                   auto tailc) {
+    constexpr int g = decltype(gg)::value, ring0 = decltype(ring0c)::value;
+    constexpr bool tail = decltype(tailc)::value;   // this group belongs to the slice before (ca, cb): registers only
+    constexpr int s2 = g / NJ, j = g % NJ;
+    static_for<MI>([&](auto ii) __attribute__((always_inline)) {
+      constexpr int i = decltype(ii)::value;
+      // as text with the accumulator tied to itself in an AGPR: through the builtin the allocator rotated accumulators
+      // through spare registers and copied them back behind the MFMAs (36 dependent copies per slice)
+      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fa[s2][i]), "v"(fb[(ring0 + g) & 7]));
+      if constexpr (!tail) {
+        // B fragment kAhead groups ahead, with the first MFMA of the group
+        if constexpr (i == 0 && g + kAhead < NB) fb[(ring0 + g + kAhead) & 7] = read_b(cb, g + kAhead);
+        // A fragments of the second k-step, one per group, in the middle of the first
+        if constexpr (i == 1 && g >= 2 && g < 2 + MI) fa[1][g - 2] = read_a(ca, 1, g - 2);
+        constexpr int q = g * MI + i;
+        if constexpr (q >= LFIRST && (q - LFIRST) % LSTEP == 0 && (q - LFIRST) / LSTEP < NL)
+          load_one((q - LFIRST) / LSTEP, na, nb, k0);
+        if constexpr (g == NB - kTail - 1 && i < NPF) warm_one(i, kpf);   // younger than every load of the slice
+      } else {
+        // tail of the slice before: (ca, cb) is the stage just released by the barrier; its first fragments
+        constexpr int q = (g - (NB - kTail)) * MI + i;   // slot within the tail
+        if constexpr (q < MI) fa[0][q] = read_a(ca, 0, q);
+        else if constexpr (q - MI < kAhead) fb[(ring0 + NB + (q - MI)) & 7] = read_b(cb, q - MI);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  static_assert(kTail * MI >= MI + kAhead, "the tail has a slot for each first read of the next slice");
+
+  // One slice on stage (ca, cb), whose first fragments are already on their way: groups 0 .. NB - kTail - 1, the
+  // waits and the barrier, then the last kTail groups from registers with the first reads of the next stage (na, nb).
+  auto slice = [&](auto ring0c, const uint8_t *ca, const uint8_t *cb, uint8_t *na, uint8_t *nb, uint32_t t) {
+    const uint32_t k0 = min(kbeg + (t + 1) * kDBK, klast), kpf = min(kbeg + (t + pf_dist) * kDBK, klast);
+    static_for<NB - kTail>([&](auto gg) __attribute__((always_inline)) {
+      group(gg, ring0c, ca, cb, na, nb, k0, kpf, std::false_type{});
+    });
+    // every read of this stage has been issued at least two groups ago; the next slice has landed in (na, nb)
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(NPF) : "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<kTail>([&](auto tt) __attribute__((always_inline)) {
+      group(std::integral_constant<int, NB - kTail + decltype(tt)::value>{}, ring0c, na, nb, nullptr, nullptr, 0, 0, std::true_type{});
+    });
+  };
+
+  for (uint32_t d = 1; d < p.pf_dist; ++d)
+#pragma unroll
+    for (int i = 0; i < NPF; ++i) warm_one(i, min(kbeg + d * kDBK, klast));
+#pragma unroll
+  for (int l = 0; l < NL; ++l) load_one(l, sA0, sB0, kbeg);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  // first fragments of the first slice (what a tail would have read)
+#pragma unroll
+  for (int i = 0; i < MI; ++i) fa[0][i] = read_a(sA0, 0, i);
+#pragma unroll
+  for (int t = 0; t < kAhead; ++t) fb[t] = read_b(sB0, t);
+  for (uint32_t t = 0; t < nsl; t += 2) {  // nsl is even (host check)
+    slice(std::integral_constant<int, 0>{}, sA0, sB0, sA1, sB1, t);
+    slice(std::integral_constant<int, NB & 7>{}, sA1, sB1, sA0, sB0, t + 1);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last warm-up loads: nothing may land after the exit
+
+  // C through LDS, a 32-row stripe (two rows of 16 x 16 tiles) at a time.  Register r of lane l of a tile: row
+  // 4 (l >> 4) + r, column l & 15.
+  __syncthreads();
+  constexpr int NJ32 = NJ / 2;
+  lds_f32 *stage = (lds_f32 *)(lds_u8 *)(lds) + wave * stripe_floats<NJ32>();
+  void *cbase = p.C;
+  uint32_t ldc = p.strideC;
+  int c_f16 = p.c_f16;
+  Epilogue epi = p.epi;
+  if (p.ksplit > 1) {
+    cbase = p.partial + (size_t)split * p.M * p.N;
+    ldc = p.N;
+    c_f16 = 0;
+    epi.kind = CUTHIP_EPI_NONE;
+  }
+  const bool vec = p.ksplit > 1 ? p.N % 4 == 0 : p.vec_store != 0;
+  const int fast = !vec ? 0 : (!c_f16 ? (epi.kind == CUTHIP_EPI_NONE ? 3 : 0)
+                               : epi.kind == CUTHIP_EPI_NONE ? 1
+                               : (epi.kind == CUTHIP_EPI_BINARY && epi.op == CUTHIP_BINARY_ADD) ? 2 : 0);
+  static_for<MI / 2>([&](auto ii) __attribute__((always_inline)) {
+    constexpr int i2 = decltype(ii)::value;
+    static_for<2 * NJ>([&](auto tt) __attribute__((always_inline)) {
+      constexpr int h = decltype(tt)::value / NJ, j = decltype(tt)::value % NJ;   // h: upper / lower 16 rows of the stripe
+      lds_f32 *wr = stage + (16 * h + 4 * (lane >> 4)) * stripe_ld<NJ32>() + 16 * j + (lane & 15);
+      const f32x4 a = acc[2 * i2 + h][j];
+      static_for<4>([&](auto rr) __attribute__((always_inline)) { wr[decltype(rr)::value * stripe_ld<NJ32>()] = a[decltype(rr)::value]; });
+    });
+    const uint32_t r0 = m0 + wm * (BM / WM) + 32 * i2, c0 = n0 + wn * (BN / WN);
+    if (fast == 1) store_staged32<NJ32, 1>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    else if (fast == 2) store_staged32<NJ32, 2>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    else if (fast == 3) store_staged32<NJ32, 3>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    else store_staged32<NJ32, 0>(stage, r0, c0, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+  });
+#endif
+}
+
 // fp32 [M, strideA] -> fp16 [M, K] (round to nearest even), 8 elements per thread
 __global__ void __launch_bounds__(256) cvt_rows_kernel(const float *src, half_t *dst, uint32_t K, uint32_t strideA,
                                                        uint32_t chunks) {
@@ -378,8 +595,13 @@ template <int BM, int BN, int WM = 2> static int launch_dense_bm(DenseParams p, 
     set_error("cuthip_matmul_gguf_ws: problem too large for one launch");
     return CUTHIP_ERR_INVALID;
   }
-  auto kern = gemm_dense_kernel<BM, BN, WM>;
-  hipLaunchKernelGGL(kern, dim3((uint32_t)grid), dim3(256), 0, stream, p);
+  // the 16 x 16 x 32 kernel unless CUT_HIP_DENSE_MFMA16=0 asks for the 32 x 32 x 16 one (kept for comparison)
+  static const bool mfma16 = [] {
+    const char *env = getenv("CUT_HIP_DENSE_MFMA16");
+    return !env || atoi(env) != 0;
+  }();
+  if (mfma16) hipLaunchKernelGGL((gemm_dense16_kernel<BM, BN, WM>), dim3((uint32_t)grid), dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL((gemm_dense_kernel<BM, BN, WM>), dim3((uint32_t)grid), dim3(256), 0, stream, p);
   return check_hip(hipGetLastError(), "dense gemm launch");
 }
 
