@@ -8,8 +8,10 @@
 // inner loop contains nothing but MFMAs, LDS fragment reads and copy instructions.
 // Supersedes MatMulQ{4,8}CoopMatTiled.cu (operators/impl/matmul) for large M.
 //
-// The GEMM: a workgroup of four waves owns a BM x 256 tile of C (BM = 256 or 128),
-// each wave a (BM/2) x 128 sub-tile in fp32 accumulators (AGPRs), K walked in slices
+// The GEMM (two kernels on the same tiles, loads and LDS image: gemm_dense16_kernel on 16 x 16 x 32 MFMAs, the one that
+// runs, and gemm_dense_kernel on 32 x 32 x 16 MFMAs, kept behind CUT_HIP_DENSE_MFMA16=0 for comparison; what follows
+// describes the latter, the former says where it differs): a workgroup of four waves owns a BM x BN tile of C,
+// each wave a sub-tile in fp32 accumulators (AGPRs), K walked in slices
 // of 64.  Both operands go global -> LDS with global_load_lds_dwordx4 (no VGPR
 // round trip): one instruction fills 8 tile rows x 128 bytes = 1 KB of LDS, lane i
 // at byte 16 i; the lane fetches the chunk of its row that belongs at that position
@@ -301,7 +303,8 @@ __global__ void __launch_bounds__(256, 1) gemm_dense16_kernel(DenseParams p) {
   constexpr int WN = 4 / WM;
   constexpr int MI = BM / (16 * WM), NJ = BN / (16 * WN);   // 16 x 16 MFMA tiles per wave
   constexpr int NB = 2 * NJ;                                 // B fragments per slice (two k-steps of 32)
-  constexpr int kAhead = 6, kTail = 3;                       // B fragments read ahead; groups multiplied behind the barrier
+  // B fragments read ahead; groups multiplied behind the barrier (2..6 ahead and tails of 2..4 measured within noise)
+  constexpr int kAhead = 6, kTail = 3;
   constexpr int NLA = BM / 32, NL = (BM + BN) / 32;          // LDS-direct loads per wave per slice (A, total)
   constexpr int NPF = 2;
   constexpr int LFIRST = 0, LLAST = (NB - kTail - 1) * MI;   // MFMA slots of a slice that carry a load
@@ -676,7 +679,7 @@ size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
 // Cost models in microseconds for the automatic choice between the two-pass path and the single-launch GEMM, fitted to
 // a sweep over the weight shapes of an 8B model (all formats, M = 16 .. 2048, HIP-graph replay, MI355X):
 //   two-pass      3 + N K (bytes per weight + 2) / 6.0 MB   the dequantization (reads the blocks, writes fp16)
-//                 + 17 + 2 ceil128(M) N K / 1.15 PFLOP/s     the dense GEMM (tiles are at least 128 rows high)
+//                 + 17 + 2 ceil128(M) N K / 1.25 PFLOP/s     the dense GEMM (tiles are at least 128 rows high)
 //   single launch K x c_fmt x max(1, tiles / 256)            c = 14.7 ns (Q4_K, Q4_0), 19.6 ns (Q8_0), 23.5 ns (Q6_K):
 //                 a workgroup decodes its K-long strip of weights once per 128 rows of A, and nothing overlaps that
 //                 walk until every CU holds more than one 128 x 128 tile.
@@ -684,7 +687,7 @@ size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
 // 173 / 203, 256 x 28672 x 4096 147 / 107; Q6_K 64 x 14336 x 4096 79 / 104.
 double dense_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
   const double nk = (double)N * K, bpw = (double)fmt_bytes(fmt) / fmt_elems(fmt);
-  return 3.0 + nk * (bpw + 2.0) / 6.0e6 + 17.0 + 2.0 * (double)((M + 127) / 128 * 128) * nk / 1.15e9;
+  return 3.0 + nk * (bpw + 2.0) / 6.0e6 + 17.0 + 2.0 * (double)((M + 127) / 128 * 128) * nk / 1.25e9;
 }
 double single_launch_rows_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
   const double c = fmt == CUTHIP_Q6_K ? 23.5e-3 : fmt == CUTHIP_Q8_0 ? 19.6e-3 : 14.7e-3;
