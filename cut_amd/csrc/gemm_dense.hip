@@ -308,7 +308,9 @@ __global__ void __launch_bounds__(256, 1) gemm_dense16_kernel(DenseParams p) {
   constexpr int NLA = BM / 32, NL = (BM + BN) / 32;          // LDS-direct loads per wave per slice (A, total)
   constexpr int NPF = 2;
   constexpr int LFIRST = 0, LLAST = (NB - kTail - 1) * MI;   // MFMA slots of a slice that carry a load
-  constexpr int LSTEP = (LLAST - LFIRST) / NL;
+  // one load every fourth MFMA at most: the last one then has half a slice to land (every second measured 4 % slower,
+  // every sixth 1 % slower)
+  constexpr int LSTEP = (LLAST - LFIRST) / NL < 4 ? (LLAST - LFIRST) / NL : 4;
   static_assert(NB % 8 == 0 || (2 * NB) % 8 == 0, "the B ring of eight must close over the two slices of a loop trip");
   static_assert(NJ >= kAhead + 2 && LSTEP >= 1 && MI >= 2, "tile shape");
   static_assert((BM + BN) * 128 * 2 <= 160 * 1024, "two LDS stages");
