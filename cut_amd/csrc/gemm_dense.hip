@@ -312,7 +312,9 @@ __global__ void __launch_bounds__(256, 1) gemm_dense16_kernel(DenseParams p) {
   // every sixth 1 % slower)
   constexpr int LSTEP = (LLAST - LFIRST) / NL < 4 ? (LLAST - LFIRST) / NL : 4;
   static_assert(NB % 8 == 0 || (2 * NB) % 8 == 0, "the B ring of eight must close over the two slices of a loop trip");
+  constexpr int kARd = (MI + NJ - 4) / (NJ - 3);             // A-fragment reads per group: the last one a group before k-step 1
   static_assert(NJ >= kAhead + 2 && LSTEP >= 1 && MI >= 2, "tile shape");
+  static_assert(kARd < MI && 2 + (MI + kARd - 1) / kARd <= NJ - 1, "the A fragments of k-step 1 are read during k-step 0");
   static_assert((BM + BN) * 128 * 2 <= 160 * 1024, "two LDS stages");
   static_assert(4 * stripe_floats<NJ / 2>() * 4 <= (BM + BN) * 128 * 2, "the output staging reuses the operand stages");
   __shared__ __attribute__((aligned(1024))) uint8_t lds[(BM + BN) * 128 * 2];
@@ -415,8 +417,9 @@ __global__ void __launch_bounds__(256, 1) gemm_dense16_kernel(DenseParams p) {
       if constexpr (!tail) {
         // B fragment kAhead groups ahead, with the first MFMA of the group
         if constexpr (i == 0 && g + kAhead < NB) fb[(ring0 + g + kAhead) & 7] = read_b(cb, g + kAhead);
-        // A fragments of the second k-step, one per group, in the middle of the first
-        if constexpr (i == 1 && g >= 2 && g < 2 + MI) fa[1][g - 2] = read_a(ca, 1, g - 2);
+        // A fragments of the second k-step, kARd per group from group 2 on, all on their way before that step begins
+        if constexpr (i >= 1 && i <= kARd && g >= 2 && (g - 2) * kARd + (i - 1) < MI)
+          fa[1][(g - 2) * kARd + (i - 1)] = read_a(ca, 1, (g - 2) * kARd + (i - 1));
         constexpr int q = g * MI + i;
         if constexpr (q >= LFIRST && (q - LFIRST) % LSTEP == 0 && (q - LFIRST) / LSTEP < NL)
           load_one((q - LFIRST) / LSTEP, na, nb, k0);
@@ -601,10 +604,8 @@ template <int BM, int BN, int WM = 2> static int launch_dense_bm(DenseParams p, 
     return CUTHIP_ERR_INVALID;
   }
   // the 16 x 16 x 32 kernel unless CUT_HIP_DENSE_MFMA16=0 asks for the 32 x 32 x 16 one (kept for comparison)
-  static const bool mfma16 = [] {
-    const char *env = getenv("CUT_HIP_DENSE_MFMA16");
-    return !env || atoi(env) != 0;
-  }();
+  const char *env16 = getenv("CUT_HIP_DENSE_MFMA16");   // read at every launch, like CUT_HIP_DENSE_TILE: a tuning aid
+  const bool mfma16 = !env16 || atoi(env16) != 0;
   if (mfma16) hipLaunchKernelGGL((gemm_dense16_kernel<BM, BN, WM>), dim3((uint32_t)grid), dim3(256), 0, stream, p);
   else hipLaunchKernelGGL((gemm_dense_kernel<BM, BN, WM>), dim3((uint32_t)grid), dim3(256), 0, stream, p);
   return check_hip(hipGetLastError(), "dense gemm launch");

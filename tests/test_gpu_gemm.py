@@ -236,6 +236,34 @@ def test_dense_gemm_128x448_tiles(ops):
     assert normwise_rel_err(got[np.ix_(rows, cols)], want) < TOL_GEMM
 
 
+@pytest.mark.parametrize("mfma16", ["1", "0"])
+@pytest.mark.parametrize("tile", ["256,224", "128,448", "256,256", "128,256", "128,256,2", "256,256,4"])
+def test_dense_gemm_every_tile_shape_and_both_kernels(ops, monkeypatch, tile, mfma16):
+    """Every tile shape of the dense GEMM (with and without a K split) under both of its kernels (16 x 16 x 32 MFMAs,
+    the default, and 32 x 32 x 16), forced through the library's tuning variables, on a problem with ragged tiles on
+    both sides: every output against the single-launch GEMM, sampled rows and columns against the oracle, and the
+    residual-add epilogue (the short output loop with an operand)."""
+    monkeypatch.setenv("CUT_HIP_DENSE_TILE", tile)
+    monkeypatch.setenv("CUT_HIP_DENSE_MFMA16", mfma16)
+    fmt = oracle.Q4_K
+    bn = int(tile.split(",")[1])
+    M, N, K = 700, 3 * bn - 8, 1024
+    W = quantized_weights(fmt, N, K, seed=151)
+    A = gauss_acts((M, K), seed=152, dtype=np.float16)
+    got = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float16)
+    ref = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=2)
+    assert normwise_rel_err(got, ref) < 5e-4      # fp16 output rounding
+    rng = np.random.default_rng(7)
+    rows = np.unique(np.concatenate([[0, 255, 256, M - 1], rng.integers(0, M, 12)]))
+    cols = np.unique(np.concatenate([[0, bn - 1, bn, N - 1], rng.integers(0, N, 150)]))
+    Ws = np.ascontiguousarray(W.reshape(N, oracle.n_bytes(fmt, K))[cols]).reshape(-1)
+    want = oracle.matmul_gguf(fmt, Ws, A[rows].astype(np.float32), len(cols), f64=True)
+    assert normwise_rel_err(got[np.ix_(rows, cols)], want) < TOL_GEMM
+    D = gauss_acts((M, N), seed=153, dtype=np.float16)
+    with_d = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float16, binary="add", d=torch.from_numpy(D).cuda())
+    assert normwise_rel_err(with_d - D.astype(np.float32), ref) < 1e-3
+
+
 def test_workspace_paths_under_hip_graph_replay(ops):
     """The two-pass GEMM (dequant + GEMM, with and without split K) and the K-split batched GEMV captured into one HIP
     graph and replayed with eager work in between: every replay equals the eager result (no allocation, no host
