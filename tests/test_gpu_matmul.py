@@ -290,6 +290,33 @@ def test_rows8_kernel_shapes(ops, name, M, N, K):
     assert normwise_rel_err(got0, want) < TOL_F16_ACT
 
 
+# (row groups, K ranges) of a workgroup with step counts the shape is chosen for: K ranges of unequal length, a range
+# longer than one staging batch, and N that fills neither the last wave's 8 rows nor the last workgroup's row groups
+FORCED_ROWS8 = [("4,1", 1024, [1, 2, 4, 8]), ("4,1", 4096 + 256, [1, 3, 8]), ("8,1", 2304, [1, 2, 5, 8]),
+                ("2,2", 1024, [1, 2, 4, 8]), ("2,2", 2304, [1, 3, 8]), ("1,4", 2048, [1, 2, 4, 8]), ("1,4", 3328, [1, 7]),
+                ("1,4", 4352, [1, 2, 4, 8]), ("2,4", 8448, [1, 2]), ("1,8", 4096, [1, 2, 4, 8]), ("1,8", 5376, [1, 4])]
+
+
+@pytest.mark.parametrize("name", list(oracle.FORMATS))
+@pytest.mark.parametrize("shape,K,batches", FORCED_ROWS8)
+def test_rows8_every_workgroup_shape(ops, monkeypatch, name, shape, K, batches):
+    """Every workgroup shape of the 8-row GEMV, forced through the library's tuning variable instead of left to the
+    choice by N and K (which reaches only one shape per problem), for every format and batch class, with a fused
+    residual add: against the oracle."""
+    monkeypatch.setenv("CUT_HIP_ROWS8_SHAPE", shape)
+    fmt = oracle.FORMATS[name]
+    N = 8 * 37 + 3
+    W = quantized_weights(fmt, N, K, seed=K + 1)
+    for M in batches:
+        A = gauss_acts((M, K), seed=M + 40, dtype=np.float16)
+        D = gauss_acts((M, N), seed=M + 80)
+        want = oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)
+        got = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=3)
+        assert normwise_rel_err(got, want) < TOL_F16_ACT, (shape, K, M)
+        got = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=3, binary="add", d=torch.from_numpy(D).cuda())
+        assert normwise_rel_err(got - D, want) < 10 * TOL_F16_ACT, (shape, K, M)
+
+
 def test_rows8_refuses_what_does_not_fit_and_auto_falls_back(ops):
     from cut_amd import lib
     fmt = oracle.Q4_K
