@@ -317,6 +317,24 @@ def test_rows8_every_workgroup_shape(ops, monkeypatch, name, shape, K, batches):
         assert normwise_rel_err(got - D, want) < 10 * TOL_F16_ACT, (shape, K, M)
 
 
+@pytest.mark.parametrize("name", list(oracle.FORMATS))
+@pytest.mark.parametrize("shape", ["1,1", "1,2", "1,4", "1,8", "2,1", "2,2", "2,4", "2,8"])
+def test_fallback_gemv_every_workgroup_shape(ops, monkeypatch, name, shape):
+    """The fallback GEMV (variant 0; 32 weight rows per workgroup, or 16 with two K parts per wave) under every
+    (parts, waves) shape, forced through the tuning variable: step counts that take the straight-line instances
+    (2, 4 and 7 steps per wave) and the generic loop, batch 1 to 8 in one pass and 20 rows as a 32-row pass."""
+    monkeypatch.setenv("CUT_HIP_GEMV_SHAPE", shape)
+    fmt = oracle.FORMATS[name]
+    N = 3 * 32 + 5
+    for K, batches in [(2048, [1, 2, 4, 8, 20]), (7168, [1, 3]), (2304, [1, 5, 20])]:
+        W = quantized_weights(fmt, N, K, seed=K + 3)
+        for M in batches:
+            A = gauss_acts((M, K), seed=M + 60, dtype=np.float16)
+            want = oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)
+            got = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=0)
+            assert normwise_rel_err(got, want) < TOL_F16_ACT, (shape, K, M)
+
+
 def test_rows8_refuses_what_does_not_fit_and_auto_falls_back(ops):
     from cut_amd import lib
     fmt = oracle.Q4_K
