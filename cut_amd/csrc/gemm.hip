@@ -41,9 +41,17 @@ struct GemmParams {
   uint32_t mtiles, ntiles;
   int a_f16, c_f16;
   int vec_store;   // C (and a binary epilogue's operand) allow 16-byte accesses
+  // K split over ksplit workgroups per tile (ranges of kper elements, a multiple of the slice): each writes fp32
+  // partial products [split][M][N] and a reduce kernel applies the epilogue; 1 = the tile's workgroup writes C itself
+  uint32_t ksplit, kper;
+  float *partial;
 };
 
 constexpr int kBN = 128, kBK = 64, kLdsRow = kBK + 8;  // halfs per LDS row
+
+// defined with the two-pass GEMM: C = epilogue(sum of the fp32 partial products)
+int launch_splitk_reduce(const float *partial, uint32_t ksplit, uint32_t M, uint32_t N, void *C, uint32_t strideC, Epilogue epi,
+                         int c_f16, hipStream_t stream);
 
 // ---- decode of one 32-element sub-block -------------------------------------
 // sub: index of the 32-element sub-block inside its row (k = 32*sub .. +31).
@@ -171,7 +179,8 @@ __global__ void __launch_bounds__(256, 2) gemm_kernel(GemmParams p) {
 
   // XCD-aware tile order: ids id, id+8, id+16, ... share an XCD; give them the
   // M-tiles of the same weight panel.
-  uint32_t id = blockIdx.x, mt, nt;
+  const uint32_t tiles = p.mtiles * p.ntiles, split = blockIdx.x / tiles;
+  uint32_t id = blockIdx.x - split * tiles, mt, nt;
   if (p.ntiles % 8 == 0) {
     uint32_t xcd = id & 7, slot = id >> 3;
     nt = (slot / p.mtiles) * 8 + xcd;
@@ -264,18 +273,20 @@ __global__ void __launch_bounds__(256, 2) gemm_kernel(GemmParams p) {
     }
   };
 
-  const uint32_t nfull = p.K / kBK, nslices = (p.K + kBK - 1) / kBK;
-  load_slice(0);
+  // this workgroup's K range [kb, ke): all of K without a split; only the last range can end in a partial slice
+  const uint32_t kb = split * p.kper, ke = min(p.K, kb + p.kper);
+  const uint32_t nfull = (ke - kb) / kBK, nslices = (ke - kb + kBK - 1) / kBK;
+  load_slice(kb);
   for (uint32_t t = 0; t < nfull; ++t) {
     __syncthreads();           // everyone is done reading the previous slice
-    store_slice(t * kBK, std::false_type{});
+    store_slice(kb + t * kBK, std::false_type{});
     __syncthreads();
-    if (t + 1 < nslices) load_slice((t + 1) * kBK);
+    if (t + 1 < nslices) load_slice(kb + (t + 1) * kBK);
     mma_slice();
   }
   if (nfull < nslices) {
     __syncthreads();
-    store_slice(nfull * kBK, std::true_type{});
+    store_slice(kb + nfull * kBK, std::true_type{});
     __syncthreads();
     mma_slice();
   }
@@ -285,13 +296,21 @@ __global__ void __launch_bounds__(256, 2) gemm_kernel(GemmParams p) {
   static_assert(4 * stripe_floats<2>() * 4 <= (BM + kBN) * kLdsRow * 2, "the output staging reuses the operand tiles");
   __syncthreads();
   lds_f32 *stage = (lds_f32 *)(lds_u8g *)(lds) + wave * stripe_floats<2>();
-  const Epilogue epi = p.epi;
-  const uint32_t Mrows = p.M, Ncols = p.N, ldc = p.strideC;
-  void *const cbase = p.C;
-  const int c_f16 = p.c_f16;
-  const bool vec = p.vec_store != 0;
-  // the common cases get the short store loops: no operator, or the residual add
-  const int fast = !(vec && c_f16) ? 0 : epi.kind == CUTHIP_EPI_NONE ? 1
+  Epilogue epi = p.epi;
+  const uint32_t Mrows = p.M, Ncols = p.N;
+  uint32_t ldc = p.strideC;
+  void *cbase = p.C;
+  int c_f16 = p.c_f16;
+  bool vec = p.vec_store != 0;
+  if (p.ksplit > 1) {   // fp32 partial products of this K range; the reduce kernel owns the epilogue
+    cbase = p.partial + (size_t)split * p.M * p.N;
+    ldc = p.N;
+    c_f16 = 0;
+    epi.kind = CUTHIP_EPI_NONE;
+    vec = p.N % 4 == 0;
+  }
+  // the common cases get the short store loops: no operator, or the residual add; fp32 partial products
+  const int fast = !vec ? 0 : !c_f16 ? (p.ksplit > 1 ? 3 : 0) : epi.kind == CUTHIP_EPI_NONE ? 1
                    : (epi.kind == CUTHIP_EPI_BINARY && epi.op == CUTHIP_BINARY_ADD) ? 2 : 0;
   static_for<MI>([&](auto ii) __attribute__((always_inline)) {
     constexpr int i = decltype(ii)::value;
@@ -299,6 +318,7 @@ __global__ void __launch_bounds__(256, 2) gemm_kernel(GemmParams p) {
     stage_tile32<2>(stage, 1, acc[i][1], lane);
     if (fast == 1) store_staged32<2, 1>(stage, m0 + wm * (BM / 2) + 32 * i, n0 + wn * 64, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
     else if (fast == 2) store_staged32<2, 2>(stage, m0 + wm * (BM / 2) + 32 * i, n0 + wn * 64, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
+    else if (fast == 3) store_staged32<2, 3>(stage, m0 + wm * (BM / 2) + 32 * i, n0 + wn * 64, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
     else store_staged32<2, 0>(stage, m0 + wm * (BM / 2) + 32 * i, n0 + wn * 64, Mrows, Ncols, cbase, ldc, c_f16, epi, vec, lane);
   });
 }
@@ -314,13 +334,32 @@ template <int FMT, int BM, bool AF16> static int launch_gemm_bm(GemmParams p, hi
                            "hipFuncSetAttribute"))
       return rc;
   }
-  uint64_t grid = (uint64_t)p.mtiles * p.ntiles;
+  // K split: with a scratch area at hand and too few tiles for the chip, up to sixteen K ranges of at least eight
+  // slices each (a workgroup walks its slices one memory round trip at a time, so short of two workgroups per CU
+  // the launch is bound by that latency: 14336 x 4096 at 64 rows 66 us unsplit)
+  const uint64_t tiles = (uint64_t)p.mtiles * p.ntiles;
+  const uint32_t nslices = (p.K + kBK - 1) / kBK;
+  uint32_t ks = 1;
+  if (p.partial && BM == 128) {
+    while (ks < 16 && tiles * ks < 384 && nslices / (2 * ks) >= 8 && (uint64_t)2 * ks * p.M * p.N * 4 <= p.kper) ks *= 2;
+    if (const char *env = getenv("CUT_HIP_GEMM_KSPLIT")) {   // tuning aid
+      const uint32_t want = (uint32_t)atoi(env);
+      if (want >= 1 && want <= 16 && (uint64_t)want * p.M * p.N * 4 <= p.kper) ks = want;
+    }
+  }
+  const uint32_t per = (nslices + ks - 1) / ks;
+  p.kper = per * kBK;                      // (on entry: bytes of scratch behind partial)
+  p.ksplit = (nslices + per - 1) / per;    // no empty range
+  if (p.ksplit == 1) p.kper = p.K + kBK;
+  uint64_t grid = tiles * p.ksplit;
   if (grid > 0x7FFFFFFFull) {
     set_error("cuthip_matmul_gguf: problem too large for one launch");
     return CUTHIP_ERR_INVALID;
   }
   hipLaunchKernelGGL(kern, dim3((uint32_t)grid), dim3(256), lds, stream, p);
-  return check_hip(hipGetLastError(), "gemm launch");
+  if (int rc = check_hip(hipGetLastError(), "gemm launch")) return rc;
+  if (p.ksplit == 1) return CUTHIP_OK;
+  return launch_splitk_reduce(p.partial, p.ksplit, p.M, p.N, p.C, p.strideC, p.epi, p.c_f16, stream);
 }
 
 template <int FMT> static int launch_gemm_fmt(const GemmParams &p, hipStream_t stream) {
@@ -334,8 +373,9 @@ template <int FMT> static int launch_gemm_fmt(const GemmParams &p, hipStream_t s
   return launch_gemm_bm<FMT, 128, true>(p, stream);
 }
 
+// scratch: 16-byte aligned room for fp32 partial products of a K split (nullptr / 0: none, one workgroup per tile)
 int launch_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K, uint32_t N,
-                uint32_t strideA, uint32_t strideC, Epilogue epi, hipStream_t stream) {
+                uint32_t strideA, uint32_t strideC, Epilogue epi, hipStream_t stream, void *scratch, size_t scratch_bytes) {
   GemmParams p;
   p.W = reinterpret_cast<const uint8_t *>(W);
   p.A = A;
@@ -346,6 +386,9 @@ int launch_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c
   p.mtiles = p.ntiles = 0;
   p.a_f16 = a_f16; p.c_f16 = c_f16;
   p.vec_store = store8_aligned(C, strideC, c_f16, epi) ? 1 : 0;
+  p.ksplit = 1;
+  p.partial = scratch && (uintptr_t)scratch % 16 == 0 ? reinterpret_cast<float *>(scratch) : nullptr;
+  p.kper = (uint32_t)(scratch_bytes < 0xFFFFFFFFull ? scratch_bytes : 0xFFFFFFFFull);   // launch_gemm_bm turns it into the range
   switch (fmt) {
   case CUTHIP_Q8_0: return launch_gemm_fmt<CUTHIP_Q8_0>(p, stream);
   case CUTHIP_Q4_0: return launch_gemm_fmt<CUTHIP_Q4_0>(p, stream);

@@ -106,7 +106,7 @@ GemvShape pick_gemv_shape(uint32_t N, uint32_t nsteps, int mt) {
 }
 
 int launch_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K, uint32_t N,
-                uint32_t strideA, uint32_t strideC, Epilogue epi, hipStream_t stream);
+                uint32_t strideA, uint32_t strideC, Epilogue epi, hipStream_t stream, void *scratch, size_t scratch_bytes);
 
 bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a_f16, const void *A);
 size_t dense_gemm_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16);
@@ -158,9 +158,23 @@ static double passes_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
   const double f = K >= 8192 ? (fmt == CUTHIP_Q6_K ? 1.55 : 1.45) : (fmt == CUTHIP_Q6_K ? 1.5 : 1.0);
   return ((M + 7) / 8) * (6.5 + weight_bytes(fmt, K, N) / 4.3e6) * f;
 }
-static double single_launch_cost_us(int fmt, uint32_t K, uint32_t N) { return 62.0 + weight_bytes(fmt, K, N) / 7e6; }
-static bool passes_preferred(int fmt, uint32_t M, uint32_t K, uint32_t N) {
-  return M > 8 && M <= kPassesMaxRows && (K >= 8192 || passes_cost_us(fmt, M, K, N) <= single_launch_cost_us(fmt, K, N));
+// The tiled GEMM with its K split over workgroups (scratch memory at hand, up to 256 rows): 9.5 us + the decode of the
+// matrix at 0.37 (Q4_K) to 0.64 (Q6_K) us per million weights per 128-row tile, + 0.07 us per row beyond 16
+// (14336 x 4096 Q4_K: 31 us at 16-64 rows, 38 at 128, 58 at 256; unsplit 65 at every M up to 128, 216 on K = 14336).
+static bool tiled_split_applies(uint32_t M, uint32_t N, const void *scratch, size_t scratch_bytes) {
+  return scratch && (uintptr_t)scratch % 16 == 0 && M > 8 && M <= 256 && scratch_bytes >= (size_t)4 * M * N * sizeof(float);
+}
+static double tiled_split_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
+  const double c = fmt == CUTHIP_Q6_K ? 0.644 : fmt == CUTHIP_Q8_0 ? 0.46 : fmt == CUTHIP_Q4_0 ? 0.40 : 0.372;
+  const uint32_t mt = (M + 127) / 128, rows = M < 128 ? M : 128;
+  return mt * (9.5 + c * 1e-6 * N * K) * (mt == 2 ? 0.93 : 1.0) + 0.07 * (rows > 16 ? rows - 16 : 0);
+}
+static double single_launch_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N, bool split) {
+  return split ? tiled_split_cost_us(fmt, M, K, N) : 62.0 + weight_bytes(fmt, K, N) / 7e6;
+}
+static bool passes_preferred(int fmt, uint32_t M, uint32_t K, uint32_t N, bool split) {
+  return M > 8 && M <= kPassesMaxRows &&
+         ((K >= 8192 && !split) || passes_cost_us(fmt, M, K, N) <= single_launch_cost_us(fmt, M, K, N, split));
 }
 
 // Argument checks shared by the matmul entry points: 0 = go on, 1 = empty problem (success), < 0 = error.
@@ -208,16 +222,18 @@ static int check_matmul_args(int fmt, const void *W, const void *A, int a_dtype,
   return 0;
 }
 
-extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M,
-                                  uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue,
-                                  int epilogue_op, const void *D, int variant, void *stream) {
+// cuthip_matmul_gguf with optional scratch memory (the workspace of cuthip_matmul_gguf_ws, or none): the tiled GEMM
+// splits K through it where it has too few tiles for the chip
+static int matmul_gguf_scratch(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M,
+                               uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue,
+                               int epilogue_op, const void *D, int variant, void *stream, void *scratch, size_t scratch_bytes) {
   using namespace cuthip;
   if (int rc = check_matmul_args(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, D))
     return rc > 0 ? CUTHIP_OK : rc;
   if (int rc = check_epilogue_op("cuthip_matmul_gguf", epilogue, epilogue_op)) return rc;
   if (epilogue_op_long(epilogue, epilogue_op)) {   // unfused matmul, then the operator as an elementwise launch
-    if (int rc = cuthip_matmul_gguf(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, CUTHIP_EPI_NONE, 0, nullptr,
-                                    variant, stream))
+    if (int rc = matmul_gguf_scratch(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, CUTHIP_EPI_NONE, 0, nullptr,
+                                     variant, stream, scratch, scratch_bytes))
       return rc;
     return launch_long_epilogue(C, c_dtype == CUTHIP_F16, M, N, strideC, epilogue, epilogue_op, D,
                                 reinterpret_cast<hipStream_t>(stream));
@@ -248,14 +264,14 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
   // 9-40 rows, automatic choice: passes of 8 rows through the decode kernels.  Measured on 14336 x 4096: 14 us per
   // pass, against 69-87 us for the 32-row skinny kernel and 73-80 us for one launch of the tiled GEMM, whose cost
   // is the decode of the whole weight matrix whatever M is.
-  if (variant == -1 && passes_preferred(fmt, M, K, N)) {
+  if (variant == -1 && passes_preferred(fmt, M, K, N, tiled_split_applies(M, N, scratch, scratch_bytes))) {
     const size_t asz = a_dtype == CUTHIP_F16 ? 2 : 4, csz = c_dtype == CUTHIP_F16 ? 2 : 4;
     for (uint32_t m0 = 0; m0 < M; m0 += 8) {
       const uint8_t *a = reinterpret_cast<const uint8_t *>(A) + (size_t)m0 * strideA * asz;
       uint8_t *c = reinterpret_cast<uint8_t *>(C) + (size_t)m0 * strideC * csz;
       const uint8_t *d = D ? reinterpret_cast<const uint8_t *>(D) + (size_t)m0 * strideC * csz : nullptr;
-      if (int rc = cuthip_matmul_gguf(fmt, W, a, a_dtype, c, c_dtype, min(8u, M - m0), K, N, strideA, strideC, epilogue,
-                                      epilogue_op, d, -1, stream))
+      if (int rc = matmul_gguf_scratch(fmt, W, a, a_dtype, c, c_dtype, min(8u, M - m0), K, N, strideA, strideC, epilogue,
+                                       epilogue_op, d, -1, stream, nullptr, 0))
         return rc;
     }
     return CUTHIP_OK;
@@ -266,7 +282,7 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
       return CUTHIP_ERR_INVALID;
     }
     return launch_gemm(fmt, W, A, a_dtype == CUTHIP_F16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC, epi,
-                       reinterpret_cast<hipStream_t>(stream));
+                       reinterpret_cast<hipStream_t>(stream), scratch, scratch_bytes);
   }
   GemvParams p = gemv_params(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epi);
   // variant 3 (and the automatic choice for M <= 8): 8 rows x 128-byte runs per wave instruction
@@ -284,6 +300,13 @@ extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_d
     return CUTHIP_ERR_INVALID;
   }
   return launch_gemv(fmt, p, reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M,
+                                  uint32_t K, uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue,
+                                  int epilogue_op, const void *D, int variant, void *stream) {
+  return matmul_gguf_scratch(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, variant,
+                             stream, nullptr, 0);
 }
 extern "C" {
 
@@ -476,8 +499,8 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
                           int variant, void *workspace, size_t workspace_bytes, void *stream) {
   using namespace cuthip;
   if ((variant != 4 && variant != 5 && variant != -1) || epilogue == CUTHIP_EPI_SWIGLU_PAIRS)
-    return cuthip_matmul_gguf(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, variant,
-                              stream);
+    return matmul_gguf_scratch(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, variant,
+                               stream, workspace, workspace ? workspace_bytes : 0);
   if (int rc = check_matmul_args(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, D))
     return rc > 0 ? CUTHIP_OK : rc;
   if (int rc = check_epilogue_op("cuthip_matmul_gguf_ws", epilogue, epilogue_op)) return rc;
@@ -499,9 +522,10 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
       blaslt_preferred()) {
     const double nk = (double)N * K;
     const double t5 = 14.0 + nk * (nk <= 64e6 ? 0.65e-6 : 0.95e-6) + 2.0 * M * nk / 1.6e9;
+    const bool split = tiled_split_applies(M, N, workspace, workspace_bytes);
     double other;
-    if (passes_preferred(fmt, M, K, N)) other = passes_cost_us(fmt, M, K, N);
-    else other = K >= 8192 ? 65.0 + 0.19 * M : single_launch_cost_us(fmt, K, N);
+    if (passes_preferred(fmt, M, K, N, split)) other = passes_cost_us(fmt, M, K, N);
+    else other = split ? tiled_split_cost_us(fmt, M, K, N) : K >= 8192 ? 65.0 + 0.19 * M : single_launch_cost_us(fmt, M, K, N, false);
     if (t5 < 0.95 * other) {
       const int rc = launch_dense_gemm(fmt, W, A, a_f16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC,
                                        Epilogue{CUTHIP_EPI_NONE, 0, nullptr}, workspace,
@@ -515,13 +539,14 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   const bool fits = dense_gemm_fits(M, K, N, strideA, a_f16, A);
   const size_t need = dense_gemm_workspace(M, K, N, a_f16);
   const bool ws_ok = workspace && (uintptr_t)workspace % 256 == 0 && workspace_bytes >= need;
+  const bool split = tiled_split_applies(M, N, workspace, workspace_bytes);
   bool dense_first = false;
   if (variant == -1 && M > 8 && fits && ws_ok) {
     const double t4 = dense_cost_us(fmt, M, K, N);
-    dense_first = M >= 1024 || (passes_preferred(fmt, M, K, N) ? t4 < 0.9 * passes_cost_us(fmt, M, K, N)
-                                                               : t4 < 0.95 * single_launch_rows_cost_us(fmt, M, K, N));
+    const double tiled = split ? tiled_split_cost_us(fmt, M, K, N) : single_launch_rows_cost_us(fmt, M, K, N);
+    dense_first = M >= 1024 || (passes_preferred(fmt, M, K, N, split) ? t4 < 0.9 * passes_cost_us(fmt, M, K, N) : t4 < 0.95 * tiled);
   }
-  if (variant == -1 && !dense_first && passes_preferred(fmt, M, K, N)) {   // 8-row passes, each with the workspace (K split on long rows)
+  if (variant == -1 && !dense_first && passes_preferred(fmt, M, K, N, split)) {   // 8-row passes, each with the workspace (K split on long rows)
     const size_t asz = a_f16 ? 2 : 4, csz = c_dtype == CUTHIP_F16 ? 2 : 4;
     for (uint32_t m0 = 0; m0 < M; m0 += 8) {
       const uint8_t *a = reinterpret_cast<const uint8_t *>(A) + (size_t)m0 * strideA * asz;
@@ -556,8 +581,8 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   // matrix against a single-launch GEMM that decodes the weights once per 128 rows (M = 512, N = 14336: 86 us against 110)
   const bool lt_ok = variant == -1 && epilogue == CUTHIP_EPI_NONE && fits && ws_ok && blaslt_preferred();
   if (variant == -1 && !((dense_first || (lt_ok && M >= 384)) && fits && ws_ok))
-    return cuthip_matmul_gguf(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, -1,
-                              stream);
+    return matmul_gguf_scratch(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, -1,
+                               stream, workspace, workspace ? workspace_bytes : 0);
   if (!fits) {
     set_error("cuthip_matmul_gguf_ws: variants 4 and 5 need K a multiple of 128, 16-byte aligned rows of A and operands "
               "below 4 GiB (M %u, K %u, N %u, strideA %u)", M, K, N, strideA);

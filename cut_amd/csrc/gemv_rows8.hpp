@@ -929,11 +929,12 @@ static int launch_rows8_pair(const GemvParams &pa, const GemvParams &pb, hipStre
   return check_hip(hipGetLastError(), "gemv pair launch");
 }
 
-// parts of K for the split across workgroups: enough parts for two workgroups per CU, at least 4 steps per part
+// parts of K for the split across workgroups: enough parts for one workgroup of eight waves per CU, at least 4 steps per
+// part (4096 x 14336 at batch 8: four parts of 14 steps 14.8 us per launch of an FFN step, eight parts of 7 steps 16.5)
 inline uint32_t rows8_ksplit_parts(uint32_t N, uint32_t nsteps) {
   const uint32_t blocks = ((N + 7) / 8 + 7) / 8;
   uint32_t s = 1;
-  while (s < 16 && blocks * s < 512 && nsteps / (2 * s) >= 4) s *= 2;
+  while (s < 16 && blocks * s < 256 && nsteps / (2 * s) >= 4) s *= 2;
   return s;
 }
 

@@ -236,6 +236,34 @@ def test_dense_gemm_128x448_tiles(ops):
     assert normwise_rel_err(got[np.ix_(rows, cols)], want) < TOL_GEMM
 
 
+@pytest.mark.parametrize("name,K", [("Q4_K", 4096), ("Q6_K", 2048), ("Q8_0", 4128), ("Q4_0", 2080), ("Q4_K", 14336)])
+@pytest.mark.parametrize("M", [9, 70, 128, 200])
+def test_tiled_gemm_splits_k_through_the_workspace(ops, monkeypatch, name, K, M):
+    """The single-launch GEMM (variant 2) with a workspace at hand: few tiles, so K is split over workgroups (fp32
+    partial products, summed by the reduce kernel, which also applies the epilogue).  Ragged tiles, a K whose last
+    range ends in a partial slice, fp16 and fp32 activations, the residual add, and a forced split of 3 ranges of
+    unequal length: against the oracle and the unsplit launch."""
+    fmt = oracle.FORMATS[name]
+    N = 300
+    W = quantized_weights(fmt, N, K, seed=K + M)
+    A = gauss_acts((M, K), seed=M + 7, dtype=np.float16)
+    want = oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)
+    unsplit = gpu_matmul(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=2)
+    got = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=2)
+    assert normwise_rel_err(got, want) < TOL_GEMM
+    assert normwise_rel_err(got, unsplit) < 1e-6      # the same products, summed in another order
+    auto = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=-1)
+    assert normwise_rel_err(auto, want) < TOL_GEMM
+    D = gauss_acts((M, N), seed=M + 9, dtype=np.float16)
+    got16 = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float16, variant=2, binary="add", d=torch.from_numpy(D).cuda())
+    assert normwise_rel_err(got16 - D.astype(np.float32), want) < 2e-3   # fp16 rounding of sum + D
+    got32 = gpu_matmul_ws(ops, fmt, W, A.astype(np.float32), N, K, out_dtype=torch.float32, variant=2)
+    assert normwise_rel_err(got32, want) < TOL_GEMM
+    monkeypatch.setenv("CUT_HIP_GEMM_KSPLIT", "3")
+    got3 = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=2)
+    assert normwise_rel_err(got3, unsplit) < 1e-6
+
+
 @pytest.mark.parametrize("mfma16", ["1", "0"])
 @pytest.mark.parametrize("tile", ["256,224", "128,448", "256,256", "128,256", "128,256,2", "256,256,4"])
 def test_dense_gemm_every_tile_shape_and_both_kernels(ops, monkeypatch, tile, mfma16):
