@@ -79,6 +79,10 @@ static const cuthip_variant_info_t kMatMulGgufVariants[] = {
     {"MatMulGgufDequantBlasLt", 256, 1, 256, 256,
      "large-M prefill in two launches: the weights are dequantized once to an fp16 workspace, then hipBLASLt's dense fp16 "
      "GEMM (opened at run time; no fused epilogue; needs cuthip_matmul_gguf_ws)"},
+    {"MatMulGgufStreamMfma", 256, 1, 16, 64,
+     "5..32 rows of A on Q4_K: 16 weight rows per wave, nibbles and 6-bit scales multiplied as integers into fp16 "
+     "subnormals, 16x16x32 f16 MFMA chains per super-block, activations staged once per workgroup (long K split over "
+     "workgroups through the workspace of cuthip_matmul_gguf_ws)"},
 };
 
 // Separated-layout matmuls: the reference's tables, name for name and index for index

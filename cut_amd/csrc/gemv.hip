@@ -115,6 +115,10 @@ double single_launch_rows_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N);
 int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K,
                       uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream,
                       int use_blaslt);
+bool stream_gemm_fits(int fmt, uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a_f16, const void *A);
+size_t stream_gemm_scratch(uint32_t M, uint32_t K, uint32_t N);
+int launch_stream_gemm(const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K, uint32_t N,
+                       uint32_t strideA, uint32_t strideC, Epilogue epi, void *scratch, size_t scratch_bytes, hipStream_t stream);
 bool blaslt_available();
 bool blaslt_preferred();
 size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16);
@@ -222,6 +226,13 @@ static int check_matmul_args(int fmt, const void *W, const void *A, int a_dtype,
   return 0;
 }
 
+static bool stream_preferred(int fmt, uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a_f16, const void *A,
+                             const void *scratch, size_t scratch_bytes) {
+  if (M < 9 || M > 32 || !cuthip::stream_gemm_fits(fmt, M, K, N, strideA, a_f16, A)) return false;
+  const size_t need = cuthip::stream_gemm_scratch(M, K, N);
+  return need == 0 || (scratch && (uintptr_t)scratch % 16 == 0 && scratch_bytes >= need);
+}
+
 // cuthip_matmul_gguf with optional scratch memory (the workspace of cuthip_matmul_gguf_ws, or none): the tiled GEMM
 // splits K through it where it has too few tiles for the chip
 static int matmul_gguf_scratch(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M,
@@ -249,7 +260,7 @@ static int matmul_gguf_scratch(int fmt, const void *W, const void *A, int a_dtyp
     return CUTHIP_ERR_INVALID;
   }
   // variant table: 0 streaming GEMV (M <= 8; beyond, as -1), 1 skinny passes of 32 rows, 2 LDS-tiled GEMM,
-  // 3 the 8-row GEMV, 4 / 5 dequantize + dense GEMM (workspace entry point only)
+  // 3 the 8-row GEMV, 4 / 5 dequantize + dense GEMM (workspace entry point only), 6 the streaming MFMA kernel (Q4_K, M <= 32)
   Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
   if (epilogue == CUTHIP_EPI_SWIGLU_PAIRS && variant != -1 && variant != 3) {
     set_error("cuthip_matmul_gguf: the SwiGLU row-pair epilogue exists in variant 3 only (got variant %d)", variant);
@@ -261,6 +272,19 @@ static int matmul_gguf_scratch(int fmt, const void *W, const void *A, int a_dtyp
   }
   // the table's default entry is valid for every M: beyond the 8 rows its GEMV takes it is the choice by shape
   if (variant == 0 && M > 8) variant = -1;
+  // 9-32 rows on Q4_K: the streaming MFMA kernel (9-16 rows of 14336 x 4096: 15.8 us against 25 for two 8-row
+  // passes; 17-32 rows: 26 us against 30 for the tiled GEMM with K split), wherever the scratch memory it needs
+  // for long rows or two activation tiles is at hand
+  if (variant == -1 && stream_preferred(fmt, M, K, N, strideA, a_dtype == CUTHIP_F16, A, scratch, scratch_bytes)) variant = 6;
+  // variant 6: the streaming MFMA kernel (Q4_K, up to 32 rows); scratch only where K has to be split over workgroups
+  if (variant == 6) {
+    if (!stream_gemm_fits(fmt, M, K, N, strideA, a_dtype == CUTHIP_F16, A)) {
+      set_error("cuthip_matmul_gguf: variant 6 takes Q4_K, M <= 32 and 16-byte aligned rows of A (fmt %d, M %u, K %u)", fmt, M, K);
+      return CUTHIP_ERR_INVALID;
+    }
+    return launch_stream_gemm(W, A, a_dtype == CUTHIP_F16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC, epi, scratch,
+                              scratch_bytes, reinterpret_cast<hipStream_t>(stream));
+  }
   // 9-40 rows, automatic choice: passes of 8 rows through the decode kernels.  Measured on 14336 x 4096: 14 us per
   // pass, against 69-87 us for the 32-row skinny kernel and 73-80 us for one launch of the tiled GEMM, whose cost
   // is the decode of the whole weight matrix whatever M is.
@@ -512,6 +536,9 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
                                 reinterpret_cast<hipStream_t>(stream));
   }
   const int a_f16 = a_dtype == CUTHIP_F16;
+  if (variant == -1 && stream_preferred(fmt, M, K, N, strideA, a_f16, A, workspace, workspace ? workspace_bytes : 0))
+    return matmul_gguf_scratch(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, 6, stream,
+                               workspace, workspace_bytes);
   // 9..383 rows with the vendor GEMM at hand: dequantize + hipBLASLt against what the automatic choice would run
   // otherwise, by a cost model fitted to a sweep over the FFN / attention shapes of an 8B model (microseconds;
   // Q4_K, graph replay): an 8-row pass 6.5 + weight bytes / 4.3 MB (x 1.45 on rows of K >= 8192), the

@@ -200,9 +200,10 @@ int cuthip_dequant(int fmt, const void *blocks, void *out, int out_dtype, uint32
  *          epilogue (residual add etc.), else NULL
  * K must be a multiple of the block size; fp32 accumulation throughout.
  * variant: index into the CUTHIP_OP_MATMUL_GGUF table, or -1 = choose by shape
- *          (M <= 8 -> streaming GEMV, 9..40 -> passes of 8 rows through it, else the
- *          LDS-tiled MFMA GEMM); variant 4 needs
- *          cuthip_matmul_gguf_ws. */
+ *          (M <= 8 -> streaming GEMV; 9..16 rows of Q4_K with K <= 4096 -> variant 6, the
+ *          streaming MFMA kernel; other 9..40 -> passes of 8 rows through the GEMV; else
+ *          the LDS-tiled MFMA GEMM); variants 4 and 5 need cuthip_matmul_gguf_ws, which
+ *          also gives variants 2 and 6 the scratch memory they split K through. */
 int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M, uint32_t K,
                        uint32_t N, uint32_t strideA, uint32_t strideC, int epilogue, int epilogue_op, const void *D,
                        int variant, void *stream);
@@ -234,7 +235,16 @@ int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void 
  *            few output tiles that the single-launch GEMM would leave most of the chip
  *            idle, from M = 256, and from M = 41 when K >= 8192; K is then split and
  *            the partial products summed), else
- *            as cuthip_matmul_gguf; 0..3 = as cuthip_matmul_gguf (workspace unused).
+ *            as cuthip_matmul_gguf; 0, 1, 3 = as cuthip_matmul_gguf (workspace unused);
+ *            2 = the single-launch GEMM, which with a workspace at hand splits K over
+ *            workgroups where its tiles alone would not fill the chip (up to 256 rows:
+ *            fp32 partial products in the workspace, summed in a second launch);
+ *            6 = MatMulGgufStreamMfma (Q4_K, M <= 32, 16-byte aligned rows of A, else an
+ *            error): the weights stay packed until they are multiplied (integer-scaled
+ *            nibbles as fp16 subnormals into 16x16x32 MFMAs, results exact up to the
+ *            order of the fp32 sums); K above 4096 (2048 beyond 16 rows) is split over
+ *            workgroups through the workspace, an error without one.  With variant -1
+ *            it is what runs for 9..32 rows of Q4_K.
  * With variant -1 the workspace also serves batch 3-8 on long rows (K >= 8192) of few (N < 12288): the 8-row GEMV
  * then splits K across workgroups, writes fp32 partial products to the workspace and sums them in a second launch
  * (the unsplit kernel would have to stage all of the activations in every workgroup).

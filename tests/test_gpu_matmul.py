@@ -335,6 +335,50 @@ def test_fallback_gemv_every_workgroup_shape(ops, monkeypatch, name, shape):
             assert normwise_rel_err(got, want) < TOL_F16_ACT, (shape, K, M)
 
 
+@pytest.mark.parametrize("M", [1, 5, 8, 16, 17, 32])
+@pytest.mark.parametrize("N,K", [(200, 2048), (70, 256), (1030, 4096), (64, 14336), (300, 8192 + 256)])
+def test_streaming_mfma_matmul(ops, M, N, K):
+    """Variant 6 (Q4_K, up to 32 rows): integer-scaled nibbles as fp16 subnormals through 16 x 16 x 32 MFMAs.  One and
+    two activation tiles, ragged N, one step, K ranges split over workgroups (needs the workspace) with ranges of
+    unequal length, fp16 and fp32 activations, a fused residual add: the products are exact, so the bound is that of
+    the fp32 summation order."""
+    fmt = oracle.Q4_K
+    W = quantized_weights(fmt, N, K, seed=N + K)
+    A = gauss_acts((M, K), seed=M + 3, dtype=np.float16)
+    want = oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)
+    a, w = torch.from_numpy(A).cuda(), torch.from_numpy(W).cuda()
+    ws = ops.matmul_gguf_workspace(fmt, M, K, N, a.dtype, "cuda")
+    ws.fill_(0xFF)
+    got = ops.matmul_gguf(a, w, fmt, N, K, out_dtype=torch.float32, variant=6, workspace=ws)
+    torch.cuda.synchronize()
+    assert normwise_rel_err(got.cpu().numpy(), want) < TOL_F16_ACT
+    D = gauss_acts((M, N), seed=M + 5, dtype=np.float16)
+    got16 = ops.matmul_gguf(a, w, fmt, N, K, out_dtype=torch.float16, variant=6, workspace=ws, binary="add",
+                            d=torch.from_numpy(D).cuda())
+    torch.cuda.synchronize()
+    assert normwise_rel_err(got16.float().cpu().numpy() - D.astype(np.float32), want) < 2e-3   # fp16 rounding of sum + D
+    got32 = ops.matmul_gguf(a.float(), w, fmt, N, K, out_dtype=torch.float32, variant=6, workspace=ws)
+    torch.cuda.synchronize()
+    assert normwise_rel_err(got32.cpu().numpy(), want) < TOL_F16_ACT
+    if K <= 4096 and M <= 16:      # one K range: no workspace needed
+        alone = ops.matmul_gguf(a, w, fmt, N, K, out_dtype=torch.float32, variant=6)
+        torch.cuda.synchronize()
+        assert normwise_rel_err(alone.cpu().numpy(), want) < TOL_F16_ACT
+
+
+def test_streaming_mfma_matmul_refusals(ops):
+    from cut_amd import lib
+    K, N = 512, 64
+    a = torch.zeros((33, K), dtype=torch.float16, device="cuda")
+    for fmt, rows in ((oracle.Q4_K, 33), (oracle.Q6_K, 8)):
+        w = torch.from_numpy(quantized_weights(fmt, N, K, seed=1)).cuda()
+        with pytest.raises(lib.CutHipError, match="variant 6"):
+            ops.matmul_gguf(a[:rows], w, fmt, N, K, variant=6)
+    w = torch.from_numpy(quantized_weights(oracle.Q4_K, 64, 14336, seed=2)).cuda()
+    with pytest.raises(lib.CutHipError, match="scratch"):       # K = 14336 is split over workgroups: workspace needed
+        ops.matmul_gguf(torch.zeros((8, 14336), dtype=torch.float16, device="cuda"), w, oracle.Q4_K, 64, 14336, variant=6)
+
+
 def test_rows8_refuses_what_does_not_fit_and_auto_falls_back(ops):
     from cut_amd import lib
     fmt = oracle.Q4_K
