@@ -323,6 +323,15 @@ __global__ void __launch_bounds__(256, 2) gemm_kernel(GemmParams p) {
   });
 }
 
+// K ranges per 128-row tile for a problem of 128 x 128 tiles with scratch_bytes of room for the partial products
+uint32_t tiled_gemm_ksplit(uint32_t M, uint32_t K, uint32_t N, size_t scratch_bytes) {
+  const uint64_t tiles = (uint64_t)((M + 127) / 128) * ((N + kBN - 1) / kBN);
+  const uint32_t nslices = (K + kBK - 1) / kBK;
+  uint32_t ks = 1;
+  while (ks < 16 && tiles * ks < 384 && nslices / (2 * ks) >= 8 && (uint64_t)2 * ks * M * N * 4 <= scratch_bytes) ks *= 2;
+  return ks;
+}
+
 template <int FMT, int BM, bool AF16> static int launch_gemm_bm(GemmParams p, hipStream_t stream) {
   p.mtiles = (p.M + BM - 1) / BM;
   p.ntiles = (p.N + kBN - 1) / kBN;
@@ -341,7 +350,7 @@ template <int FMT, int BM, bool AF16> static int launch_gemm_bm(GemmParams p, hi
   const uint32_t nslices = (p.K + kBK - 1) / kBK;
   uint32_t ks = 1;
   if (p.partial && BM == 128) {
-    while (ks < 16 && tiles * ks < 384 && nslices / (2 * ks) >= 8 && (uint64_t)2 * ks * p.M * p.N * 4 <= p.kper) ks *= 2;
+    ks = tiled_gemm_ksplit(p.M, p.K, p.N, p.kper);
     if (const char *env = getenv("CUT_HIP_GEMM_KSPLIT")) {   // tuning aid
       const uint32_t want = (uint32_t)atoi(env);
       if (want >= 1 && want <= 16 && (uint64_t)want * p.M * p.N * 4 <= p.kper) ks = want;

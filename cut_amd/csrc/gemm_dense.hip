@@ -688,9 +688,11 @@ size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
 //                 walk until every CU holds more than one 128 x 128 tile.
 // Measured against them (Q4_K, M x N x K): 64 x 4096 x 4096 38 / 62 us, 512 x 14336 x 4096 99 / 105, 512 x 28672 x 4096
 // 173 / 203, 256 x 28672 x 4096 147 / 107; Q6_K 64 x 14336 x 4096 79 / 104.
+//                 + 5 where the GEMM splits K (a third launch sums the partial products): 1024 x 1024 x 4096 36 us
 double dense_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
   const double nk = (double)N * K, bpw = (double)fmt_bytes(fmt) / fmt_elems(fmt);
-  return 3.0 + nk * (bpw + 2.0) / 6.0e6 + 17.0 + 2.0 * (double)((M + 127) / 128 * 128) * nk / 1.25e9;
+  const double split = pick_dense_shape(M, K, N).ksplit > 1 ? 5.0 : 0.0;
+  return 3.0 + nk * (bpw + 2.0) / 6.0e6 + 17.0 + 2.0 * (double)((M + 127) / 128 * 128) * nk / 1.25e9 + split;
 }
 double single_launch_rows_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
   const double c = fmt == CUTHIP_Q6_K ? 23.5e-3 : fmt == CUTHIP_Q8_0 ? 19.6e-3 : 14.7e-3;

@@ -115,6 +115,7 @@ double single_launch_rows_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N);
 int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K,
                       uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream,
                       int use_blaslt);
+uint32_t tiled_gemm_ksplit(uint32_t M, uint32_t K, uint32_t N, size_t scratch_bytes);
 bool stream_gemm_fits(int fmt, uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a_f16, const void *A);
 size_t stream_gemm_scratch(uint32_t M, uint32_t K, uint32_t N);
 int launch_stream_gemm(const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K, uint32_t N,
@@ -162,21 +163,24 @@ static double passes_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
   const double f = K >= 8192 ? (fmt == CUTHIP_Q6_K ? 1.55 : 1.45) : (fmt == CUTHIP_Q6_K ? 1.5 : 1.0);
   return ((M + 7) / 8) * (6.5 + weight_bytes(fmt, K, N) / 4.3e6) * f;
 }
-// The tiled GEMM with its K split over workgroups (scratch memory at hand, up to 256 rows): 9.5 us + the decode of the
-// matrix at 0.37 (Q4_K) to 0.64 (Q6_K) us per million weights per 128-row tile, + 0.07 us per row beyond 16
-// (14336 x 4096 Q4_K: 31 us at 16-64 rows, 38 at 128, 58 at 256; unsplit 65 at every M up to 128, 216 on K = 14336).
-static bool tiled_split_applies(uint32_t M, uint32_t N, const void *scratch, size_t scratch_bytes) {
-  return scratch && (uintptr_t)scratch % 16 == 0 && M > 8 && M <= 256 && scratch_bytes >= (size_t)4 * M * N * sizeof(float);
+// The tiled GEMM with its K split over workgroups (scratch memory at hand, so few 128 x 128 tiles that the launch rule
+// of gemm.hip splits): 9.5 us for the two launches + 0.66 us (Q4_K; Q6_K x 1.84, Q8_0 x 1.31) per slice of 64 that a
+// CU walks + the partial products written and read back at 6 MB/us.  14336 x 4096 Q4_K: 31 us at 32 rows, 38 at 128,
+// 62 at 256 (unsplit 65 at every M up to 128; 216 on K = 14336); 4096 x 1024: 19 at 256 rows, 20 at 512, 28 at 1024.
+static bool tiled_split_applies(uint32_t M, uint32_t K, uint32_t N, const void *scratch, size_t scratch_bytes) {
+  return scratch && (uintptr_t)scratch % 16 == 0 && M > 8 && cuthip::tiled_gemm_ksplit(M, K, N, scratch_bytes) > 1;
 }
-static double tiled_split_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
-  const double c = fmt == CUTHIP_Q6_K ? 0.644 : fmt == CUTHIP_Q8_0 ? 0.46 : fmt == CUTHIP_Q4_0 ? 0.40 : 0.372;
-  const uint32_t mt = (M + 127) / 128, rows = M < 128 ? M : 128;
-  return mt * (9.5 + c * 1e-6 * N * K) * (mt == 2 ? 0.93 : 1.0) + 0.07 * (rows > 16 ? rows - 16 : 0);
+static double tiled_split_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N, size_t scratch_bytes) {
+  const double f = fmt == CUTHIP_Q6_K ? 1.84 : fmt == CUTHIP_Q8_0 ? 1.31 : fmt == CUTHIP_Q4_0 ? 1.1 : 1.0;
+  const double tiles = (double)((M + 127) / 128) * ((N + 127) / 128), slices = (K + 63) / 64;
+  const uint32_t ks = cuthip::tiled_gemm_ksplit(M, K, N, scratch_bytes);
+  return 9.5 + 0.66 * f * tiles * slices / 256.0 + (double)ks * M * N * 8.0 / 6e6;
 }
-static double single_launch_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N, bool split) {
-  return split ? tiled_split_cost_us(fmt, M, K, N) : 62.0 + weight_bytes(fmt, K, N) / 7e6;
+// split: bytes of scratch the tiled GEMM may split K through, 0 = none (or the launch would not split)
+static double single_launch_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N, size_t split) {
+  return split ? tiled_split_cost_us(fmt, M, K, N, split) : 62.0 + weight_bytes(fmt, K, N) / 7e6;
 }
-static bool passes_preferred(int fmt, uint32_t M, uint32_t K, uint32_t N, bool split) {
+static bool passes_preferred(int fmt, uint32_t M, uint32_t K, uint32_t N, size_t split) {
   return M > 8 && M <= kPassesMaxRows &&
          ((K >= 8192 && !split) || passes_cost_us(fmt, M, K, N) <= single_launch_cost_us(fmt, M, K, N, split));
 }
@@ -288,7 +292,7 @@ static int matmul_gguf_scratch(int fmt, const void *W, const void *A, int a_dtyp
   // 9-40 rows, automatic choice: passes of 8 rows through the decode kernels.  Measured on 14336 x 4096: 14 us per
   // pass, against 69-87 us for the 32-row skinny kernel and 73-80 us for one launch of the tiled GEMM, whose cost
   // is the decode of the whole weight matrix whatever M is.
-  if (variant == -1 && passes_preferred(fmt, M, K, N, tiled_split_applies(M, N, scratch, scratch_bytes))) {
+  if (variant == -1 && passes_preferred(fmt, M, K, N, tiled_split_applies(M, K, N, scratch, scratch_bytes) ? scratch_bytes : 0)) {
     const size_t asz = a_dtype == CUTHIP_F16 ? 2 : 4, csz = c_dtype == CUTHIP_F16 ? 2 : 4;
     for (uint32_t m0 = 0; m0 < M; m0 += 8) {
       const uint8_t *a = reinterpret_cast<const uint8_t *>(A) + (size_t)m0 * strideA * asz;
@@ -549,10 +553,10 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
       blaslt_preferred()) {
     const double nk = (double)N * K;
     const double t5 = 14.0 + nk * (nk <= 64e6 ? 0.65e-6 : 0.95e-6) + 2.0 * M * nk / 1.6e9;
-    const bool split = tiled_split_applies(M, N, workspace, workspace_bytes);
+    const size_t split = tiled_split_applies(M, K, N, workspace, workspace_bytes) ? workspace_bytes : 0;
     double other;
     if (passes_preferred(fmt, M, K, N, split)) other = passes_cost_us(fmt, M, K, N);
-    else other = split ? tiled_split_cost_us(fmt, M, K, N) : K >= 8192 ? 65.0 + 0.19 * M : single_launch_cost_us(fmt, M, K, N, false);
+    else other = split ? tiled_split_cost_us(fmt, M, K, N, split) : K >= 8192 ? 65.0 + 0.19 * M : single_launch_cost_us(fmt, M, K, N, 0);
     if (t5 < 0.95 * other) {
       const int rc = launch_dense_gemm(fmt, W, A, a_f16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC,
                                        Epilogue{CUTHIP_EPI_NONE, 0, nullptr}, workspace,
@@ -566,12 +570,12 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   const bool fits = dense_gemm_fits(M, K, N, strideA, a_f16, A);
   const size_t need = dense_gemm_workspace(M, K, N, a_f16);
   const bool ws_ok = workspace && (uintptr_t)workspace % 256 == 0 && workspace_bytes >= need;
-  const bool split = tiled_split_applies(M, N, workspace, workspace_bytes);
+  const size_t split = tiled_split_applies(M, K, N, workspace, workspace ? workspace_bytes : 0) ? workspace_bytes : 0;
   bool dense_first = false;
   if (variant == -1 && M > 8 && fits && ws_ok) {
     const double t4 = dense_cost_us(fmt, M, K, N);
-    const double tiled = split ? tiled_split_cost_us(fmt, M, K, N) : single_launch_rows_cost_us(fmt, M, K, N);
-    dense_first = M >= 1024 || (passes_preferred(fmt, M, K, N, split) ? t4 < 0.9 * passes_cost_us(fmt, M, K, N) : t4 < 0.95 * tiled);
+    const double tiled = split ? tiled_split_cost_us(fmt, M, K, N, split) : single_launch_rows_cost_us(fmt, M, K, N);
+    dense_first = (M >= 1024 && !split) || (passes_preferred(fmt, M, K, N, split) ? t4 < 0.9 * passes_cost_us(fmt, M, K, N) : t4 < 0.95 * tiled);
   }
   if (variant == -1 && !dense_first && passes_preferred(fmt, M, K, N, split)) {   // 8-row passes, each with the workspace (K split on long rows)
     const size_t asz = a_f16 ? 2 : 4, csz = c_dtype == CUTHIP_F16 ? 2 : 4;
