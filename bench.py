@@ -432,6 +432,25 @@ def main():
         for b in (2, 4, 8):
             wall_b, ev_b, _ = timed_graph(torch, ffn_step(b), 120, 12)
             extras[f"q4k_ffn_gemv_batch{b}_GBps"] = round(ffn_bytes(b) * 120 / wall_b / 1e9, 1)
+        # 16-128 rows (batched decode, short prefill chunks): the same three matmuls through cuthip_matmul_gguf_ws,
+        # whose workspace lets the streaming MFMA kernel and the tiled GEMM split K; GB/s over the same bytes
+        xb = torch.from_numpy(rng.standard_normal((128, N_EMBD), dtype=np.float32).astype(np.float16)).to(dev)
+        hb = torch.from_numpy(rng.standard_normal((128, N_FF), dtype=np.float32).astype(np.float16)).to(dev)
+        yb_ff = torch.empty((128, N_FF), dtype=torch.float16, device=dev)
+        yb_em = torch.empty((128, N_EMBD), dtype=torch.float16, device=dev)
+        for b in (16, 32, 64, 128):
+            ws_b = ops.matmul_gguf_workspace("Q4_K", b, N_FF, N_EMBD, torch.float16, dev)
+
+            def mid_step(s, b=b, ws_b=ws_b):
+                i = s % COPIES
+                ops.matmul_gguf(xb[:b], gate[i], "Q4_K", N_FF, N_EMBD, out=yb_ff[:b], workspace=ws_b)
+                ops.matmul_gguf(xb[:b], up[i], "Q4_K", N_FF, N_EMBD, out=yb_ff[:b], workspace=ws_b)
+                ops.matmul_gguf(hb[:b], down[i], "Q4_K", N_EMBD, N_FF, out=yb_em[:b], workspace=ws_b)
+            wall_b, ev_b, _ = timed_graph(torch, mid_step, 60, 6)
+            extras[f"q4k_ffn_matmul_batch{b}_GBps"] = round(ffn_bytes(b) * 60 / wall_b / 1e9, 1)
+            extras[f"q4k_ffn_matmul_batch{b}_us_per_matmul"] = round(wall_b * 1e6 / 180, 1)
+            del ws_b
+        del xb, hb, yb_ff, yb_em
         # gate and up as one launch (rows concatenated, the reference's fused w_gate_up: llama.cpp:1288-1330)
         gate_up = [torch.cat([gate[i], up[i]]) for i in range(COPIES)]
         y_gu = torch.empty((1, 2 * N_FF), dtype=torch.float16, device=dev)
