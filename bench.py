@@ -292,6 +292,8 @@ def main():
     ap.add_argument("--prepare-only", action="store_true", help="only run the load-time preparation kernels")
     ap.add_argument("--q8-only", action="store_true",
                     help="only run the Q8_0 prefill GEMMs at M = 2048 (int8-activation variant and fp16 path)")
+    ap.add_argument("--matmul-batch-only", type=int, default=0, metavar="B",
+                    help="only run the FFN step at B rows (9..256) through the workspace entry point, for profiling")
     ap.add_argument("--gemv-batch-only", type=int, default=0, metavar="B",
                     help="only run the FFN GEMV step at batch B (2..8), for profiling")
     ap.add_argument("--decode-only", action="store_true",
@@ -388,6 +390,28 @@ def main():
     def ffn_bytes(b):
         return 3 * w_bytes + b * 2 * (2 * (N_EMBD + N_FF) + (N_FF + N_EMBD))
 
+    def ffn_step_ws(b):
+        # 9 rows and more: the three matmuls through cuthip_matmul_gguf_ws, whose workspace lets the streaming MFMA
+        # kernel and the tiled GEMM split K
+        xb = torch.from_numpy(rng.standard_normal((b, N_EMBD), dtype=np.float32).astype(np.float16)).to(dev)
+        hb = torch.from_numpy(rng.standard_normal((b, N_FF), dtype=np.float32).astype(np.float16)).to(dev)
+        yb_ff = torch.empty((b, N_FF), dtype=torch.float16, device=dev)
+        yb_em = torch.empty((b, N_EMBD), dtype=torch.float16, device=dev)
+        ws_b = ops.matmul_gguf_workspace("Q4_K", b, N_FF, N_EMBD, torch.float16, dev)
+
+        def step(s):
+            i = s % COPIES
+            ops.matmul_gguf(xb, gate[i], "Q4_K", N_FF, N_EMBD, out=yb_ff, workspace=ws_b)
+            ops.matmul_gguf(xb, up[i], "Q4_K", N_FF, N_EMBD, out=yb_ff, workspace=ws_b)
+            ops.matmul_gguf(hb, down[i], "Q4_K", N_EMBD, N_FF, out=yb_em, workspace=ws_b)
+        return step
+
+    if args.matmul_batch_only:
+        b = args.matmul_batch_only
+        wall_b, ev_b, _ = timed_graph(torch, ffn_step_ws(b), 60, 6)
+        print(json.dumps({f"q4k_ffn_matmul_batch{b}_GBps": round(ffn_bytes(b) * 60 / wall_b / 1e9, 1),
+                          "us_per_matmul": round(ev_b * 1e3 / 180, 2)}))
+        return
     if args.gemv_batch_only:
         b = args.gemv_batch_only
         wall_b, ev_b, _ = timed_graph(torch, ffn_step(b), 120, 12)
@@ -432,25 +456,12 @@ def main():
         for b in (2, 4, 8):
             wall_b, ev_b, _ = timed_graph(torch, ffn_step(b), 120, 12)
             extras[f"q4k_ffn_gemv_batch{b}_GBps"] = round(ffn_bytes(b) * 120 / wall_b / 1e9, 1)
-        # 16-128 rows (batched decode, short prefill chunks): the same three matmuls through cuthip_matmul_gguf_ws,
-        # whose workspace lets the streaming MFMA kernel and the tiled GEMM split K; GB/s over the same bytes
-        xb = torch.from_numpy(rng.standard_normal((128, N_EMBD), dtype=np.float32).astype(np.float16)).to(dev)
-        hb = torch.from_numpy(rng.standard_normal((128, N_FF), dtype=np.float32).astype(np.float16)).to(dev)
-        yb_ff = torch.empty((128, N_FF), dtype=torch.float16, device=dev)
-        yb_em = torch.empty((128, N_EMBD), dtype=torch.float16, device=dev)
+        # 16-128 rows (batched decode, short prefill chunks): the same three matmuls through cuthip_matmul_gguf_ws;
+        # GB/s over the same bytes
         for b in (16, 32, 64, 128):
-            ws_b = ops.matmul_gguf_workspace("Q4_K", b, N_FF, N_EMBD, torch.float16, dev)
-
-            def mid_step(s, b=b, ws_b=ws_b):
-                i = s % COPIES
-                ops.matmul_gguf(xb[:b], gate[i], "Q4_K", N_FF, N_EMBD, out=yb_ff[:b], workspace=ws_b)
-                ops.matmul_gguf(xb[:b], up[i], "Q4_K", N_FF, N_EMBD, out=yb_ff[:b], workspace=ws_b)
-                ops.matmul_gguf(hb[:b], down[i], "Q4_K", N_EMBD, N_FF, out=yb_em[:b], workspace=ws_b)
-            wall_b, ev_b, _ = timed_graph(torch, mid_step, 60, 6)
+            wall_b, ev_b, _ = timed_graph(torch, ffn_step_ws(b), 60, 6)
             extras[f"q4k_ffn_matmul_batch{b}_GBps"] = round(ffn_bytes(b) * 60 / wall_b / 1e9, 1)
             extras[f"q4k_ffn_matmul_batch{b}_us_per_matmul"] = round(wall_b * 1e6 / 180, 1)
-            del ws_b
-        del xb, hb, yb_ff, yb_em
         # gate and up as one launch (rows concatenated, the reference's fused w_gate_up: llama.cpp:1288-1330)
         gate_up = [torch.cat([gate[i], up[i]]) for i in range(COPIES)]
         y_gu = torch.empty((1, 2 * N_FF), dtype=torch.float16, device=dev)
