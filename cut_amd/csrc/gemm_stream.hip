@@ -22,7 +22,7 @@
 // keeps kStreamDepth steps of weight loads in flight in a register ring and waits only for the step it multiplies.
 //
 // Measured (MI355X, HIP-graph replay, Q4_K 14336 x 4096): 15.8 us at 9-16 rows (two passes of the 8-row GEMV: 25),
-// 26 us at 17-32 rows (tiled GEMM with K split: 30); at 8 rows and fewer the 8-row GEMV is the faster one (13 us):
+// 21 us at 17-32 rows (tiled GEMM with K split: 30); at 8 rows and fewer the 8-row GEMV is the faster one (13 us):
 // both spend about 0.05 vector instructions per weight on the unpack, which bounds them well before HBM does.
 #include <type_traits>
 
@@ -40,7 +40,7 @@ struct StreamParams {
   Epilogue epi;
   uint32_t M, K, N, strideA, strideC, row_bytes;
   int a_f16, c_f16;
-  uint32_t nblocks;       // workgroups along N (64 weight rows each)
+  uint32_t nblocks;       // workgroups along N (16 RG weight rows each)
   uint32_t range_steps;   // 256-element steps per K range
   uint32_t ksplit;
   float *partial;         // [ksplit][M][N] when ksplit > 1
@@ -59,21 +59,22 @@ __device__ __forceinline__ half8_t as_frag(uint32_t a, uint32_t b, uint32_t c, u
   return __builtin_bit_cast(half8_t, u32x4{a, b, c, d});
 }
 
-// MT: activation tiles of 16 rows (1 or 2); KW: waves that share 16 weight rows, each on its own part of the steps
-// (two waves per SIMD: one wave alone cannot hide its own LDS and matrix-core latencies)
-template <int MT, int KW>
-__global__ void __launch_bounds__(256 * KW) gemm_stream_q4k_kernel(StreamParams p) {
+// MT: activation tiles of 16 rows (1 or 2); RG: groups of 16 weight rows per workgroup; KW: waves that share a group,
+// each on its own part of the steps.  RG x KW = 8 waves wherever the range is long enough (two waves per SIMD: one
+// wave alone cannot hide its own LDS and matrix-core latencies).
+template <int MT, int KW, int RG>
+__global__ void __launch_bounds__(64 * RG * KW) gemm_stream_q4k_kernel(StreamParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  constexpr int D = kStreamDepth, THREADS = 256 * KW;
+  constexpr int D = kStreamDepth, THREADS = 64 * RG * KW;
   const uint32_t split = blockIdx.x / p.nblocks, bid = blockIdx.x - split * p.nblocks;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, rg = wave & 3, kw = wave >> 2;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, rg = wave % RG, kw = wave / RG;
   const uint32_t s_lo = split * p.range_steps, nsteps = p.K / 256;
   const uint32_t rcnt = min(p.range_steps, nsteps - s_lo);   // steps of this workgroup; the host launches no empty range
   const uint32_t range_k = rcnt * 256, pitch = range_k * 2 + 16;   // bytes per staged activation row
   const uint32_t strip0 = 16 * MT * (p.range_steps * 512 + 16);     // the weight strips lie behind the activations
   const uint32_t sb = rcnt * kw / KW, cnt = rcnt * (kw + 1) / KW - sb;   // this wave's steps: [sb, sb + cnt) of the range
 
-  const uint32_t n = (bid * 4 + rg) * 16 + (lane & 15), kq = lane >> 4;
+  const uint32_t n = (bid * RG + rg) * 16 + (lane & 15), kq = lane >> 4;
 
   // The 16 blocks of a step (16 rows x 144 bytes) are fetched as 144 pieces of 16 bytes, piece c = row c / 9, part
   // c % 9, by lanes c, c - 64, c - 128: neighbouring lanes read neighbouring bytes, every cache line is requested
@@ -84,7 +85,7 @@ __global__ void __launch_bounds__(256 * KW) gemm_stream_q4k_kernel(StreamParams 
 #pragma unroll
   for (int j = 0; j < 3; ++j) {
     const uint32_t c = min((uint32_t)lane + 64u * j, 143u), r = c / 9, part = c - 9 * r;
-    piece[j] = p.W + (size_t)min((bid * 4 + rg) * 16 + r, p.N - 1) * p.row_bytes + (size_t)(s_lo + sb) * 144 + 16 * part;
+    piece[j] = p.W + (size_t)min((bid * RG + rg) * 16 + r, p.N - 1) * p.row_bytes + (size_t)(s_lo + sb) * 144 + 16 * part;
   }
   struct Raw { u32x4 c[3]; };
   auto load = [&](Raw &r, uint32_t step) __attribute__((always_inline)) {
@@ -230,8 +231,8 @@ __global__ void __launch_bounds__(256 * KW) gemm_stream_q4k_kernel(StreamParams 
   // the K parts of a row group meet in LDS (the staged activations are no longer needed)
   if constexpr (KW > 1) {
     __syncthreads();
-    // [KW - 1][4 row groups][MT * 4 registers][64 lanes]
-    float *red = reinterpret_cast<float *>(lds) + ((size_t)(kw > 0 ? kw - 1 : 0) * 4 + rg) * 64 * MT * 4 + lane;
+    // [KW - 1][RG row groups][MT * 4 registers][64 lanes]
+    float *red = reinterpret_cast<float *>(lds) + ((size_t)(kw > 0 ? kw - 1 : 0) * RG + rg) * 64 * MT * 4 + lane;
     if (kw > 0) {
 #pragma unroll
       for (int t = 0; t < MT; ++t)
@@ -245,7 +246,7 @@ __global__ void __launch_bounds__(256 * KW) gemm_stream_q4k_kernel(StreamParams 
 #pragma unroll
       for (int t = 0; t < MT; ++t)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[t][e] += red[((size_t)(w - 1) * 4 * 64 * MT * 4) + (t * 4 + e) * 64];
+        for (int e = 0; e < 4; ++e) acc[t][e] += red[((size_t)(w - 1) * RG * 64 * MT * 4) + (t * 4 + e) * 64];
   }
   // accumulator register e of lane l, tile t: row 16 t + 4 (l >> 4) + e, column (weight row) n
   if (n < p.N) {
@@ -265,8 +266,16 @@ __global__ void __launch_bounds__(256 * KW) gemm_stream_q4k_kernel(StreamParams 
 // K ranges of the streaming kernel: as few as LDS allows (one range of up to kStreamLdsMax bytes of staged
 // activations), more while the grid has fewer workgroups than CUs and a range keeps at least 8 steps
 // (and the scratch memory holds the partial products of twice as many)
+// Weight rows per workgroup: 64 (four row groups, two waves each), or with two activation tiles 128 (eight row groups
+// of one wave: half as many workgroups stage the activations; 14336 x 4096 at 32 rows 21 us against 26) wherever that
+// still leaves a workgroup for every second CU (4096 x 4096: 18 us against 14 otherwise)
+static uint32_t stream_block_rows(uint32_t M, uint32_t K, uint32_t N) {
+  if (M <= 16) return 64;
+  const uint32_t ks_lds = (K / 256 + 7) / 8;   // ranges of at most eight steps with 32 staged rows
+  return (N + 127) / 128 * ks_lds >= 128 ? 128 : 64;
+}
 static void stream_layout(uint32_t M, uint32_t K, uint32_t N, size_t scratch_bytes, uint32_t *range_steps, uint32_t *ksplit) {
-  const uint32_t mt = (M + 15) / 16, nsteps = K / 256, nblocks = (N + 63) / 64;
+  const uint32_t mt = (M + 15) / 16, nsteps = K / 256, nblocks = (N + stream_block_rows(M, K, N) - 1) / stream_block_rows(M, K, N);
   const uint32_t max_steps = (kStreamLdsMax / (16 * mt) - 16) / 512;
   uint32_t ks = (nsteps + max_steps - 1) / max_steps;
   while (ks < 16 && nblocks * ks < 192 && nsteps / (2 * ks) >= 8 && scratch_bytes >= (size_t)2 * ks * M * N * sizeof(float)) ks *= 2;
@@ -296,7 +305,8 @@ int launch_stream_gemm(const void *W, const void *A, int a_f16, void *C, int c_f
   p.M = M; p.K = K; p.N = N; p.strideA = strideA; p.strideC = strideC;
   p.row_bytes = K / 256 * 144;
   p.a_f16 = a_f16; p.c_f16 = c_f16;
-  p.nblocks = (N + 63) / 64;
+  const uint32_t block_rows = stream_block_rows(M, K, N);
+  p.nblocks = (N + block_rows - 1) / block_rows;
   if (!scratch || (uintptr_t)scratch % 16 != 0) scratch_bytes = 0;
   stream_layout(M, K, N, scratch_bytes, &p.range_steps, &p.ksplit);
   p.partial = reinterpret_cast<float *>(scratch);
@@ -307,16 +317,19 @@ int launch_stream_gemm(const void *W, const void *A, int a_f16, void *C, int c_f
   }
   const uint32_t mt = (M + 15) / 16;
   const size_t lds = (size_t)16 * mt * ((size_t)p.range_steps * 512 + 16) + 8 * kStripBytes;
-  const bool two = p.range_steps >= 4;   // two waves per row group once each keeps at least two steps
-  auto kern = mt == 1 ? (two ? gemm_stream_q4k_kernel<1, 2> : gemm_stream_q4k_kernel<1, 1>)
-                      : (two ? gemm_stream_q4k_kernel<2, 2> : gemm_stream_q4k_kernel<2, 1>);
+  // four row groups: two waves each once a wave keeps at least two steps
+  const bool two = block_rows == 64 && p.range_steps >= 4;
+  auto kern = block_rows == 128 ? gemm_stream_q4k_kernel<2, 1, 8>
+              : mt == 1 ? (two ? gemm_stream_q4k_kernel<1, 2, 4> : gemm_stream_q4k_kernel<1, 1, 4>)
+                        : (two ? gemm_stream_q4k_kernel<2, 2, 4> : gemm_stream_q4k_kernel<2, 1, 4>);
+  const uint32_t threads = block_rows == 128 || two ? 512 : 256;
   if (lds > 64 * 1024) {
     if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                                (int)lds),
                            "hipFuncSetAttribute"))
       return rc;
   }
-  hipLaunchKernelGGL(kern, dim3(p.nblocks * p.ksplit), dim3(two ? 512 : 256), lds, stream, p);
+  hipLaunchKernelGGL(kern, dim3(p.nblocks * p.ksplit), dim3(threads), lds, stream, p);
   if (int rc = check_hip(hipGetLastError(), "streaming matmul launch")) return rc;
   if (p.ksplit == 1) return CUTHIP_OK;
   return launch_splitk_reduce(p.partial, p.ksplit, M, N, C, strideC, epi, c_f16, stream);

@@ -277,7 +277,7 @@ static int matmul_gguf_scratch(int fmt, const void *W, const void *A, int a_dtyp
   // the table's default entry is valid for every M: beyond the 8 rows its GEMV takes it is the choice by shape
   if (variant == 0 && M > 8) variant = -1;
   // 9-32 rows on Q4_K: the streaming MFMA kernel (9-16 rows of 14336 x 4096: 15.8 us against 25 for two 8-row
-  // passes; 17-32 rows: 26 us against 30 for the tiled GEMM with K split), wherever the scratch memory it needs
+  // passes; 17-32 rows: 21 us against 30 for the tiled GEMM with K split), wherever the scratch memory it needs
   // for long rows or two activation tiles is at hand
   if (variant == -1 && stream_preferred(fmt, M, K, N, strideA, a_dtype == CUTHIP_F16, A, scratch, scratch_bytes)) variant = 6;
   // variant 6: the streaming MFMA kernel (Q4_K, up to 32 rows); scratch only where K has to be split over workgroups
