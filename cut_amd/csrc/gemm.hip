@@ -3,7 +3,7 @@
 //
 // Supersedes MatMulQ{4,8}CoopMatTiled.cu (operators/impl/matmul): 32x32x16
 // tiles with one 16x16x16 MMA per warp between two barriers.  Here a workgroup
-// of four waves owns a BM x 128 tile of C (BM = 256 or 128), each wave a
+// of four waves owns a BM x 128 tile of C (BM = 256, 128 or - up to 64 rows of A - 64), each wave a
 // (BM/2) x 64 sub-tile held in fp32 accumulators, and walks K in slices of 64.
 // Per slice the workgroup
 //   * copies the A slice to LDS as fp16 (fp32 activations are rounded once),
@@ -293,7 +293,7 @@ __global__ void __launch_bounds__(256, 2) gemm_kernel(GemmParams p) {
 
   // C tile through LDS, a 32-row stripe of the wave's sub-tile at a time (gemm_store.hpp); the operand tiles are free
   // once every wave has multiplied the last slice
-  static_assert(4 * stripe_floats<2>() * 4 <= (BM + kBN) * kLdsRow * 2, "the output staging reuses the operand tiles");
+  // the output staging reuses the operand tiles (the launch asks for the larger of the two)
   __syncthreads();
   lds_f32 *stage = (lds_f32 *)(lds_u8g *)(lds) + wave * stripe_floats<2>();
   Epilogue epi = p.epi;
@@ -336,6 +336,7 @@ template <int FMT, int BM, bool AF16> static int launch_gemm_bm(GemmParams p, hi
   p.mtiles = (p.M + BM - 1) / BM;
   p.ntiles = (p.N + kBN - 1) / kBN;
   size_t lds = (size_t)(BM + kBN) * kLdsRow * 2;
+  if (lds < 4 * stripe_floats<2>() * 4) lds = 4 * stripe_floats<2>() * 4;
   auto kern = gemm_kernel<FMT, BM, AF16>;
   if (lds > 64 * 1024) {
     if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -349,7 +350,7 @@ template <int FMT, int BM, bool AF16> static int launch_gemm_bm(GemmParams p, hi
   const uint64_t tiles = (uint64_t)p.mtiles * p.ntiles;
   const uint32_t nslices = (p.K + kBK - 1) / kBK;
   uint32_t ks = 1;
-  if (p.partial && BM == 128) {
+  if (p.partial && BM <= 128) {
     ks = tiled_gemm_ksplit(p.M, p.K, p.N, p.kper);
     if (const char *env = getenv("CUT_HIP_GEMM_KSPLIT")) {   // tuning aid
       const uint32_t want = (uint32_t)atoi(env);
@@ -374,11 +375,13 @@ template <int FMT, int BM, bool AF16> static int launch_gemm_bm(GemmParams p, hi
 template <int FMT> static int launch_gemm_fmt(const GemmParams &p, hipStream_t stream) {
   // 256-row tiles once they fill the chip (>= 2 workgroups per CU), else 128-row tiles.
   // fp32 activations and Q6_K need more staging registers and always take 128 rows.
-  if (!p.a_f16) return launch_gemm_bm<FMT, 128, false>(p, stream);
+  if (!p.a_f16) return p.M <= 64 ? launch_gemm_bm<FMT, 64, false>(p, stream) : launch_gemm_bm<FMT, 128, false>(p, stream);
   uint64_t tiles256 = (uint64_t)((p.M + 255) / 256) * ((p.N + kBN - 1) / kBN);
   if constexpr (FMT != CUTHIP_Q6_K) {
     if (tiles256 >= 512) return launch_gemm_bm<FMT, 256, true>(p, stream);
   }
+  // up to 64 rows: 64-row tiles, half the matrix-core work per slice (14336 x 4096 at 33-64 rows 28-29 us against 33-34)
+  if (p.M <= 64) return launch_gemm_bm<FMT, 64, true>(p, stream);
   return launch_gemm_bm<FMT, 128, true>(p, stream);
 }
 
