@@ -85,6 +85,32 @@ def test_q4k_ffn_shapes_fp16_io(ops, N, K, M):
         assert np.all(np.abs(one[0] - got[0]) <= np.abs(got[0]) * 2.0 ** -10 + 1e-4 * rms)
 
 
+@pytest.mark.parametrize("M", [16, 32, 64, 128])
+@pytest.mark.parametrize("N,K", [(14336, 4096), (4096, 14336)])
+def test_q4k_ffn_shapes_at_9_to_128_rows(ops, N, K, M):
+    """The FFN shapes at the row counts between the GEMV and prefill, through the workspace entry point with the
+    library's own choice (streaming MFMA kernel up to 32 rows, tiled GEMM with K split over workgroups beyond): fp32
+    output against the float64 oracle on a sample of weight rows, and batch rows are independent: rows 0 and M - 1
+    of the call agree with the same rows computed alone by the GEMV."""
+    fmt = oracle.Q4_K
+    W = quantized_weights(fmt, N, K, seed=0)
+    A = gauss_acts((M, K), seed=M, dtype=np.float16)
+    a, w = torch.from_numpy(A).cuda(), torch.from_numpy(W).cuda()
+    ws = ops.matmul_gguf_workspace(fmt, M, K, N, a.dtype, "cuda")
+    ws.fill_(0xFF)
+    got = ops.matmul_gguf(a, w, fmt, N, K, out_dtype=torch.float32, workspace=ws)
+    torch.cuda.synchronize()
+    got = got.cpu().numpy()
+    rows = np.unique(np.concatenate([np.arange(0, 64), np.arange(N - 64, N), np.random.default_rng(0).integers(0, N, 384)]))
+    Ws = W.reshape(N, oracle.n_bytes(fmt, K))[rows].reshape(-1)
+    want = oracle.matmul_gguf(fmt, Ws, A.astype(np.float32), len(rows), f64=True)
+    assert normwise_rel_err(got[:, rows], want) < (TOL_F16_ACT if M <= 32 else 5e-4)   # exact products / fp16-decoded weights
+    for r in (0, M - 1):
+        one = ops.matmul_gguf(a[r:r + 1], w, fmt, N, K, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        assert normwise_rel_err(got[r:r + 1], one.cpu().numpy()) < (TOL_F16_ACT if M <= 32 else 5e-4)
+
+
 def test_linearity_and_row_permutation(ops):
     fmt = oracle.Q4_K
     N, K = 4096, 4096
