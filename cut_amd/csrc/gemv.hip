@@ -165,8 +165,9 @@ static double passes_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
 }
 // The tiled GEMM with its K split over workgroups (scratch memory at hand, so few 128 x 128 tiles that the launch rule
 // of gemm.hip splits): 9.5 us for the two launches + 0.66 us (Q4_K; Q6_K x 1.84, Q8_0 x 1.31) per slice of 64 that a
-// CU walks + the partial products written and read back at 6 MB/us.  14336 x 4096 Q4_K: 31 us at 32 rows, 38 at 128,
-// 62 at 256 (unsplit 65 at every M up to 128; 216 on K = 14336); 4096 x 1024: 19 at 256 rows, 20 at 512, 28 at 1024.
+// CU walks (x 0.85 with the 64-row tiles of up to 64 rows) + the partial products written and read back at 6 MB/us.
+// 14336 x 4096 Q4_K: 27 us at 32 rows, 29 at 64, 38 at 128, 62 at 256 (unsplit 65 at every M up to 128; 216 on
+// K = 14336); 4096 x 1024: 19 at 256 rows, 20 at 512, 28 at 1024.
 static bool tiled_split_applies(uint32_t M, uint32_t K, uint32_t N, const void *scratch, size_t scratch_bytes) {
   return scratch && (uintptr_t)scratch % 16 == 0 && M > 8 && cuthip::tiled_gemm_ksplit(M, K, N, scratch_bytes) > 1;
 }
