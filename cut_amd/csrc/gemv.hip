@@ -168,8 +168,11 @@ static double passes_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
 // CU walks (x 0.85 with the 64-row tiles of up to 64 rows) + the partial products written and read back at 6 MB/us.
 // 14336 x 4096 Q4_K: 27 us at 32 rows, 29 at 64, 38 at 128, 62 at 256 (unsplit 65 at every M up to 128; 216 on
 // K = 14336); 4096 x 1024: 19 at 256 rows, 20 at 512, 28 at 1024.
+// Beyond 256 rows only for matrices of fewer than 32 M weights: on 4096 x 14336 at 512 rows the model says 89 us and
+// the launch takes 102, against 93 for the two-pass path.
 static bool tiled_split_applies(uint32_t M, uint32_t K, uint32_t N, const void *scratch, size_t scratch_bytes) {
-  return scratch && (uintptr_t)scratch % 16 == 0 && M > 8 && cuthip::tiled_gemm_ksplit(M, K, N, scratch_bytes) > 1;
+  return scratch && (uintptr_t)scratch % 16 == 0 && M > 8 && (M <= 256 || (uint64_t)N * K < 32000000ull) &&
+         cuthip::tiled_gemm_ksplit(M, K, N, scratch_bytes) > 1;
 }
 static double tiled_split_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N, size_t scratch_bytes) {
   const double f = fmt == CUTHIP_Q6_K ? 1.84 : fmt == CUTHIP_Q8_0 ? 1.31 : fmt == CUTHIP_Q4_0 ? 1.1 : 1.0;
