@@ -24,6 +24,7 @@ def main():
     ap.add_argument("--output", default=os.path.join(os.path.dirname(os.path.abspath(__file__)), "tuning_data.json"))
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--formats", default=",".join(FORMATS))
+    ap.add_argument("--batches", default=",".join(str(b) for b in BATCHES), help="rows of activations to sweep (comma separated)")
     ap.add_argument("--measurements", default=None, help="also write every timing of the sweep to this JSON file")
     ap.add_argument("--with-vendor", action="store_true",
                     help="let rules name the dequantize + hipBLASLt variant too (it is timed and logged either way)")
@@ -43,7 +44,7 @@ def main():
             tile = Q.quantize(fmt, np.random.default_rng(0).standard_normal(1024 * K, dtype=np.float32) * np.float32(0.02))
             w = torch.from_numpy(tile).to(dev).repeat(N // 1024)
             copies = [w.clone() for _ in range(max(2, min(8, int(3e8 // w.numel()))))]
-            for M in BATCHES:
+            for M in [int(b) for b in args.batches.split(",")]:
                 a = torch.randn((M, K), dtype=torch.float16, device=dev)
                 c = torch.empty((M, N), dtype=torch.float16, device=dev)
                 ws = ops.matmul_gguf_workspace(fmt, M, K, N, a.dtype, dev)

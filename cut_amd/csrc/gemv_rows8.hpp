@@ -43,6 +43,13 @@ namespace cuthip {
 #define CUTHIP_ROWS8_DOTMAX 1
 #endif
 constexpr int kRows8DotMax = CUTHIP_ROWS8_DOTMAX;   // batch rows up to which the dot-product path is taken
+// Q6_K keeps the dot-product path up to four rows: its matrix-core path pays 16 sub-block scalings of every
+// accumulator per step (14336 x 4096 at 2 / 4 rows: 15.1 / 18.0 us against 18.9 / 20.2; Q4_K and Q8_0 at 2 rows are
+// faster through the matrix core: 9.4 against 11.3 us, 17.0 against 17.3)
+#ifndef CUTHIP_ROWS8_DOTMAX_Q6K
+#define CUTHIP_ROWS8_DOTMAX_Q6K 4
+#endif
+template <int FMT> constexpr int rows8_dot_max() { return FMT == CUTHIP_Q6_K ? CUTHIP_ROWS8_DOTMAX_Q6K : kRows8DotMax; }
 constexpr int kXGroup = 72;             // halfs per staged 64-element group (64 + 8 pad)
 constexpr int kXStep = 4 * kXGroup;     // halfs per 256-element step
 
@@ -527,7 +534,7 @@ template <int SUBK, int THREADS, int MT, int XR, bool PRO> struct XStage {
 template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO>
 __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t bid) {
   using S = Rows8<FMT>;
-  constexpr bool DOT = MT <= kRows8DotMax;
+  constexpr bool DOT = MT <= rows8_dot_max<FMT>();
   constexpr int WAVES = RWG * KW, THREADS = 64 * WAVES;
   // accumulators: dot path one per batch row; matrix-core path rows 4m + g of C, RQ quads of four pieces
   constexpr int R = DOT ? MT : 2 * MT, RQ = DOT ? MT : R / 4;
