@@ -377,8 +377,8 @@ def main():
     w_bytes = ops.n_bytes("Q4_K", N_FF, N_EMBD)  # 33,030,144 for either shape
 
     def ffn_step(b):
-        # batch 3-8: with a workspace the long-row down projection splits K across workgroups
-        ws_down = ops.matmul_gguf_workspace("Q4_K", b, N_FF, N_EMBD, torch.float16, dev) if b > 2 else None
+        # batch 2-8: with a workspace the long-row down projection splits K across workgroups
+        ws_down = ops.matmul_gguf_workspace("Q4_K", b, N_FF, N_EMBD, torch.float16, dev) if b >= 2 else None
 
         def step(s):
             i = s % COPIES

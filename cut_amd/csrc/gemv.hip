@@ -56,10 +56,10 @@ int launch_splitk_reduce(const float *partial, uint32_t ksplit, uint32_t M, uint
 
 // The split across workgroups pays where one row group per workgroup would re-stage long activations for few rows:
 // batch 2-8, rows of at least 32 steps, and not enough row groups to fill the chip without splitting K.
-static bool ksplit_gemv_preferred(uint32_t M, uint32_t K, uint32_t N) {
-  // from 3 batch rows on (two rows of K = 14336 still fit the LDS budget of the unsplit kernel, which then measures
-  // faster: 13.3 us against 16 us for 4096 x 14336)
-  return M >= 3 && M <= 8 && K >= 8192 && (N + 7) / 8 < 1536;
+static bool ksplit_gemv_preferred(int fmt, uint32_t M, uint32_t K, uint32_t N) {
+  // from 2 batch rows on (4096 x 14336 at two rows: Q4_K 11.6 us against 12.6 unsplit, Q8_0 18.2 against 19.6); Q6_K
+  // from 3: its two rows run the dot-product path, unsplit 17.4 us against 18.2
+  return M >= (fmt == CUTHIP_Q6_K ? 3u : 2u) && M <= 8 && K >= 8192 && (N + 7) / 8 < 1536;
 }
 static size_t ksplit_gemv_workspace(uint32_t M, uint32_t K, uint32_t N) {
   return (size_t)rows8_ksplit_parts(N, (K + 255) / 256) * M * N * sizeof(float);
@@ -524,7 +524,7 @@ int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, in
 
 size_t cuthip_matmul_gguf_workspace_bytes(int fmt, uint32_t M, uint32_t K, uint32_t N, int a_dtype) {
   (void)fmt;
-  if (cuthip::ksplit_gemv_preferred(M, K, N)) return cuthip::ksplit_gemv_workspace(M, K, N);
+  if (cuthip::ksplit_gemv_preferred(fmt, M, K, N)) return cuthip::ksplit_gemv_workspace(M, K, N);
   return cuthip::dense_gemm_workspace(M, K, N, a_dtype == CUTHIP_F16);
 }
 
@@ -596,7 +596,7 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
     return CUTHIP_OK;
   }
   // batch 3-8 on long rows: the 8-row GEMV with K split across workgroups, partial products in the workspace
-  if (variant == -1 && !dense_first && ksplit_gemv_preferred(M, K, N) && workspace && (uintptr_t)workspace % 16 == 0 &&
+  if (variant == -1 && !dense_first && ksplit_gemv_preferred(fmt, M, K, N) && workspace && (uintptr_t)workspace % 16 == 0 &&
       workspace_bytes >= ksplit_gemv_workspace(M, K, N) && (uintptr_t)A % 16 == 0 && (strideA * (a_f16 ? 2 : 4)) % 16 == 0) {
     const GemvParams p = gemv_params(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC,
                                      Epilogue{CUTHIP_EPI_NONE, 0, nullptr});

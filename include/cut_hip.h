@@ -245,7 +245,7 @@ int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void 
  *            order of the fp32 sums); K above 4096 (2048 beyond 16 rows) is split over
  *            workgroups through the workspace, an error without one.  With variant -1
  *            it is what runs for 9..32 rows of Q4_K.
- * With variant -1 the workspace also serves batch 3-8 on long rows (K >= 8192) of few (N < 12288): the 8-row GEMV
+ * With variant -1 the workspace also serves batch 2-8 (Q6_K: 3-8) on long rows (K >= 8192) of few (N < 12288): the 8-row GEMV
  * then splits K across workgroups, writes fp32 partial products to the workspace and sums them in a second launch
  * (the unsplit kernel would have to stage all of the activations in every workgroup).
  * Other arguments and numerics as cuthip_matmul_gguf. */

@@ -444,9 +444,10 @@ def test_pair_launch_equals_two_matmuls(ops, fa, fb, Na, Nb, K):
 
 
 @pytest.mark.parametrize("name", list(oracle.FORMATS))
-@pytest.mark.parametrize("M,N,K", [(4, 4096, 14336), (8, 4096, 14336), (3, 4096, 14336), (3, 100, 8192), (5, 9, 8192 + 32)])
+@pytest.mark.parametrize("M,N,K", [(2, 4096, 14336), (4, 4096, 14336), (8, 4096, 14336), (3, 4096, 14336), (3, 100, 8192), (5, 9, 8192 + 32),
+                                   (2, 100, 8192 + 256)])
 def test_batched_gemv_with_k_split_across_workgroups(ops, name, M, N, K):
-    """Batch 3-8 on long rows with a workspace: K ranges go to different workgroups, fp32 partial products are summed by
+    """Batch 2-8 on long rows with a workspace: K ranges go to different workgroups, fp32 partial products are summed by
     a second kernel, which also applies the epilogue.  Against the oracle (sampled columns for the big shapes) and
     against the launch without a workspace."""
     fmt = oracle.FORMATS[name]
