@@ -1014,7 +1014,8 @@ template <int FA, int FB> bool launch_rows8_pair_fmt(const GemvParams &pa, const
   constexpr int D = 4;
   if (s.kw == 1 && s.rwg < 8) *rc = launch_rows8_pair<FA, FB, 4, 1, D, 2>(pa, pb, stream);
   else if (s.kw == 2) *rc = launch_rows8_pair<FA, FB, 2, 2, D, 4>(pa, pb, stream);
-  else if (s.kw == 4 && pa.nsteps <= 16) *rc = launch_rows8_pair<FA, FB, 1, 4, D, 2>(pa, pb, stream);
+  // four steps per wave: a ring of two (1.730 against 1.750 ms per token of an 8B decode step with a ring of four)
+  else if (s.kw == 4 && pa.nsteps <= 16) *rc = launch_rows8_pair<FA, FB, 1, 4, 2, 2>(pa, pb, stream);
   else return false;
   return true;
 }
