@@ -295,6 +295,21 @@ __global__ void __launch_bounds__(128) attn_merge_kernel(const float *partial, c
   float ov[kPre];
 #pragma unroll
   for (uint32_t s = 0; s < kPre; ++s) ov[s] = (pre && s < used && tid < headDim) ? base[(size_t)s * rec + 2 + tid] : 0.0f;
+  if (pre) {
+    // up to 32 splits: every wave holds all (max, sum) pairs, one per lane, and folds them by itself: no LDS, no
+    // workgroup barrier; the weight of split s comes out of lane s
+    const uint32_t ls = tid & 63;
+    const bool have = ls < used;
+    const float ms = have ? base[(size_t)ls * rec] : -INFINITY, lsum = have ? base[(size_t)ls * rec + 1] : 0.0f;
+    const float M = wave_max(ms);
+    const float w = ms == -INFINITY ? 0.0f : expf(ms - M);   // an empty split (and an empty sequence: M = -inf) weighs nothing
+    const float L = wave_sum(lsum * w);
+    float o = 0.0f;   // every lane takes part in the shuffles; threads beyond the head dimension hold zeros
+#pragma unroll
+    for (uint32_t s = 0; s < kPre; ++s) o = fmaf(ov[s], __shfl(w, (int)s), o);
+    if (tid < headDim) st_act(out, out_f16, (size_t)h * headDim + tid, L > 0.0f ? o / L : 0.0f);
+    return;
+  }
   float m = -INFINITY;
   for (uint32_t s = tid; s < used; s += 128) m = fmaxf(m, base[(size_t)s * rec]);
   m = wave_max(m);
@@ -314,13 +329,8 @@ __global__ void __launch_bounds__(128) attn_merge_kernel(const float *partial, c
   const float L = red[2] + red[3];
   if (tid < headDim) {
     float o = 0.0f;
-    if (pre) {
-#pragma unroll
-      for (uint32_t s = 0; s < kPre; ++s) o = fmaf(ov[s], s < used ? Ws[s] : 0.0f, o);
-    } else {
 #pragma unroll 8
-      for (uint32_t s = 0; s < used; ++s) o = fmaf(base[(size_t)s * rec + 2 + tid], Ws[s], o);
-    }
+    for (uint32_t s = 0; s < used; ++s) o = fmaf(base[(size_t)s * rec + 2 + tid], Ws[s], o);
     st_act(out, out_f16, (size_t)h * headDim + tid, L > 0.0f ? o / L : 0.0f);
   }
 }
