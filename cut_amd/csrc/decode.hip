@@ -212,15 +212,18 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_
     const uint32_t rep = rep0 + wave;
     const bool live = rep < nRep;
     const uint32_t h = kvH * nRep + (live ? rep : 0);
-    __syncthreads();   // K, V staged (first pass) / Qs, Ps free again (later passes)
     if (rep0 == 0) {
+      // the first pass' query goes to LDS ahead of the staging barrier (each wave reads only its own), so that the
+      // pass costs one workgroup barrier, not two
 #pragma unroll
       for (int e = 0; e < 2; ++e)
         if (lane + 64 * e < headDim) Qs[wave * kAttnMaxHd + lane + 64 * e] = q_pre[e];
+      __syncthreads();   // K, V staged
     } else {
+      __syncthreads();   // Qs, Ps free again
       for (uint32_t d = lane; d < headDim; d += 64) Qs[wave * kAttnMaxHd + d] = ld_act(q, q_f16, (size_t)h * headDim + d);
+      __syncthreads();
     }
-    __syncthreads();
     // score of position t0 + lane: q is read as broadcast 16-byte pieces
     float sc = 0.0f;
     const half_t *krow = Ks + lane * kAttnRow;
