@@ -21,7 +21,7 @@
 // of the two-pass GEMM, which applies the epilogue).  After the staging barrier the loop has no barrier: each lane
 // keeps kStreamDepth steps of weight loads in flight in a register ring and waits only for the step it multiplies.
 //
-// Measured (MI355X, HIP-graph replay, Q4_K 14336 x 4096): 15.8 us at 9-16 rows (two passes of the 8-row GEMV: 25),
+// Measured (MI355X, HIP-graph replay, Q4_K 14336 x 4096): 15.0 us at 9-16 rows (two passes of the 8-row GEMV: 25),
 // 21 us at 17-32 rows (tiled GEMM with K split: 30); at 8 rows and fewer the 8-row GEMV is the faster one (13 us):
 // both spend about 0.05 vector instructions per weight on the unpack, which bounds them well before HBM does.
 #include <type_traits>
@@ -49,7 +49,7 @@ struct StreamParams {
 typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) uint8_t lds_u8s;
 
-constexpr int kStreamDepth = 4;
+constexpr int kStreamDepth = 2;   // steps of weight loads in flight per lane (waves have 4 to 8 steps: 15.0 us against 16.5 with four)
 constexpr uint32_t kStripBytes = 192 * 16;          // LDS per wave for the blocks of a step
 constexpr uint32_t kStreamLdsMax = 132 * 1024;     // staged activations: 16 rows of 4096 (the strips of eight waves take 24 KB more)
 
