@@ -486,6 +486,18 @@ def main():
         extras["q6k_lm_head_128256x4096_gemv_GBps"] = round((head.numel() + 2 * (4096 + 128256)) * 20 / (ev_h * 1e-3) / 1e9, 1)
         del head, logits
         torch.cuda.empty_cache()
+        # Q6_K at the FFN down-projection shape (half the down projections of a Q4_K_M file are Q6_K): 48 MB per launch,
+        # six copies rotated
+        q6_h = make_q_weights("Q6_K", N_EMBD, N_FF, 4)
+        q6 = [torch.from_numpy(q6_h).to(dev).clone() for _ in range(COPIES)]
+        y6 = torch.empty((1, N_EMBD), dtype=torch.float16, device=dev)
+
+        def q6_down(s):
+            ops.matmul_gguf(h[:1], q6[s % COPIES], "Q6_K", N_EMBD, N_FF, out=y6)
+        wall_6, ev_6, _ = timed_graph(torch, q6_down, 60, 6)
+        extras["q6k_gemv_4096x14336_GBps"] = round((q6[0].numel() + 2 * (N_FF + N_EMBD)) * 60 / (ev_6 * 1e-3) / 1e9, 1)
+        del q6, y6
+        torch.cuda.empty_cache()
         # config 5: prefill GEMM, Q4_K weights, fp16 activations, fp16 MFMA with fp32 accumulate.  The headline keys
         # (q4k_prefill_gemm_*_TFLOPs, *_pct_of_f16_mfma_peak) are this library's own kernels through its own choice
         # by shape; the vendor library's GEMM behind the same dequantization (variant 5, opt-in) is reported under
