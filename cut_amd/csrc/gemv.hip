@@ -34,12 +34,14 @@ Rows8Shape pick_rows8_shape(uint32_t N, uint32_t nsteps) {
   int kw = 1;
   // 1536 waves exactly (the q | k | v pair of an 8B model: 6144 rows, split once) still gain from a second split:
   // 5.8 us against 6.2 us for 6144 x 4096
-  while (kw < 8 && (uint64_t)groups * kw < (kw == 1 ? 1536u : 1537u) && nsteps / (uint32_t)(2 * kw) >= 2) kw *= 2;
+  // (the split into eight only while a wave keeps four steps: 1024 x 4096 Q6_K 4.8 us with four ranges, 6.2 with eight)
+  while (kw < 8 && (uint64_t)groups * kw < (kw == 1 ? 1536u : 1537u) && nsteps / (uint32_t)(2 * kw) >= (kw < 4 ? 2u : 4u)) kw *= 2;
   // rows split four ways: two row groups per workgroup share one staging of x (28 KB at K = 14336, which every
   // workgroup reads from L2): 9.8 us against 10.7 us for 4096 x 14336; 4096 x 4096 (16 steps) 5.2 us against 5.4, and
   // 1.3 us per layer of an 8B decode step, whose attention output projection has that shape (batch 1 only: the
-  // launch keeps one row group per workgroup for more batch rows)
-  if (kw == 4) return Rows8Shape{2, 4};
+  // launch keeps one row group per workgroup for more batch rows); from 4096 rows on: 1024 x 4096 is faster with
+  // one row group per workgroup (Q6_K 4.8 us against 5.5)
+  if (kw == 4) return Rows8Shape{groups >= 512 ? 2 : 1, 4};
   // eight row groups per workgroup from 28672 rows on (fused gate + up of an 8B model: 15.6 us against 16.0-16.2 us)
   return Rows8Shape{groups >= 3584 ? 8 : 4, kw};
 }
