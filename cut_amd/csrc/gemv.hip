@@ -25,13 +25,28 @@ CUTHIP_EXTERN_ROWS8(CUTHIP_Q6_K)
 
 // Workgroup shape of the rows8 GEMV: split K (kw step ranges per 8-row group)
 // while the grid has fewer than ~6 waves per CU and each wave keeps >= 2 steps.
-Rows8Shape pick_rows8_shape(uint32_t N, uint32_t nsteps) {
+Rows8Shape pick_rows8_shape(int fmt, uint32_t M, uint32_t N, uint32_t nsteps) {
   if (const char *env = std::getenv("CUT_HIP_ROWS8_SHAPE")) {   // "rwg,kw" tuning aid
     int rwg = 0, kw = 0;
     if (sscanf(env, "%d,%d", &rwg, &kw) == 2 && (kw == 1 || kw == 2 || kw == 4 || kw == 8)) return Rows8Shape{rwg, kw};
   }
+  (void)fmt;   // one rule for all formats so far
   uint32_t groups = (N + 7) / 8;
   int kw = 1;
+  if (M > 4) {
+    // 5-8 batch rows: every workgroup stages all eight rows of activations (72-80 KB at K = 4096, two workgroups per
+    // CU), so fewer, larger workgroups win earlier than at batch 1.  Measured at K = 4096, batch 8, us with
+    // (row groups, K ranges) = (1,8) / (1,4) / (2,2) / (8,1):
+    //   1024 rows  Q4_K  6.0 /  8.6 /  9.5 / 10.8    Q6_K  8.1 /  9.3 / 12.1 / 17.8    Q8_0  8.1 /  9.3 / 11.6 / 17.9
+    //   2048 rows  Q4_K  6.5 /  9.0 /  9.7 / 11.2    Q6_K  8.5 /  9.9 / 12.4 / 18.0    Q8_0  8.3 /  9.6 / 11.6 / 18.1
+    //   4096 rows  Q4_K 10.8 / 10.4 /  9.9 / 11.3    Q6_K 14.9 / 11.9 / 12.9 / 18.0    Q8_0 14.5 / 11.8 / 12.0 / 18.0
+    //   6144 rows  Q4_K 15.5 / 16.8 / 11.6 / 11.5    Q6_K 21.3 / 18.4 / 14.9 / 18.2    Q8_0 20.7 / 18.6 / 14.6 / 18.1
+    //   8192 rows  Q4_K 19.4 / 18.5 / 11.8 / 11.6    Q6_K 27.9 / 21.3 / 16.2 / 19.8    Q8_0 27.5 / 22.1 / 16.0 / 19.4
+    //  14336 rows  Q4_K 32.1 / 32.1 / 21.0 / 12.6    Q6_K 51.4 / 39.3 / 30.4 / 22.8    Q8_0 47.4 / 39.9 / 29.4 / 20.9
+    const int want = groups <= 256 ? 8 : groups <= 512 ? 4 : groups < 1536 ? 2 : 1;
+    while (kw < want && nsteps / (uint32_t)(2 * kw) >= 2u) kw *= 2;
+    return Rows8Shape{kw == 1 ? 8 : kw == 2 ? 2 : 1, kw};
+  }
   // 1536 waves exactly (the q | k | v pair of an 8B model: 6144 rows, split once) still gain from a second split:
   // 5.8 us against 6.2 us for 6144 x 4096
   // (the split into eight only while a wave keeps four steps: 1024 x 4096 Q6_K 4.8 us with four ranges, 6.2 with eight)
@@ -61,12 +76,16 @@ int launch_splitk_reduce(const float *partial, uint32_t ksplit, uint32_t M, uint
 // The split across workgroups pays where one row group per workgroup would re-stage long activations for few rows:
 // batch 2-8, rows of at least 32 steps, and not enough row groups to fill the chip without splitting K.
 static bool ksplit_gemv_preferred(int fmt, uint32_t M, uint32_t K, uint32_t N) {
+  if (M < 2 || M > 8) return false;
+  // whatever the number of weight rows where the unsplit kernel cannot hold the activations in LDS (8 rows of K >= 8192):
+  // what would run otherwise is the 32-row fallback
+  if (rows8_lds_bytes_rt(fmt, (K + 255) / 256, rows8_batch_class(M)) > kRows8LdsBudget) return true;
   // from 2 batch rows on (4096 x 14336 at two rows: Q4_K 11.6 us against 12.6 unsplit, Q8_0 18.2 against 19.6); Q6_K
   // from 3: its two rows run the dot-product path, unsplit 17.4 us against 18.2
-  return M >= (fmt == CUTHIP_Q6_K ? 3u : 2u) && M <= 8 && K >= 8192 && (N + 7) / 8 < 1536;
+  return M >= (fmt == CUTHIP_Q6_K ? 3u : 2u) && K >= 8192 && (N + 7) / 8 < 1536;
 }
-static size_t ksplit_gemv_workspace(uint32_t M, uint32_t K, uint32_t N) {
-  return (size_t)rows8_ksplit_parts(N, (K + 255) / 256) * M * N * sizeof(float);
+static size_t ksplit_gemv_workspace(int fmt, uint32_t M, uint32_t K, uint32_t N) {
+  return (size_t)rows8_ksplit_parts(fmt, M, N, (K + 255) / 256) * M * N * sizeof(float);
 }
 
 #define CUTHIP_EXTERN_PAIR(FA, FB) \
@@ -332,6 +351,27 @@ static int matmul_gguf_scratch(int fmt, const void *W, const void *A, int a_dtyp
       set_error("cuthip_matmul_gguf: variant 3 needs M <= 8 and the activations to fit in LDS (M = %u, K = %u)", M, K);
       return CUTHIP_ERR_INVALID;
     }
+    // The batch rows do not fit the 8-row GEMV's LDS budget together (8 rows of K = 8192, 3 of K = 14336) and no scratch
+    // memory is at hand for its K split: passes over fewer rows at a time where those beat the 32-row fallback kernel,
+    // which is slow on every format but Q4_K.  Measured, us, fallback against passes: 28672 x 8192 at 8 rows Q6_K 248 / 123,
+    // Q8_0 196 / 119, Q4_0 125 / 88; 4096 x 14336 at 4 rows Q6_K 80 / 30, Q8_0 61 / 36, at 8 rows Q6_K 87 / 58,
+    // Q8_0 70 / 75; Q4_K 4096 x 14336 at 4 rows 21 / 25: its fallback stays.
+    if (fmt != CUTHIP_Q4_K) {
+      uint32_t rows = 4;
+      while (rows >= 1 && (rows >= M || rows8_lds_bytes_rt(fmt, (K + 255) / 256, (int)rows) > kRows8LdsBudget)) rows /= 2;
+      if (rows >= 1 && (M + rows - 1) / rows <= (fmt == CUTHIP_Q6_K ? 4u : 2u)) {
+        const size_t asz = a_dtype == CUTHIP_F16 ? 2 : 4, csz = c_dtype == CUTHIP_F16 ? 2 : 4;
+        for (uint32_t m0 = 0; m0 < M; m0 += rows) {
+          const uint8_t *a = reinterpret_cast<const uint8_t *>(A) + (size_t)m0 * strideA * asz;
+          uint8_t *c = reinterpret_cast<uint8_t *>(C) + (size_t)m0 * strideC * csz;
+          const uint8_t *d = D ? reinterpret_cast<const uint8_t *>(D) + (size_t)m0 * strideC * csz : nullptr;
+          if (int rc2 = matmul_gguf_scratch(fmt, W, a, a_dtype, c, c_dtype, min(rows, M - m0), K, N, strideA, strideC, epilogue,
+                                            epilogue_op, d, -1, stream, nullptr, 0))
+            return rc2;
+        }
+        return CUTHIP_OK;
+      }
+    }
   }
   if (epilogue == CUTHIP_EPI_SWIGLU_PAIRS) {
     set_error("cuthip_matmul_gguf: the SwiGLU row-pair epilogue exists in variant 3 only (got variant %d)", variant);
@@ -431,7 +471,7 @@ int cuthip_matmul_gguf_argmax(int fmt, const void *W, const void *A, int a_dtype
   apply_carry(p, carry, false);
   // the arg-max rides in the matmul's epilogue where the 8-row GEMV runs one K range per wave (any vocabulary-sized N)
   // and the caller brought room for the per-group winners; otherwise the logits are scanned by the second launch
-  const bool fused = pick_rows8_shape(N, p.nsteps).kw == 1 && workspace && (uintptr_t)workspace % 8 == 0 &&
+  const bool fused = pick_rows8_shape(fmt, 1, N, p.nsteps).kw == 1 && workspace && (uintptr_t)workspace % 8 == 0 &&
                      workspace_bytes >= cuthip_matmul_gguf_argmax_workspace_bytes(N);
   if (fused) p.argmax_parts = reinterpret_cast<ArgmaxPart *>(workspace);
   bool taken = false;
@@ -528,7 +568,7 @@ int cuthip_matmul_gguf_pair(int fmt_a, const void *Wa, uint32_t Na, void *Ca, in
 
 size_t cuthip_matmul_gguf_workspace_bytes(int fmt, uint32_t M, uint32_t K, uint32_t N, int a_dtype) {
   (void)fmt;
-  if (cuthip::ksplit_gemv_preferred(fmt, M, K, N)) return cuthip::ksplit_gemv_workspace(M, K, N);
+  if (cuthip::ksplit_gemv_preferred(fmt, M, K, N)) return cuthip::ksplit_gemv_workspace(fmt, M, K, N);
   return cuthip::dense_gemm_workspace(M, K, N, a_dtype == CUTHIP_F16);
 }
 
@@ -601,7 +641,7 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   }
   // batch 3-8 on long rows: the 8-row GEMV with K split across workgroups, partial products in the workspace
   if (variant == -1 && !dense_first && ksplit_gemv_preferred(fmt, M, K, N) && workspace && (uintptr_t)workspace % 16 == 0 &&
-      workspace_bytes >= ksplit_gemv_workspace(M, K, N) && (uintptr_t)A % 16 == 0 && (strideA * (a_f16 ? 2 : 4)) % 16 == 0) {
+      workspace_bytes >= ksplit_gemv_workspace(fmt, M, K, N) && (uintptr_t)A % 16 == 0 && (strideA * (a_f16 ? 2 : 4)) % 16 == 0) {
     const GemvParams p = gemv_params(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC,
                                      Epilogue{CUTHIP_EPI_NONE, 0, nullptr});
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);

@@ -594,7 +594,7 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
   // the weight ring, one share per thread, folded per wave and across the waves through LDS at the staging barrier
   // (the order of the additions depends on the launch shape only)
   constexpr int CP = 4;
-  const uint32_t nparts = p.sumsq_parts ? (p.K + 7) / 8 : 0u;
+  const uint32_t nparts = (MT == 1 && p.sumsq_parts) ? (p.K + 7) / 8 : 0u;   // batch 1 only: the LDS of larger batches has no room for it
   float cpart[CP];
 #pragma unroll
   for (int jj = 0; jj < CP; ++jj) {
@@ -870,8 +870,10 @@ __global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_pair_kernel(GemvP
     rows8_body<FB, 1, RWG, KW, D, XWANT, false>(pb, blockIdx.x - blocks_a);
 }
 
+inline size_t rows8_lds_bytes_rt(int fmt, uint32_t nsteps, int mt);
 template <int FMT> static size_t rows8_lds_bytes(const GemvParams &p, int mt) {
-  return (size_t)mt * ((size_t)p.nsteps * kXStep * 2 + (size_t)p.nsteps * Rows8<FMT>::NSUB * 4 + 8 * 4);   // + [8 waves] floats
+  static_assert(Rows8<FMT>::NSUB == (FMT == CUTHIP_Q6_K ? 16 : 8), "rows8_lds_bytes_rt assumes these sub-block counts");
+  return rows8_lds_bytes_rt(FMT, p.nsteps, mt);
 }
 
 template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO = false>
@@ -936,18 +938,37 @@ static int launch_rows8_pair(const GemvParams &pa, const GemvParams &pb, hipStre
   return check_hip(hipGetLastError(), "gemv pair launch");
 }
 
+// LDS of one workgroup of the 8-row GEMV: mt batch rows of staged activations and their per-sub-block sums (Q6_K has 16
+// sub-blocks per 256 elements, the other formats 8); at batch 1 eight more floats, the per-wave shares of sum(x^2) of
+// the RMSNorm prologue and of the carried norm, which exist at batch 1 only.  Without them 8 rows of K = 4096 and 4 rows
+// of K = 8192 of Q6_K take exactly 80 KB, so that two workgroups share a CU.
+inline size_t rows8_lds_bytes_rt(int fmt, uint32_t nsteps, int mt) {
+  const size_t nsub = fmt == CUTHIP_Q6_K ? 16 : 8;
+  return (size_t)mt * ((size_t)nsteps * kXStep * 2 + (size_t)nsteps * nsub * 4) + (mt == 1 ? 8 * 4 : 0);
+}
+
+// LDS a workgroup may ask for.  More would fit (160 KB per CU), but every workgroup stages all of its activations:
+// at 129 KB (4 batch rows, K = 14336) the staging traffic makes this kernel slower than the 32-row fallback
+// (30 us against 23.5 us for 4096 x 14336), so such shapes stay with the fallback.
+constexpr size_t kRows8LdsBudget = 96 * 1024;
+
+inline int rows8_batch_class(uint32_t M) { return M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8)); }
+
 // parts of K for the split across workgroups: enough parts for one workgroup of eight waves per CU, at least 4 steps per
-// part (4096 x 14336 at batch 8: four parts of 14 steps 14.8 us per launch of an FFN step, eight parts of 7 steps 16.5)
-inline uint32_t rows8_ksplit_parts(uint32_t N, uint32_t nsteps) {
+// part (4096 x 14336 at batch 8: four parts of 14 steps 14.8 us per launch of an FFN step, eight parts of 7 steps 16.5),
+// and as many more as it takes for the activations of one part to fit the LDS budget (8 rows of K = 28672: 8 parts)
+inline uint32_t rows8_ksplit_parts(int fmt, uint32_t M, uint32_t N, uint32_t nsteps) {
   const uint32_t blocks = ((N + 7) / 8 + 7) / 8;
   uint32_t s = 1;
   while (s < 16 && blocks * s < 256 && nsteps / (2 * s) >= 4) s *= 2;
+  const int mt = rows8_batch_class(M < 2 ? 2 : M);
+  while (s < nsteps && rows8_lds_bytes_rt(fmt, (nsteps + s - 1) / s, mt) > kRows8LdsBudget) s *= 2;
   return s;
 }
 
 // steps per part and the number of non-empty parts (rounding the steps up can leave the last of the wanted parts empty)
-inline void rows8_ksplit_layout(uint32_t N, uint32_t nsteps, uint32_t *part_steps, uint32_t *parts) {
-  const uint32_t want = rows8_ksplit_parts(N, nsteps);
+inline void rows8_ksplit_layout(int fmt, uint32_t M, uint32_t N, uint32_t nsteps, uint32_t *part_steps, uint32_t *parts) {
+  const uint32_t want = rows8_ksplit_parts(fmt, M, N, nsteps);
   *part_steps = (nsteps + want - 1) / want;
   *parts = (nsteps + *part_steps - 1) / *part_steps;
 }
@@ -955,7 +976,7 @@ inline void rows8_ksplit_layout(uint32_t N, uint32_t nsteps, uint32_t *part_step
 template <int FMT, int MT> static int launch_rows8_ksplit_mt(const GemvParams &p, float *partial, hipStream_t stream) {
   constexpr int D = 4;
   uint32_t parts, part_steps;
-  rows8_ksplit_layout(p.N, p.nsteps, &part_steps, &parts);
+  rows8_ksplit_layout(FMT, p.M, p.N, p.nsteps, &part_steps, &parts);
   GemvParams q = p;
   q.K = min(p.K, part_steps * 256u);
   q.nsteps = part_steps;
@@ -975,29 +996,23 @@ template <int FMT, int MT> static int launch_rows8_ksplit_mt(const GemvParams &p
 // M = 2..8; returns the number of parts through *parts_out (the caller sums them)
 template <int FMT> int launch_rows8_ksplit(const GemvParams &p, float *partial, uint32_t *parts_out, hipStream_t stream) {
   uint32_t part_steps;
-  rows8_ksplit_layout(p.N, p.nsteps, &part_steps, parts_out);
+  rows8_ksplit_layout(FMT, p.M, p.N, p.nsteps, &part_steps, parts_out);
   if (p.M <= 2) return launch_rows8_ksplit_mt<FMT, 2>(p, partial, stream);
   if (p.M <= 4) return launch_rows8_ksplit_mt<FMT, 4>(p, partial, stream);
   return launch_rows8_ksplit_mt<FMT, 8>(p, partial, stream);
 }
 
 struct Rows8Shape { int rwg, kw; };
-Rows8Shape pick_rows8_shape(uint32_t N, uint32_t nsteps);
-
-// LDS a workgroup may ask for.  More would fit (160 KB per CU), but every workgroup stages all of its activations:
-// at 129 KB (4 batch rows, K = 14336) the staging traffic makes this kernel slower than the 32-row fallback
-// (30 us against 23.5 us for 4096 x 14336), so such shapes stay with the fallback.
-constexpr size_t kRows8LdsBudget = 96 * 1024;
+Rows8Shape pick_rows8_shape(int fmt, uint32_t M, uint32_t N, uint32_t nsteps);
 
 // true if the rows8 kernel can take the problem (activations must fit in LDS)
 template <int FMT> bool rows8_fits(const GemvParams &p) {
   if (p.M > 8) return false;
-  int mt = p.M <= 1 ? 1 : (p.M <= 2 ? 2 : (p.M <= 4 ? 4 : 8));
-  return rows8_lds_bytes<FMT>(p, mt) <= kRows8LdsBudget;
+  return rows8_lds_bytes<FMT>(p, rows8_batch_class(p.M)) <= kRows8LdsBudget;
 }
 
 template <int FMT> int launch_rows8_fmt(const GemvParams &p, hipStream_t stream) {
-  Rows8Shape s = pick_rows8_shape(p.N, p.nsteps);
+  Rows8Shape s = pick_rows8_shape(FMT, p.M, p.N, p.nsteps);
   if (FMT == CUTHIP_Q6_K && s.rwg > 4) s.rwg = 4;   // measured on the 128256 x 4096 head: 103 us against 110-114 with 8 row groups
   if (p.M <= 1) return launch_rows8_shape<FMT, 1>(p, s.rwg, s.kw, stream);
   if (p.M <= 2) return launch_rows8_shape<FMT, 2>(p, s.rwg, s.kw, stream);
@@ -1010,7 +1025,7 @@ template <int FMT> int launch_rows8_fmt(const GemvParams &p, hipStream_t stream)
 template <int FA, int FB> bool launch_rows8_pair_fmt(const GemvParams &pa, const GemvParams &pb, hipStream_t stream, int *rc) {
   if (pa.M != 1 || pb.M != 1 || pa.K != pb.K || pa.pro || pb.pro) return false;
   if (rows8_lds_bytes<FA>(pa, 1) > kRows8LdsBudget || rows8_lds_bytes<FB>(pb, 1) > kRows8LdsBudget) return false;
-  Rows8Shape s = pick_rows8_shape(pa.N + pb.N, pa.nsteps);
+  Rows8Shape s = pick_rows8_shape(FA, 1, pa.N + pb.N, pa.nsteps);
   constexpr int D = 4;
   if (s.kw == 1 && s.rwg < 8) *rc = launch_rows8_pair<FA, FB, 4, 1, D, 2>(pa, pb, stream);
   else if (s.kw == 2) *rc = launch_rows8_pair<FA, FB, 2, 2, D, 4>(pa, pb, stream);

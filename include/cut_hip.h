@@ -247,7 +247,11 @@ int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void 
  *            it is what runs for 9..32 rows of Q4_K.
  * With variant -1 the workspace also serves batch 2-8 (Q6_K: 3-8) on long rows (K >= 8192) of few (N < 12288): the 8-row GEMV
  * then splits K across workgroups, writes fp32 partial products to the workspace and sums them in a second launch
- * (the unsplit kernel would have to stage all of the activations in every workgroup).
+ * (the unsplit kernel would have to stage all of the activations in every workgroup).  The same for any N where the
+ * batch rows times K exceed the 96 KB of LDS the unsplit kernel stages them in (8 rows of K >= 8192, 4 of K >= 16384): K
+ * is split into as many parts as that takes (28672 x 8192 at 8 rows: Q4_K 47 us against 80 without a workspace, Q6_K 77
+ * against 123, Q8_0 80 against 119).  Without a workspace such shapes run as passes over fewer rows where those fit
+ * (all formats but Q4_K), else on the 32-row fallback kernel.
  * Other arguments and numerics as cuthip_matmul_gguf. */
 size_t cuthip_matmul_gguf_workspace_bytes(int fmt, uint32_t M, uint32_t K, uint32_t N, int a_dtype);
 int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t M, uint32_t K,

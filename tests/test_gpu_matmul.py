@@ -473,6 +473,33 @@ def test_batched_gemv_with_k_split_across_workgroups(ops, name, M, N, K):
 
 
 @pytest.mark.parametrize("name", list(oracle.FORMATS))
+@pytest.mark.parametrize("M,N,K", [(8, 16, 90112), (7, 16384, 8192), (5, 12288, 8192), (3, 256, 28672)])
+def test_batched_gemv_k_split_where_the_activations_exceed_lds(ops, name, M, N, K):
+    """Batch rows x K beyond what one workgroup stages in LDS: with a workspace the K split takes as many parts as it
+    needs for one part to fit (8 rows of K = 90112: 32 parts; 7 rows of K = 8192 on 16384 weight rows: 2 parts, where
+    the chip would be full without any), whatever the number of weight rows.  Against the oracle on sampled columns and
+    against the launch without a workspace (the 32-row fallback kernel).  The weights repeat a block of 256 rows."""
+    fmt = oracle.FORMATS[name]
+    rows = min(N, 256)
+    tile = quantized_weights(fmt, rows, K, seed=140)
+    W = np.tile(tile, N // rows)
+    A = gauss_acts((M, K), seed=141, dtype=np.float16)
+    a, w = torch.from_numpy(A).cuda(), torch.from_numpy(W).cuda()
+    ws = ops.matmul_gguf_workspace(fmt, M, K, N, a.dtype, "cuda")
+    assert ws is not None and ws.numel() > 0
+    ws.fill_(0xFF)
+    got = ops.matmul_gguf(a, w, fmt, N, K, out_dtype=torch.float32, workspace=ws)
+    ref = ops.matmul_gguf(a, w, fmt, N, K, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    got, ref = got.cpu().numpy(), ref.cpu().numpy()
+    assert normwise_rel_err(got, ref) < 2e-5
+    cols = np.unique(np.concatenate([[0, N - 1], np.random.default_rng(8).integers(0, N, min(N, 64))]))
+    Ws = np.ascontiguousarray(W.reshape(N, oracle.n_bytes(fmt, K))[cols]).reshape(-1)
+    want = oracle.matmul_gguf(fmt, Ws, A.astype(np.float32), len(cols), f64=True)
+    assert normwise_rel_err(got[:, cols], want) < TOL_F16_ACT
+
+
+@pytest.mark.parametrize("name", list(oracle.FORMATS))
 @pytest.mark.parametrize("M", [9, 19, 40])
 def test_mid_size_batches_run_as_eight_row_passes(ops, name, M):
     """9-40 rows with the automatic choice: passes of 8 rows through the decode kernel, with strided A / C / D and a
