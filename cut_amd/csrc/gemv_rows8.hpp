@@ -457,15 +457,15 @@ template <int SUBK, int THREADS, int MT, int XR, bool PRO> struct XStage {
       if (m < p.M && k < p.K) {
         const uint8_t *src = reinterpret_cast<const uint8_t *>(p.A) + ((size_t)m * p.strideA + k) * esz;
         ra[u] = ld_u32x4(src);
-        if (PRO && p.pro == CUTHIP_PRO_SWIGLU) {
-          rb[u] = ld_u32x4(src + (size_t)p.K * 2);   // the "up" half of [gate | up] (fp16 only)
-        } else {
-          if (!p.a_f16) rb[u] = ld_u32x4(src + 16);
-          if (PRO && p.pro == CUTHIP_PRO_RMSNORM) {
-            const uint8_t *w = reinterpret_cast<const uint8_t *>(p.norm_w + k);
-            wa[u] = ld_u32x4(w);
-            wb[u] = ld_u32x4(w + 16);
-          }
+        // one load site per register array (a branch per source would let the compiler merge the stores of different
+        // arrays into one with a run-time slot, which moves the arrays to scratch memory)
+        const bool swiglu = PRO && p.pro == CUTHIP_PRO_SWIGLU;
+        // second half of the group: the "up" half of [gate | up] (fp16 only), or elements 4..7 of an fp32 group
+        if (swiglu || !p.a_f16) rb[u] = ld_u32x4(swiglu ? src + (size_t)p.K * 2 : src + 16);
+        if (PRO && p.pro == CUTHIP_PRO_RMSNORM) {
+          const uint8_t *w = reinterpret_cast<const uint8_t *>(p.norm_w + k);
+          wa[u] = ld_u32x4(w);
+          wb[u] = ld_u32x4(w + 16);
         }
       }
     }

@@ -73,9 +73,9 @@ class DecodeStep:
         2 = RMSNorm is fused into the following matmuls as well.  Level 2 saves three more launches per layer but
         every workgroup of those matmuls then stages fp32 x and the norm weights (4x the bytes of fp16 x), which
         lengthens their start-up; likewise every workgroup of w_down recomputes SiLU * up for its whole input.  On
-        MI355X both levels measured slower than separate launches (2.43 / 2.70 / 2.85 ms per token for 0 / 1 / 2 at
-        the 8B shape); fusing into the producer has no such cost.  The fused entry point stays for shapes where
-        launches dominate."""
+        MI355X neither level gains over separate launches (2.05 / 2.07 / 2.09 ms per token for 0 / 1 / 2 at the 8B
+        shape, 1.96 / 1.72 for 3 / 4); fusing into the producer has no such cost.  The fused entry point stays for
+        shapes where launches dominate."""
         if fuse >= 3:
             layers = [dict(L, gate_up=interleave_gate_up(L["gate_up"], cfg.ffn)) for L in layers]
         if fuse == 4:   # rows of q | k interleaved inside every head for the RoPE epilogue
