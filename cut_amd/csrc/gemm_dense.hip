@@ -683,7 +683,8 @@ size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
 // a sweep over the weight shapes of an 8B model (all formats, M = 16 .. 2048, HIP-graph replay, MI355X):
 //   two-pass      3 + N K (bytes per weight + 2) / 6.0 MB   the dequantization (reads the blocks, writes fp16)
 //                 + 17 + 2 ceil128(M) N K / 1.25 PFLOP/s     the dense GEMM (tiles are at least 128 rows high)
-//   single launch K x c_fmt x max(1, tiles / 256)            c = 14.7 ns (Q4_K, Q4_0), 19.6 ns (Q8_0), 23.5 ns (Q6_K):
+//   single launch K x c_fmt x max(1, tiles / 256)            c = 14.7 ns (Q4_K, Q4_0), 17 ns (Q8_0: 256 x 28672 x 4096 122 us,
+//                 512 rows 220, 256 x 14336 x 4096 73-76), 23.5 ns (Q6_K):
 //                 a workgroup decodes its K-long strip of weights once per 128 rows of A, and nothing overlaps that
 //                 walk until every CU holds more than one 128 x 128 tile.
 // Measured against them (Q4_K, M x N x K): 64 x 4096 x 4096 38 / 62 us, 512 x 14336 x 4096 99 / 105, 512 x 28672 x 4096
@@ -695,7 +696,7 @@ double dense_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
   return 3.0 + nk * (bpw + 2.0) / 6.0e6 + 17.0 + 2.0 * (double)((M + 127) / 128 * 128) * nk / 1.25e9 + split;
 }
 double single_launch_rows_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
-  const double c = fmt == CUTHIP_Q6_K ? 23.5e-3 : fmt == CUTHIP_Q8_0 ? 19.6e-3 : 14.7e-3;
+  const double c = fmt == CUTHIP_Q6_K ? 23.5e-3 : fmt == CUTHIP_Q8_0 ? 17.0e-3 : 14.7e-3;
   const double tiles = (double)((M + 127) / 128) * ((N + 127) / 128);
   return K * c * (tiles > 256.0 ? tiles / 256.0 : 1.0);
 }
