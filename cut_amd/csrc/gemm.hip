@@ -104,17 +104,20 @@ template <> struct Sub<CUTHIP_Q6_K> {
     uint32_t s = sub & 3;
     float d = f16bits_to_f32(r.d);
     float dsc0 = d * (float)(int)(int8_t)(r.sc & 0xFF), dsc1 = d * (float)(int)(int8_t)(r.sc >> 8);
+    const float off0 = -32.0f * dsc0, off1 = -32.0f * dsc1;
     uint32_t lsh = (s >> 1) * 4, hsh = 2 * s;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       uint32_t wl = i < 4 ? r.ql[0][i] : r.ql[1][i - 4], wh = i < 4 ? r.qh[0][i] : r.qh[1][i - 4];
       uint32_t q6 = ((wl >> lsh) & 0x0F0F0F0Fu) | (((wh >> hsh) & 0x03030303u) << 4);
       asm volatile("" : "+v"(q6));
-      float dsc = i < 4 ? dsc0 : dsc1;  // elements 0-15 / 16-31 of the 32
-      w[4 * i + 0] = (half_t)(dsc * (cvt_ubyte0(q6) - 32.0f));
-      w[4 * i + 1] = (half_t)(dsc * (cvt_ubyte1(q6) - 32.0f));
-      w[4 * i + 2] = (half_t)(dsc * (cvt_ubyte2(q6) - 32.0f));
-      w[4 * i + 3] = (half_t)(dsc * (cvt_ubyte3(q6) - 32.0f));
+      // dsc * (q - 32) as one fused multiply-add with the exact constant -32 dsc: the same real number rounded once,
+      // hence the same bits, and one instruction per weight less
+      const float dsc = i < 4 ? dsc0 : dsc1, off = i < 4 ? off0 : off1;  // elements 0-15 / 16-31 of the 32
+      w[4 * i + 0] = (half_t)__builtin_fmaf(dsc, cvt_ubyte0(q6), off);
+      w[4 * i + 1] = (half_t)__builtin_fmaf(dsc, cvt_ubyte1(q6), off);
+      w[4 * i + 2] = (half_t)__builtin_fmaf(dsc, cvt_ubyte2(q6), off);
+      w[4 * i + 3] = (half_t)__builtin_fmaf(dsc, cvt_ubyte3(q6), off);
     }
   }
 };
@@ -128,14 +131,14 @@ template <> struct Sub<CUTHIP_Q8_0> {
     r.q[1] = ld_u32x4(blk + 18);
   }
   __device__ static void decode(const Raw &r, uint32_t, half_t (&w)[32]) {
-    float d = f16bits_to_f32(r.d);
+    const float d = f16bits_to_f32(r.d), off = -128.0f * d;   // d * (q + 128 - 128) as one exact fused multiply-add
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       uint32_t word = (i < 4 ? r.q[0][i] : r.q[1][i - 4]) ^ 0x80808080u;  // q + 128 as unsigned bytes
-      w[4 * i + 0] = (half_t)(d * (cvt_ubyte0(word) - 128.0f));
-      w[4 * i + 1] = (half_t)(d * (cvt_ubyte1(word) - 128.0f));
-      w[4 * i + 2] = (half_t)(d * (cvt_ubyte2(word) - 128.0f));
-      w[4 * i + 3] = (half_t)(d * (cvt_ubyte3(word) - 128.0f));
+      w[4 * i + 0] = (half_t)__builtin_fmaf(d, cvt_ubyte0(word), off);
+      w[4 * i + 1] = (half_t)__builtin_fmaf(d, cvt_ubyte1(word), off);
+      w[4 * i + 2] = (half_t)__builtin_fmaf(d, cvt_ubyte2(word), off);
+      w[4 * i + 3] = (half_t)__builtin_fmaf(d, cvt_ubyte3(word), off);
     }
   }
 };
@@ -148,18 +151,18 @@ template <> struct Sub<CUTHIP_Q4_0> {
     r.q = ld_u32x4(blk + 2);
   }
   __device__ static void decode(const Raw &r, uint32_t, half_t (&w)[32]) {
-    float d = f16bits_to_f32(r.d);
+    const float d = f16bits_to_f32(r.d), off = -8.0f * d;   // d * (q - 8) as one exact fused multiply-add
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       uint32_t lo = r.q[i] & 0x0F0F0F0Fu, hi = (r.q[i] >> 4) & 0x0F0F0F0Fu;
-      w[4 * i + 0] = (half_t)(d * (cvt_ubyte0(lo) - 8.0f));
-      w[4 * i + 1] = (half_t)(d * (cvt_ubyte1(lo) - 8.0f));
-      w[4 * i + 2] = (half_t)(d * (cvt_ubyte2(lo) - 8.0f));
-      w[4 * i + 3] = (half_t)(d * (cvt_ubyte3(lo) - 8.0f));
-      w[16 + 4 * i + 0] = (half_t)(d * (cvt_ubyte0(hi) - 8.0f));
-      w[16 + 4 * i + 1] = (half_t)(d * (cvt_ubyte1(hi) - 8.0f));
-      w[16 + 4 * i + 2] = (half_t)(d * (cvt_ubyte2(hi) - 8.0f));
-      w[16 + 4 * i + 3] = (half_t)(d * (cvt_ubyte3(hi) - 8.0f));
+      w[4 * i + 0] = (half_t)__builtin_fmaf(d, cvt_ubyte0(lo), off);
+      w[4 * i + 1] = (half_t)__builtin_fmaf(d, cvt_ubyte1(lo), off);
+      w[4 * i + 2] = (half_t)__builtin_fmaf(d, cvt_ubyte2(lo), off);
+      w[4 * i + 3] = (half_t)__builtin_fmaf(d, cvt_ubyte3(lo), off);
+      w[16 + 4 * i + 0] = (half_t)__builtin_fmaf(d, cvt_ubyte0(hi), off);
+      w[16 + 4 * i + 1] = (half_t)__builtin_fmaf(d, cvt_ubyte1(hi), off);
+      w[16 + 4 * i + 2] = (half_t)__builtin_fmaf(d, cvt_ubyte2(hi), off);
+      w[16 + 4 * i + 3] = (half_t)__builtin_fmaf(d, cvt_ubyte3(hi), off);
     }
   }
 };
