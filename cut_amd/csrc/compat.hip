@@ -17,6 +17,7 @@
 // several workgroups the partial sums go to a caller-provided workspace and a
 // second kernel adds them and applies the epilogue.
 #include <cstdint>
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -39,22 +40,92 @@ struct SepParams {
   int affine;
 };
 
-template <bool Q4, int MT>
+// RAGGED: N is not a multiple of 16, so the last lane of a row holds fewer columns and reads them byte by byte; the
+// instance for whole lanes carries none of that code (32 rows x a divergent byte loop each made the kernel 10,000
+// instructions long, more than the instruction cache holds).
+template <bool Q4, int MT, bool RAGGED>
 __global__ void __launch_bounds__(64 * kSepWaves, 2) sep_gemv_kernel(SepParams p) {
-  __shared__ float xs[MT][kSepWaves * kSepKC];
-  __shared__ float red[MT][kSepTile];
+  // activations of the workgroup's k range, [MT][128] floats, rounded up to one slot per thread and load
+  constexpr int XL = (MT * kSepWaves * kSepKC + 64 * kSepWaves - 1) / (64 * kSepWaves);
+  __shared__ float xs[XL * 64 * kSepWaves];
+  __shared__ f32x4 red[kSepWaves - 1][MT][kSepCols / 4][64];   // lane-contiguous 16-byte slots: no bank conflicts
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t c0 = blockIdx.x * kSepTile + lane * kSepCols;
   const uint32_t kwg = blockIdx.y * (kSepWaves * kSepKC);   // first k-row of this workgroup
   const uint32_t k0 = kwg + wave * kSepKC;                  // this wave's block
   const uint32_t blocksK = p.K / 32;
+  const uint32_t ncols = c0 < p.N ? min((uint32_t)kSepCols, p.N - c0) : 0u;
+  const bool work = k0 < p.K && ncols;
+  // The instance for whole lanes issues every load unconditionally (lanes and waves without work read column 0 of
+  // block 0 and drop it): with loads under a condition the compiler waits for all of them at the first use of any.
+  const uint32_t cb = (RAGGED || work) ? c0 : 0u, kb = (RAGGED || work) ? k0 : 0u;
 
-  // activations of the workgroup's k range
-  for (int i = tid; i < MT * kSepWaves * kSepKC; i += 64 * kSepWaves) {
-    int m = i / (kSepWaves * kSepKC), kk = i % (kSepWaves * kSepKC);
-    uint32_t row = p.m0 + m, k = kwg + kk;
-    xs[m][kk] = (row < p.M && k < p.K) ? p.A[(size_t)row * p.strideA + k] : 0.0f;
+  // One k-row of this lane's 16 columns: 16 bytes of int8 or 8 bytes of nibbles.
+  using Row = typename std::conditional<Q4, u32x2, u32x4>::type;
+  auto load_row = [&](uint32_t k) -> Row {
+    Row w{};
+    if (Q4) {
+      const uint8_t *src = p.B + (size_t)k * p.strideB + cb / 2;
+      if (!RAGGED || ncols == kSepCols) {
+        const u32x2 v = ld_u32x2(src);
+        w[0] = v.x;
+        w[1] = v.y;
+      } else {   // last lane of a ragged row: byte loads inside the row
+        for (uint32_t b = 0; b < (ncols + 1) / 2; ++b) w[b >> 2] |= (uint32_t)src[b] << (8 * (b & 3));
+      }
+    } else {
+      const uint8_t *src = p.B + (size_t)k * p.strideB + cb;
+      if (!RAGGED || ncols == kSepCols) {
+        const u32x4 v = ld_u32x4(src);
+        w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+      } else {
+        for (uint32_t b = 0; b < ncols; ++b) w[b >> 2] |= (uint32_t)src[b] << (8 * (b & 3));
+      }
+    }
+    return w;
+  };
+
+  // Every load of the wave's block is requested before anything is used: G rows per lane in flight (all 32 where the
+  // registers allow), then the block's scales (and minima), then the activations of the workgroup's k range.  With
+  // four groups of eight rows, each used right after the next was requested, the kernel waited for four memory round
+  // trips in turn and took 20 us for 14336 x 4096 whatever the format.
+  // The activations of the workgroup's k range are requested first and unconditionally (threads without an element
+  // read element 0 and drop it), so that they arrive ahead of the weights and the wait for them leaves the weight
+  // loads in flight: memory returns in issue order.
+  float xv[XL];
+#pragma unroll
+  for (int u = 0; u < XL; ++u) {
+    const int i = tid + u * 64 * kSepWaves, m = i / (kSepWaves * kSepKC), kk = i % (kSepWaves * kSepKC);
+    const uint32_t row = p.m0 + m, k = kwg + kk;
+    const bool ok = m < MT && row < p.M && k < p.K;
+    xv[u] = p.A[ok ? (size_t)row * p.strideA + k : (size_t)0];
+    if (!ok) xv[u] = 0.0f;
   }
+  __builtin_amdgcn_sched_barrier(0);   // the requests above stay ahead of the weight loads
+  constexpr int G = MT <= 2 ? kSepKC : kSepKC / 4;   // four batch rows leave registers for eight weight rows in flight
+  Row wbuf[G];
+  if (!RAGGED || work) {
+#pragma unroll
+    for (int j = 0; j < G; ++j) wbuf[j] = load_row(kb + j);
+  }
+  const uint32_t blk = kb / 32;
+  const uint16_t *srow = p.S + (size_t)blk * p.scaleStride + cb;
+  // without minima the second pair of loads repeats the scales (dropped later): no condition around a load
+  const uint16_t *mrow = p.S + (size_t)((Q4 && p.affine ? blocksK : 0u) + blk) * p.scaleStride + cb;
+  // whole lanes: the launcher has checked that every lane's scales are 16-byte aligned
+  const bool svec = !RAGGED || (work && ncols == kSepCols && ((uintptr_t)srow & 15u) == 0 && ((uintptr_t)mrow & 15u) == 0);
+  u32x4 sraw[2] = {u32x4{0, 0, 0, 0}, u32x4{0, 0, 0, 0}}, mraw[2] = {u32x4{0, 0, 0, 0}, u32x4{0, 0, 0, 0}};
+  if (svec) {
+    sraw[0] = ld_u32x4(reinterpret_cast<const uint8_t *>(srow));
+    sraw[1] = ld_u32x4(reinterpret_cast<const uint8_t *>(srow) + 16);
+    if (Q4 && (!RAGGED || p.affine)) {
+      mraw[0] = ld_u32x4(reinterpret_cast<const uint8_t *>(mrow));
+      mraw[1] = ld_u32x4(reinterpret_cast<const uint8_t *>(mrow) + 16);
+    }
+  }
+  // every thread stores (slots beyond [MT][128] are never read): a store under a condition would take its load along
+#pragma unroll
+  for (int u = 0; u < XL; ++u) xs[tid + u * 64 * kSepWaves] = xv[u];
   __syncthreads();
 
   // a wave handles exactly one quantization block of k, so the per-block sums become the result in place
@@ -66,84 +137,42 @@ __global__ void __launch_bounds__(64 * kSepWaves, 2) sep_gemv_kernel(SepParams p
     for (int c = 0; c < kSepCols; ++c) bs[m][c] = 0.0f;
   }
 
-  const uint32_t ncols = c0 < p.N ? min((uint32_t)kSepCols, p.N - c0) : 0u;
-  if (k0 < p.K && ncols) {
-    const float *xw = &xs[0][wave * kSepKC];
-    // One k-row of this lane's 16 columns: 16 bytes of int8 or 8 bytes of nibbles (as the low half of a u32x4).
-    auto load_row = [&](uint32_t k) -> u32x4 {
-      u32x4 w = u32x4{0, 0, 0, 0};
-      if (Q4) {
-        const uint8_t *src = p.B + (size_t)k * p.strideB + c0 / 2;
-        if (ncols == kSepCols) {
-          const u32x2 v = ld_u32x2(src);
-          w.x = v.x;
-          w.y = v.y;
-        } else {   // last lane of a ragged row: byte loads inside the row
-          for (uint32_t b = 0; b < (ncols + 1) / 2; ++b) w[b >> 2] |= (uint32_t)src[b] << (8 * (b & 3));
+  if (work) {
+    const float *xw = &xs[wave * kSepKC];
+    auto row_fma = [&](const Row &w, int kk) {
+      float q[kSepCols];
+      if constexpr (Q4) {
+        // low and high nibbles of four bytes at a time (one mask, one shift + mask), then a byte-to-float conversion each
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          uint32_t lo = w[h] & 0x0F0F0F0Fu, hi = (w[h] >> 4) & 0x0F0F0F0Fu;
+          asm volatile("" : "+v"(lo), "+v"(hi));   // known bits would turn every conversion into a bit-field extract + convert
+          q[8 * h + 0] = cvt_ubyte0(lo); q[8 * h + 1] = cvt_ubyte0(hi);
+          q[8 * h + 2] = cvt_ubyte1(lo); q[8 * h + 3] = cvt_ubyte1(hi);
+          q[8 * h + 4] = cvt_ubyte2(lo); q[8 * h + 5] = cvt_ubyte2(hi);
+          q[8 * h + 6] = cvt_ubyte3(lo); q[8 * h + 7] = cvt_ubyte3(hi);
         }
       } else {
-        const uint8_t *src = p.B + (size_t)k * p.strideB + c0;
-        if (ncols == kSepCols) {
-          w = ld_u32x4(src);
-        } else {
-          for (uint32_t b = 0; b < ncols; ++b) w[b >> 2] |= (uint32_t)src[b] << (8 * (b & 3));
-        }
+#pragma unroll
+        for (int c = 0; c < kSepCols; ++c) q[c] = (float)(int)(int8_t)((w[c >> 2] >> (8 * (c & 3))) & 0xFF);
       }
-      return w;
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        float x = xw[m * (kSepWaves * kSepKC) + kk];
+        sx[m] += x;
+#pragma unroll
+        for (int c = 0; c < kSepCols; ++c) bs[m][c] = fmaf(x, q[c], bs[m][c]);
+      }
     };
-    // the block's scales (and minima), fp16 [k/32][scaleStride]: requested before the rows, used after them
-    const uint32_t blk = k0 / 32;
-    const uint16_t *srow = p.S + (size_t)blk * p.scaleStride + c0;
-    const uint16_t *mrow = p.S + (size_t)(blocksK + blk) * p.scaleStride + c0;
-    const bool svec = ncols == kSepCols && ((uintptr_t)srow & 15u) == 0 && ((uintptr_t)mrow & 15u) == 0;
-    u32x4 sraw[2] = {u32x4{0, 0, 0, 0}, u32x4{0, 0, 0, 0}}, mraw[2] = {u32x4{0, 0, 0, 0}, u32x4{0, 0, 0, 0}};
-    if (svec) {
-      sraw[0] = ld_u32x4(reinterpret_cast<const uint8_t *>(srow));
-      sraw[1] = ld_u32x4(reinterpret_cast<const uint8_t *>(srow) + 16);
-      if (Q4 && p.affine) {
-        mraw[0] = ld_u32x4(reinterpret_cast<const uint8_t *>(mrow));
-        mraw[1] = ld_u32x4(reinterpret_cast<const uint8_t *>(mrow) + 16);
-      }
-    }
-    // The 32 rows in four groups of eight: the loads of a group are in flight while the group before it is multiplied
-    // (one load per iteration with its use right behind it left every load's latency exposed: 1.7 TB/s).
-    constexpr int G = 8;
-    u32x4 wbuf[2][G];
 #pragma unroll
-    for (int j = 0; j < G; ++j) wbuf[0][j] = load_row(k0 + j);
-#pragma unroll
-    for (int g = 0; g < kSepKC / G; ++g) {
-      if (g + 1 < kSepKC / G) {
-#pragma unroll
-        for (int j = 0; j < G; ++j) wbuf[(g + 1) & 1][j] = load_row(k0 + (g + 1) * G + j);
-      }
-#pragma unroll
-      for (int j = 0; j < G; ++j) {
-        const u32x4 w = wbuf[g & 1][j];
-        const int kk = g * G + j;
-        float q[kSepCols];
-        if (Q4) {
-#pragma unroll
-          for (int c = 0; c < 8; ++c) {
-            q[c] = (float)((w.x >> (4 * c)) & 0xF);
-            q[8 + c] = (float)((w.y >> (4 * c)) & 0xF);
-          }
-        } else {
-#pragma unroll
-          for (int c = 0; c < kSepCols; ++c) q[c] = (float)(int)(int8_t)((w[c >> 2] >> (8 * (c & 3))) & 0xFF);
-        }
-#pragma unroll
-        for (int m = 0; m < MT; ++m) {
-          float x = xw[m * (kSepWaves * kSepKC) + kk];
-          sx[m] += x;
-#pragma unroll
-          for (int c = 0; c < kSepCols; ++c) bs[m][c] = fmaf(x, q[c], bs[m][c]);
-        }
-      }
+    for (int j = 0; j < kSepKC; ++j) {
+      row_fma(wbuf[j % G], j);
+      if (j + G < kSepKC) wbuf[j % G] = load_row(kb + j + G);   // G < 32: the slot is refilled as soon as it is used
+      if constexpr (G < kSepKC) __builtin_amdgcn_sched_barrier(0);   // keeps the refills from being hoisted into spills
     }
 #pragma unroll
     for (int c = 0; c < kSepCols; ++c) {
-      if ((uint32_t)c < ncols) {
+      if (!RAGGED || (uint32_t)c < ncols) {
         float s, mn = 0.0f;
         if (svec) {
           s = f16bits_to_f32((sraw[c >> 3][(c >> 1) & 3] >> (16 * (c & 1))) & 0xFFFFu);
@@ -161,35 +190,44 @@ __global__ void __launch_bounds__(64 * kSepWaves, 2) sep_gemv_kernel(SepParams p
     }
   }
 
-  // fold the four waves (k blocks) of the workgroup into wave 0, one wave at a time through LDS
-  for (int w = 1; w < kSepWaves; ++w) {
-    if (wave == w) {
+  // fold the four waves (k blocks) of the workgroup into wave 0: one trip through LDS, added in wave order
+  if (wave > 0) {
 #pragma unroll
-      for (int m = 0; m < MT; ++m)
+    for (int m = 0; m < MT; ++m)
 #pragma unroll
-        for (int c = 0; c < kSepCols; ++c) red[m][lane * kSepCols + c] = bs[m][c];
-    }
-    __syncthreads();
-    if (wave == 0) {
-#pragma unroll
-      for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int c = 0; c < kSepCols; ++c) bs[m][c] += red[m][lane * kSepCols + c];
-    }
-    __syncthreads();
+      for (int c4 = 0; c4 < kSepCols / 4; ++c4)
+        red[wave - 1][m][c4][lane] = f32x4{bs[m][4 * c4], bs[m][4 * c4 + 1], bs[m][4 * c4 + 2], bs[m][4 * c4 + 3]};
   }
+  __syncthreads();
   if (wave == 0 && ncols) {
+#pragma unroll
+    for (int w = 0; w < kSepWaves - 1; ++w)
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int c4 = 0; c4 < kSepCols / 4; ++c4) {
+          const f32x4 v = red[w][m][c4][lane];
+          bs[m][4 * c4] += v.x; bs[m][4 * c4 + 1] += v.y; bs[m][4 * c4 + 2] += v.z; bs[m][4 * c4 + 3] += v.w;
+        }
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
       const uint32_t row = p.m0 + m;
+      if (row >= p.M) continue;
+      if (p.nsplit > 1) {   // workspace [split][M][N]
+        float *dst = p.C + ((size_t)blockIdx.y * p.M + row) * p.N + c0;
+        if ((!RAGGED || ncols == kSepCols) && ((uintptr_t)dst & 15u) == 0) {
 #pragma unroll
-      for (int c = 0; c < kSepCols; ++c) {
-        if (row < p.M && (uint32_t)c < ncols) {
-          if (p.nsplit == 1)
-            store_out(p.C, p.epi, 0, (size_t)row * p.strideC + c0 + c, bs[m][c]);
-          else
-            p.C[((size_t)blockIdx.y * p.M + row) * p.N + c0 + c] = bs[m][c];   // workspace [split][M][N]
+          for (int c4 = 0; c4 < kSepCols / 4; ++c4)
+            reinterpret_cast<f32x4 *>(dst)[c4] = f32x4{bs[m][4 * c4], bs[m][4 * c4 + 1], bs[m][4 * c4 + 2], bs[m][4 * c4 + 3]};
+        } else {
+#pragma unroll
+          for (int c = 0; c < kSepCols; ++c)
+            if (!RAGGED || (uint32_t)c < ncols) dst[c] = bs[m][c];
         }
+      } else {
+#pragma unroll
+        for (int c = 0; c < kSepCols; ++c)
+          if (!RAGGED || (uint32_t)c < ncols) store_out(p.C, p.epi, 0, (size_t)row * p.strideC + c0 + c, bs[m][c]);
       }
     }
   }
@@ -206,15 +244,45 @@ __global__ void __launch_bounds__(256) sep_reduce_kernel(const float *ws, float 
   store_out(C, epi, 0, (size_t)row * strideC + n, v);
 }
 
+// The same for four consecutive columns per thread (N a multiple of 4, 16-byte aligned workspace): 16 partial sums
+// requested at a time instead of eight single floats, added in the same order.
+__global__ void __launch_bounds__(256) sep_reduce4_kernel(const float *ws, float *C, Epilogue epi, uint32_t M, uint32_t N,
+                                                          uint32_t strideC, uint32_t m0, uint32_t mcount, uint32_t nsplit) {
+  const uint32_t n4 = N / 4, i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= mcount * n4) return;
+  const uint32_t row = m0 + i / n4, n = (i % n4) * 4;
+  const float *src = ws + (size_t)row * N + n;
+  const size_t step = (size_t)M * N;
+  f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+  uint32_t s = 0;
+  for (; s + 16 <= nsplit; s += 16) {
+    f32x4 t[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) t[u] = *reinterpret_cast<const f32x4 *>(src + (s + u) * step);
+#pragma unroll
+    for (int u = 0; u < 16; ++u) v += t[u];
+  }
+  for (; s < nsplit; ++s) v += *reinterpret_cast<const f32x4 *>(src + s * step);
+#pragma unroll
+  for (int c = 0; c < 4; ++c) store_out(C, epi, 0, (size_t)row * strideC + n + c, v[c]);
+}
+
 template <bool Q4, int MT> static int launch_sep(SepParams p, uint32_t mcount, float *C, void *workspace, hipStream_t stream) {
   dim3 grid((p.N + kSepTile - 1) / kSepTile, p.nsplit);
   float *out = p.nsplit == 1 ? C : reinterpret_cast<float *>(workspace);
   p.C = out;
-  hipLaunchKernelGGL((sep_gemv_kernel<Q4, MT>), grid, dim3(64 * kSepWaves), 0, stream, p);
+  // whole lanes: every lane holds 16 columns and its scales are 16-byte aligned
+  if (p.N % kSepCols == 0 && (uintptr_t)p.S % 16 == 0 && p.scaleStride % 8 == 0)
+    hipLaunchKernelGGL((sep_gemv_kernel<Q4, MT, false>), grid, dim3(64 * kSepWaves), 0, stream, p);
+  else hipLaunchKernelGGL((sep_gemv_kernel<Q4, MT, true>), grid, dim3(64 * kSepWaves), 0, stream, p);
   if (int rc = check_hip(hipGetLastError(), "separated-layout matmul launch")) return rc;
   if (p.nsplit > 1) {
-    hipLaunchKernelGGL(sep_reduce_kernel, dim3((mcount * p.N + 255) / 256), dim3(256), 0, stream,
-                       reinterpret_cast<const float *>(workspace), C, p.epi, p.M, p.N, p.strideC, p.m0, mcount, p.nsplit);
+    if (p.N % 4 == 0 && (uintptr_t)workspace % 16 == 0)
+      hipLaunchKernelGGL(sep_reduce4_kernel, dim3((mcount * (p.N / 4) + 255) / 256), dim3(256), 0, stream,
+                         reinterpret_cast<const float *>(workspace), C, p.epi, p.M, p.N, p.strideC, p.m0, mcount, p.nsplit);
+    else
+      hipLaunchKernelGGL(sep_reduce_kernel, dim3((mcount * p.N + 255) / 256), dim3(256), 0, stream,
+                         reinterpret_cast<const float *>(workspace), C, p.epi, p.M, p.N, p.strideC, p.m0, mcount, p.nsplit);
     return check_hip(hipGetLastError(), "separated-layout reduce launch");
   }
   return CUTHIP_OK;
