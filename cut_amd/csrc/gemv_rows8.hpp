@@ -210,7 +210,13 @@ template <> struct Rows8<CUTHIP_Q6_K> {
   __device__ static void compute(const Raw &r, const half_t *xa, const float *const *sx, const LaneCtx &c,
                                  float (&acc)[R], float (&cacc)[(R + 3) / 4]) {
     constexpr uint32_t kH45 = 0x00300030u, kH89 = 0x03000300u;
-    uint32_t ql[4] = {r.ql.x, r.ql.y, r.ql.z, r.ql.w}, qh[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
+    // The swaps below work in place on single registers.  The ring's 16-byte values pass through this pin as whole
+    // tuples: without it the compiler keeps their halves in separate registers across the loop and copies them out
+    // of a load's destination right behind the load, i.e. it waits for loads it has just issued (s_waitcnt vmcnt(3)
+    // with four steps in flight) and the ring runs one step at a time.
+    u32x4 tql = r.ql, tqh = r.qh;
+    asm volatile("" : "+v"(tql), "+v"(tqh));
+    uint32_t ql[4] = {tql.x, tql.y, tql.z, tql.w}, qh[4] = {tqh.x, tqh.y, tqh.z, tqh.w};
     swap_halves(ql[0], ql[2]); swap_halves(ql[1], ql[3]);
     swap_halves(qh[0], qh[2]); swap_halves(qh[1], qh[3]);
     float d = f16bits_to_f32(r.d);
@@ -301,15 +307,17 @@ template <> struct Rows8<CUTHIP_Q6_K> {
 // 8kg..+7 / 16+8kg..+7 of block 2g and (2,3) / (6,7) those of block 2g+1.
 template <> struct Rows8<CUTHIP_Q8_0> {
   static constexpr int NSUB = 8, SUBK = 32;
-  struct Raw { u32x4 q0, q1; uint32_t d; };
+  // keep: 0xFFFF, or 0 for a block past K (its scale is masked to zero where it is used: touching the loaded value
+  // here would make the load wait for itself and every load before it, and the ring of steps would run in turn)
+  struct Raw { u32x4 q0, q1; uint32_t d, keep; };
   __device__ static void init(LaneCtx &c) { c.c0 = c.c1 = c.c2 = c.c3 = 0; }
   __device__ static void load(Raw &r, const uint8_t *row, uint32_t step, const LaneCtx &c, uint32_t K) {
     uint32_t nblk = K / 32, b = step * 8 + 2 * c.g + c.kg;
     const uint8_t *p = row + (size_t)min(b, nblk - 1) * 34;
     r.q0 = ld_u32x4(p + 2);
     r.q1 = ld_u32x4(p + 18);
-    uint32_t d = ld_u16(p);
-    r.d = b < nblk ? d : 0u;   // blocks past K contribute zero
+    r.d = ld_u16(p);
+    r.keep = b < nblk ? 0xFFFFu : 0u;   // blocks past K contribute zero
   }
   template <int R>
   __device__ static void compute(const Raw &r, const half_t *xa, const float *const *sx, const LaneCtx &c,
@@ -319,7 +327,7 @@ template <> struct Rows8<CUTHIP_Q8_0> {
                      r.q1.x ^ kFlip, r.q1.y ^ kFlip, r.q1.z ^ kFlip, r.q1.w ^ kFlip};
     swap_halves(w[0], w[2]); swap_halves(w[1], w[3]);
     swap_halves(w[4], w[6]); swap_halves(w[5], w[7]);
-    uint32_t da = r.d, db = r.d;
+    uint32_t da = r.d & r.keep, db = da;
     swap_halves(da, db);   // lanes 0-31: (own, partner) ; lanes 32-63: (partner, own) = (block 2g, block 2g+1)
     float d_a = f16bits_to_f32(da), d_b = f16bits_to_f32(db);
     const half8_t *x8 = reinterpret_cast<const half8_t *>(xa);   // elements 64g + 8kg + {0, 16, 32, 48}
@@ -349,7 +357,7 @@ template <> struct Rows8<CUTHIP_Q8_0> {
     constexpr uint32_t kByte = 0x00FF00FFu, kFlip = 0x80808080u;
     const uint32_t w[8] = {r.q0.x ^ kFlip, r.q0.y ^ kFlip, r.q0.z ^ kFlip, r.q0.w ^ kFlip,
                            r.q1.x ^ kFlip, r.q1.y ^ kFlip, r.q1.z ^ kFlip, r.q1.w ^ kFlip};
-    float d = f16bits_to_f32(r.d);
+    float d = f16bits_to_f32(r.d & r.keep);
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
       const u32x4 *x4 = reinterpret_cast<const u32x4 *>(xa + m * xrow);
@@ -370,21 +378,23 @@ template <> struct Rows8<CUTHIP_Q8_0> {
 // of block 2g and (2,3) those of block 2g+1.
 template <> struct Rows8<CUTHIP_Q4_0> {
   static constexpr int NSUB = 8, SUBK = 32;
-  struct Raw { u32x4 q; uint32_t d; };
+  struct Raw { u32x4 q; uint32_t d, keep; };   // keep: as for Q8_0
   __device__ static void init(LaneCtx &c) { c.c0 = c.c1 = c.c2 = c.c3 = 0; }
   __device__ static void load(Raw &r, const uint8_t *row, uint32_t step, const LaneCtx &c, uint32_t K) {
     uint32_t nblk = K / 32, b = step * 8 + 2 * c.g + c.kg;
     const uint8_t *p = row + (size_t)min(b, nblk - 1) * 18;
     r.q = ld_u32x4(p + 2);
-    uint32_t d = ld_u16(p);
-    r.d = b < nblk ? d : 0u;
+    r.d = ld_u16(p);
+    r.keep = b < nblk ? 0xFFFFu : 0u;
   }
   template <int R>
   __device__ static void compute(const Raw &r, const half_t *xa, const float *const *sx, const LaneCtx &c,
                                  float (&acc)[R], float (&cacc)[(R + 3) / 4]) {
-    uint32_t w[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+    u32x4 tq = r.q;
+    asm volatile("" : "+v"(tq));   // the ring's value as a whole tuple up to here (see the Q6_K path)
+    uint32_t w[4] = {tq.x, tq.y, tq.z, tq.w};
     swap_halves(w[0], w[2]); swap_halves(w[1], w[3]);
-    uint32_t da = r.d, db = r.d;
+    uint32_t da = r.d & r.keep, db = da;
     swap_halves(da, db);
     float d_a = f16bits_to_f32(da), d_b = f16bits_to_f32(db);
     const half8_t *x8 = reinterpret_cast<const half8_t *>(xa);   // elements 64g + 8kg + {0, 16, 32, 48}
@@ -414,7 +424,7 @@ template <> struct Rows8<CUTHIP_Q4_0> {
   template <int MT>
   __device__ static void dot(const Raw &r, const half_t *xa, int xrow, const float *sx, int sxrow, const LaneCtx &c,
                              float (&acc)[MT], float (&cacc)[MT]) {
-    float d = f16bits_to_f32(r.d);
+    float d = f16bits_to_f32(r.d & r.keep);
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
       const u32x4 *x4 = reinterpret_cast<const u32x4 *>(xa + m * xrow);
