@@ -37,13 +37,13 @@ Rows8Shape pick_rows8_shape(int fmt, uint32_t M, uint32_t N, uint32_t nsteps) {
     // 5-8 batch rows: every workgroup stages all eight rows of activations (72-80 KB at K = 4096, two workgroups per
     // CU), so fewer, larger workgroups win earlier than at batch 1.  Measured at K = 4096, batch 8, us with
     // (row groups, K ranges) = (1,8) / (1,4) / (2,2) / (8,1):
-    //   1024 rows  Q4_K  6.0 /  8.6 /  9.5 / 10.8    Q6_K  8.1 /  9.3 / 12.1 / 17.8    Q8_0  8.1 /  9.3 / 11.6 / 17.9
-    //   2048 rows  Q4_K  6.5 /  9.0 /  9.7 / 11.2    Q6_K  8.5 /  9.9 / 12.4 / 18.0    Q8_0  8.3 /  9.6 / 11.6 / 18.1
-    //   4096 rows  Q4_K 10.8 / 10.4 /  9.9 / 11.3    Q6_K 14.9 / 11.9 / 12.9 / 18.0    Q8_0 14.5 / 11.8 / 12.0 / 18.0
-    //   6144 rows  Q4_K 15.5 / 16.8 / 11.6 / 11.5    Q6_K 21.3 / 18.4 / 14.9 / 18.2    Q8_0 20.7 / 18.6 / 14.6 / 18.1
-    //   8192 rows  Q4_K 19.4 / 18.5 / 11.8 / 11.6    Q6_K 27.9 / 21.3 / 16.2 / 19.8    Q8_0 27.5 / 22.1 / 16.0 / 19.4
-    //  14336 rows  Q4_K 32.1 / 32.1 / 21.0 / 12.6    Q6_K 51.4 / 39.3 / 30.4 / 22.8    Q8_0 47.4 / 39.9 / 29.4 / 20.9
-    const int want = groups <= 256 ? 8 : groups <= 512 ? 4 : groups < 1536 ? 2 : 1;
+    //   1024 rows  Q4_K  6.0 /  8.5 /  9.5 / 10.8    Q6_K  8.1 /  9.2 / 10.8 / 15.8    Q8_0  8.1 /  9.2 / 10.2 / 16.9
+    //   2048 rows  Q4_K  6.6 /  9.1 /  9.7 / 11.2    Q6_K  8.5 /  9.9 / 11.0 / 15.9    Q8_0  8.5 /  9.6 / 10.3 / 16.9
+    //   4096 rows  Q4_K 11.0 / 10.4 / 10.0 / 11.2    Q6_K 14.7 / 12.1 / 11.6 / 15.9    Q8_0 14.7 / 11.9 / 10.7 / 16.9
+    //   6144 rows  Q4_K 15.1 / 16.5 / 11.5 / 11.3    Q6_K 20.8 / 18.6 / 14.1 / 16.0    Q8_0 20.6 / 18.8 / 13.3 / 17.0
+    //   8192 rows  Q4_K 19.6 / 18.6 / 12.0 / 11.6    Q6_K 26.9 / 21.1 / 14.8 / 16.3    Q8_0 27.6 / 22.3 / 14.7 / 17.7
+    //  14336 rows  Q4_K 32.3 / 32.4 / 21.2 / 12.7    Q6_K 49.7 / 39.8 / 27.1 / 19.7    Q8_0 46.9 / 40.5 / 25.7 / 18.8
+    const int want = groups <= 256 ? 8 : groups < 512 ? 4 : groups < 1536 ? 2 : 1;
     while (kw < want && nsteps / (uint32_t)(2 * kw) >= 2u) kw *= 2;
     return Rows8Shape{kw == 1 ? 8 : kw == 2 ? 2 : 1, kw};
   }
