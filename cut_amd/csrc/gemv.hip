@@ -178,12 +178,13 @@ static cuthip::GemvParams gemv_params(int fmt, const void *W, const void *A, int
 constexpr uint32_t kPassesMaxRows = 40;   // up to here 8-row passes of the decode kernels can beat one tiled GEMM launch
 
 // Costs in microseconds fitted to a sweep over the weight shapes of an 8B model (HIP-graph replay, MI355X): an 8-row
-// pass of the decode kernels 6.5 + weight bytes / 4.3 MB (x 1.45 on rows of K >= 8192, x 1.5 for Q6_K, x 1.55 for both), one launch of
+// pass of the decode kernels 6.5 + weight bytes / 4.3 MB (x 1.45 on rows of K >= 8192, x 1.05 for Q6_K: 14336 x 4096 18.6 us,
+// 28672 x 4096 34.4; x 1.55 for both), one launch of
 // the tiled GEMM on the blocks 62 + weight bytes / 7 MB (its cost is the decode of the whole matrix whatever M is; on
 // rows of K >= 8192 it has too few tiles and is never the better one).
 static double weight_bytes(int fmt, uint32_t K, uint32_t N) { return (double)N * K / cuthip::fmt_elems(fmt) * cuthip::fmt_bytes(fmt); }
 static double passes_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
-  const double f = K >= 8192 ? (fmt == CUTHIP_Q6_K ? 1.55 : 1.45) : (fmt == CUTHIP_Q6_K ? 1.5 : 1.0);
+  const double f = K >= 8192 ? (fmt == CUTHIP_Q6_K ? 1.55 : 1.45) : (fmt == CUTHIP_Q6_K ? 1.05 : 1.0);
   return ((M + 7) / 8) * (6.5 + weight_bytes(fmt, K, N) / 4.3e6) * f;
 }
 // The tiled GEMM with its K split over workgroups (scratch memory at hand, so few 128 x 128 tiles that the launch rule
