@@ -114,7 +114,7 @@ __global__ void __launch_bounds__(256, 2) gemm_q8_i8_kernel(I8Params p) {
   //   B: 128 rows x 4 blocks = 512 blocks, 2 per thread (row = idx >> 2, block = idx & 3): 2 x 16 bytes + scale each
   //   a_scale: threads 0-127 take the four floats of one row
   i32x4 araw[4], braw[2][2];
-  uint32_t bd[2];
+  uint32_t bd[2], bkeep[2];
   f32x4 sraw = {0.0f, 0.0f, 0.0f, 0.0f};
 
   auto load_slice = [&](uint32_t kb0) {   // kb0: first block of the slice
@@ -131,8 +131,11 @@ __global__ void __launch_bounds__(256, 2) gemm_q8_i8_kernel(I8Params p) {
       const uint32_t r = min(n0 + (uint32_t)(idx >> 2), p.N - 1);
       const uint32_t kb = kb0 + (uint32_t)(idx & 3);
       const uint8_t *blk = p.W + (size_t)r * p.row_bytes + (size_t)min(kb, p.nblk - 1) * 34;
-      const uint32_t d = ld_u16(blk);
-      bd[v] = kb < p.nblk ? d : 0u;   // blocks past K get a zero scale: whatever the matrix core sums for them counts nothing
+      bd[v] = ld_u16(blk);
+      // blocks past K get a zero scale (whatever the matrix core sums for them counts nothing): a mask applied where the
+      // scale is used, since a select here would wait for the load, and every load before it, ahead of the MFMAs of
+      // the slice that is meant to hide them
+      bkeep[v] = kb < p.nblk ? 0xFFFFu : 0u;
       braw[v][0] = __builtin_bit_cast(i32x4, ld_u32x4(blk + 2));
       braw[v][1] = __builtin_bit_cast(i32x4, ld_u32x4(blk + 18));
     }
@@ -154,7 +157,7 @@ __global__ void __launch_bounds__(256, 2) gemm_q8_i8_kernel(I8Params p) {
       const int idx = v * 256 + tid, row = idx >> 2, blk = idx & 3;
       *reinterpret_cast<i32x4 *>(Bs + row * kI8Pitch + blk * 32) = braw[v][0];
       *reinterpret_cast<i32x4 *>(Bs + row * kI8Pitch + blk * 32 + 16) = braw[v][1];
-      sw_s[blk][row] = f16bits_to_f32(bd[v]);
+      sw_s[blk][row] = f16bits_to_f32(bd[v] & bkeep[v]);
     }
     if (tid < kI8BM) {
 #pragma unroll
