@@ -237,15 +237,18 @@ template <> struct Step<CUTHIP_Q6_K> {
 // i.e. the fp16 subnormal (q + 128) * 2^-24, and the +128 goes to the sum term.
 template <> struct Step<CUTHIP_Q8_0> {
   static constexpr int NSUB = 8, SUBK = 32;
-  struct Raw { u32x4 q[8]; uint32_t d[8]; };
+  // keep: bit i set if block i of the step lies inside K (blocks past K contribute zero: their scale is dropped where
+  // it is used; a select or a condition around the load here would make the loads of a step wait for each other)
+  struct Raw { u32x4 q[8]; uint32_t d[8]; uint32_t keep; };
   __device__ static void load(Raw &r, const uint8_t *row, uint32_t step, int kg, uint32_t K) {
     uint32_t nblk = K / 32, b0 = step * 8;
+    r.keep = b0 + 8 <= nblk ? 0xFFu : (b0 < nblk ? (1u << (nblk - b0)) - 1u : 0u);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       uint32_t b = min(b0 + i, nblk - 1);
       const uint8_t *p = row + (size_t)b * 34;
       r.q[i] = ld_u32x4(p + 2 + 16 * kg);
-      r.d[i] = (b0 + i < nblk) ? ld_u16(p) : 0u;   // blocks past K contribute zero
+      r.d[i] = ld_u16(p);
     }
   }
   template <int R, int SXROW>
@@ -263,7 +266,7 @@ template <> struct Step<CUTHIP_Q8_0> {
       half8_t bb = as_half8(w.z & kByte, (w.z >> 8) & kByte, w.w & kByte, (w.w >> 8) & kByte);
       f32x16 p = mfma(xa[4 * i + 0], ba, zero16());
       p = mfma(xa[4 * i + 1], bb, p);
-      float d = f16bits_to_f32(valid ? r.d[i] : 0u);
+      float d = f16bits_to_f32((valid && ((r.keep >> i) & 1u)) ? r.d[i] : 0u);
 #pragma unroll
       for (int r_ = 0; r_ < R; ++r_) {
         float t = fmaf(p[r_], kTwo24, -128.0f * sxr[r_][i]);
@@ -277,15 +280,16 @@ template <> struct Step<CUTHIP_Q8_0> {
 // j+16, value (nib - 8) * d.  Lane kg takes bytes 8kg .. 8kg+7 of each block.
 template <> struct Step<CUTHIP_Q4_0> {
   static constexpr int NSUB = 8, SUBK = 32;
-  struct Raw { u32x2 q[8]; uint32_t d[8]; };
+  struct Raw { u32x2 q[8]; uint32_t d[8]; uint32_t keep; };   // keep: as for Q8_0
   __device__ static void load(Raw &r, const uint8_t *row, uint32_t step, int kg, uint32_t K) {
     uint32_t nblk = K / 32, b0 = step * 8;
+    r.keep = b0 + 8 <= nblk ? 0xFFu : (b0 < nblk ? (1u << (nblk - b0)) - 1u : 0u);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       uint32_t b = min(b0 + i, nblk - 1);
       const uint8_t *p = row + (size_t)b * 18;
       r.q[i] = ld_u32x2(p + 2 + 8 * kg);
-      r.d[i] = (b0 + i < nblk) ? ld_u16(p) : 0u;
+      r.d[i] = ld_u16(p);
     }
   }
   template <int R, int SXROW>
@@ -304,7 +308,7 @@ template <> struct Step<CUTHIP_Q4_0> {
       // elements 32i + 8kg + j (low) and 32i + 16 + 8kg + j (high)
       f32x16 p = mfma(xa[4 * i + 0], lo, zero16());
       p = mfma(xa[4 * i + 2], hi, p);
-      float d = f16bits_to_f32(valid ? r.d[i] : 0u);
+      float d = f16bits_to_f32((valid && ((r.keep >> i) & 1u)) ? r.d[i] : 0u);
 #pragma unroll
       for (int r_ = 0; r_ < R; ++r_) {
         float t = fmaf(p[r_], kTwo24, -8.0f * sxr[r_][i]);
