@@ -43,11 +43,12 @@ namespace cuthip {
 #define CUTHIP_ROWS8_DOTMAX 1
 #endif
 constexpr int kRows8DotMax = CUTHIP_ROWS8_DOTMAX;   // batch rows up to which the dot-product path is taken
-// Q6_K keeps the dot-product path up to four rows: its matrix-core path pays 16 sub-block scalings of every
-// accumulator per step (14336 x 4096 at 2 / 4 rows: 15.1 / 18.0 us against 18.9 / 20.2; Q4_K and Q8_0 at 2 rows are
-// faster through the matrix core: 9.4 against 11.3 us, 17.0 against 17.3)
+// Q6_K keeps the dot-product path for two rows (14336 x 4096: 15.3 us either way, 28672 x 4096 25.4 against 26.0) and
+// takes the matrix core from three (3 / 4 rows: 15.6 / 15.8 us against 17.2 / 17.3; before that path's ring of loads
+// was repaired it lost up to four rows, 18.9 / 20.2 against 15.1 / 18.0); Q4_K and Q8_0 at 2 rows are faster through
+// the matrix core: 9.4 against 11.3 us, 17.0 against 17.3
 #ifndef CUTHIP_ROWS8_DOTMAX_Q6K
-#define CUTHIP_ROWS8_DOTMAX_Q6K 4
+#define CUTHIP_ROWS8_DOTMAX_Q6K 2
 #endif
 template <int FMT> constexpr int rows8_dot_max() { return FMT == CUTHIP_Q6_K ? CUTHIP_ROWS8_DOTMAX_Q6K : kRows8DotMax; }
 constexpr int kXGroup = 72;             // halfs per staged 64-element group (64 + 8 pad)
