@@ -30,7 +30,6 @@ Rows8Shape pick_rows8_shape(int fmt, uint32_t M, uint32_t N, uint32_t nsteps) {
     int rwg = 0, kw = 0;
     if (sscanf(env, "%d,%d", &rwg, &kw) == 2 && (kw == 1 || kw == 2 || kw == 4 || kw == 8)) return Rows8Shape{rwg, kw};
   }
-  (void)fmt;   // one rule for all formats so far
   uint32_t groups = (N + 7) / 8;
   int kw = 1;
   if (M > 4) {
@@ -56,7 +55,11 @@ Rows8Shape pick_rows8_shape(int fmt, uint32_t M, uint32_t N, uint32_t nsteps) {
   // 1.3 us per layer of an 8B decode step, whose attention output projection has that shape (batch 1 only: the
   // launch keeps one row group per workgroup for more batch rows); from 4096 rows on: 1024 x 4096 is faster with
   // one row group per workgroup (Q6_K 4.8 us against 5.5)
-  if (kw == 4) return Rows8Shape{groups >= 512 ? 2 : 1, 4};
+  // (5120 and 6144 rows again with one: Q8_0 8.7 us against 9.8, Q6_K 7.3 against 8.1, Q4_K 6.2 against 6.3)
+  if (kw == 4) return Rows8Shape{groups >= 512 && groups < 640 ? 2 : 1, 4};
+  // Q8_0, whose rows are twice as long in bytes, gains from two K ranges on very many rows as well (batch 1, 28672 x
+  // 4096: 27.7 us against 30.4 with eight row groups and one range; 128256 x 4096: 105 against 108)
+  if (fmt == CUTHIP_Q8_0 && M <= 1 && groups >= 3584) return Rows8Shape{2, 2};
   // eight row groups per workgroup from 28672 rows on (fused gate + up of an 8B model: 15.6 us against 16.0-16.2 us)
   return Rows8Shape{groups >= 3584 ? 8 : 4, kw};
 }
