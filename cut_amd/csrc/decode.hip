@@ -182,31 +182,63 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_
   const uint32_t t0 = split * kAttnChunk;
   const uint32_t nvalid = t0 < seqLen ? min((uint32_t)kAttnChunk, seqLen - t0) : 0u;
 
-  // the query of the first pass is requested before anything else: it does not depend on the sequence length, and
-  // loaded after the staging barrier it would cost a memory round trip of its own
-  float q_pre[2] = {0.0f, 0.0f};
+  // Every load of the start-up is requested before the first of them is used, so that the kernel begins with one
+  // memory round trip: the query of the first pass (raw bits, converted later: a conversion right behind the load is a
+  // use, and the compiler then waits for it on the spot), then the chunk of K and V.  Written as a loop with the
+  // store right behind each load, the staging waited for four round trips in turn, and the query for two more.
+  uint32_t q_raw[2] = {0u, 0u};
   {
     const uint32_t h0 = kvH * nRep + (wave < nRep ? wave : 0);
-#pragma unroll
-    for (int e = 0; e < 2; ++e)
-      if (lane + 64 * e < headDim) q_pre[e] = ld_act(q, q_f16, (size_t)h0 * headDim + lane + 64 * e);
-  }
-  // stage the chunk of K and V (16-byte pieces; rows past the sequence are zero)
-  const uint32_t pieces = headDim / 8;
-  for (uint32_t i = tid; i < kAttnChunk * pieces; i += 256) {
-    uint32_t r = i / pieces, c8 = i % pieces;
-    // the loads do not wait for the sequence length (every row below the cache capacity is readable); rows past
-    // the sequence are zeroed afterwards
-    size_t off = (size_t)min(t0 + r, maxSeqLen - 1) * alignedKvDim + kvH * headDim + c8 * 8;
-    u32x4 kv = ld_u32x4(reinterpret_cast<const uint8_t *>(kCache + off));
-    u32x4 vv = ld_u32x4(reinterpret_cast<const uint8_t *>(vCache + off));
-    if (r >= nvalid) {
-      kv = u32x4{0, 0, 0, 0};
-      vv = u32x4{0, 0, 0, 0};
+    const size_t qi = (size_t)h0 * headDim + min(lane, headDim - 1);   // lanes beyond the head dimension read a valid element
+    const size_t qj = (size_t)h0 * headDim + min(lane + 64, headDim - 1);
+    if (q_f16) {
+      q_raw[0] = reinterpret_cast<const uint16_t *>(q)[qi];
+      q_raw[1] = reinterpret_cast<const uint16_t *>(q)[qj];
+    } else {
+      q_raw[0] = reinterpret_cast<const uint32_t *>(q)[qi];
+      q_raw[1] = reinterpret_cast<const uint32_t *>(q)[qj];
     }
-    *reinterpret_cast<u32x4 *>(Ks + r * kAttnRow + c8 * 8) = kv;
-    *reinterpret_cast<u32x4 *>(Vs + r * kAttnRow + c8 * 8) = vv;
   }
+  // stage the chunk of K and V (16-byte pieces; rows past the sequence are zero).  The loads do not wait for the
+  // sequence length (every row below the cache capacity is readable); rows past the sequence are zeroed afterwards.
+  const uint32_t pieces = headDim / 8;
+  if constexpr (HD != 0) {
+    constexpr int IT = kAttnChunk * (HD / 8) / 256;
+    static_assert(IT * 256 == kAttnChunk * (HD / 8), "one 16-byte piece per thread and round");
+    u32x4 kraw[IT], vraw[IT];
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+      const uint32_t i = tid + 256u * it, r = i / (HD / 8), c8 = i % (HD / 8);
+      const size_t off = (size_t)min(t0 + r, maxSeqLen - 1) * alignedKvDim + kvH * headDim + c8 * 8;
+      kraw[it] = ld_u32x4(reinterpret_cast<const uint8_t *>(kCache + off));
+      vraw[it] = ld_u32x4(reinterpret_cast<const uint8_t *>(vCache + off));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+      const uint32_t i = tid + 256u * it, r = i / (HD / 8), c8 = i % (HD / 8);
+      const bool past = r >= nvalid;
+      *reinterpret_cast<u32x4 *>(Ks + r * kAttnRow + c8 * 8) = past ? u32x4{0, 0, 0, 0} : kraw[it];
+      *reinterpret_cast<u32x4 *>(Vs + r * kAttnRow + c8 * 8) = past ? u32x4{0, 0, 0, 0} : vraw[it];
+    }
+  } else {
+    for (uint32_t i = tid; i < kAttnChunk * pieces; i += 256) {
+      uint32_t r = i / pieces, c8 = i % pieces;
+      size_t off = (size_t)min(t0 + r, maxSeqLen - 1) * alignedKvDim + kvH * headDim + c8 * 8;
+      u32x4 kv = ld_u32x4(reinterpret_cast<const uint8_t *>(kCache + off));
+      u32x4 vv = ld_u32x4(reinterpret_cast<const uint8_t *>(vCache + off));
+      if (r >= nvalid) {
+        kv = u32x4{0, 0, 0, 0};
+        vv = u32x4{0, 0, 0, 0};
+      }
+      *reinterpret_cast<u32x4 *>(Ks + r * kAttnRow + c8 * 8) = kv;
+      *reinterpret_cast<u32x4 *>(Vs + r * kAttnRow + c8 * 8) = vv;
+    }
+  }
+  float q_pre[2];
+#pragma unroll
+  for (int e = 0; e < 2; ++e)
+    q_pre[e] = q_f16 ? (float)__builtin_bit_cast(half_t, (uint16_t)q_raw[e]) : __builtin_bit_cast(float, q_raw[e]);
   // query heads of this KV head are handled four at a time, one per wave
   for (uint32_t rep0 = 0; rep0 < nRep; rep0 += 4) {
     const uint32_t rep = rep0 + wave;
