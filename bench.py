@@ -498,6 +498,20 @@ def main():
         extras["q6k_gemv_4096x14336_GBps"] = round((q6[0].numel() + 2 * (N_FF + N_EMBD)) * 60 / (ev_6 * 1e-3) / 1e9, 1)
         del q6, y6
         torch.cuda.empty_cache()
+        # the other three formats at the gate / up shape, batch 1 (the headline is the same launch on Q4_K): bytes of the
+        # blocks + fp16 x and y over the launch time, six copies rotated
+        yf = torch.empty((1, N_FF), dtype=torch.float16, device=dev)
+        for fname in ("Q4_0", "Q6_K", "Q8_0"):
+            wf_h = torch.from_numpy(make_q_weights(fname, 1024, N_EMBD, 7)).to(dev).repeat(N_FF // 1024)   # 1024 rows, repeated
+            wf = [wf_h.clone() for _ in range(COPIES)]
+
+            def gemv_f(s):
+                ops.matmul_gguf(x[:1], wf[s % COPIES], fname, N_FF, N_EMBD, out=yf)
+            _, ev_f, _ = timed_graph(torch, gemv_f, 60, 6)
+            extras[f"{fname.lower()}_gemv_14336x4096_GBps"] = round((wf[0].numel() + 2 * (N_FF + N_EMBD)) * 60 / (ev_f * 1e-3) / 1e9, 1)
+            del wf, wf_h
+            torch.cuda.empty_cache()
+        del yf
         # config 5: prefill GEMM, Q4_K weights, fp16 activations, fp16 MFMA with fp32 accumulate.  The headline keys
         # (q4k_prefill_gemm_*_TFLOPs, *_pct_of_f16_mfma_peak) are this library's own kernels through its own choice
         # by shape; the vendor library's GEMM behind the same dequantization (variant 5, opt-in) is reported under
