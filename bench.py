@@ -298,6 +298,8 @@ def main():
                     help="only run the FFN GEMV step at batch B (2..8), for profiling")
     ap.add_argument("--decode-only", action="store_true",
                     help="only run the 8B-shape decode step (target of rocprofv3 runs)")
+    ap.add_argument("--head-only", action="store_true",
+                    help="only run the batch-1 GEMV at the output-head shape (128256 x 4096) on Q6_K and on Q4_K, for profiling")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it")
@@ -329,6 +331,23 @@ def main():
         return
     if args.q8_only:
         print(json.dumps(bench_q8_prefill(torch, ops, dev, shapes=((2048, N_FF, N_EMBD),), reps=5)))
+        return
+    if args.head_only:
+        res = {}
+        xh = torch.randn((1, N_EMBD), dtype=torch.float16, device=dev)
+        logits = torch.empty((1, 128256), dtype=torch.float16, device=dev)
+        for fname in ("Q6_K", "Q4_K"):
+            head = torch.from_numpy(make_q_weights(fname, 4008, N_EMBD, 3)).to(dev).repeat(32)   # 4008 rows, repeated
+            heads = [head, head.clone()]
+
+            def lm_head(s_):
+                ops.matmul_gguf(xh, heads[s_ % 2], fname, 128256, N_EMBD, out=logits)
+            _, ev_h, _ = timed_graph(torch, lm_head, 20, 3)
+            res[f"{fname.lower()}_gemv_128256x4096_GBps"] = round((head.numel() + 2 * (N_EMBD + 128256)) * 20 / (ev_h * 1e-3) / 1e9, 1)
+            res[f"{fname.lower()}_gemv_128256x4096_us"] = round(ev_h * 1e3 / 20, 1)
+            del heads, head
+            torch.cuda.empty_cache()
+        print(json.dumps(res))
         return
     if args.decode_only:
         x_h = np.random.default_rng(1).standard_normal((8, N_EMBD), dtype=np.float32).astype(np.float16)
