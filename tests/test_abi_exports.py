@@ -83,6 +83,33 @@ def test_separated_layout_entry_points_take_the_variant_index():
     assert lib.cuthip_matmul_sep_workspace_bytes_for(L.OP_MATMUL_Q4, 4, 1, 4096, 4096) >= 4096 * 4096 * 2
 
 
+def test_batched_gemv_workspace_covers_the_k_ranges_its_lds_budget_forces():
+    """Host logic of the workspace sizing for 2..8 batch rows (no device needed): the K split of the 8-row GEMV takes
+    enough ranges for one workgroup of eight waves per CU, and beyond that as many as it needs for the activations of
+    one range (8 batch rows x 576 + 32 bytes per 256 elements; 640 for Q6_K) to fit 96 KB of LDS; the workspace holds
+    one fp32 [M, N] per range.  Ranges are a power of two."""
+    lib = L.load()
+    Q4_K, Q6_K = L.FORMATS["Q4_K"], L.FORMATS["Q6_K"]
+
+    def ranges(fmt, M, K, N):
+        b = lib.cuthip_matmul_gguf_workspace_bytes(fmt, M, K, N, L.F16)
+        assert b % (M * N * 4) == 0
+        return b // (M * N * 4)
+    # few weight rows: the occupancy rule alone (16 ranges at most from it), 4096 x 14336 at batch 8: 4 ranges of 14 steps
+    assert ranges(Q4_K, 8, 14336, 4096) == 4
+    # many weight rows on K = 8192: the chip is full without a split, but 8 rows x 32 steps x 608 B = 152 KB: 2 ranges
+    assert ranges(Q4_K, 8, 8192, 28672) == 2
+    assert ranges(Q6_K, 8, 8192, 28672) == 2
+    # 4 rows of K = 8192 fit (76 / 80 KB): no K split is preferred for that many weight rows, the workspace is the
+    # prefill one (fp16 copy of the weights) as for any other shape
+    assert lib.cuthip_matmul_gguf_workspace_bytes(Q4_K, 4, 8192, 28672, L.F16) >= 28672 * 8192 * 2
+    # very long rows on few weight rows: 16 ranges from the occupancy rule leave 22 steps each, 8 x 22 x 608 B = 107 KB:
+    # doubled once more
+    assert ranges(Q4_K, 8, 90112, 16) == 32
+    # two rows of K = 28672 (2 x 112 x 608 B = 136 KB)
+    assert ranges(Q4_K, 2, 28672, 8192) >= 2
+
+
 def test_default_variant_of_the_gguf_table_is_valid_for_every_m():
     lib = L.load()
     assert lib.cuthip_variant_default(L.OP_MATMUL_GGUF) == 0
