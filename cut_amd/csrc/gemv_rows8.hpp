@@ -197,7 +197,16 @@ template <> struct Rows8<CUTHIP_Q6_K> {
   // (one 16-byte load per lane, the same address for the 8 lanes of a row, 2-byte aligned) cost a tenth of the kernel:
   // 128256 x 4096 at batch 1 102.6 us with the 16-byte load, 94.3 with this one, 104.9 with two 2-byte loads of just
   // the byte pairs a lane uses (an instruction more), 78 without any scale load.
-  struct Raw { u32x4 ql, qh; u32x2 sc; uint32_t d; };
+  // qh: this lane's half (8 bytes: sigma picks which) of the 16 high-bit bytes that it shares with its neighbour of the
+  // other sigma; the two halves are exchanged with DPP moves inside the quad where they are used
+  struct Raw { u32x4 ql; u32x2 qh, sc; uint32_t d; };
+  __device__ static void high_bits(const u32x2 &h, uint32_t (&qh)[4]) {
+    const int a = (int)h.x, b = (int)h.y;
+    qh[0] = (uint32_t)__builtin_amdgcn_mov_dpp(a, 0xA0, 0xF, 0xF, true);   // quad_perm [0,0,2,2]: the sigma = 0 lane's half
+    qh[1] = (uint32_t)__builtin_amdgcn_mov_dpp(b, 0xA0, 0xF, 0xF, true);
+    qh[2] = (uint32_t)__builtin_amdgcn_mov_dpp(a, 0xF5, 0xF, 0xF, true);   // quad_perm [1,1,3,3]: the sigma = 1 lane's half
+    qh[3] = (uint32_t)__builtin_amdgcn_mov_dpp(b, 0xF5, 0xF, 0xF, true);
+  }
   __device__ static void init(LaneCtx &c) {
     c.c0 = 2u * (c.g & 1);        // qh bit offset of quarter sigma
     c.c1 = 16u * (c.g & 1);       // bit offset of scale byte pair (2 sigma, 2 sigma + 1) inside its dword
@@ -207,7 +216,7 @@ template <> struct Rows8<CUTHIP_Q6_K> {
   __device__ static void load(Raw &r, const uint8_t *row, uint32_t step, const LaneCtx &c, uint32_t) {
     const uint8_t *p = row + (size_t)step * 210;
     r.ql = ld_u32x4(p + 32 * c.g + 16 * c.kg);
-    r.qh = ld_u32x4(p + 128 + 32 * (c.g >> 1) + 16 * c.kg);
+    r.qh = ld_u32x2(p + 128 + 32 * (c.g >> 1) + 16 * c.kg + 8 * (c.g & 1));
     r.sc = ld_u32x2(p + 192 + 8 * c.c2);
     r.d = ld_u16(p + 208);
   }
@@ -219,9 +228,11 @@ template <> struct Rows8<CUTHIP_Q6_K> {
     // tuples: without it the compiler keeps their halves in separate registers across the loop and copies them out
     // of a load's destination right behind the load, i.e. it waits for loads it has just issued (s_waitcnt vmcnt(3)
     // with four steps in flight) and the ring runs one step at a time.
-    u32x4 tql = r.ql, tqh = r.qh;
+    u32x4 tql = r.ql;
+    u32x2 tqh = r.qh;
     asm volatile("" : "+v"(tql), "+v"(tqh));
-    uint32_t ql[4] = {tql.x, tql.y, tql.z, tql.w}, qh[4] = {tqh.x, tqh.y, tqh.z, tqh.w};
+    uint32_t ql[4] = {tql.x, tql.y, tql.z, tql.w}, qh[4];
+    high_bits(tqh, qh);
     swap_halves(ql[0], ql[2]); swap_halves(ql[1], ql[3]);
     swap_halves(qh[0], qh[2]); swap_halves(qh[1], qh[3]);
     float d = f16bits_to_f32(r.d);
@@ -269,7 +280,9 @@ template <> struct Rows8<CUTHIP_Q6_K> {
   __device__ static void dot(const Raw &r, const half_t *xa, int xrow, const float *sx, int sxrow, const LaneCtx &c,
                              float (&acc)[MT], float (&cacc)[MT]) {
     constexpr uint32_t kH45 = 0x00300030u, kH89 = 0x03000300u;
-    const uint32_t ql[4] = {r.ql.x, r.ql.y, r.ql.z, r.ql.w}, qh[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
+    const uint32_t ql[4] = {r.ql.x, r.ql.y, r.ql.z, r.ql.w};
+    uint32_t qh[4];
+    high_bits(r.qh, qh);
     uint32_t vl[8], vh[8];   // 6-bit quants as fp16 subnormals: q * 2^-24 (quarter sigma) and q * 2^-20 (quarter sigma+2)
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
