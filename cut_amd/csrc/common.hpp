@@ -34,10 +34,12 @@ __host__ __device__ inline int fmt_bytes(int fmt) {
 // serves unaligned vector loads from global memory, so wide loads go through
 // packed views and the compiler still emits global_load_dwordx2/x4.
 struct __attribute__((packed, aligned(2))) U16x1 { uint16_t v; };
+struct __attribute__((packed, aligned(2))) U32x1p { uint32_t v; };
 struct __attribute__((packed, aligned(2))) U32x2p { uint32_t v[2]; };
 struct __attribute__((packed, aligned(2))) U32x4p { uint32_t v[4]; };
 
 __device__ inline uint32_t ld_u16(const uint8_t *p) { return reinterpret_cast<const U16x1 *>(p)->v; }
+__device__ inline uint32_t ld_u32(const uint8_t *p) { return reinterpret_cast<const U32x1p *>(p)->v; }
 __device__ inline u32x2 ld_u32x2(const uint8_t *p) {
   U32x2p t = *reinterpret_cast<const U32x2p *>(p);
   return u32x2{t.v[0], t.v[1]};
