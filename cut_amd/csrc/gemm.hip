@@ -90,13 +90,17 @@ template <> struct Sub<CUTHIP_Q4_K> {
 };
 
 template <> struct Sub<CUTHIP_Q6_K> {
-  struct Raw { u32x4 ql[2]; u32x4 qh[2]; uint32_t sc, d; };
+  // qh1: half of the 32 high-bit bytes of the block's half H.  The two threads of a pair (tid, tid ^ 1: the two
+  // sub-blocks of one weight row in a slice) need the same 32 bytes; the even one loads the first 16, the odd one the
+  // second 16, and decode() exchanges them inside the quad.  The blocks are 2-byte aligned, and what such loads return
+  // through the vector memory path is what the decode of this format is short of.
+  struct Raw { u32x4 ql[2]; u32x4 qh1; uint32_t sc, d; };
   __device__ static void load(Raw &r, const uint8_t *row, uint32_t sub) {
     const uint8_t *blk = row + (size_t)(sub >> 3) * 210;
     uint32_t H = (sub >> 2) & 1, s = sub & 3;
     const uint8_t *ql = blk + 64 * H + 32 * (s & 1), *qh = blk + 128 + 32 * H;
     r.ql[0] = ld_u32x4(ql); r.ql[1] = ld_u32x4(ql + 16);
-    r.qh[0] = ld_u32x4(qh); r.qh[1] = ld_u32x4(qh + 16);
+    r.qh1 = ld_u32x4(qh + 16 * (threadIdx.x & 1));
     r.sc = ld_u16(blk + 192 + 8 * H + 2 * s);
     r.d = ld_u16(blk + 208);
   }
@@ -106,9 +110,15 @@ template <> struct Sub<CUTHIP_Q6_K> {
     float dsc0 = d * (float)(int)(int8_t)(r.sc & 0xFF), dsc1 = d * (float)(int)(int8_t)(r.sc >> 8);
     const float off0 = -32.0f * dsc0, off1 = -32.0f * dsc1;
     uint32_t lsh = (s >> 1) * 4, hsh = 2 * s;
+    uint32_t qh[8];   // quad_perm [0,0,2,2]: the even thread's 16 bytes; [1,1,3,3]: the odd thread's
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      qh[i] = (uint32_t)__builtin_amdgcn_mov_dpp((int)r.qh1[i], 0xA0, 0xF, 0xF, true);
+      qh[4 + i] = (uint32_t)__builtin_amdgcn_mov_dpp((int)r.qh1[i], 0xF5, 0xF, 0xF, true);
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      uint32_t wl = i < 4 ? r.ql[0][i] : r.ql[1][i - 4], wh = i < 4 ? r.qh[0][i] : r.qh[1][i - 4];
+      uint32_t wl = i < 4 ? r.ql[0][i] : r.ql[1][i - 4], wh = qh[i];
       uint32_t q6 = ((wl >> lsh) & 0x0F0F0F0Fu) | (((wh >> hsh) & 0x03030303u) << 4);
       asm volatile("" : "+v"(q6));
       // dsc * (q - 32) as one fused multiply-add with the exact constant -32 dsc: the same real number rounded once,
