@@ -682,9 +682,12 @@ size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
 // Cost models in microseconds for the automatic choice between the two-pass path and the single-launch GEMM, fitted to
 // a sweep over the weight shapes of an 8B model (all formats, M = 16 .. 2048, HIP-graph replay, MI355X):
 //   two-pass      3 + N K (bytes per weight + 2) / 6.0 MB   the dequantization (reads the blocks, writes fp16)
-//                 + 17 + 2 ceil128(M) N K / 1.25 PFLOP/s     the dense GEMM (tiles are at least 128 rows high)
+//                 + 17 + max(2 ceil128(M) N K / 1.25 PFLOP/s,  the dense GEMM (tiles are at least 128 rows high; up to 256 rows
+//                            2 N K / 3.5 MB)                  it is bound by reading the fp16 weights: 128 and 256 x 28672 x 4096
+//                                                             both take 147-148 us on Q6_K, 14336 x 4096 76 and 79)
 //   single launch K x c_fmt x max(1, tiles / 256)            c = 14.7 ns (Q4_K, Q4_0), 17 ns (Q8_0: 256 x 28672 x 4096 122 us,
-//                 512 rows 220, 256 x 14336 x 4096 73-76), 23.5 ns (Q6_K):
+//                 512 rows 220, 256 x 14336 x 4096 73-76), 19.5 ns (Q6_K: 256 x 28672 x 4096 133-139 us,
+//                 512 x 14336 x 4096 139):
 //                 a workgroup decodes its K-long strip of weights once per 128 rows of A, and nothing overlaps that
 //                 walk until every CU holds more than one 128 x 128 tile.
 // Measured against them (Q4_K, M x N x K): 64 x 4096 x 4096 38 / 62 us, 512 x 14336 x 4096 99 / 105, 512 x 28672 x 4096
@@ -693,10 +696,11 @@ size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16) {
 double dense_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
   const double nk = (double)N * K, bpw = (double)fmt_bytes(fmt) / fmt_elems(fmt);
   const double split = pick_dense_shape(M, K, N).ksplit > 1 ? 5.0 : 0.0;
-  return 3.0 + nk * (bpw + 2.0) / 6.0e6 + 17.0 + 2.0 * (double)((M + 127) / 128 * 128) * nk / 1.25e9 + split;
+  const double mfma = 2.0 * (double)((M + 127) / 128 * 128) * nk / 1.25e9, stream = 2.0 * nk / 3.5e6;
+  return 3.0 + nk * (bpw + 2.0) / 6.0e6 + 17.0 + (mfma > stream ? mfma : stream) + split;
 }
 double single_launch_rows_cost_us(int fmt, uint32_t M, uint32_t K, uint32_t N) {
-  const double c = fmt == CUTHIP_Q6_K ? 23.5e-3 : fmt == CUTHIP_Q8_0 ? 17.0e-3 : 14.7e-3;
+  const double c = fmt == CUTHIP_Q6_K ? 19.5e-3 : fmt == CUTHIP_Q8_0 ? 17.0e-3 : 14.7e-3;
   const double tiles = (double)((M + 127) / 128) * ((N + 127) / 128);
   return K * c * (tiles > 256.0 ? tiles / 256.0 : 1.0);
 }
