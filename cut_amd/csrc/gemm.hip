@@ -94,20 +94,24 @@ template <> struct Sub<CUTHIP_Q6_K> {
   // sub-blocks of one weight row in a slice) need the same 32 bytes; the even one loads the first 16, the odd one the
   // second 16, and decode() exchanges them inside the quad.  The blocks are 2-byte aligned, and what such loads return
   // through the vector memory path is what the decode of this format is short of.
-  struct Raw { u32x4 ql[2]; u32x4 qh1; uint32_t sc, d; };
+  // sd: the even thread loads the pair's two scale bytes (they are adjacent), the odd one the last scale bytes and d;
+  // one small load per thread and slice instead of two.
+  struct Raw { u32x4 ql[2]; u32x4 qh1; uint32_t sd; };
   __device__ static void load(Raw &r, const uint8_t *row, uint32_t sub) {
     const uint8_t *blk = row + (size_t)(sub >> 3) * 210;
     uint32_t H = (sub >> 2) & 1, s = sub & 3;
     const uint8_t *ql = blk + 64 * H + 32 * (s & 1), *qh = blk + 128 + 32 * H;
     r.ql[0] = ld_u32x4(ql); r.ql[1] = ld_u32x4(ql + 16);
     r.qh1 = ld_u32x4(qh + 16 * (threadIdx.x & 1));
-    r.sc = ld_u16(blk + 192 + 8 * H + 2 * s);
-    r.d = ld_u16(blk + 208);
+    r.sd = ld_u32((threadIdx.x & 1) ? blk + 206 : blk + 192 + 8 * H + 2 * (s & 2));
   }
   __device__ static void decode(const Raw &r, uint32_t sub, half_t (&w)[32]) {
     uint32_t s = sub & 3;
-    float d = f16bits_to_f32(r.d);
-    float dsc0 = d * (float)(int)(int8_t)(r.sc & 0xFF), dsc1 = d * (float)(int)(int8_t)(r.sc >> 8);
+    const uint32_t sc2 = (uint32_t)__builtin_amdgcn_mov_dpp((int)r.sd, 0xA0, 0xF, 0xF, true);   // the pair's scales
+    const uint32_t dd = (uint32_t)__builtin_amdgcn_mov_dpp((int)r.sd, 0xF5, 0xF, 0xF, true);    // d in the high half
+    const uint32_t sc = (threadIdx.x & 1) ? sc2 >> 16 : sc2 & 0xFFFF;
+    float d = f16bits_to_f32(dd >> 16);
+    float dsc0 = d * (float)(int)(int8_t)(sc & 0xFF), dsc1 = d * (float)(int)(int8_t)(sc >> 8);
     const float off0 = -32.0f * dsc0, off1 = -32.0f * dsc1;
     uint32_t lsh = (s >> 1) * 4, hsh = 2 * s;
     uint32_t qh[8];   // quad_perm [0,0,2,2]: the even thread's 16 bytes; [1,1,3,3]: the odd thread's
