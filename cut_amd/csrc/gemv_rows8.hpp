@@ -199,7 +199,10 @@ template <> struct Rows8<CUTHIP_Q6_K> {
   // the byte pairs a lane uses (an instruction more), 78 without any scale load.
   // qh: this lane's half (8 bytes: sigma picks which) of the 16 high-bit bytes that it shares with its neighbour of the
   // other sigma; the two halves are exchanged with DPP moves inside the quad where they are used
-  struct Raw { u32x4 ql; u32x2 qh; uint32_t sc, d; };   // sc: scale dword 2H + sigma; the neighbour of the other sigma holds the other one
+  // sd: one dword.  In the kg = 0 lane scale dword 2H + sigma (the neighbour of the other sigma holds the other one of
+  // the half), in the kg = 1 lane bytes 206-209 of the block (d in the upper half); the two lanes exchange them where
+  // they are used, one load per lane and step less than with d loaded by every lane.
+  struct Raw { u32x4 ql; u32x2 qh; uint32_t sd; };
   __device__ static void high_bits(const u32x2 &h, uint32_t (&qh)[4]) {
     const int a = (int)h.x, b = (int)h.y;
     qh[0] = (uint32_t)__builtin_amdgcn_mov_dpp(a, 0xA0, 0xF, 0xF, true);   // quad_perm [0,0,2,2]: the sigma = 0 lane's half
@@ -211,14 +214,20 @@ template <> struct Rows8<CUTHIP_Q6_K> {
     c.c0 = 2u * (c.g & 1);        // qh bit offset of quarter sigma
     c.c1 = 16u * (c.g & 1);       // bit offset of scale byte pair (2 sigma, 2 sigma + 1) inside its dword
     c.c2 = (uint32_t)(c.g >> 1);  // H
-    c.c3 = 0;
+    c.c3 = c.kg ? 206u : 192u + 8u * c.c2 + 2u * c.c0;   // byte offset of this lane's dword sd
+  }
+  // both lanes of a pair: the scale dword of its kg = 0 lane and d from its kg = 1 lane
+  __device__ static void scales_and_d(uint32_t sd, uint32_t &sc, float &d) {
+    uint32_t a = sd, b = sd;
+    swap_halves(a, b);
+    sc = a;
+    d = f16bits_to_f32(b >> 16);
   }
   __device__ static void load(Raw &r, const uint8_t *row, uint32_t step, const LaneCtx &c, uint32_t) {
     const uint8_t *p = row + (size_t)step * 210;
     r.ql = ld_u32x4(p + 32 * c.g + 16 * c.kg);
     r.qh = ld_u32x2(p + 128 + 32 * (c.g >> 1) + 16 * c.kg + 8 * (c.g & 1));
-    r.sc = ld_u32(p + 192 + 8 * c.c2 + 2 * c.c0);   // c0 = 2 sigma
-    r.d = ld_u16(p + 208);
+    r.sd = ld_u32(p + c.c3);
   }
   template <int R>
   __device__ static void compute(const Raw &r, const half_t *xa, const float *const *sx, const LaneCtx &c,
@@ -235,9 +244,11 @@ template <> struct Rows8<CUTHIP_Q6_K> {
     high_bits(tqh, qh);
     swap_halves(ql[0], ql[2]); swap_halves(ql[1], ql[3]);
     swap_halves(qh[0], qh[2]); swap_halves(qh[1], qh[3]);
-    float d = f16bits_to_f32(r.d);
-    uint32_t wlo = (uint32_t)__builtin_amdgcn_mov_dpp((int)r.sc, 0xA0, 0xF, 0xF, true);   // dword 2H (quarter sigma), from the sigma = 0 lane
-    uint32_t whi = (uint32_t)__builtin_amdgcn_mov_dpp((int)r.sc, 0xF5, 0xF, 0xF, true);   // dword 2H+1 (quarter sigma+2), from the sigma = 1 lane
+    float d;
+    uint32_t sc;
+    scales_and_d(r.sd, sc, d);
+    uint32_t wlo = (uint32_t)__builtin_amdgcn_mov_dpp((int)sc, 0xA0, 0xF, 0xF, true);   // dword 2H (quarter sigma), from the sigma = 0 lane
+    uint32_t whi = (uint32_t)__builtin_amdgcn_mov_dpp((int)sc, 0xF5, 0xF, 0xF, true);   // dword 2H+1 (quarter sigma+2), from the sigma = 1 lane
     const half8_t *x8 = reinterpret_cast<const half8_t *>(xa);
     // x8 offsets (in 8-half chunks): quarter sigma, lam: 2*lam ; quarter sigma+2, lam: 9 + 2*lam  (72 halfs = 9 chunks)
 #pragma unroll
@@ -293,9 +304,11 @@ template <> struct Rows8<CUTHIP_Q6_K> {
       vh[2 * k] = (w & kNibHi) | (hl & kH89);
       vh[2 * k + 1] = (w8 & kNibHi) | (hr & kH89);
     }
-    float d = f16bits_to_f32(r.d);
-    uint32_t wlo = (uint32_t)__builtin_amdgcn_mov_dpp((int)r.sc, 0xA0, 0xF, 0xF, true);
-    uint32_t whi = (uint32_t)__builtin_amdgcn_mov_dpp((int)r.sc, 0xF5, 0xF, 0xF, true);
+    float d;
+    uint32_t sc;
+    scales_and_d(r.sd, sc, d);
+    uint32_t wlo = (uint32_t)__builtin_amdgcn_mov_dpp((int)sc, 0xA0, 0xF, 0xF, true);
+    uint32_t whi = (uint32_t)__builtin_amdgcn_mov_dpp((int)sc, 0xF5, 0xF, 0xF, true);
     float dlo = d * (float)(int)__builtin_amdgcn_sbfe((int)wlo, c.c1, 8);
     float dhi = d * (float)(int)__builtin_amdgcn_sbfe((int)whi, c.c1, 8);
     const int j_lo = 8 * (c.g >> 1) + 2 * (c.g & 1) + c.kg;
