@@ -46,14 +46,19 @@ __global__ void __launch_bounds__(256) long_epilogue_kernel(void *C, int c_f16, 
   store_plain(C, c_f16, idx, v);
 }
 
+int check_long_epilogue_alias(int epilogue, int op, const void *C, const void *D) {
+  if (epilogue == CUTHIP_EPI_BINARY && D == C) {
+    set_error("binary operator %d is applied after the matmul, in a launch of its own: D must not alias C", op);
+    return CUTHIP_ERR_INVALID;
+  }
+  return CUTHIP_OK;
+}
+
 int launch_long_epilogue(void *C, int c_f16, uint32_t M, uint32_t N, uint32_t strideC, int epilogue, int op, const void *D,
                          hipStream_t stream) {
   const uint64_t total = (uint64_t)M * N;
   if (total == 0) return CUTHIP_OK;
-  if (epilogue == CUTHIP_EPI_BINARY && D == C) {   // the unfused matmul has already overwritten what D held
-    set_error("binary operator %d is applied after the matmul, in a launch of its own: D must not alias C", op);
-    return CUTHIP_ERR_INVALID;
-  }
+  if (int rc = check_long_epilogue_alias(epilogue, op, C, D)) return rc;   // (the entry points check before the matmul)
   hipLaunchKernelGGL(long_epilogue_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, stream, C, c_f16, M, N,
                      strideC, epilogue, op, D);
   return check_hip(hipGetLastError(), "epilogue launch");
@@ -146,8 +151,46 @@ __global__ void __launch_bounds__(256) read_probe_kernel(const u32x4 *src, size_
 
 namespace cuthip {
 bool blaslt_available();
-bool blaslt_preferred();
 int attn_static_setup();
+Tuning g_tuning;
+
+// One key of the launch-shape overrides; value nullptr or "" restores the library's own choice for that key.
+static int set_tuning_key(const char *key, const char *value) {
+  const bool clear = !value || !value[0];
+  int a = 0, b = 0, c = 1;
+  if (!strcmp(key, "rows8_shape")) {
+    if (clear) { g_tuning.rows8_rwg = g_tuning.rows8_kw = 0; return CUTHIP_OK; }
+    if (sscanf(value, "%d,%d", &a, &b) == 2 && a >= 1 && (b == 1 || b == 2 || b == 4 || b == 8)) {
+      g_tuning.rows8_rwg = a; g_tuning.rows8_kw = b; return CUTHIP_OK;
+    }
+  } else if (!strcmp(key, "gemv_shape")) {
+    if (clear) { g_tuning.gemv_kp = g_tuning.gemv_waves = 0; return CUTHIP_OK; }
+    if (sscanf(value, "%d,%d", &a, &b) == 2 && (a == 1 || a == 2) && (b == 1 || b == 2 || b == 4 || b == 8)) {
+      g_tuning.gemv_kp = a; g_tuning.gemv_waves = b; return CUTHIP_OK;
+    }
+  } else if (!strcmp(key, "gemm_ksplit")) {
+    if (clear) { g_tuning.gemm_ksplit = 0; return CUTHIP_OK; }
+    if (sscanf(value, "%d", &a) == 1 && a >= 1 && a <= 16) { g_tuning.gemm_ksplit = a; return CUTHIP_OK; }
+  } else if (!strcmp(key, "dense_tile")) {
+    if (clear) { g_tuning.dense_bm = g_tuning.dense_bn = 0; g_tuning.dense_ks = 1; return CUTHIP_OK; }
+    const int got = sscanf(value, "%d,%d,%d", &a, &b, &c);
+    if (got >= 2 && ((b == 256 && (a == 256 || a == 128)) || (b == 448 && a == 128) || (b == 224 && a == 256)) &&
+        (c == 1 || c == 2 || c == 4 || c == 8)) {
+      g_tuning.dense_bm = a; g_tuning.dense_bn = b; g_tuning.dense_ks = c; return CUTHIP_OK;
+    }
+  } else if (!strcmp(key, "dense_mfma16")) {
+    if (clear) { g_tuning.dense_mfma16 = 1; return CUTHIP_OK; }
+    if (sscanf(value, "%d", &a) == 1) { g_tuning.dense_mfma16 = a != 0; return CUTHIP_OK; }
+  } else if (!strcmp(key, "dense_pf")) {
+    if (clear) { g_tuning.dense_pf = -1; return CUTHIP_OK; }
+    if (sscanf(value, "%d", &a) == 1 && a >= 0) { g_tuning.dense_pf = a; return CUTHIP_OK; }
+  } else {
+    set_error("cuthip_set_tuning: unknown key '%s' (rows8_shape, gemv_shape, gemm_ksplit, dense_tile, dense_mfma16, dense_pf)", key);
+    return CUTHIP_ERR_INVALID;
+  }
+  set_error("cuthip_set_tuning: value '%s' is not valid for key '%s'", value, key);
+  return CUTHIP_ERR_INVALID;
+}
 }
 using namespace cuthip;
 
@@ -173,10 +216,13 @@ int cuthip_init(int device) {
     set_error("cuthip_init: device %d is %s; this library is built for gfx950 only", device, p.gcnArchName);
     return CUTHIP_ERR_NO_DEVICE;
   }
-  // hipBLASLt (variant 5 of the prefill matmul) is opt-in: a process that sets CUT_HIP_VENDOR_GEMM opens it now,
-  // because its handle must not be created inside a stream capture, where the first matmul of a caller may well
-  // run; absence of the library is not an error
-  (void)cuthip::blaslt_preferred();
+  // the launch-shape overrides of the environment are taken over here, once: no launcher calls getenv.  A value that
+  // does not parse is ignored, as an unset variable is.
+  static const struct { const char *env, *key; } kEnv[] = {
+      {"CUT_HIP_ROWS8_SHAPE", "rows8_shape"}, {"CUT_HIP_GEMV_SHAPE", "gemv_shape"},   {"CUT_HIP_GEMM_KSPLIT", "gemm_ksplit"},
+      {"CUT_HIP_DENSE_TILE", "dense_tile"},   {"CUT_HIP_DENSE_MFMA16", "dense_mfma16"}, {"CUT_HIP_DENSE_PF", "dense_pf"}};
+  for (const auto &e : kEnv)
+    if (const char *v = getenv(e.env)) (void)set_tuning_key(e.key, v);
   // device address of the built-in attention scratch on this device (cuthip_attn_decode_static)
   return cuthip::attn_static_setup();
 }
@@ -225,7 +271,21 @@ int cuthip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream) {
   return check_hip(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream), "hipMemcpyAsync d2d");
 }
 int cuthip_memset(void *dst, int value, size_t bytes, void *stream) {
+  // not under capture: memset nodes have given wrong results on replays of a graph on this part
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (stream && hipStreamIsCapturing((hipStream_t)stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone) {
+    set_error("cuthip_memset: the stream is capturing; clear the memory before the capture or with a kernel of the sequence");
+    return CUTHIP_ERR_INVALID;
+  }
   return check_hip(hipMemsetAsync(dst, value, bytes, (hipStream_t)stream), "hipMemsetAsync");
+}
+
+int cuthip_set_tuning(const char *key, const char *value) {
+  if (!key) {
+    set_error("cuthip_set_tuning: null key");
+    return CUTHIP_ERR_INVALID;
+  }
+  return set_tuning_key(key, value);
 }
 
 int cuthip_stream_create(void **stream) {

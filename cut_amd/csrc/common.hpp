@@ -233,5 +233,20 @@ int check_epilogue_op(const char *who, int epilogue, int op);
 // matmul whose fused operator is one of those (C and D are [M, strideC] of fp16 or fp32)
 int launch_long_epilogue(void *C, int c_f16, uint32_t M, uint32_t N, uint32_t strideC, int epilogue, int op, const void *D,
                          hipStream_t stream);
+// CUTHIP_ERR_INVALID (error set) when a binary operator that runs as a launch of its own would find its operand D
+// already overwritten by the matmul (D == C); checked by the entry points before the unfused matmul is launched
+int check_long_epilogue_alias(int epilogue, int op, const void *C, const void *D);
+
+// Launch-shape overrides for tests and tuning sweeps.  Written by cuthip_set_tuning and, once, by cuthip_init from the
+// CUT_HIP_* environment variables; the launchers only read this struct (no getenv on a launch path).  0 / -1 = unset.
+struct Tuning {
+  int rows8_rwg = 0, rows8_kw = 0;               // "rows8_shape"  = "rwg,kw"
+  int gemv_kp = 0, gemv_waves = 0;               // "gemv_shape"   = "kp,waves"
+  int gemm_ksplit = 0;                           // "gemm_ksplit"  = "n"
+  int dense_bm = 0, dense_bn = 0, dense_ks = 1;  // "dense_tile"   = "bm,bn[,ksplit]"
+  int dense_mfma16 = 1;                          // "dense_mfma16" = "0" | "1"
+  int dense_pf = -1;                             // "dense_pf"     = prefetch distance in slices
+};
+extern Tuning g_tuning;
 
 }  // namespace cuthip

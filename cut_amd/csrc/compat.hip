@@ -297,7 +297,6 @@ constexpr uint32_t kSepDenseRows = 32;
 
 bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a_f16, const void *A);
 size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16);
-bool blaslt_preferred();
 int launch_dense_gemm(int fmt, const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K,
                       uint32_t N, uint32_t strideA, uint32_t strideC, Epilogue epi, void *workspace, hipStream_t stream,
                       int use_blaslt);
@@ -459,6 +458,7 @@ static int matmul_sep(bool q4, const float *A, const void *B, const void *S, con
   }
   if (int rc = check_epilogue_op(who, epilogue, epilogue_op)) return rc;
   if (epilogue_op_long(epilogue, epilogue_op)) {   // unfused matmul, then the operator as an elementwise launch
+    if (int rc = check_long_epilogue_alias(epilogue, epilogue_op, C, D)) return rc;   // before anything is written
     if (int rc = matmul_sep(q4, A, B, S, nullptr, C, M, K, N, strideA, strideB, strideC, scaleStride, CUTHIP_EPI_NONE, 0, affine,
                             variant, workspace, workspace_bytes, stream))
       return rc;
@@ -485,7 +485,7 @@ static int matmul_sep(bool q4, const float *A, const void *B, const void *S, con
     Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
     return launch_dense_gemm(-1, w16, A, 0, C, 0, M, K, N, strideA, strideC, epi,
                              reinterpret_cast<uint8_t *>(workspace) + sep_w16_bytes(K, N), stream,
-                             (epilogue == CUTHIP_EPI_NONE && blaslt_preferred()) ? 2 : 0);
+                             0);
   }
   SepParams p;
   p.A = A;

@@ -178,7 +178,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_
   __shared__ __attribute__((aligned(16))) float Ps[4 * kAttnChunk];
   const uint32_t kvH = blockIdx.x, split = blockIdx.y, nRep = nHeads / nKvHeads;
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const uint32_t seqLen = params[1];
+  const uint32_t seqLen = min(params[1], maxSeqLen);   // a length beyond the cache capacity attends the capacity only
   const uint32_t t0 = split * kAttnChunk;
   const uint32_t nvalid = t0 < seqLen ? min((uint32_t)kAttnChunk, seqLen - t0) : 0u;
 
@@ -469,22 +469,22 @@ __global__ void __launch_bounds__(1024) argmax_finish_kernel(const ArgmaxPart *p
   uint32_t idx = 0xFFFFFFFFu;
   if (tid < n_pen) ptok[tid] = pen_tokens[tid];
   __syncthreads();
-  if (tid < n_pen) {
-    const int32_t t = ptok[tid];
-    bool effective = t >= 0 && (uint32_t)t < n;
-    for (uint32_t k = tid + 1; effective && k < n_pen; ++k) effective = ptok[k] != t;   // a later entry of the same token wins
-    float v = 0.0f;
-    if (effective) {
-      const float l = ld_act(logits, x_f16, (size_t)t), f = pen_factors[tid];
-      v = l > 0.0f ? l / f : l * f;
-      st_act(logits, x_f16, (size_t)t, v);
-      if (x_f16) v = (float)(half_t)v;   // as stored
-    }
-    __syncthreads();            // every entry has read its token before any is marked
+  // every barrier below is reached by all threads: the per-entry work is predicated, never the barrier
+  const bool mine = tid < n_pen;
+  const int32_t t = mine ? ptok[tid] : -1;
+  bool effective = mine && t >= 0 && (uint32_t)t < n;
+  for (uint32_t k = tid + 1; effective && k < n_pen; ++k) effective = ptok[k] != t;   // a later entry of the same token wins
+  float v = 0.0f;
+  if (effective) {
+    const float l = ld_act(logits, x_f16, (size_t)t), f = pen_factors[tid];
+    v = l > 0.0f ? l / f : l * f;
+    st_act(logits, x_f16, (size_t)t, v);
+    if (x_f16) v = (float)(half_t)v;   // as stored
+  }
+  __syncthreads();            // every entry has read its token before any is marked
+  if (mine) {
     if (!effective) ptok[tid] = -1;
     pval[tid] = v;
-  } else {
-    __syncthreads();
   }
   __syncthreads();
   // value of row r as the penalised logits hold it: listed rows from the table above (their stores may not be
@@ -671,10 +671,17 @@ static __device__ __align__(256) unsigned char scratch[kAttnStaticBytes];
 static void *g_scratch_ptr[kMaxDevices];   // per device; written under g_scratch_mu
 static std::mutex g_scratch_mu;
 
-// Device address of `scratch` on the current device (looked up on first use there); nullptr after set_error.
-static void *attn_static_ptr() {
-  int dev = -1;
-  if (check_hip(hipGetDevice(&dev), "hipGetDevice")) return nullptr;
+// Device address of `scratch` on the device that owns `stream` (the current device for the null stream), looked up
+// on first use there with that device current; nullptr after set_error.
+static void *attn_static_ptr(hipStream_t stream) {
+  int cur = -1, dev = -1;
+  if (check_hip(hipGetDevice(&cur), "hipGetDevice")) return nullptr;
+  dev = cur;
+  if (stream) {
+    hipDevice_t sd = 0;
+    if (check_hip(hipStreamGetDevice(stream, &sd), "hipStreamGetDevice")) return nullptr;
+    dev = (int)sd;
+  }
   if (dev < 0 || dev >= kMaxDevices) {
     set_error("attention scratch: device index %d beyond %d", dev, kMaxDevices);
     return nullptr;
@@ -682,14 +689,17 @@ static void *attn_static_ptr() {
   std::lock_guard<std::mutex> lock(g_scratch_mu);
   if (!g_scratch_ptr[dev]) {
     void *ptr = nullptr;
-    if (check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return nullptr;
+    if (dev != cur && check_hip(hipSetDevice(dev), "hipSetDevice")) return nullptr;
+    const int rc = check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+    if (dev != cur) (void)hipSetDevice(cur);
+    if (rc) return nullptr;
     g_scratch_ptr[dev] = ptr;
   }
   return g_scratch_ptr[dev];
 }
 
 // called by cuthip_init with the chosen device current
-int attn_static_setup() { return attn_static_ptr() ? CUTHIP_OK : CUTHIP_ERR_HIP; }
+int attn_static_setup() { return attn_static_ptr(nullptr) ? CUTHIP_OK : CUTHIP_ERR_HIP; }
 }  // namespace cuthip
 
 extern "C" {
@@ -710,7 +720,7 @@ int cuthip_attn_decode_static(const void *q, int q_dtype, const void *k_cache, c
               max_seq_len, need, kAttnStaticBytes);
     return CUTHIP_ERR_INVALID;
   }
-  void *ptr = attn_static_ptr();
+  void *ptr = attn_static_ptr((hipStream_t)stream);
   if (!ptr) return CUTHIP_ERR_HIP;
   // every split record of this call's launch shape is written before the merge reads it, so nothing of an earlier
   // call's contents is read and nothing needs clearing

@@ -369,10 +369,8 @@ template <int FMT, int BM, bool AF16> static int launch_gemm_bm(GemmParams p, hi
   uint32_t ks = 1;
   if (p.partial && BM <= 128) {
     ks = tiled_gemm_ksplit(p.M, p.K, p.N, p.kper);
-    if (const char *env = getenv("CUT_HIP_GEMM_KSPLIT")) {   // tuning aid
-      const uint32_t want = (uint32_t)atoi(env);
-      if (want >= 1 && want <= 16 && (uint64_t)want * p.M * p.N * 4 <= p.kper) ks = want;
-    }
+    const uint32_t want = (uint32_t)g_tuning.gemm_ksplit;   // forced by a test or a sweep
+    if (want >= 1 && want <= 16 && (uint64_t)want * p.M * p.N * 4 <= p.kper) ks = want;
   }
   const uint32_t per = (nslices + ks - 1) / ks;
   p.kper = per * kBK;                      // (on entry: bytes of scratch behind partial)

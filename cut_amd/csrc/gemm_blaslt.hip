@@ -108,12 +108,6 @@ bool blaslt_available() {
   return hipGetDevice(&dev) == hipSuccess && dev == lt.device;   // the handle belongs to one device
 }
 
-// the library's own choice by shape may take the vendor GEMM only when the process asks for it
-bool blaslt_preferred() {
-  const char *on = std::getenv("CUT_HIP_VENDOR_GEMM");
-  return on && on[0] && on[0] != '0' && blaslt_available();
-}
-
 // Row-major C = A . Wd^T is, column-major, C^T (N x M) = op_T(Wd as K x N) . (A as K x M).
 // Returns CUTHIP_OK, or CUTHIP_ERR_INVALID with the error set when the library has no kernel for the problem.
 int launch_blaslt_gemm(const void *Wd, const void *A16, void *C, int c_f16, uint32_t M, uint32_t K, uint32_t N, uint32_t strideA,

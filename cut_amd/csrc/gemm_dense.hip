@@ -597,15 +597,14 @@ template <int BM, int BN, int WM = 2> static int launch_dense_bm(DenseParams p, 
     p.pf_asplit = panels < per_xcd ? panels : per_xcd;
     if (p.pf_asplit == 0) p.pf_asplit = 1;
   }
-  if (const char *env = getenv("CUT_HIP_DENSE_PF")) p.pf_dist = (uint32_t)atoi(env);
+  if (g_tuning.dense_pf >= 0) p.pf_dist = (uint32_t)g_tuning.dense_pf;
   uint64_t grid = (uint64_t)p.mtiles * p.ntiles * p.ksplit;
   if (grid > 0x7FFFFFFFull) {
     set_error("cuthip_matmul_gguf_ws: problem too large for one launch");
     return CUTHIP_ERR_INVALID;
   }
-  // the 16 x 16 x 32 kernel unless CUT_HIP_DENSE_MFMA16=0 asks for the 32 x 32 x 16 one (kept for comparison)
-  const char *env16 = getenv("CUT_HIP_DENSE_MFMA16");   // read at every launch, like CUT_HIP_DENSE_TILE: a tuning aid
-  const bool mfma16 = !env16 || atoi(env16) != 0;
+  // the 16 x 16 x 32 kernel unless the tuning key dense_mfma16 = 0 asks for the 32 x 32 x 16 one (kept for comparison)
+  const bool mfma16 = g_tuning.dense_mfma16 != 0;
   if (mfma16) hipLaunchKernelGGL((gemm_dense16_kernel<BM, BN, WM>), dim3((uint32_t)grid), dim3(256), 0, stream, p);
   else hipLaunchKernelGGL((gemm_dense_kernel<BM, BN, WM>), dim3((uint32_t)grid), dim3(256), 0, stream, p);
   return check_hip(hipGetLastError(), "dense gemm launch");
@@ -631,13 +630,8 @@ bool dense_gemm_fits(uint32_t M, uint32_t K, uint32_t N, uint32_t strideA, int a
 // tiles instead (partials in the workspace, summed by a second kernel).
 struct DenseShape { int bm, bn; uint32_t ksplit; };
 static DenseShape pick_dense_shape(uint32_t M, uint32_t K, uint32_t N) {
-  if (const char *env = getenv("CUT_HIP_DENSE_TILE")) {   // "bm,bn[,ksplit]" tuning aid: 256,224 / 128,448 / 128,256 / 256,256
-    int bm = 0, bn = 0, ks = 1;
-    const int got = sscanf(env, "%d,%d,%d", &bm, &bn, &ks);   // optional third field: K ranges (1, 2, 4, 8)
-    if (got >= 2 && ((bn == 256 && (bm == 256 || bm == 128)) || (bn == 448 && bm == 128) || (bn == 224 && bm == 256)) &&
-        (ks == 1 || ks == 2 || ks == 4 || ks == 8) && K % (ks * 128) == 0)
-      return DenseShape{bm, bn, (uint32_t)ks};
-  }
+  if (g_tuning.dense_bn && K % ((uint32_t)g_tuning.dense_ks * 128) == 0)   // forced by a test or a sweep
+    return DenseShape{g_tuning.dense_bm, g_tuning.dense_bn, (uint32_t)g_tuning.dense_ks};
   static const struct { int bm, bn; double cost; } cands[] = {{256, 224, 0.96}, {128, 448, 1.00}, {256, 256, 1.03}, {128, 256, 1.24}};
   int best = 0;
   double best_t = 0.0;

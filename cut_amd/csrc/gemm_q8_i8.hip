@@ -281,6 +281,7 @@ int cuthip_matmul_q8_i8(const void *W, const void *A, int a_dtype, void *C, int 
   }
   if (int rc = check_epilogue_op("cuthip_matmul_q8_i8", epilogue, epilogue_op)) return rc;
   if (epilogue_op_long(epilogue, epilogue_op)) {
+    if (int rc = check_long_epilogue_alias(epilogue, epilogue_op, C, D)) return rc;   // before anything is written
     if (int rc = cuthip_matmul_q8_i8(W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, CUTHIP_EPI_NONE, 0, nullptr, workspace,
                                      workspace_bytes, stream))
       return rc;

@@ -26,10 +26,7 @@ CUTHIP_EXTERN_ROWS8(CUTHIP_Q6_K)
 // Workgroup shape of the rows8 GEMV: split K (kw step ranges per 8-row group)
 // while the grid has fewer than ~6 waves per CU and each wave keeps >= 2 steps.
 Rows8Shape pick_rows8_shape(int fmt, uint32_t M, uint32_t N, uint32_t nsteps) {
-  if (const char *env = std::getenv("CUT_HIP_ROWS8_SHAPE")) {   // "rwg,kw" tuning aid
-    int rwg = 0, kw = 0;
-    if (sscanf(env, "%d,%d", &rwg, &kw) == 2 && (kw == 1 || kw == 2 || kw == 4 || kw == 8)) return Rows8Shape{rwg, kw};
-  }
+  if (g_tuning.rows8_kw) return Rows8Shape{g_tuning.rows8_rwg, g_tuning.rows8_kw};   // forced by a test or a sweep
   uint32_t groups = (N + 7) / 8;
   int kw = 1;
   if (M > 4) {
@@ -112,14 +109,7 @@ static int launch_rows8_any(int fmt, const GemvParams &p, hipStream_t stream, bo
 }
 
 GemvShape pick_gemv_shape(uint32_t N, uint32_t nsteps, int mt) {
-  // CUT_HIP_GEMV_SHAPE="kp,waves" overrides the heuristic (tuning aid).
-  if (const char *env = std::getenv("CUT_HIP_GEMV_SHAPE")) {
-    int kp = 0, w = 0;
-    if (sscanf(env, "%d,%d", &kp, &w) == 2 && (kp == 1 || kp == 2) && (w == 1 || w == 2 || w == 4 || w == 8)) {
-      if (mt > 8) kp = 1;
-      return GemvShape{kp, w};
-    }
-  }
+  if (g_tuning.gemv_waves) return GemvShape{mt > 8 ? 1 : g_tuning.gemv_kp, g_tuning.gemv_waves};   // forced by a test or a sweep
   // Measured on MI355X at the projection shapes of an 8B model: two parts per
   // wave (16 weight rows per workgroup) win for M <= 2 unless N is huge, and
   // K is split over as many waves as keep >= 2 steps of 256 per part.
@@ -147,7 +137,6 @@ size_t stream_gemm_scratch(uint32_t M, uint32_t K, uint32_t N);
 int launch_stream_gemm(const void *W, const void *A, int a_f16, void *C, int c_f16, uint32_t M, uint32_t K, uint32_t N,
                        uint32_t strideA, uint32_t strideC, Epilogue epi, void *scratch, size_t scratch_bytes, hipStream_t stream);
 bool blaslt_available();
-bool blaslt_preferred();
 size_t dense_f16_workspace(uint32_t M, uint32_t K, uint32_t N, int a_f16);
 
 static int launch_gemv(int fmt, const GemvParams &p, hipStream_t stream) {
@@ -280,6 +269,7 @@ static int matmul_gguf_scratch(int fmt, const void *W, const void *A, int a_dtyp
     return rc > 0 ? CUTHIP_OK : rc;
   if (int rc = check_epilogue_op("cuthip_matmul_gguf", epilogue, epilogue_op)) return rc;
   if (epilogue_op_long(epilogue, epilogue_op)) {   // unfused matmul, then the operator as an elementwise launch
+    if (int rc = check_long_epilogue_alias(epilogue, epilogue_op, C, D)) return rc;   // before anything is written
     if (int rc = matmul_gguf_scratch(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, CUTHIP_EPI_NONE, 0, nullptr,
                                      variant, stream, scratch, scratch_bytes))
       return rc;
@@ -413,6 +403,7 @@ int cuthip_matmul_gguf_carry(int fmt, const void *W, const void *A, int a_dtype,
   if (int rc = check_matmul_args(fmt, W, A, a_dtype, C, c_dtype, 1, K, N, K, n_out, epilogue, D)) return rc > 0 ? CUTHIP_OK : rc;
   if (int rc = check_epilogue_op("cuthip_matmul_gguf_carry", epilogue, epilogue_op)) return rc;
   if (epilogue_op_long(epilogue, epilogue_op)) {
+    if (int rc = check_long_epilogue_alias(epilogue, epilogue_op, C, D)) return rc;   // before anything is written
     if (carry && (carry->next_norm_weight || carry->next_x16 || carry->next_sumsq_parts)) {
       set_error("cuthip_matmul_gguf_carry: operator %d runs as a launch of its own after the matmul and cannot feed the "
                 "producer side of a carried RMSNorm", epilogue_op);
@@ -587,6 +578,7 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
     return rc > 0 ? CUTHIP_OK : rc;
   if (int rc = check_epilogue_op("cuthip_matmul_gguf_ws", epilogue, epilogue_op)) return rc;
   if (epilogue_op_long(epilogue, epilogue_op)) {
+    if (int rc = check_long_epilogue_alias(epilogue, epilogue_op, C, D)) return rc;   // before anything is written
     if (int rc = cuthip_matmul_gguf_ws(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, CUTHIP_EPI_NONE, 0, nullptr,
                                        variant, workspace, workspace_bytes, stream))
       return rc;
@@ -597,27 +589,6 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
   if (variant == -1 && stream_preferred(fmt, M, K, N, strideA, a_f16, A, workspace, workspace ? workspace_bytes : 0))
     return matmul_gguf_scratch(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, 6, stream,
                                workspace, workspace_bytes);
-  // 9..383 rows with the vendor GEMM at hand: dequantize + hipBLASLt against what the automatic choice would run
-  // otherwise, by a cost model fitted to a sweep over the FFN / attention shapes of an 8B model (microseconds;
-  // Q4_K, graph replay): an 8-row pass 6.5 + weight bytes / 4.3 MB (x 1.45 on rows of K >= 8192), the
-  // single-launch GEMM 62 + weight bytes / 7 MB (K >= 8192: the split two-pass GEMM, 65 + 0.19 M), the vendor path
-  // 14 + N K x 0.65e-6 (0.95e-6 once the fp16 copy outgrows the 256 MB cache) + 2 M N K / 1.6 PFLOP/s.
-  if (variant == -1 && M > 8 && M < 384 && epilogue == CUTHIP_EPI_NONE && workspace && (uintptr_t)workspace % 256 == 0 &&
-      dense_gemm_fits(M, K, N, strideA, a_f16, A) && workspace_bytes >= dense_gemm_workspace(M, K, N, a_f16) &&
-      blaslt_preferred()) {
-    const double nk = (double)N * K;
-    const double t5 = 14.0 + nk * (nk <= 64e6 ? 0.65e-6 : 0.95e-6) + 2.0 * M * nk / 1.6e9;
-    const size_t split = tiled_split_applies(M, K, N, workspace, workspace_bytes) ? workspace_bytes : 0;
-    double other;
-    if (passes_preferred(fmt, M, K, N, split)) other = passes_cost_us(fmt, M, K, N);
-    else other = split ? tiled_split_cost_us(fmt, M, K, N, split) : K >= 8192 ? 65.0 + 0.19 * M : single_launch_cost_us(fmt, M, K, N, 0);
-    if (t5 < 0.95 * other) {
-      const int rc = launch_dense_gemm(fmt, W, A, a_f16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC,
-                                       Epilogue{CUTHIP_EPI_NONE, 0, nullptr}, workspace,
-                                       reinterpret_cast<hipStream_t>(stream), 2);
-      return rc;
-    }
-  }
   // Beyond 8 rows, with a workspace at hand: dequantize + dense GEMM where its modelled cost is below that of what
   // would run otherwise (8-row passes up to 40 rows where those beat the single-launch GEMM, else that GEMM); against
   // either only by a margin (a tenth, a twentieth): the models are rough.  From 1024 rows always.
@@ -662,10 +633,7 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
     Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
     return launch_splitk_reduce(partial, parts, M, N, C, strideC, epi, c_dtype == CUTHIP_F16, s);
   }
-  // with the vendor GEMM behind the dequantization the two-pass path pays earlier: 25 us of dequantization for an FFN
-  // matrix against a single-launch GEMM that decodes the weights once per 128 rows (M = 512, N = 14336: 86 us against 110)
-  const bool lt_ok = variant == -1 && epilogue == CUTHIP_EPI_NONE && fits && ws_ok && blaslt_preferred();
-  if (variant == -1 && !((dense_first || (lt_ok && M >= 384)) && fits && ws_ok))
+  if (variant == -1 && !(dense_first && fits && ws_ok))
     return matmul_gguf_scratch(fmt, W, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, epilogue, epilogue_op, D, -1,
                                stream, workspace, workspace ? workspace_bytes : 0);
   if (!fits) {
@@ -682,8 +650,8 @@ int cuthip_matmul_gguf_ws(int fmt, const void *W, const void *A, int a_dtype, vo
     set_error("cuthip_matmul_gguf_ws: variant 5 (dequantize, then the vendor GEMM) has no fused epilogue: use variant 4");
     return CUTHIP_ERR_INVALID;
   }
-  // the dense GEMM of the automatic choice: the vendor library where it is present and nothing is fused
-  const int use_blaslt = variant == 5 ? 1 : lt_ok ? 2 : 0;
+  // the vendor GEMM runs for variant 5 only; the automatic choice never takes it
+  const int use_blaslt = variant == 5 ? 1 : 0;
   Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
   return launch_dense_gemm(fmt, W, A, a_f16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC, epi, workspace,
                            reinterpret_cast<hipStream_t>(stream), use_blaslt);
@@ -713,6 +681,7 @@ int cuthip_matmul_dense_f16(const void *W16, const void *A, int a_dtype, void *C
   }
   if (int rc = check_epilogue_op("cuthip_matmul_dense_f16", epilogue, epilogue_op)) return rc;
   if (epilogue_op_long(epilogue, epilogue_op)) {
+    if (int rc = check_long_epilogue_alias(epilogue, epilogue_op, C, D)) return rc;   // before anything is written
     if (int rc = cuthip_matmul_dense_f16(W16, A, a_dtype, C, c_dtype, M, K, N, strideA, strideC, CUTHIP_EPI_NONE, 0, nullptr,
                                          workspace, workspace_bytes, stream))
       return rc;
@@ -731,10 +700,9 @@ int cuthip_matmul_dense_f16(const void *W16, const void *A, int a_dtype, void *C
               workspace ? workspace_bytes : (size_t)0);
     return CUTHIP_ERR_INVALID;
   }
-  const int use_blaslt = (epilogue == CUTHIP_EPI_NONE && blaslt_preferred()) ? 2 : 0;
   Epilogue epi{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr};
   return launch_dense_gemm(-1, W16, A, a_f16, C, c_dtype == CUTHIP_F16, M, K, N, strideA, strideC, epi, workspace,
-                           reinterpret_cast<hipStream_t>(stream), use_blaslt);
+                           reinterpret_cast<hipStream_t>(stream), 0);
 }
 
 int cuthip_matmul_gguf_pro(int fmt, const void *W, const void *A, int a_dtype, void *C, int c_dtype, uint32_t K, uint32_t N,
@@ -751,6 +719,7 @@ int cuthip_matmul_gguf_pro(int fmt, const void *W, const void *A, int a_dtype, v
   }
   if (int rc = check_epilogue_op("cuthip_matmul_gguf_pro", epilogue, epilogue_op)) return rc;
   if (epilogue_op_long(epilogue, epilogue_op)) {
+    if (int rc = check_long_epilogue_alias(epilogue, epilogue_op, C, D)) return rc;   // before anything is written
     if (int rc = cuthip_matmul_gguf_pro(fmt, W, A, a_dtype, C, c_dtype, K, N, CUTHIP_EPI_NONE, 0, nullptr, prologue, norm_weight,
                                         eps, stream))
       return rc;

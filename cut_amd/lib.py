@@ -28,7 +28,7 @@ BLOCK_BYTES = {Q8_0: 34, Q4_0: 18, Q4_K: 144, Q6_K: 210}
 
 # every symbol include/cut_hip.h declares
 EXPORTS = [
-    "cuthip_init", "cuthip_last_error", "cuthip_device_info",
+    "cuthip_init", "cuthip_last_error", "cuthip_device_info", "cuthip_set_tuning",
     "cuthip_malloc", "cuthip_free", "cuthip_memcpy_h2d", "cuthip_memcpy_d2h", "cuthip_memcpy_d2d", "cuthip_memset",
     "cuthip_stream_create", "cuthip_stream_destroy", "cuthip_stream_sync",
     "cuthip_event_create", "cuthip_event_destroy", "cuthip_event_record", "cuthip_event_sync", "cuthip_event_elapsed_ms",
@@ -94,6 +94,7 @@ def load() -> C.CDLL:
     lib.cuthip_last_error.argtypes = []
     lib.cuthip_init.argtypes = [i]
     lib.cuthip_device_info.argtypes = [C.POINTER(DeviceInfo)]
+    lib.cuthip_set_tuning.argtypes = [C.c_char_p, C.c_char_p]
     lib.cuthip_malloc.argtypes = [C.POINTER(vp), C.c_size_t]
     lib.cuthip_free.argtypes = [vp]
     for n in ("cuthip_memcpy_h2d", "cuthip_memcpy_d2h", "cuthip_memcpy_d2d"):
@@ -186,3 +187,8 @@ def device_info() -> dict:
     d = DeviceInfo()
     check(load().cuthip_device_info(C.byref(d)))
     return {f: (getattr(d, f).decode() if isinstance(getattr(d, f), bytes) else getattr(d, f)) for f, _ in d._fields_}
+
+
+def set_tuning(key: str, value: str | None) -> None:
+    """Forces a launch shape (tests, sweeps); value None restores the library's own choice (cuthip_set_tuning)."""
+    check(load().cuthip_set_tuning(key.encode(), value.encode() if value is not None else None))

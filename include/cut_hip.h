@@ -105,9 +105,20 @@ typedef struct {
 /* ---- library / device -------------------------------------------------- */
 
 /* Selects the device and checks that it is gfx950.  Replaces the backend
- * constructor's device pick-up (core/backends/cuda/CudaCompute.cpp:60-100). */
+ * constructor's device pick-up (core/backends/cuda/CudaCompute.cpp:60-100).
+ * Also takes over, once, the launch-shape overrides of the environment (CUT_HIP_ROWS8_SHAPE, CUT_HIP_GEMV_SHAPE,
+ * CUT_HIP_GEMM_KSPLIT, CUT_HIP_DENSE_TILE, CUT_HIP_DENSE_MFMA16, CUT_HIP_DENSE_PF: the values cuthip_set_tuning takes);
+ * no launch reads the environment. */
 int cuthip_init(int device);
 const char *cuthip_last_error(void);
+/* Forces a launch shape for tests and tuning sweeps, process-wide, until changed; value NULL or "" restores the
+ * library's own choice.  Keys: "rows8_shape" = "rwg,kw" (8-row GEMV: row groups per workgroup, K ranges 1/2/4/8),
+ * "gemv_shape" = "kp,waves" (fallback GEMV), "gemm_ksplit" = "n" (K ranges of the single-launch GEMM, 1..16),
+ * "dense_tile" = "bm,bn[,ksplit]" (256,224 / 128,448 / 128,256 / 256,256), "dense_mfma16" = "0" | "1",
+ * "dense_pf" = prefetch distance in slices.  Not synchronised with launches in flight on other threads.  The
+ * reference's counterpart is the per-operator `spec` argument that its tests and op_bench pass
+ * (operators/impl/matmul/MatMulOp.cpp:336-374); an unknown key or a malformed value is CUTHIP_ERR_INVALID. */
+int cuthip_set_tuning(const char *key, const char *value);
 /* DeviceCaps + DeviceInfo of the reference (core/api/include/ComputeCommon.h:92-97). */
 int cuthip_device_info(cuthip_device_info_t *info);
 
@@ -120,6 +131,7 @@ int cuthip_free(void *device_ptr);
 int cuthip_memcpy_h2d(void *device_dst, const void *host_src, size_t bytes, void *stream);
 int cuthip_memcpy_d2h(void *host_dst, const void *device_src, size_t bytes, void *stream);
 int cuthip_memcpy_d2d(void *device_dst, const void *device_src, size_t bytes, void *stream);
+/* hipMemsetAsync; CUTHIP_ERR_INVALID while `stream` is capturing (memset nodes are kept out of graphs). */
 int cuthip_memset(void *device_dst, int value, size_t bytes, void *stream);
 int cuthip_stream_create(void **stream);
 int cuthip_stream_destroy(void *stream);
@@ -134,8 +146,8 @@ int cuthip_event_elapsed_ms(void *start, void *stop, float *ms);
  * (core/backends/cuda/CudaCommandBuffer.cpp:261-285: cuStreamBeginCapture, the dispatches, cuStreamEndCapture,
  * cuGraphInstantiate once, then cuGraphLaunch per token).  Between begin and end every cuthip_* launch on `stream`
  * (a stream from cuthip_stream_create, not the default one) is recorded instead of run; no entry point of this
- * library allocates, so all of them may be captured (cuthip_memset is the exception: clear memory before the capture
- * or with a kernel of the sequence).  Values that change between replays (position, sequence length, token ids,
+ * library allocates, so all of them may be captured (cuthip_memset is the exception and refuses a capturing stream:
+ * clear memory before the capture or with a kernel of the sequence).  Values that change between replays (position, sequence length, token ids,
  * penalty lists) are read from device memory by the kernels, so the host updates those buffers and launches the same
  * graph again.  The handle owns both the graph and its executable form. */
 int cuthip_graph_begin_capture(void *stream);
@@ -223,15 +235,15 @@ int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void 
  *            rows of A are not 16-byte aligned or the workspace is too small);
  *            5 = MatMulGgufDequantBlasLt: the same dequantization, then hipBLASLt's
  *            dense fp16 GEMM (the weights are plain fp16 by then, so it is a library
- *            GEMM; the library is opened with dlopen by cuthip_init and its handle is
- *            created then (outside any stream capture), the only allocation this
- *            library ever causes; the first matmul of a new shape asks the library's
- *            heuristic for a kernel, on the host; an error if
- *            the library is absent or an epilogue is asked for; CUT_HIP_NO_BLASLT=1 in
- *            the environment keeps it closed);
- *            -1 = choose by shape: the two-pass path (variant 5 where hipBLASLt is
- *            present, has a kernel for the shape and no epilogue is fused, else
- *            variant 4) when it applies and M >= 1024 (or, with so
+ *            GEMM; the library is opened with dlopen, and its handle created, by the first
+ *            cuthip_variant_available(CUTHIP_OP_MATMUL_GGUF, 5) or the first call with this index:
+ *            a caller that captures streams does one of these before it captures; it is the
+ *            only allocation this library ever causes; the first matmul of a new shape asks the
+ *            library's heuristic for a kernel, on the host; an error if the library is absent or
+ *            an epilogue is asked for; CUT_HIP_NO_BLASLT=1 in the environment keeps it closed).
+ *            Variant 5 runs only when this index is passed: no automatic choice takes it;
+ *            -1 = choose by shape among the hand-written kernels: the two-pass path (variant 4)
+ *            when it applies and M >= 1024 (or, with so
  *            few output tiles that the single-launch GEMM would leave most of the chip
  *            idle, from M = 256, and from M = 41 when K >= 8192; K is then split and
  *            the partial products summed), else
@@ -241,8 +253,11 @@ int cuthip_matmul_gguf(int fmt, const void *W, const void *A, int a_dtype, void 
  *            fp32 partial products in the workspace, summed in a second launch);
  *            6 = MatMulGgufStreamMfma (Q4_K, M <= 32, 16-byte aligned rows of A, else an
  *            error): the weights stay packed until they are multiplied (integer-scaled
- *            nibbles as fp16 subnormals into 16x16x32 MFMAs, results exact up to the
- *            order of the fp32 sums); K above 4096 (2048 beyond 16 rows) is split over
+ *            nibbles as fp16 subnormals into 16x16x32 MFMAs: the products are exact and
+ *            the result differs from fp32 FMAs only by the order of the fp32 sums, given
+ *            fp16 activations; fp32 activations are rounded to fp16, nearest even, when they
+ *            are staged - 2^-11 relative per element, |a| > 65504 becomes inf - as on the 8-row
+ *            GEMV and the GEMMs); K above 4096 (2048 beyond 16 rows) is split over
  *            workgroups through the workspace, an error without one.  With variant -1
  *            it is what runs for 9..32 rows of Q4_K.
  * With variant -1 the workspace also serves batch 2-8 (Q6_K: 3-8) on long rows (K >= 8192) of few (N < 12288): the 8-row GEMV

@@ -293,6 +293,156 @@ private:
   Tensor output_;
 };
 
+// ---- MatMulOpNode: the reference's 3-input quantized matmul ------------------------------------
+// operators/impl/matmul/MatMulOp.h:16-70, MatMulOp.cpp:271-383 on the loader's separated tensors: A fp32 [K] or
+// [M, K]; packedB [K, N] int8 (Q8) or [K, N/2] nibble bytes (Q4); scalesB fp16 [K/32, N], or [2K/32, N] when the
+// lower half holds the per-block minima (affine Q4).  The format is inferred from the shapes, the variant from the
+// shape unless `spec` names one, exactly as the reference does it; the messages of the errors are the reference's.
+enum class QuantFormat : int { None = 0, Q8 = 1, Q4 = 2 };
+// What the constructor reads of store.caps() (core/api/include/ComputeCommon.h:92-97); gfx950 always has matrix cores.
+struct DeviceCaps {
+  bool cooperativeMatrix = true;
+  // the matrix-core route of this backend (dequantize to fp16, dense MFMA GEMM) takes K in multiples of 128; where the
+  // reference's K % 16 == 0 holds but this does not, the automatic choice stays with the tiled variant
+  uint32_t cooperativeMatrixK = 128;
+};
+// Sizes of the reference's variant tables and their defaults (MatMulQ8Variants.generated.h:20-21,
+// MatMulQ4Variants.generated.h:20-21); the library's CUTHIP_OP_MATMUL_Q8 / _Q4 tables hold the same numbers.
+constexpr uint32_t kMatMulQ8VariantCount = 8, kMatMulQ8DefaultVariant = 2, kMatMulQ4VariantCount = 5, kMatMulQ4DefaultVariant = 0;
+
+// Everything the constructor derives from the shapes, without touching the device (MatMulOp.cpp:283-374).
+struct QuantMatMulPlan {
+  QuantFormat format = QuantFormat::None;
+  uint32_t M = 0, K = 0, N = 0;
+  bool q4Affine = false;            // scales carry the minima in their lower half
+  bool autoSpec = false;            // no explicit spec from the caller
+  uint32_t spec = 0;                // index into the Q8 / Q4 variant table
+  uint32_t fusionFallbackSpec = 0;  // the fusion-capable variant of the same shape class
+  // push constants (MatMulOp.cpp:514-541): rows are padded to four elements
+  uint32_t strideA = 0, strideB = 0, strideC = 0, scaleStride = 0;
+};
+inline QuantMatMulPlan planQuantMatMul(const std::vector<uint32_t> &shapeA, const std::vector<uint32_t> &shapePB,
+                                       const std::vector<uint32_t> &shapeSB, DataType scalesDtype,
+                                       std::optional<uint32_t> spec = {}, DeviceCaps caps = {}) {
+  QuantMatMulPlan p;
+  if (shapePB.size() != 2 || shapeSB.size() != 2) throw std::runtime_error("matmul requires 2D B and scales matrices");
+  if (shapeA.size() == 1) {   // [K] is [1, K]: the optimizer may have removed the reshape
+    p.M = 1;
+    p.K = shapeA[0];
+  } else if (shapeA.size() == 2) {
+    p.M = shapeA[0];
+    p.K = shapeA[1];
+  } else {
+    throw std::runtime_error("matmul: A must be 1D or 2D");
+  }
+  if (shapePB[0] != p.K)
+    throw std::runtime_error("matmul: B rows (" + std::to_string(shapePB[0]) + ") must match A cols (" + std::to_string(p.K) + ")");
+  const uint32_t bCols = shapePB[1], sCols = shapeSB[1];
+  if (bCols == sCols) {
+    p.format = QuantFormat::Q8;
+    p.N = bCols;
+  } else if (bCols * 2 == sCols) {
+    p.format = QuantFormat::Q4;
+    p.N = sCols;
+    p.q4Affine = shapeSB[0] == 2u * ((p.K + 31u) / 32u);
+  } else {
+    throw std::runtime_error("matmul: cannot determine quant format from B cols (" + std::to_string(bCols) +
+                             ") and scales cols (" + std::to_string(sCols) + ")");
+  }
+  p.autoSpec = !spec.has_value();
+  if (p.format == QuantFormat::Q8)
+    p.fusionFallbackSpec = p.M == 1 ? (p.N >= 8 ? 4u : 3u) : kMatMulQ8DefaultVariant;   // GemvKPar8 / GemvKPar / VecT16R4x4
+  else
+    p.fusionFallbackSpec = p.M == 1 ? (p.N >= 8 ? 3u : 2u) : kMatMulQ4DefaultVariant;   // Q4GemvKPar8 / Q4GemvKPar / tiled
+  const bool coop = p.M > 1 && caps.cooperativeMatrix && scalesDtype == DataType::Float16 && p.K % 16 == 0 && p.N % 32 == 0 &&
+                    p.K % (caps.cooperativeMatrixK ? caps.cooperativeMatrixK : 1u) == 0;
+  if (spec.has_value()) p.spec = *spec;
+  else if (p.format == QuantFormat::Q8 && coop) p.spec = kMatMulQ8VariantCount - 1;   // MatMulQ8CoopMatTiled
+  else if (p.format == QuantFormat::Q4 && coop) p.spec = 4;                          // MatMulQ4CoopMatTiled
+  else p.spec = p.fusionFallbackSpec;
+  p.strideA = (p.K + 3) & ~3u;
+  p.strideB = ((p.format == QuantFormat::Q4 ? p.N / 2 : p.N) + 3) & ~3u;
+  p.strideC = p.scaleStride = (p.N + 3) & ~3u;
+  return p;
+}
+
+class MatMulOpNode {
+public:
+  MatMulOpNode(const Tensor &a, const Tensor &packedB, const Tensor &scalesB, std::optional<uint32_t> spec = {}, DeviceCaps caps = {})
+      : a_(a), b_(packedB), s_(scalesB), plan_(planQuantMatMul(a.shape, packedB.shape, scalesB.shape, scalesB.dtype, spec, caps)) {
+    const QuantMatMulPlan &p = plan_;
+    if (p.M == 0 || p.K == 0 || p.N == 0) throw std::runtime_error("matmul: empty dimension");
+    if (p.K % 32 != 0) throw std::runtime_error("matmul: K must be a multiple of the 32-element quantization block");
+    if (p.spec >= (p.format == QuantFormat::Q8 ? kMatMulQ8VariantCount : kMatMulQ4VariantCount))
+      throw std::runtime_error("matmul: variant index " + std::to_string(p.spec) + " is outside the table");
+    if (a.dtype != DataType::Float32) throw std::runtime_error("matmul: the quantized matmul takes Float32 activations");
+    if (scalesB.dtype != DataType::Float16) throw std::runtime_error("matmul: scales must be Float16");
+    // the reference's tensors are rows padded to four elements; a tensor that states another stride is refused
+    if ((a.rowStride && a.rowStride != p.strideA) || (packedB.rowStride && packedB.rowStride != p.strideB) ||
+        (scalesB.rowStride && scalesB.rowStride != p.scaleStride))
+      throw std::runtime_error("matmul: row strides must be the dimensions padded to four elements");
+    const size_t scaleRows = (size_t)(p.q4Affine ? 2u : 1u) * (p.K / 32);
+    if (!a.buffer || a.buffer->bytes() < ((size_t)(p.M - 1) * p.strideA + p.K) * 4 || !packedB.buffer ||
+        packedB.buffer->bytes() < (size_t)(p.K - 1) * p.strideB + (p.format == QuantFormat::Q4 ? p.N / 2 : p.N) ||
+        !scalesB.buffer || scalesB.buffer->bytes() < ((scaleRows - 1) * p.scaleStride + p.N) * 2)
+      throw std::runtime_error("matmul: a tensor holds fewer bytes than its shape and padded stride need");
+    if (shapeRows(scalesB) < scaleRows) throw std::runtime_error("matmul: scales must have K/32 rows");
+    storage_ = DeviceBuffer((size_t)p.M * p.strideC * 4);
+    output_ = Tensor{&storage_, {p.M, p.N}, DataType::Float32, p.strideC};
+    scratch_ = DeviceBuffer(cuthip_matmul_sep_workspace_bytes_for(op(), (int)p.spec, p.M, p.K, p.N));
+  }
+  MatMulOpNode(MatMulOpNode &&) = delete;   // output() points into this node
+  // MatMulOp.cpp:389-419: the quantized cooperative-matrix variants have a fusion epilogue, so nothing falls back
+  void setFusion(MatMulFusion fusion, int fusionOp = 0, const Tensor &d = {}) {
+    if (fusion == MatMulFusion::Binary) {
+      if (!d.buffer) throw std::runtime_error("matmul: Binary fusion needs the tensor d");
+      if (d.dtype != DataType::Float32 || d.stride() != plan_.strideC) throw std::runtime_error("matmul: d must match the output");
+    }
+    fusion_ = fusion;
+    fusionOp_ = fusionOp;
+    d_ = d;
+  }
+  QuantFormat format() const { return plan_.format; }
+  MatMulFusion fusion() const { return fusion_; }
+  const QuantMatMulPlan &plan() const { return plan_; }
+  DataType outputDtype() const { return DataType::Float32; }   // MatMulOp.cpp:436-438: always Float32
+  std::vector<uint32_t> outputShape() const { return {plan_.M, plan_.N}; }
+  std::string displayName() const {   // MatMulOp.cpp:572-603
+    std::string name = plan_.format == QuantFormat::Q8 ? "MatMulQ8" : "MatMulQ4";
+    if (fusion_ == MatMulFusion::Unary) name += "Unary";
+    if (fusion_ == MatMulFusion::Binary) name += "Binary";
+    return name;
+  }
+  std::string variantName() const { return variantInfo(op(), plan_.spec).name; }
+  const Tensor &output() const { return output_; }
+  void dispatch(void *stream = nullptr) const {
+    const QuantMatMulPlan &p = plan_;
+    const float *A = static_cast<const float *>(a_.data()), *D = static_cast<const float *>(d_.data());
+    float *C = static_cast<float *>(output_.data());
+    const uint16_t *S = static_cast<const uint16_t *>(s_.data());
+    if (p.format == QuantFormat::Q8)
+      check(cuthip_matmul_q8_sep(A, static_cast<const int8_t *>(b_.data()), S, D, C, p.M, p.K, p.N, p.strideA, p.strideB,
+                                 p.strideC, p.scaleStride, (int)fusion_, fusionOp_, (int)p.spec, scratch_.data(),
+                                 scratch_.bytes(), stream),
+            "cuthip_matmul_q8_sep");
+    else
+      check(cuthip_matmul_q4_sep(A, static_cast<const uint8_t *>(b_.data()), S, D, C, p.M, p.K, p.N, p.strideA, p.strideB,
+                                 p.strideC, p.scaleStride, (int)fusion_, fusionOp_, p.q4Affine ? 1 : 0, (int)p.spec,
+                                 scratch_.data(), scratch_.bytes(), stream),
+            "cuthip_matmul_q4_sep");
+  }
+
+private:
+  static size_t shapeRows(const Tensor &t) { return t.shape.empty() ? 0 : t.shape[0]; }
+  cuthip_op op() const { return plan_.format == QuantFormat::Q8 ? CUTHIP_OP_MATMUL_Q8 : CUTHIP_OP_MATMUL_Q4; }
+  Tensor a_, b_, s_, d_;
+  QuantMatMulPlan plan_;
+  MatMulFusion fusion_ = MatMulFusion::None;
+  int fusionOp_ = 0;
+  DeviceBuffer storage_, scratch_;
+  Tensor output_;
+};
+
 // ---- MatMulDenseF16OpNode ----------------------------------------------------------------
 // Prefill matmul on weights kept dequantized: w16 is the fp16 [N, K] output of a DequantOpNode (DataType::Float16,
 // row stride K); the float-path matmul of the reference's runner on its fp16 weight tensors (llama.cpp:800-815).

@@ -19,3 +19,16 @@ def golden():
 
     path = os.path.join(ROOT, "tests", "golden", "dequant_golden.npz")
     return np.load(path, allow_pickle=False)
+
+
+TUNING_KEYS = ("rows8_shape", "gemv_shape", "gemm_ksplit", "dense_tile", "dense_mfma16", "dense_pf")
+
+
+@pytest.fixture
+def tuning():
+    """Forces launch shapes through cuthip_set_tuning for the duration of one test; every key is restored afterwards."""
+    from cut_amd import lib
+
+    yield lib.set_tuning
+    for key in TUNING_KEYS:
+        lib.set_tuning(key, None)

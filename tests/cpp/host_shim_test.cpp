@@ -78,6 +78,76 @@ static void test_validation() {
   EXPECT(throws([&] { prepareSeparated(sw, raw, GgufFormat::Q8_0, 4, 64); }));  // raw too small
 }
 
+template <class F> static std::string message_of(F f) {
+  try {
+    f();
+  } catch (const std::runtime_error &e) {
+    return e.what();
+  }
+  return "";
+}
+
+// Every branch of the 3-input MatMulOpNode constructor (MatMulOp.cpp:283-374): format inference from the shapes, the
+// reference's error texts, the variant it would pick, the padded strides of its push constants.
+static void test_matmul_plan() {
+  using V = std::vector<uint32_t>;
+  const DataType f16 = DataType::Float16;
+  // Q8: B.cols == scales.cols
+  QuantMatMulPlan p = planQuantMatMul(V{4096}, V{4096, 14336}, V{128, 14336}, f16);
+  EXPECT(p.format == QuantFormat::Q8 && p.M == 1 && p.K == 4096 && p.N == 14336 && !p.q4Affine && p.autoSpec);
+  EXPECT(p.spec == 4 && p.fusionFallbackSpec == 4);                       // M == 1: MatMulQ8GemvKPar8
+  EXPECT(variantInfo(CUTHIP_OP_MATMUL_Q8, p.spec).name == "MatMulQ8GemvKPar8");
+  p = planQuantMatMul(V{1, 64}, V{64, 6}, V{2, 6}, f16);
+  EXPECT(p.spec == 3 && p.strideA == 64 && p.strideB == 8 && p.strideC == 8 && p.scaleStride == 8);   // N < 8: GemvKPar
+  p = planQuantMatMul(V{33, 4096}, V{4096, 4096}, V{128, 4096}, f16);
+  EXPECT(p.M == 33 && p.spec == kMatMulQ8VariantCount - 1 && p.fusionFallbackSpec == kMatMulQ8DefaultVariant);   // CoopMatTiled
+  p = planQuantMatMul(V{33, 4096}, V{4096, 4100}, V{128, 4100}, f16);
+  EXPECT(p.spec == kMatMulQ8DefaultVariant);                               // N % 32 != 0: tiled
+  p = planQuantMatMul(V{33, 4096}, V{4096, 4096}, V{128, 4096}, DataType::Float32);
+  EXPECT(p.spec == kMatMulQ8DefaultVariant);                               // scales not Float16: tiled
+  DeviceCaps nocoop;
+  nocoop.cooperativeMatrix = false;
+  p = planQuantMatMul(V{33, 4096}, V{4096, 4096}, V{128, 4096}, f16, {}, nocoop);
+  EXPECT(p.spec == kMatMulQ8DefaultVariant);
+  p = planQuantMatMul(V{33, 4112}, V{4112, 4096}, V{129, 4096}, f16);
+  EXPECT(p.spec == kMatMulQ8DefaultVariant);                               // K % 16 == 0 but not a multiple of 128: tiled here
+  DeviceCaps refcaps;
+  refcaps.cooperativeMatrixK = 16;
+  p = planQuantMatMul(V{33, 4112}, V{4112, 4096}, V{129, 4096}, f16, {}, refcaps);
+  EXPECT(p.spec == kMatMulQ8VariantCount - 1);                             // the reference's own condition
+  p = planQuantMatMul(V{33, 4096}, V{4096, 4096}, V{128, 4096}, f16, 5u);
+  EXPECT(p.spec == 5 && !p.autoSpec);                                      // explicit spec is kept
+  // Q4: 2 * B.cols == scales.cols; affine when the scales have twice the rows
+  p = planQuantMatMul(V{4096}, V{4096, 7168}, V{128, 14336}, f16);
+  EXPECT(p.format == QuantFormat::Q4 && p.N == 14336 && !p.q4Affine && p.spec == 3 && p.strideB == 7168);   // Q4GemvKPar8
+  p = planQuantMatMul(V{4096}, V{4096, 7168}, V{256, 14336}, f16);
+  EXPECT(p.q4Affine && p.spec == 3);
+  p = planQuantMatMul(V{1, 64}, V{64, 3}, V{2, 6}, f16);
+  EXPECT(p.spec == 2 && p.strideB == 4 && p.scaleStride == 8);             // N < 8: Q4GemvKPar
+  p = planQuantMatMul(V{512, 4096}, V{4096, 7168}, V{256, 14336}, f16);
+  EXPECT(p.spec == 4 && p.fusionFallbackSpec == kMatMulQ4DefaultVariant && p.q4Affine);   // MatMulQ4CoopMatTiled
+  p = planQuantMatMul(V{512, 4096}, V{4096, 7170}, V{128, 14340}, f16);
+  EXPECT(p.spec == kMatMulQ4DefaultVariant);
+  // the reference's messages
+  EXPECT(message_of([&] { planQuantMatMul(V{64}, V{64}, V{2, 6}, f16); }) == "matmul requires 2D B and scales matrices");
+  EXPECT(message_of([&] { planQuantMatMul(V{64}, V{64, 6}, V{12}, f16); }) == "matmul requires 2D B and scales matrices");
+  EXPECT(message_of([&] { planQuantMatMul(V{1, 2, 64}, V{64, 6}, V{2, 6}, f16); }) == "matmul: A must be 1D or 2D");
+  EXPECT(message_of([&] { planQuantMatMul(V{96}, V{64, 6}, V{2, 6}, f16); }) == "matmul: B rows (64) must match A cols (96)");
+  EXPECT(message_of([&] { planQuantMatMul(V{64}, V{64, 5}, V{2, 6}, f16); }) ==
+         "matmul: cannot determine quant format from B cols (5) and scales cols (6)");
+  // the node validates before it touches the device
+  DeviceBuffer none;
+  Tensor a{&none, {64}, DataType::Float32, 0}, b{&none, {64, 8}, DataType::Float32, 0}, sc{&none, {2, 8}, DataType::Float16, 0};
+  EXPECT(throws([&] { MatMulOpNode n(a, b, sc); }));                         // buffers too small
+  EXPECT(message_of([&] { MatMulOpNode n(a, b, sc, 8u); }).find("outside the table") != std::string::npos);
+  Tensor a16{&none, {64}, DataType::Float16, 0};
+  EXPECT(message_of([&] { MatMulOpNode n(a16, b, sc); }).find("Float32 activations") != std::string::npos);
+  Tensor a48{&none, {48}, DataType::Float32, 0}, b48{&none, {48, 8}, DataType::Float32, 0};
+  EXPECT(message_of([&] { MatMulOpNode n(a48, b48, sc); }).find("multiple of the 32-element") != std::string::npos);
+  Tensor as{&none, {2, 64}, DataType::Float32, 70};
+  EXPECT(message_of([&] { MatMulOpNode n(as, b, sc); }).find("padded to four") != std::string::npos);
+}
+
 static double normwise(const std::vector<float> &got, const std::vector<double> &want) {
   double num = 0, den = 0;
   for (size_t i = 0; i < got.size(); ++i) {
@@ -255,6 +325,72 @@ static void test_gpu() {
       EXPECT(err < 1e-3);
     }
   }
+  // The 3-input MatMulOpNode on the reference's known answers (tests/harness/OpRegistry.h:1995-2086): format and
+  // variant inferred from the shapes, rows padded to four elements as the reference's tensors are.
+  {
+    auto run = [&](uint32_t M, uint32_t K, uint32_t N, bool q4, const std::vector<uint8_t> &bvals, const std::vector<float> &scales,
+                   uint32_t scaleRows, std::optional<uint32_t> spec) {
+      const uint32_t cols = q4 ? N / 2 : N, sB = (cols + 3) & ~3u, sS = (N + 3) & ~3u, sA = (K + 3) & ~3u;
+      std::vector<float> a((size_t)M * sA, 1.0f);
+      std::vector<uint8_t> b((size_t)K * sB, 0);
+      for (uint32_t k = 0; k < K; ++k)
+        for (uint32_t c = 0; c < cols; ++c) b[(size_t)k * sB + c] = bvals[(size_t)k * cols + c];
+      std::vector<uint16_t> s((size_t)scaleRows * sS, 0);
+      for (uint32_t r = 0; r < scaleRows; ++r)
+        for (uint32_t n = 0; n < N; ++n) s[(size_t)r * sS + n] = orc_f32_to_f16(scales[(size_t)r * N + n]);
+      DeviceBuffer adev(a.data(), a.size() * 4), bdev(b.data(), b.size()), sdev(s.data(), s.size() * 2);
+      Tensor at{&adev, M == 1 ? std::vector<uint32_t>{K} : std::vector<uint32_t>{M, K}, DataType::Float32, 0};
+      Tensor bt{&bdev, {K, cols}, DataType::Float32, 0}, st{&sdev, {scaleRows, N}, DataType::Float16, 0};
+      MatMulOpNode mm(at, bt, st, spec);
+      EXPECT(mm.format() == (q4 ? QuantFormat::Q4 : QuantFormat::Q8));
+      mm.dispatch();
+      std::vector<float> c((size_t)M * mm.plan().strideC);
+      mm.output().buffer->download(c.data(), c.size() * 4);
+      return c;
+    };
+    // q8_simple: A = 1, B[k, 0] = 1, B[k, 1] = 2, scales 1 -> [32, 64]
+    std::vector<uint8_t> b8(32 * 2);
+    for (uint32_t k = 0; k < 32; ++k) { b8[2 * k] = 1; b8[2 * k + 1] = 2; }
+    auto c = run(1, 32, 2, false, b8, {1.0f, 1.0f}, 1, {});
+    EXPECT(std::fabs(c[0] - 32.0f) < 1e-3f && std::fabs(c[1] - 64.0f) < 1e-3f);
+    // q8_withscales: K = 64, B = 4, scales {0.5, 2} / {1, 0.25} -> [192, 288]
+    c = run(1, 64, 2, false, std::vector<uint8_t>(64 * 2, 4), {0.5f, 2.0f, 1.0f, 0.25f}, 2, {});
+    EXPECT(std::fabs(c[0] - 192.0f) < 1.0f && std::fabs(c[1] - 288.0f) < 1.0f);
+    // q4: nibbles 9 / 10 (values 1 / 2) -> [32, 64]; nibble 12 with the scales above -> [192, 288]
+    c = run(1, 32, 2, true, std::vector<uint8_t>(32, 9 | (10 << 4)), {1.0f, 1.0f}, 1, {});
+    EXPECT(std::fabs(c[0] - 32.0f) < 1e-3f && std::fabs(c[1] - 64.0f) < 1e-3f);
+    c = run(1, 64, 2, true, std::vector<uint8_t>(64, 12 | (12 << 4)), {0.5f, 2.0f, 1.0f, 0.25f}, 2, {});
+    EXPECT(std::fabs(c[0] - 192.0f) < 1.0f && std::fabs(c[1] - 288.0f) < 1.0f);
+    // every variant index of both tables on the same case, and at M = 3 (the reference's q8/q4AllVariantsVerify)
+    for (uint32_t spec = 0; spec < kMatMulQ8VariantCount; ++spec)
+      for (uint32_t M : {1u, 3u}) {
+        if (spec == kMatMulQ8VariantCount - 1) continue;   // the matrix-core variant needs K % 128 == 0: below
+        c = run(M, 64, 2, false, std::vector<uint8_t>(64 * 2, 4), {0.5f, 2.0f, 1.0f, 0.25f}, 2, spec);
+        EXPECT(std::fabs(c[0] - 192.0f) < 1.0f && std::fabs(c[1] - 288.0f) < 1.0f);
+      }
+    for (uint32_t spec = 0; spec + 1 < kMatMulQ4VariantCount; ++spec)
+      for (uint32_t M : {1u, 3u}) {
+        c = run(M, 64, 2, true, std::vector<uint8_t>(64, 12 | (12 << 4)), {0.5f, 2.0f, 1.0f, 0.25f}, 2, spec);
+        EXPECT(std::fabs(c[0] - 192.0f) < 1.0f && std::fabs(c[1] - 288.0f) < 1.0f);
+      }
+    // M > 1 on a shape the matrix-core variants take (chosen automatically): q = 1, scales 0.5 -> K / 2 everywhere;
+    // affine Q4 with nibble 9 (value 1), scale 0.5, minimum 0.25 -> K * 0.75
+    {
+      const uint32_t M = 40, K = 256, N = 64;
+      c = run(M, K, N, false, std::vector<uint8_t>((size_t)K * N, 1), std::vector<float>((size_t)(K / 32) * N, 0.5f), K / 32, {});
+      bool ok = true;
+      for (uint32_t m = 0; m < M && ok; ++m)
+        for (uint32_t n = 0; n < N && ok; ++n) ok = std::fabs(c[(size_t)m * N + n] - K * 0.5f) < 1e-2f;
+      EXPECT(ok);
+      std::vector<float> sm((size_t)(2 * K / 32) * N, 0.5f);
+      for (size_t i = (size_t)(K / 32) * N; i < sm.size(); ++i) sm[i] = 0.25f;
+      c = run(M, K, N, true, std::vector<uint8_t>((size_t)K * N / 2, 9 | (9 << 4)), sm, 2 * K / 32, {});
+      ok = true;
+      for (uint32_t m = 0; m < M && ok; ++m)
+        for (uint32_t n = 0; n < N && ok; ++n) ok = std::fabs(c[(size_t)m * N + n] - K * 0.75f) < 1e-2f;
+      EXPECT(ok);
+    }
+  }
   // an explicit variant that cannot take the shape is an error, not a silent fallback
   {
     std::vector<uint8_t> blocks(ggufBytes(GgufFormat::Q8_0, 64 * 64), 0);
@@ -275,6 +411,7 @@ int main(int argc, char **argv) {
   std::string mode = argc > 1 ? argv[1] : "--cpu";
   test_tables();
   test_validation();
+  test_matmul_plan();
   if (mode == "--gpu") test_gpu();
   std::printf("%s: %d failure(s)\n", mode.c_str(), g_fail);
   return g_fail ? 1 : 0;

@@ -238,6 +238,121 @@ def test_repetition_penalty_and_penalized_argmax(ops):
             assert np.array_equal(d.cpu().numpy(), want_l)
 
 
+@pytest.mark.parametrize("n_pen", [66, 100, 1000])
+def test_penalized_argmax_with_lists_longer_than_a_wave(ops, n_pen):
+    """Penalty lists of more than 64 entries (the runner's default window is 64 tokens plus the suppressed ones,
+    llama.cpp:2566-2592): entries handled by the second and later waves of the finishing workgroup, a list length that
+    is not a multiple of 64, the unpenalised winner and the runners-up listed late in the list, padding entries of -1,
+    and a winner after the penalty that sits in a row scanned by a thread of another wave.  Against the oracle's dense
+    penalty followed by arg-max, on the logits directly and through the matmul's per-wave winners."""
+    rng = np.random.default_rng(70 + n_pen)
+    n = 40000
+    lg = (rng.standard_normal(n) * 2).astype(np.float32)
+    order = np.argsort(lg)
+    top = [int(t) for t in order[-5:][::-1]]                  # the five largest logits, largest first
+    toks = [int(t) for t in rng.choice(n, n_pen, replace=False)]
+    # the winners sit at the end of the list; the largest is listed twice and its last entry (the last of the list,
+    # handled by the last thread that has an entry) is the one that counts
+    toks = [t for t in toks if t not in top][:n_pen - 9] + [-1] * 3 + top + [top[0]]
+    assert len(toks) == n_pen
+    facs = [float(f) for f in rng.uniform(1.1, 3.0, n_pen)]
+    for i, t in enumerate(toks):
+        if t in top:
+            facs[i] = 1e6
+    facs[n_pen - 6] = 1.0                                     # the first entry of the largest: overridden
+    dense = np.ones(n, np.float32)
+    for t, f in zip(toks, facs):
+        if 0 <= t < n:
+            dense[t] = f
+    idx = torch.full((1,), -1, dtype=torch.int32, device="cuda")
+    for dt in (np.float32, np.float16):
+        l_h = lg.astype(dt)
+        want_l = oracle.repetition_penalty(l_h.astype(np.float32), dense).astype(dt)
+        want = int(np.argmax(want_l))
+        assert want not in top
+        if dt is np.float32:
+            assert (want % 1024) >= 64                        # found by a thread outside the first wave
+        d = dev(l_h.copy())
+        ops.argmax_penalized(d, idx, dev(np.array(toks, np.int32)), dev(np.array(facs, np.float32)))
+        torch.cuda.synchronize()
+        assert int(idx.item()) == want, (dt, n_pen)
+        assert np.array_equal(d.cpu().numpy(), want_l)
+    # through the head matmul: per-wave winners in the workspace, the listed groups re-derived from the logits
+    fmt, N, K = oracle.Q8_0, 12296, 512
+    W = dev(quantized_weights(fmt, N, K, seed=71))
+    a = dev(gauss_acts((1, K), seed=72, dtype=np.float16)).view(-1)
+    ref = ops.matmul_gguf(a, W, fmt, N, K, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    ref = ref.cpu().numpy()[0]
+    order = np.argsort(ref)
+    top = [int(t) for t in order[-5:][::-1]]
+    toks = [int(t) for t in rng.choice(N, n_pen, replace=False) if int(t) not in top][:n_pen - 6] + [-1] + top
+    toks = (toks + [-1] * n_pen)[:n_pen]
+    facs = [1e6 if t in top else 1.5 for t in toks]
+    dense = np.ones(N, np.float32)
+    for t, f in zip(toks, facs):
+        if 0 <= t < N:
+            dense[t] = f
+    want_l = oracle.repetition_penalty(ref, dense)
+    for ws in (ops.lm_head_workspace(N, "cuda"), None):
+        logits = torch.empty(N, dtype=torch.float32, device="cuda")
+        ops.matmul_gguf_argmax(a, W, fmt, N, K, logits, idx, pen_tokens=dev(np.array(toks, np.int32)),
+                               pen_factors=dev(np.array(facs, np.float32)), workspace=ws)
+        torch.cuda.synchronize()
+        assert np.array_equal(logits.cpu().numpy(), want_l)
+        assert int(idx.item()) == int(np.argmax(want_l)), (n_pen, ws is None)
+
+
+@pytest.mark.parametrize("max_ctx,seq", [(100, 120), (100, 128), (64, 1000), (130, 131)])
+def test_attention_decode_clamps_the_length_to_the_cache_capacity(ops, max_ctx, seq):
+    """A device-side sequence length beyond max_seq_len attends the max_seq_len cached positions once each (capacities
+    that are not a multiple of the 64-position chunk included), through the workspace entry point and the
+    allocation-free one."""
+    n_heads, n_kv, hd = 8, 2, 64
+    rng = np.random.default_rng(max_ctx + seq)
+    q = rng.standard_normal(n_heads * hd).astype(np.float32)
+    K = (rng.standard_normal((max_ctx, n_kv * hd)) * 0.5).astype(np.float16)
+    V = rng.standard_normal((max_ctx, n_kv * hd)).astype(np.float16)
+    scale = 1 / math.sqrt(hd)
+    want = oracle.attention_decode(q, K.view(np.uint16), V.view(np.uint16), max_ctx, n_heads, n_kv, hd, scale)
+    ws = ops.attn_decode_workspace(n_heads, hd, max_ctx, "cuda")
+    params = dev(np.array([seq - 1, seq], np.int32))
+    out = torch.empty(n_heads * hd, dtype=torch.float32, device="cuda")
+    ops.attn_decode(dev(q), dev(K), dev(V), params, n_heads, n_kv, hd, scale, ws, out)
+    torch.cuda.synchronize()
+    assert normwise_rel_err(out.cpu().numpy(), want) < 2e-6
+    out2 = torch.empty_like(out)
+    ops.attn_decode_static(dev(q), dev(K), dev(V), params, n_heads, n_kv, hd, scale, out2)
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+
+
+def test_memset_is_refused_on_a_capturing_stream(ops):
+    """cuthip_memset records nothing into a graph: on a capturing stream it returns an error and the capture goes on."""
+    from cut_amd import lib
+    import ctypes as C
+    L = lib.load()
+    buf = torch.full((256,), 7, dtype=torch.uint8, device="cuda")
+    st = C.c_void_p()
+    lib.check(L.cuthip_stream_create(C.byref(st)))
+    try:
+        lib.check(L.cuthip_memset(buf.data_ptr(), 1, 256, st))          # eager: allowed
+        lib.check(L.cuthip_stream_sync(st))
+        assert bool((buf == 1).all())
+        lib.check(L.cuthip_graph_begin_capture(st))
+        rc = L.cuthip_memset(buf.data_ptr(), 2, 256, st)
+        msg = L.cuthip_last_error()
+        g = C.c_void_p()
+        lib.check(L.cuthip_graph_end_capture(st, C.byref(g)))
+        assert rc != 0 and b"capturing" in msg
+        lib.check(L.cuthip_graph_launch(g, st))
+        lib.check(L.cuthip_stream_sync(st))
+        assert bool((buf == 1).all())
+        lib.check(L.cuthip_graph_destroy(g))
+    finally:
+        L.cuthip_stream_destroy(st)
+
+
 @pytest.mark.parametrize("name,N,K", [("Q6_K", 128256, 4096), ("Q4_K", 14336, 4096), ("Q8_0", 12296, 512), ("Q6_K", 1000, 512)])
 def test_head_matmul_with_argmax_in_the_epilogue(ops, name, N, K):
     """cuthip_matmul_gguf_argmax against the plain matmul followed by `penalty, then arg-max`: same logits bit for bit,
@@ -252,6 +367,11 @@ def test_head_matmul_with_argmax_in_the_epilogue(ops, name, N, K):
     plain = ops.matmul_gguf(a, W, fmt, N, K, out_dtype=torch.float32)
     torch.cuda.synchronize()
     ref = plain.cpu().numpy()[0]
+    # the logits themselves against the float64 oracle, on a sample of vocabulary rows
+    rows = np.unique(np.concatenate([[0, N - 1], np.random.default_rng(62).integers(0, N, 512)]))
+    Wh = W.cpu().numpy().reshape(N, rb)[rows].reshape(-1)
+    want_rows = oracle.matmul_gguf(fmt, Wh, a.cpu().numpy().astype(np.float32)[None], len(rows), f64=True)[0]
+    assert normwise_rel_err(ref[rows], want_rows) < 2e-5
     order = np.argsort(ref)
     top, runner_up = int(order[-1]), int(order[-2])
     ws = ops.lm_head_workspace(N, "cuda")

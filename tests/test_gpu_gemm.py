@@ -238,7 +238,7 @@ def test_dense_gemm_128x448_tiles(ops):
 
 @pytest.mark.parametrize("name,K", [("Q4_K", 4096), ("Q6_K", 2048), ("Q8_0", 4128), ("Q4_0", 2080), ("Q4_K", 14336)])
 @pytest.mark.parametrize("M", [9, 70, 128, 200])
-def test_tiled_gemm_splits_k_through_the_workspace(ops, monkeypatch, name, K, M):
+def test_tiled_gemm_splits_k_through_the_workspace(ops, tuning, name, K, M):
     """The single-launch GEMM (variant 2) with a workspace at hand: few tiles, so K is split over workgroups (fp32
     partial products, summed by the reduce kernel, which also applies the epilogue).  Ragged tiles, a K whose last
     range ends in a partial slice, fp16 and fp32 activations, the residual add, and a forced split of 3 ranges of
@@ -259,20 +259,20 @@ def test_tiled_gemm_splits_k_through_the_workspace(ops, monkeypatch, name, K, M)
     assert normwise_rel_err(got16 - D.astype(np.float32), want) < 2e-3   # fp16 rounding of sum + D
     got32 = gpu_matmul_ws(ops, fmt, W, A.astype(np.float32), N, K, out_dtype=torch.float32, variant=2)
     assert normwise_rel_err(got32, want) < TOL_GEMM
-    monkeypatch.setenv("CUT_HIP_GEMM_KSPLIT", "3")
+    tuning("gemm_ksplit", "3")
     got3 = gpu_matmul_ws(ops, fmt, W, A, N, K, out_dtype=torch.float32, variant=2)
     assert normwise_rel_err(got3, unsplit) < 1e-6
 
 
 @pytest.mark.parametrize("mfma16", ["1", "0"])
 @pytest.mark.parametrize("tile", ["256,224", "128,448", "256,256", "128,256", "128,256,2", "256,256,4"])
-def test_dense_gemm_every_tile_shape_and_both_kernels(ops, monkeypatch, tile, mfma16):
+def test_dense_gemm_every_tile_shape_and_both_kernels(ops, tuning, tile, mfma16):
     """Every tile shape of the dense GEMM (with and without a K split) under both of its kernels (16 x 16 x 32 MFMAs,
-    the default, and 32 x 32 x 16), forced through the library's tuning variables, on a problem with ragged tiles on
+    the default, and 32 x 32 x 16), forced through cuthip_set_tuning, on a problem with ragged tiles on
     both sides: every output against the single-launch GEMM, sampled rows and columns against the oracle, and the
     residual-add epilogue (the short output loop with an operand)."""
-    monkeypatch.setenv("CUT_HIP_DENSE_TILE", tile)
-    monkeypatch.setenv("CUT_HIP_DENSE_MFMA16", mfma16)
+    tuning("dense_tile", tile)
+    tuning("dense_mfma16", mfma16)
     fmt = oracle.Q4_K
     bn = int(tile.split(",")[1])
     M, N, K = 700, 3 * bn - 8, 1024

@@ -60,7 +60,7 @@ def test_gemv_fp32_activations_config1_shape(ops, name):
     assert err < TOL_F32_ACT, err
 
 
-@pytest.mark.parametrize("M", [1, 8])
+@pytest.mark.parametrize("M", [1, 2, 4, 8])
 @pytest.mark.parametrize("N,K", [(14336, 4096), (4096, 14336)])
 def test_q4k_ffn_shapes_fp16_io(ops, N, K, M):
     """BASELINE config 3: FFN shapes, fp16 in, fp32 accumulate, fp16 out.
@@ -325,11 +325,11 @@ FORCED_ROWS8 = [("4,1", 1024, [1, 2, 4, 8]), ("4,1", 4096 + 256, [1, 3, 8]), ("8
 
 @pytest.mark.parametrize("name", list(oracle.FORMATS))
 @pytest.mark.parametrize("shape,K,batches", FORCED_ROWS8)
-def test_rows8_every_workgroup_shape(ops, monkeypatch, name, shape, K, batches):
-    """Every workgroup shape of the 8-row GEMV, forced through the library's tuning variable instead of left to the
+def test_rows8_every_workgroup_shape(ops, tuning, name, shape, K, batches):
+    """Every workgroup shape of the 8-row GEMV, forced through cuthip_set_tuning instead of left to the
     choice by N and K (which reaches only one shape per problem), for every format and batch class, with a fused
     residual add: against the oracle."""
-    monkeypatch.setenv("CUT_HIP_ROWS8_SHAPE", shape)
+    tuning("rows8_shape", shape)
     fmt = oracle.FORMATS[name]
     N = 8 * 37 + 3
     W = quantized_weights(fmt, N, K, seed=K + 1)
@@ -345,11 +345,11 @@ def test_rows8_every_workgroup_shape(ops, monkeypatch, name, shape, K, batches):
 
 @pytest.mark.parametrize("name", list(oracle.FORMATS))
 @pytest.mark.parametrize("shape", ["1,1", "1,2", "1,4", "1,8", "2,1", "2,2", "2,4", "2,8"])
-def test_fallback_gemv_every_workgroup_shape(ops, monkeypatch, name, shape):
+def test_fallback_gemv_every_workgroup_shape(ops, tuning, name, shape):
     """The fallback GEMV (variant 0; 32 weight rows per workgroup, or 16 with two K parts per wave) under every
-    (parts, waves) shape, forced through the tuning variable: step counts that take the straight-line instances
+    (parts, waves) shape, forced through cuthip_set_tuning: step counts that take the straight-line instances
     (2, 4 and 7 steps per wave) and the generic loop, batch 1 to 8 in one pass and 20 rows as a 32-row pass."""
-    monkeypatch.setenv("CUT_HIP_GEMV_SHAPE", shape)
+    tuning("gemv_shape", shape)
     fmt = oracle.FORMATS[name]
     N = 3 * 32 + 5
     for K, batches in [(2048, [1, 2, 4, 8, 20]), (7168, [1, 3]), (2304, [1, 5, 20])]:
@@ -519,3 +519,46 @@ def test_mid_size_batches_run_as_eight_row_passes(ops, name, M):
     want = oracle.matmul_gguf(fmt, W, A.astype(np.float32), N, f64=True)
     assert normwise_rel_err(c_buf[:, :N].cpu().numpy() - D, want) < TOL_F16_ACT
     assert torch.all(c_buf[:, N:] == 7.0)
+
+
+@pytest.mark.parametrize("M", [16, 32])
+def test_streaming_kernel_rounds_fp32_activations_to_fp16(ops, M):
+    """Variant 6 (and the automatic choice at 9..32 rows of Q4_K) stages fp32 activations as fp16, nearest even: against
+    the float64 oracle on the fp32 values the result carries that rounding (2^-11 relative per element, a few 1e-4
+    normwise), and against the oracle on the rounded values it is as tight as with fp16 inputs."""
+    fmt = oracle.Q4_K
+    N, K = 520, 2048
+    W = quantized_weights(fmt, N, K, seed=170)
+    A = gauss_acts((M, K), seed=171)
+    a, w = torch.from_numpy(A).cuda(), torch.from_numpy(W).cuda()
+    ws = ops.matmul_gguf_workspace(fmt, M, K, N, a.dtype, "cuda")
+    for variant in (6, -1):
+        got = ops.matmul_gguf(a, w, fmt, N, K, out_dtype=torch.float32, workspace=ws, variant=variant)
+        torch.cuda.synchronize()
+        got = got.cpu().numpy()
+        assert normwise_rel_err(got, oracle.matmul_gguf(fmt, W, A, N, f64=True)) < TOL_F32_ACT
+        rounded = A.astype(np.float16).astype(np.float32)
+        assert normwise_rel_err(got, oracle.matmul_gguf(fmt, W, rounded, N, f64=True)) < TOL_F16_ACT
+
+
+@pytest.mark.parametrize("op", ["mod", "pow", "floor_div"])
+def test_long_binary_operator_refuses_aliased_operand_before_writing(ops, op):
+    """The operators that run as a launch of their own after the matmul need D intact: D == C is refused by every
+    entry point before the unfused matmul is launched, so the caller's buffer still holds D."""
+    from cut_amd import lib
+    fmt = oracle.Q4_K
+    N, K, M = 64, 512, 3
+    w = torch.from_numpy(quantized_weights(fmt, N, K, seed=180)).cuda()
+    a = torch.from_numpy(gauss_acts((M, K), seed=181, dtype=np.float16)).cuda()
+    d0 = gauss_acts((M, N), seed=182)
+    c = torch.from_numpy(d0.copy()).cuda()
+    ws = ops.matmul_gguf_workspace(fmt, M, K, N, a.dtype, "cuda")
+    L = lib.load()
+    rc = L.cuthip_matmul_gguf(fmt, w.data_ptr(), a.data_ptr(), lib.F16, c.data_ptr(), lib.F32, M, K, N, K, N, lib.EPI_BINARY,
+                              lib.BINARY[op], c.data_ptr(), -1, None)
+    assert rc != 0 and b"alias" in L.cuthip_last_error()
+    rc = L.cuthip_matmul_gguf_ws(fmt, w.data_ptr(), a.data_ptr(), lib.F16, c.data_ptr(), lib.F32, M, K, N, K, N, lib.EPI_BINARY,
+                                 lib.BINARY[op], c.data_ptr(), -1, ws.data_ptr(), ws.numel(), None)
+    assert rc != 0 and b"alias" in L.cuthip_last_error()
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy(), d0)
