@@ -568,6 +568,51 @@ template <int SUBK, int THREADS, int MT, int XR, bool PRO> struct XStage {
   }
 };
 
+// fp16 activations without a prologue (every decode matmul).  Same groups of 8 per thread as the general path (a wave's
+// load is 1 KB contiguous; whole 32-element sub-blocks per thread were tried and cost 6 % at batch 1: a load instruction
+// then touches 64 lines instead of 8), but no conversion: the sum of a group is four v_dot2 against (1, 1), the sums of
+// the 2 or 4 groups of a sub-block meet through DPP quad permutes instead of LDS shuffles, the reordering is four byte
+// permutes.  A wave issues one instruction per four cycles whatever its kind, so a shorter start-up is time won before
+// the first product.
+template <int SUBK, int THREADS, int MT, int XR> struct XStageF16 {
+  u32x4 r[MT * XR];
+  __device__ void load(const GemvParams &p, uint32_t base, int tid) {
+#pragma unroll
+    for (int u = 0; u < MT * XR; ++u) {
+      const uint32_t m = u / XR, gi = base + (u % XR) * THREADS + tid, k = gi * 8;
+      if (m < p.M && k < p.K) r[u] = ld_u32x4(reinterpret_cast<const uint8_t *>(p.A) + ((size_t)m * p.strideA + k) * 2u);
+    }
+  }
+  static __device__ __forceinline__ float quad_xor_add(float s, bool two) {
+    // every lane of the quad executes this (callers keep it outside divergent code)
+    s += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, s), 0xB1, 0xF, 0xF, true));   // lanes (1 0 3 2)
+    if (two) s += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, s), 0x4E, 0xF, 0xF, true));   // lanes (2 3 0 1)
+    return s;
+  }
+  __device__ void store(const GemvParams &p, uint32_t base, int tid, uint32_t gpr, half_t *xs, float *sxs, int xrow, int sxrow) {
+    const half2_t one{(half_t)1.0f, (half_t)1.0f};
+#pragma unroll
+    for (int u = 0; u < MT * XR; ++u) {
+      const uint32_t m = u / XR, gi = base + (u % XR) * THREADS + tid, k = gi * 8;
+      const bool active = m < p.M && gi < gpr, ok = active && k < p.K;   // groups between K and the padded length hold zeros
+      const uint32_t e0 = ok ? r[u].x : 0u, e1 = ok ? r[u].y : 0u, e2 = ok ? r[u].z : 0u, e3 = ok ? r[u].w : 0u;
+      float s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, e0), one, 0.0f, false);
+      s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, e1), one, s, false);
+      s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, e2), one, s, false);
+      s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, e3), one, s, false);
+      s = quad_xor_add(s, SUBK == 32);
+      if (active) {
+        // halves (0 1)(2 3)(4 5)(6 7) -> (0 2)(1 3)(4 6)(5 7)
+        *reinterpret_cast<u32x4 *>(xs + m * xrow + (gi >> 3) * kXGroup + (gi & 7) * 8) =
+            u32x4{__builtin_amdgcn_perm(e1, e0, 0x05040100u), __builtin_amdgcn_perm(e1, e0, 0x07060302u),
+                  __builtin_amdgcn_perm(e3, e2, 0x05040100u), __builtin_amdgcn_perm(e3, e2, 0x07060302u)};
+        constexpr uint32_t per = SUBK / 8;
+        if ((gi & (per - 1)) == 0) sxs[m * sxrow + gi / per] = s;
+      }
+    }
+  }
+};
+
 // ---- the kernel -----------------------------------------------------------------
 // MT: batch rows held (1, 2 or 4); RWG x KW waves per workgroup; D ring depth.
 // MT == 1 takes the lane-local dot-product path (v_dot2_f32_f16 on the same
@@ -629,9 +674,13 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
   // second batch (every further batch is one more memory round trip before the first step can start)
   constexpr int XCAP = 8 / MT, XR = XWANT < XCAP ? XWANT : XCAP;
   const uint32_t gpr = kpad / 8;   // 8-element groups per padded row
+  // fp16 activations and no prologue: the short staging; otherwise the general one
+  const bool fastx = !PRO && p.a_f16;
   XStage<S::SUBK, THREADS, MT, XR, PRO> xst;
+  XStageF16<S::SUBK, THREADS, MT, XR> xsf;
   xst.init();
-  xst.load(p, 0, tid, gpr);
+  if (fastx) xsf.load(p, 0, tid);
+  else xst.load(p, 0, tid, gpr);
   // carried RMSNorm, consumer side: the K / 8 partial sums of squares travel like the activations: requested ahead of
   // the weight ring, one share per thread, folded per wave and across the waves through LDS at the staging barrier
   // (the order of the additions depends on the launch shape only)
@@ -649,10 +698,18 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
     S::load(buf[i], row, min(sb + i, last), c, p.K);
     __builtin_amdgcn_sched_barrier(0);   // keep issue order = ring order, so that step i waits for its own loads only
   }
-  xst.store(p, 0, tid, gpr, xs, sxs, xrow, sxrow);
-  for (uint32_t base = THREADS * XR; base < gpr; base += THREADS * XR) {
-    xst.load(p, base, tid, gpr);
-    xst.store(p, base, tid, gpr, xs, sxs, xrow, sxrow);
+  if (fastx) {
+    xsf.store(p, 0, tid, gpr, xs, sxs, xrow, sxrow);
+    for (uint32_t base = THREADS * XR; base < gpr; base += THREADS * XR) {
+      xsf.load(p, base, tid);
+      xsf.store(p, base, tid, gpr, xs, sxs, xrow, sxrow);
+    }
+  } else {
+    xst.store(p, 0, tid, gpr, xs, sxs, xrow, sxrow);
+    for (uint32_t base = THREADS * XR; base < gpr; base += THREADS * XR) {
+      xst.load(p, base, tid, gpr);
+      xst.store(p, base, tid, gpr, xs, sxs, xrow, sxrow);
+    }
   }
   if (!PRO && nparts) {
     float t = (cpart[0] + cpart[1]) + (cpart[2] + cpart[3]);
