@@ -78,10 +78,31 @@ struct LaneCtx {
   uint32_t c0, c1, c2, c3;  // per-lane constants of the format
 };
 
+// Sums across lanes without the LDS crossbar (a ds_bpermute round trip is about a hundred cycles, and these sit on
+// the tail of every wave).  Every lane of the wave must be active.  add_xor4 / add_xor8 mirror 8 / 16 lanes, which is
+// the xor exchange once the smaller groups hold equal sums, so they are used in that order only.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float add_xor1(float v) { return v + dpp_move<0xB1>(v); }    // quad_perm (1 0 3 2)
+__device__ __forceinline__ float add_xor2(float v) { return v + dpp_move<0x4E>(v); }    // quad_perm (2 3 0 1)
+__device__ __forceinline__ float add_xor4(float v) { return v + dpp_move<0x141>(v); }   // row_half_mirror
+__device__ __forceinline__ float add_xor8(float v) { return v + dpp_move<0x140>(v); }   // row_mirror
+// (the swaps exchange the odd rows / upper half of the first operand with the even rows / lower half of the second.
+// The elements of the result are read into scalars first: __builtin_bit_cast applied to a vector element expression
+// reads element 0 whatever the index, with this compiler)
+__device__ __forceinline__ float add_xor16(float v) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, v), __builtin_bit_cast(uint32_t, v), false, false);
+  const uint32_t mine = r[0], other = r[1];
+  return __builtin_bit_cast(float, mine) + __builtin_bit_cast(float, other);
+}
+__device__ __forceinline__ float add_xor32(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, v), __builtin_bit_cast(uint32_t, v), false, false);
+  const uint32_t mine = r[0], other = r[1];
+  return __builtin_bit_cast(float, mine) + __builtin_bit_cast(float, other);
+}
 __device__ inline float wave_sum_all(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-  return v;
+  return add_xor32(add_xor16(add_xor8(add_xor4(add_xor2(add_xor1(v))))));
 }
 
 // One output row of a matmul with the RoPE / cache-append epilogue: v = this row's product, partner = the
@@ -720,9 +741,7 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
   if (PRO && p.pro == CUTHIP_PRO_RMSNORM) {
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
-      float t = xst.ssq[m];
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o);
+      const float t = wave_sum_all(xst.ssq[m]);
       if (lane == 0) nrm[m * WAVES + wave] = t;
     }
   }
@@ -801,9 +820,7 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
 #pragma unroll
     for (int q = 0; q < RQ; ++q) {
       float v = S::finish_dot(acc[q], cacc[q]);
-      v += __shfl_xor(v, 1);
-      v += __shfl_xor(v, 2);
-      v += __shfl_xor(v, 32);
+      v = add_xor32(add_xor2(add_xor1(v)));
       out[q] = (PRO ? v * xscale[q] : v) * carry_scale;   // linear in the partial sums: applied before the K ranges are folded
     }
     writer = c.g == 0 && c.kg == 0;
@@ -812,8 +829,7 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
     for (int q = 0; q < RQ; ++q) {
       float v = c.g == 0 ? acc[4 * q] : c.g == 1 ? acc[4 * q + 1] : c.g == 2 ? acc[4 * q + 2] : acc[4 * q + 3];
       v = S::finish(v, cacc[q]);
-      v += __shfl_xor(v, 1);
-      v += __shfl_xor(v, 2);
+      v = add_xor2(add_xor1(v));
       out[q] = v * carry_scale;   // batch row 2q + kg
     }
     writer = c.g == 0;
@@ -922,9 +938,7 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
       carry_sq = wave_sum_all(carry_sq);
       if (lane == 0 && n0 < p.N) p.next_sumsq_parts[n0 / 8] = carry_sq;
     } else {         // folded epilogue: thread 8 g + r of the workgroup holds row r of its g-th row group
-      carry_sq += __shfl_xor(carry_sq, 1);
-      carry_sq += __shfl_xor(carry_sq, 2);
-      carry_sq += __shfl_xor(carry_sq, 4);
+      carry_sq = add_xor4(add_xor2(add_xor1(carry_sq)));
       const uint32_t grp = bid * RWG + (uint32_t)tid / 8;
       if (tid < RWG * 8 && (tid & 7) == 0 && grp * 8 < p.N) p.next_sumsq_parts[grp] = carry_sq;
     }
