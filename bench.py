@@ -9,7 +9,8 @@ activations in and out, fp32 accumulation.  One step = the three GEMVs of one
 FFN block (gate and up 14336 x 4096, down 4096 x 14336).  Weights are resident
 in HBM before the timed region and every step reads a different copy of them
 (COPIES sets, 595 MB in total), so they stream from HBM and not from the
-256 MB Infinity Cache.  The K timed steps are replayed as one HIP graph.
+256 MB Infinity Cache.  The K timed steps are one HIP graph, replayed once untimed
+(the first replay also uploads the graph: 0.5-1 us per launch at K = 300) and once timed.
 
 Prints one JSON line: metric/value = algorithmic bytes per second over the
 whole timed region, plus "roofline" (the GEMV kernel against the 8 TB/s HBM
@@ -42,8 +43,8 @@ def make_q_weights(fmt_name, n, k, seed):
 
 
 def timed_graph(torch, fn_step, steps, warmup):
-    """Runs `warmup` eager steps, captures `steps` steps into one HIP graph and
-    replays it once.  Returns (wall_seconds, event_ms, used_graph)."""
+    """Runs `warmup` eager steps, captures `steps` steps into one HIP graph, replays it once untimed (part of the
+    warm-up) and once timed.  Returns (wall_seconds, event_ms, used_graph)."""
     for s in range(warmup):
         fn_step(s)
     torch.cuda.synchronize()
@@ -55,6 +56,7 @@ def timed_graph(torch, fn_step, steps, warmup):
                 fn_step(s)
         torch.cuda.synchronize()
         run = g.replay
+        g.replay()   # untimed: the first replay of a graph also uploads it to the device
     except Exception as e:  # noqa: BLE001
         log(f"[bench] graph capture failed ({e}); timing eager launches")
         used_graph = False
@@ -273,8 +275,8 @@ def bench_dequant(torch, ops, dev, reps=20):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=300)
-    ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
