@@ -13,8 +13,10 @@
 // where the reference takes (A, packedB, scalesB).
 #pragma once
 
+#include <cmath>
 #include <cstdint>
 #include <cstring>
+#include <initializer_list>
 #include <optional>
 #include <stdexcept>
 #include <string>
@@ -543,6 +545,494 @@ inline void prepareSeparated(SeparatedWeights &out, const Tensor &rawBlocks, Ggu
                            reinterpret_cast<uint16_t *>(out.scales.data()), out.scaleStride, stream),
         "cuthip_prepare_sep");
 }
+
+
+// ==== the operators of one decode step =================================================================
+// What LlamaModel::runLayer chains per token around the quantized matmuls (interface/runner/llama/llama.cpp:
+// RMSNorm -> q / k / v projections -> FusedRoPEKVWrite -> Attention -> wo + residual -> RMSNorm -> gate + up ->
+// SiLU * up -> w_down + residual; then the output norm, the head and the sampling).  The first three nodes mirror the
+// reference's operators one to one; the Carry / Pair / Argmax nodes below are this backend's fused forms of the same
+// chain (six launches per layer).  Every node may be given the tensor it writes (preallocOutput, as the reference's
+// AttentionOpNode takes one): the residual stream and the normed activations are shared between the nodes of a layer.
+namespace detail {
+inline size_t tensorBytes(const Tensor &t) {
+  if (t.shape.empty()) return 0;
+  size_t rows = 1;
+  for (size_t i = 0; i + 1 < t.shape.size(); ++i) rows *= t.shape[i];
+  return ((rows - 1) * (size_t)t.stride() + t.shape.back()) * dtypeBytes(t.dtype);
+}
+inline void requireBytes(const Tensor &t, size_t bytes, const char *what) {
+  if (!t.buffer || t.buffer->bytes() < bytes) throw std::runtime_error(std::string(what) + ": tensor holds fewer bytes than its shape");
+}
+inline void requireTensor(const Tensor &t, const char *what) { requireBytes(t, tensorBytes(t), what); }
+}  // namespace detail
+
+// ---- RMSNormOpNode: operators/impl/rmsnorm/RMSNormOp.h:22-44, RMSNormOp.cpp:9-47 ---------------------
+// x [dim] or [rows, dim], weight [dim]; output of x's shape.  The reference asks for a weight of x's dtype and
+// returns that dtype; here the weight is Float32 whatever x is and the output dtype may be chosen (the decode chain
+// norms an fp32 residual stream into fp16 matmul inputs).
+class RMSNormOpNode {
+public:
+  RMSNormOpNode(const Tensor &x, const Tensor &weight, float eps = 1e-5f, std::optional<DataType> outDtype = {},
+                const Tensor &preallocOutput = {})
+      : x_(x), weight_(weight), eps_(eps) {
+    if (x.shape.empty() || x.shape.size() > 2 || weight.shape.size() != 1)
+      throw std::runtime_error("RMSNorm requires 1D or 2D input, 1D weight");
+    rows_ = x.shape.size() == 2 ? x.shape[0] : 1u;
+    dim_ = x.shape.back();
+    if (weight.shape[0] != dim_) throw std::runtime_error("RMSNorm: weight dimension must match input");
+    if (weight.dtype != DataType::Float32) throw std::runtime_error("RMSNorm: weight must be Float32");
+    if (rows_ == 0 || dim_ == 0) throw std::runtime_error("RMSNorm: empty input");
+    detail::requireTensor(x, "RMSNorm");
+    detail::requireTensor(weight, "RMSNorm");
+    outDtype_ = outDtype.value_or(x.dtype);
+    if (preallocOutput.buffer) {
+      if (preallocOutput.dtype != outDtype_ || preallocOutput.shape != x.shape || preallocOutput.stride() != x.stride())
+        throw std::runtime_error("RMSNorm: preallocated output must have the input's shape and row stride");
+      detail::requireTensor(preallocOutput, "RMSNorm");
+      output_ = preallocOutput;
+    } else {
+      storage_ = DeviceBuffer((size_t)rows_ * x.stride() * dtypeBytes(outDtype_));
+      output_ = Tensor{&storage_, x.shape, outDtype_, x.stride()};
+    }
+  }
+  RMSNormOpNode(RMSNormOpNode &&) = delete;
+  DataType outputDtype() const { return outDtype_; }
+  std::vector<uint32_t> outputShape() const { return output_.shape; }
+  std::string displayName() const { return "RMSNorm"; }
+  const Tensor &output() const { return output_; }
+  void dispatch(void *stream = nullptr) const {
+    check(cuthip_rmsnorm(x_.data(), (int)x_.dtype, static_cast<const float *>(weight_.data()), output_.data(), (int)outDtype_, rows_,
+                         dim_, x_.stride(), eps_, stream),
+          "cuthip_rmsnorm");
+  }
+
+private:
+  Tensor x_, weight_;
+  float eps_;
+  uint32_t rows_ = 0, dim_ = 0;
+  DataType outDtype_ = DataType::Float32;
+  DeviceBuffer storage_;
+  Tensor output_;
+};
+
+// The runtimeParams buffer of the reference's runner: device uint32[2] = {position, sequence length}, read by the
+// kernels so that a captured graph serves the next token after an 8-byte upload.
+class RuntimeParams {
+public:
+  RuntimeParams() : buf_(8) { set(0, 1); }
+  void set(uint32_t position, uint32_t seqLen, void *stream = nullptr) {
+    const uint32_t v[2] = {position, seqLen};
+    buf_.upload(v, sizeof(v), stream);
+  }
+  const uint32_t *data() const { return static_cast<const uint32_t *>(buf_.data()); }
+
+private:
+  DeviceBuffer buf_;
+};
+
+// ---- FusedRoPEKVWriteOpNode: operators/impl/attention/AttentionOp.h:156-184, AttentionOp.cpp:553-612 -------
+// q [qDim], k [kvDim], v [kvDim] of one dtype; tables Float32 [positions, headDim / 2]; caches Float16
+// [positions, alignedKvDim].  Output: the rotated q, Float32 [qDim] (AttentionOp.cpp:576).  A position at or beyond
+// the rows of the caches or tables writes nothing (the reference would write past the cache).
+class FusedRoPEKVWriteOpNode {
+public:
+  FusedRoPEKVWriteOpNode(const Tensor &q, const Tensor &k, const Tensor &v, const RuntimeParams &runtimeParams,
+                         const Tensor &cosTable, const Tensor &sinTable, const Tensor &kCache, const Tensor &vCache,
+                         uint32_t headDim, const Tensor &preallocOutput = {})
+      : q_(q), k_(k), v_(v), cos_(cosTable), sin_(sinTable), kc_(kCache), vc_(vCache), params_(&runtimeParams), headDim_(headDim) {
+    if (q.shape.size() != 1 || k.shape.size() != 1 || v.shape.size() != 1) throw std::runtime_error("FusedRoPEKVWrite: q, k, v must be 1D");
+    qDim_ = q.shape[0];
+    kvDim_ = k.shape[0];
+    if (v.shape[0] != kvDim_ || q.dtype != k.dtype || q.dtype != v.dtype)
+      throw std::runtime_error("FusedRoPEKVWrite: k and v must have one size, q, k and v one dtype");
+    if (headDim_ == 0 || headDim_ % 2 != 0 || qDim_ % headDim_ != 0 || kvDim_ % headDim_ != 0)
+      throw std::runtime_error("FusedRoPEKVWrite: qDim and kvDim must be multiples of an even headDim");
+    if (cosTable.shape.size() != 2 || sinTable.shape != cosTable.shape || cosTable.shape[1] != headDim_ / 2 ||
+        cosTable.dtype != DataType::Float32 || sinTable.dtype != DataType::Float32)
+      throw std::runtime_error("FusedRoPEKVWrite: tables must be Float32 [positions, headDim / 2]");
+    if (kCache.shape.size() != 2 || vCache.shape != kCache.shape || kCache.shape[1] != kvDim_ || kCache.dtype != DataType::Float16 ||
+        vCache.dtype != DataType::Float16 || kCache.stride() != vCache.stride())
+      throw std::runtime_error("FusedRoPEKVWrite: caches must be Float16 [positions, kvDim] with one row stride");
+    alignedKvDim_ = kCache.stride();   // the reference pads cache rows to four elements (AttentionOp.cpp:570)
+    maxPositions_ = kCache.shape[0] < cosTable.shape[0] ? kCache.shape[0] : cosTable.shape[0];
+    for (const Tensor *t : {&q, &k, &v, &cosTable, &sinTable, &kCache, &vCache}) detail::requireTensor(*t, "FusedRoPEKVWrite");
+    if (preallocOutput.buffer) {
+      if (preallocOutput.shape != std::vector<uint32_t>{qDim_}) throw std::runtime_error("FusedRoPEKVWrite: preallocated output must be [qDim]");
+      detail::requireTensor(preallocOutput, "FusedRoPEKVWrite");
+      output_ = preallocOutput;
+    } else {
+      storage_ = DeviceBuffer((size_t)qDim_ * 4);
+      output_ = Tensor{&storage_, {qDim_}, DataType::Float32, qDim_};
+    }
+  }
+  FusedRoPEKVWriteOpNode(FusedRoPEKVWriteOpNode &&) = delete;
+  DataType outputDtype() const { return output_.dtype; }
+  std::vector<uint32_t> outputShape() const { return {qDim_}; }
+  std::string displayName() const { return "FusedRoPEKVWrite"; }
+  const Tensor &output() const { return output_; }
+  void dispatch(void *stream = nullptr) const {
+    check(cuthip_rope_kv_write(q_.data(), k_.data(), v_.data(), (int)q_.dtype, params_->data(), static_cast<const float *>(cos_.data()),
+                               static_cast<const float *>(sin_.data()), kc_.data(), vc_.data(), output_.data(), (int)output_.dtype,
+                               qDim_, kvDim_, headDim_, alignedKvDim_, maxPositions_, stream),
+          "cuthip_rope_kv_write");
+  }
+
+private:
+  Tensor q_, k_, v_, cos_, sin_, kc_, vc_;
+  const RuntimeParams *params_;
+  uint32_t headDim_, qDim_ = 0, kvDim_ = 0, alignedKvDim_ = 0, maxPositions_ = 0;
+  DeviceBuffer storage_;
+  Tensor output_;
+};
+
+// ---- AttentionOpNode: operators/impl/attention/AttentionOp.h:33-66, AttentionOp.cpp:57-86 ---------------
+// q [nHeads * headDim]; caches Float16 [maxSeqLen, kvDim]; output [nHeads * headDim] of q's dtype unless another is
+// asked for; scale = 1 / sqrt(headDim) (AttentionOp.cpp:77).  maxSeqLen bounds the launch: the capacity of the cache
+// unless the caller knows a tighter bound on the sequence length (the kernel reads that many positions).  The node
+// owns the scratch of the context splits.
+class AttentionOpNode {
+public:
+  AttentionOpNode(const Tensor &q, const Tensor &kCache, const Tensor &vCache, const RuntimeParams &runtimeParams, uint32_t nHeads,
+                  uint32_t nKvHeads, uint32_t headDim, const Tensor &preallocOutput = {}, std::optional<DataType> outDtype = {},
+                  std::optional<uint32_t> maxSeqLen = {})
+      : q_(q), kc_(kCache), vc_(vCache), params_(&runtimeParams), nHeads_(nHeads), nKvHeads_(nKvHeads), headDim_(headDim) {
+    if (nHeads == 0 || nKvHeads == 0 || headDim == 0 || nHeads % nKvHeads != 0)
+      throw std::runtime_error("Attention: nHeads must be a positive multiple of nKvHeads");
+    if (headDim > 128) throw std::runtime_error("Attention: headDim above 128 is not supported");   // Attention.cu:35-106
+    if (q.shape.size() != 1 || q.shape[0] != nHeads * headDim) throw std::runtime_error("Attention: q must be [nHeads * headDim]");
+    if (kCache.shape.size() != 2 || vCache.shape != kCache.shape || kCache.shape[1] != nKvHeads * headDim ||
+        kCache.dtype != DataType::Float16 || vCache.dtype != DataType::Float16 || kCache.stride() != vCache.stride())
+      throw std::runtime_error("Attention: caches must be Float16 [maxSeqLen, nKvHeads * headDim] with one row stride");
+    maxSeqLen_ = maxSeqLen.value_or(kCache.shape[0]);
+    if (maxSeqLen_ == 0 || maxSeqLen_ > kCache.shape[0]) throw std::runtime_error("Attention: maxSeqLen must lie within the cache");
+    for (const Tensor *t : {&q, &kCache, &vCache}) detail::requireTensor(*t, "Attention");
+    scale_ = 1.0f / std::sqrt((float)headDim);
+    const DataType odt = outDtype.value_or(q.dtype);
+    if (preallocOutput.buffer) {
+      if (preallocOutput.shape != q.shape || preallocOutput.dtype != odt) throw std::runtime_error("Attention: preallocated output must match q's shape and the output dtype");
+      detail::requireTensor(preallocOutput, "Attention");
+      output_ = preallocOutput;
+    } else {
+      storage_ = DeviceBuffer((size_t)q.shape[0] * dtypeBytes(odt));
+      output_ = Tensor{&storage_, q.shape, odt, q.shape[0]};
+    }
+    scratch_ = DeviceBuffer(cuthip_attn_decode_workspace_bytes(nHeads, headDim, maxSeqLen_));
+  }
+  AttentionOpNode(AttentionOpNode &&) = delete;
+  DataType outputDtype() const { return output_.dtype; }
+  std::vector<uint32_t> outputShape() const { return output_.shape; }
+  std::string displayName() const { return "Attention"; }
+  const Tensor &output() const { return output_; }
+  void dispatch(void *stream = nullptr) const {
+    check(cuthip_attn_decode(q_.data(), (int)q_.dtype, kc_.data(), vc_.data(), params_->data(), output_.data(), (int)output_.dtype,
+                             nHeads_, nKvHeads_, headDim_, kc_.stride(), scale_, maxSeqLen_, scratch_.data(), scratch_.bytes(), stream),
+          "cuthip_attn_decode");
+  }
+
+private:
+  Tensor q_, kc_, vc_;
+  const RuntimeParams *params_;
+  uint32_t nHeads_, nKvHeads_, headDim_, maxSeqLen_ = 0;
+  float scale_ = 0.0f;
+  DeviceBuffer storage_, scratch_;
+  Tensor output_;
+};
+
+// ---- load-time row permutations of the fused decode chain (whole block rows move; done once per tensor) ----
+// [gate rows | up rows] -> gate_0, up_0, gate_1, up_1, ...: the layout the SiLU(gate) * up epilogue reads.
+inline std::vector<uint8_t> interleaveGateUp(const std::vector<uint8_t> &blocks, uint32_t ffn) {
+  if (ffn == 0 || blocks.size() % (2 * (size_t)ffn) != 0) throw std::runtime_error("interleaveGateUp: bytes are not 2 * ffn whole rows");
+  const size_t rb = blocks.size() / (2 * (size_t)ffn);
+  std::vector<uint8_t> out(blocks.size());
+  for (uint32_t i = 0; i < ffn; ++i) {
+    std::memcpy(&out[(2 * (size_t)i) * rb], &blocks[(size_t)i * rb], rb);
+    std::memcpy(&out[(2 * (size_t)i + 1) * rb], &blocks[((size_t)ffn + i) * rb], rb);
+  }
+  return out;
+}
+// Rows of [heads * headDim, K] re-ordered inside every head to d = 0, headDim / 2, 1, headDim / 2 + 1, ...: the two
+// partners of the half-split rotation become neighbouring rows, which is what the RoPE epilogue of the pair launch reads.
+inline std::vector<uint8_t> interleaveRopeRows(const std::vector<uint8_t> &blocks, uint32_t nRows, uint32_t headDim) {
+  if (nRows == 0 || headDim == 0 || headDim % 2 != 0 || nRows % headDim != 0 || blocks.size() % nRows != 0)
+    throw std::runtime_error("interleaveRopeRows: rows must be whole heads of an even headDim");
+  const size_t rb = blocks.size() / nRows;
+  const uint32_t half = headDim / 2;
+  std::vector<uint8_t> out(blocks.size());
+  for (uint32_t h = 0; h < nRows / headDim; ++h)
+    for (uint32_t j = 0; j < half; ++j)
+      for (uint32_t t = 0; t < 2; ++t)
+        std::memcpy(&out[((size_t)h * headDim + 2 * j + t) * rb], &blocks[((size_t)h * headDim + t * half + j) * rb], rb);
+  return out;
+}
+
+// The two sides of an RMSNorm carried across batch-1 matmuls (cuthip_norm_carry_t): the matmul that forms the
+// residual stream (producer) also stores x * weight of the norm that follows as fp16 and the sum of x^2 over each
+// group of 8 outputs; the matmul that reads those activations (consumer) scales its result by
+// rsqrt(sum / K + eps).  The reference fuses RMSNorm into its consumers (runtime/graph/GraphOptimizer.cpp:46-70).
+struct NormCarry {
+  const Tensor *sumsqParts = nullptr;       // consumer: Float32 [ceil(K / 8)]
+  float eps = 0.0f;
+  const Tensor *nextNormWeight = nullptr;   // producer: Float32 [N]
+  const Tensor *nextX16 = nullptr;          // producer: Float16 [N], written
+  const Tensor *nextSumsqParts = nullptr;   // producer: Float32 [ceil(N / 8)], written
+  static NormCarry consumer(const Tensor &sumsqParts, float eps) {
+    NormCarry c;
+    c.sumsqParts = &sumsqParts;
+    c.eps = eps;
+    return c;
+  }
+  static NormCarry producer(const Tensor &nextNormWeight, const Tensor &nextX16, const Tensor &nextSumsqParts) {
+    NormCarry c;
+    c.nextNormWeight = &nextNormWeight;
+    c.nextX16 = &nextX16;
+    c.nextSumsqParts = &nextSumsqParts;
+    return c;
+  }
+  // K: length of the activations (consumer side); N: outputs (producer side)
+  cuthip_norm_carry_t lower(uint32_t K, uint32_t N) const {
+    cuthip_norm_carry_t c{};
+    if (sumsqParts) {
+      if (sumsqParts->dtype != DataType::Float32) throw std::runtime_error("NormCarry: partial sums must be Float32");
+      detail::requireBytes(*sumsqParts, (size_t)((K + 7) / 8) * 4, "NormCarry");
+      c.sumsq_parts = static_cast<const float *>(sumsqParts->data());
+      c.eps = eps;
+    }
+    if (nextNormWeight || nextX16 || nextSumsqParts) {
+      if (!nextNormWeight || !nextX16 || !nextSumsqParts) throw std::runtime_error("NormCarry: the producer side needs all three tensors");
+      if (nextNormWeight->dtype != DataType::Float32 || nextX16->dtype != DataType::Float16 || nextSumsqParts->dtype != DataType::Float32)
+        throw std::runtime_error("NormCarry: producer tensors are Float32 weight, Float16 activations, Float32 partial sums");
+      detail::requireBytes(*nextNormWeight, (size_t)N * 4, "NormCarry");
+      detail::requireBytes(*nextX16, (size_t)N * 2, "NormCarry");
+      detail::requireBytes(*nextSumsqParts, (size_t)((N + 7) / 8) * 4, "NormCarry");
+      c.next_norm_weight = static_cast<const float *>(nextNormWeight->data());
+      c.next_x16 = nextX16->data();
+      c.next_sumsq_parts = static_cast<float *>(nextSumsqParts->data());
+    }
+    return c;
+  }
+  bool any() const { return sumsqParts || nextNormWeight || nextX16 || nextSumsqParts; }
+};
+
+// ---- MatMulGgufCarryOpNode: a batch-1 MatMulGgufOpNode taking part in a carried RMSNorm -----------------
+// a [K]; output [N], or [N / 2] with the SiLU(gate) * up epilogue over interleaved rows (setSwigluPairs).  With
+// preallocOutput == the tensor d of a Binary add the node updates the residual stream in place.
+class MatMulGgufCarryOpNode {
+public:
+  MatMulGgufCarryOpNode(const Tensor &a, const Tensor &wBlocks, GgufFormat format, uint32_t N, const NormCarry &carry,
+                        DataType outDtype = DataType::Float32, const Tensor &preallocOutput = {}, bool swigluPairs = false)
+      : a_(a), w_(wBlocks), format_(format), N_(N), swiglu_(swigluPairs) {
+    if (a.shape.size() != 1) throw std::runtime_error("MatMulGgufCarryOpNode: A must be a vector (batch 1)");
+    K_ = a.shape[0];
+    if (K_ == 0 || N_ == 0 || K_ % blockElems(format) != 0) throw std::runtime_error("MatMulGgufCarryOpNode: K must be a positive multiple of the block size");
+    if (swiglu_ && N_ % 2 != 0) throw std::runtime_error("MatMulGgufCarryOpNode: row pairs need an even N");
+    detail::requireTensor(a, "MatMulGgufCarryOpNode");
+    detail::requireBytes(wBlocks, ggufBytes(format, (uint64_t)N_ * K_), "MatMulGgufCarryOpNode");
+    const uint32_t outN = swiglu_ ? N_ / 2 : N_;
+    carry_ = carry.lower(K_, outN);
+    if (preallocOutput.buffer) {
+      if (preallocOutput.shape != std::vector<uint32_t>{outN}) throw std::runtime_error("MatMulGgufCarryOpNode: preallocated output of the wrong size");
+      detail::requireTensor(preallocOutput, "MatMulGgufCarryOpNode");
+      output_ = preallocOutput;
+    } else {
+      storage_ = DeviceBuffer((size_t)outN * dtypeBytes(outDtype));
+      output_ = Tensor{&storage_, {outN}, outDtype, outN};
+    }
+  }
+  MatMulGgufCarryOpNode(MatMulGgufCarryOpNode &&) = delete;
+  void setFusion(MatMulFusion fusion, int fusionOp = 0, const Tensor &d = {}) {
+    if (swiglu_ && fusion != MatMulFusion::None) throw std::runtime_error("MatMulGgufCarryOpNode::setFusion: the row-pair epilogue takes no further fusion");
+    if (fusion == MatMulFusion::Binary) {
+      if (!d.buffer) throw std::runtime_error("MatMulGgufCarryOpNode::setFusion: Binary fusion needs the tensor d");
+      if (d.dtype != output_.dtype || d.shape != output_.shape) throw std::runtime_error("MatMulGgufCarryOpNode::setFusion: d must match the output");
+    }
+    fusion_ = fusion;
+    fusionOp_ = fusionOp;
+    d_ = d;
+  }
+  DataType outputDtype() const { return output_.dtype; }
+  std::vector<uint32_t> outputShape() const { return output_.shape; }
+  std::string displayName() const { return "MatMulGgufCarry"; }
+  const Tensor &output() const { return output_; }
+  void dispatch(void *stream = nullptr) const {
+    check(cuthip_matmul_gguf_carry((int)format_, w_.data(), a_.data(), (int)a_.dtype, output_.data(), (int)output_.dtype, K_, N_,
+                                   swiglu_ ? (int)CUTHIP_EPI_SWIGLU_PAIRS : (int)fusion_, fusionOp_, d_.data(), &carry_, stream),
+          "cuthip_matmul_gguf_carry");
+  }
+
+private:
+  Tensor a_, w_, d_;
+  GgufFormat format_;
+  uint32_t K_ = 0, N_ = 0;
+  bool swiglu_ = false;
+  cuthip_norm_carry_t carry_{};
+  MatMulFusion fusion_ = MatMulFusion::None;
+  int fusionOp_ = 0;
+  DeviceBuffer storage_;
+  Tensor output_;
+};
+
+// ---- MatMulGgufPairOpNode: two batch-1 matmuls on one activation vector in one launch -------------------
+// The q | k and v projections of a decode step, whose weights differ in format in the common GGUF mixes (the
+// reference fuses wqkv only when its loader could concatenate them, interface/runner/llama/llama.cpp:1710-1756).
+// Plain form: outputs [Na] and [Nb].  With setRopeAppend the launch is the projections plus FusedRoPEKVWriteOpNode:
+// tensor A holds the rows [q heads | k heads] in interleaveRopeRows order, tensor B the v rows; the rotated q is the
+// node's output, rotated k and v go to the cache row of the position, and the plain outputs are not written.
+class MatMulGgufPairOpNode {
+public:
+  MatMulGgufPairOpNode(const Tensor &a, const Tensor &wa, GgufFormat formatA, uint32_t Na, const Tensor &wb, GgufFormat formatB,
+                       uint32_t Nb, const NormCarry &carry = {}, DataType outDtype = DataType::Float32)
+      : a_(a), wa_(wa), wb_(wb), fa_(formatA), fb_(formatB), Na_(Na), Nb_(Nb), outDtype_(outDtype) {
+    if (a.shape.size() != 1) throw std::runtime_error("MatMulGgufPairOpNode: A must be a vector (batch 1)");
+    K_ = a.shape[0];
+    if (K_ == 0 || Na == 0 || Nb == 0 || K_ % blockElems(formatA) != 0 || K_ % blockElems(formatB) != 0)
+      throw std::runtime_error("MatMulGgufPairOpNode: K must be a positive multiple of both block sizes");
+    detail::requireTensor(a, "MatMulGgufPairOpNode");
+    detail::requireBytes(wa, ggufBytes(formatA, (uint64_t)Na * K_), "MatMulGgufPairOpNode");
+    detail::requireBytes(wb, ggufBytes(formatB, (uint64_t)Nb * K_), "MatMulGgufPairOpNode");
+    if (carry.nextNormWeight || carry.nextX16 || carry.nextSumsqParts)
+      throw std::runtime_error("MatMulGgufPairOpNode: only the consumer side of a carried norm applies");
+    hasCarry_ = carry.any();
+    carry_ = carry.lower(K_, 0);
+    storageA_ = DeviceBuffer((size_t)Na * dtypeBytes(outDtype));
+    storageB_ = DeviceBuffer((size_t)Nb * dtypeBytes(outDtype));
+    outputA_ = Tensor{&storageA_, {Na}, outDtype, Na};
+    outputB_ = Tensor{&storageB_, {Nb}, outDtype, Nb};
+  }
+  MatMulGgufPairOpNode(MatMulGgufPairOpNode &&) = delete;
+  void setRopeAppend(const RuntimeParams &runtimeParams, const Tensor &cosTable, const Tensor &sinTable, const Tensor &kCache,
+                     const Tensor &vCache, uint32_t qDim, uint32_t headDim, const Tensor &preallocQ = {}) {
+    if (headDim == 0 || headDim % 2 != 0 || qDim == 0 || qDim % headDim != 0 || qDim >= Na_ || (Na_ - qDim) % headDim != 0 || Nb_ != Na_ - qDim)
+      throw std::runtime_error("MatMulGgufPairOpNode::setRopeAppend: tensor A is [qDim + kvDim] rows, tensor B kvDim rows, whole heads");
+    if (cosTable.shape.size() != 2 || sinTable.shape != cosTable.shape || cosTable.shape[1] != headDim / 2 ||
+        cosTable.dtype != DataType::Float32 || sinTable.dtype != DataType::Float32)
+      throw std::runtime_error("MatMulGgufPairOpNode::setRopeAppend: tables must be Float32 [positions, headDim / 2]");
+    if (kCache.shape.size() != 2 || vCache.shape != kCache.shape || kCache.shape[1] != Nb_ || kCache.dtype != DataType::Float16 ||
+        vCache.dtype != DataType::Float16 || kCache.stride() != vCache.stride())
+      throw std::runtime_error("MatMulGgufPairOpNode::setRopeAppend: caches must be Float16 [positions, kvDim] with one row stride");
+    for (const Tensor *t : {&cosTable, &sinTable, &kCache, &vCache}) detail::requireTensor(*t, "MatMulGgufPairOpNode::setRopeAppend");
+    if (preallocQ.buffer) {
+      if (preallocQ.shape != std::vector<uint32_t>{qDim}) throw std::runtime_error("MatMulGgufPairOpNode::setRopeAppend: preallocated q must be [qDim]");
+      detail::requireTensor(preallocQ, "MatMulGgufPairOpNode::setRopeAppend");
+      qOut_ = preallocQ;
+    } else {
+      storageQ_ = DeviceBuffer((size_t)qDim * 4);
+      qOut_ = Tensor{&storageQ_, {qDim}, DataType::Float32, qDim};
+    }
+    rope_ = cuthip_rope_append_t{};
+    rope_.runtime_params = runtimeParams.data();
+    rope_.cos_table = static_cast<const float *>(cosTable.data());
+    rope_.sin_table = static_cast<const float *>(sinTable.data());
+    rope_.q_out = qOut_.data();
+    rope_.q_out_dtype = (int)qOut_.dtype;
+    rope_.k_cache = kCache.data();
+    rope_.v_cache = vCache.data();
+    rope_.q_dim = qDim;
+    rope_.head_dim = headDim;
+    rope_.aligned_kv_dim = kCache.stride();
+    rope_.max_positions = kCache.shape[0] < cosTable.shape[0] ? kCache.shape[0] : cosTable.shape[0];
+    hasRope_ = true;
+  }
+  std::string displayName() const { return hasRope_ ? "MatMulGgufPairRoPEKVWrite" : "MatMulGgufPair"; }
+  const Tensor &outputA() const { return outputA_; }
+  const Tensor &outputB() const { return outputB_; }
+  const Tensor &output() const {   // the rotated q once setRopeAppend was called
+    if (!hasRope_) throw std::runtime_error("MatMulGgufPairOpNode::output: no RoPE epilogue set; use outputA() / outputB()");
+    return qOut_;
+  }
+  void dispatch(void *stream = nullptr) const {
+    check(cuthip_matmul_gguf_pair((int)fa_, wa_.data(), Na_, hasRope_ ? nullptr : outputA_.data(), (int)fb_, wb_.data(), Nb_,
+                                  hasRope_ ? nullptr : outputB_.data(), a_.data(), (int)a_.dtype, (int)outDtype_, K_,
+                                  hasCarry_ ? &carry_ : nullptr, hasRope_ ? &rope_ : nullptr, stream),
+          "cuthip_matmul_gguf_pair");
+  }
+
+private:
+  Tensor a_, wa_, wb_;
+  GgufFormat fa_, fb_;
+  uint32_t Na_, Nb_, K_ = 0;
+  DataType outDtype_;
+  bool hasCarry_ = false, hasRope_ = false;
+  cuthip_norm_carry_t carry_{};
+  cuthip_rope_append_t rope_{};
+  DeviceBuffer storageA_, storageB_, storageQ_;
+  Tensor outputA_, outputB_, qOut_;
+};
+
+// ---- MatMulGgufArgmaxOpNode: the output head with the sampling folded in -----------------------------------
+// logits [N] = a [K] . dequant(W)^T, the repetition penalty on the listed tokens, the index of the first maximum
+// (the reference runs LM head, RepetitionPenaltyOpNode and ReduceArgmax as three dispatches,
+// interface/runner/llama/llama.cpp:2145-2152).  The penalty list lives on the device (setPenalties uploads it); its
+// length is fixed at construction so that a captured graph can be replayed with new entries (unused ones: token -1).
+class MatMulGgufArgmaxOpNode {
+public:
+  MatMulGgufArgmaxOpNode(const Tensor &a, const Tensor &wBlocks, GgufFormat format, uint32_t N, const NormCarry &carry = {},
+                         uint32_t penaltyWindow = 0, DataType logitsDtype = DataType::Float32)
+      : a_(a), w_(wBlocks), format_(format), N_(N), window_(penaltyWindow) {
+    if (a.shape.size() != 1) throw std::runtime_error("MatMulGgufArgmaxOpNode: A must be a vector (batch 1)");
+    K_ = a.shape[0];
+    if (K_ == 0 || N_ == 0 || K_ % blockElems(format) != 0) throw std::runtime_error("MatMulGgufArgmaxOpNode: K must be a positive multiple of the block size");
+    if (penaltyWindow > 1024) throw std::runtime_error("MatMulGgufArgmaxOpNode: at most 1024 penalised tokens");
+    detail::requireTensor(a, "MatMulGgufArgmaxOpNode");
+    detail::requireBytes(wBlocks, ggufBytes(format, (uint64_t)N_ * K_), "MatMulGgufArgmaxOpNode");
+    if (carry.nextNormWeight || carry.nextX16 || carry.nextSumsqParts)
+      throw std::runtime_error("MatMulGgufArgmaxOpNode: only the consumer side of a carried norm applies");
+    hasCarry_ = carry.any();
+    carry_ = carry.lower(K_, 0);
+    logitsStorage_ = DeviceBuffer((size_t)N_ * dtypeBytes(logitsDtype));
+    logits_ = Tensor{&logitsStorage_, {N_}, logitsDtype, N_};
+    token_ = DeviceBuffer(4);
+    scratch_ = DeviceBuffer(cuthip_matmul_gguf_argmax_workspace_bytes(N_));
+    if (window_) {
+      penTokens_ = DeviceBuffer((size_t)window_ * 4);
+      penFactors_ = DeviceBuffer((size_t)window_ * 4);
+      setPenalties({}, {});
+    }
+  }
+  MatMulGgufArgmaxOpNode(MatMulGgufArgmaxOpNode &&) = delete;
+  // The entries of the runner's factor vector that are not 1 (llama.cpp:2566-2592); the most recent ones are kept
+  // when there are more than the window holds.
+  void setPenalties(const std::vector<int32_t> &tokens, const std::vector<float> &factors, void *stream = nullptr) {
+    if (tokens.size() != factors.size()) throw std::runtime_error("MatMulGgufArgmaxOpNode::setPenalties: one factor per token");
+    if (!window_) {
+      if (!tokens.empty()) throw std::runtime_error("MatMulGgufArgmaxOpNode::setPenalties: the node was built without a penalty window");
+      return;
+    }
+    std::vector<int32_t> t(window_, -1);
+    std::vector<float> f(window_, 1.0f);
+    const size_t n = tokens.size() < window_ ? tokens.size() : window_, skip = tokens.size() - n;
+    for (size_t i = 0; i < n; ++i) {
+      t[i] = tokens[skip + i];
+      f[i] = factors[skip + i];
+    }
+    penTokens_.upload(t.data(), t.size() * 4, stream);
+    penFactors_.upload(f.data(), f.size() * 4, stream);
+  }
+  std::string displayName() const { return "MatMulGgufArgmax"; }
+  const Tensor &output() const { return logits_; }         // the (penalised) logits
+  const DeviceBuffer &token() const { return token_; }     // device uint32: the sampled token
+  uint32_t readToken(void *stream = nullptr) const {
+    uint32_t t = 0;
+    token_.download(&t, 4, stream);
+    return t;
+  }
+  void dispatch(void *stream = nullptr) const {
+    check(cuthip_matmul_gguf_argmax((int)format_, w_.data(), a_.data(), (int)a_.dtype, logits_.data(), (int)logits_.dtype, K_, N_,
+                                    hasCarry_ ? &carry_ : nullptr, static_cast<const int32_t *>(penTokens_.data()),
+                                    static_cast<const float *>(penFactors_.data()), window_, scratch_.data(), scratch_.bytes(),
+                                    static_cast<uint32_t *>(token_.data()), stream),
+          "cuthip_matmul_gguf_argmax");
+  }
+
+private:
+  Tensor a_, w_;
+  GgufFormat format_;
+  uint32_t N_, K_ = 0, window_;
+  bool hasCarry_ = false;
+  cuthip_norm_carry_t carry_{};
+  DeviceBuffer logitsStorage_, token_, scratch_, penTokens_, penFactors_;
+  Tensor logits_;
+};
 
 }  // namespace hip
 }  // namespace cut

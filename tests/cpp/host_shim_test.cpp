@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 #include <random>
 #include <string>
 #include <vector>
@@ -34,6 +35,15 @@ template <class F> static bool throws(F f) {
     return true;
   }
   return false;
+}
+
+template <class F> static std::string message_of(F f) {
+  try {
+    f();
+  } catch (const std::runtime_error &e) {
+    return e.what();
+  }
+  return "";
 }
 
 static void test_tables() {
@@ -72,19 +82,34 @@ static void test_validation() {
   EXPECT(throws([&] { MatMulDenseF16OpNode n(a200, w16); }));                   // A cols != weight cols
   Tensor a256{&none, {2, 256}, DataType::Float16, 0};
   EXPECT(throws([&] { MatMulDenseF16OpNode n(a256, w16); }));                   // weights too small
+  // the operators of a decode step: shapes are checked before any device call
+  Tensor x2{&none, {2, 64}, DataType::Float32, 64}, w64{&none, {64}, DataType::Float32, 0}, w32{&none, {32}, DataType::Float32, 0};
+  Tensor x3{&none, {1, 2, 64}, DataType::Float32, 64};
+  EXPECT(message_of([&] { RMSNormOpNode n(x3, w64); }) == "RMSNorm requires 1D or 2D input, 1D weight");   // RMSNormOp.cpp:20-22
+  EXPECT(message_of([&] { RMSNormOpNode n(x2, x2); }) == "RMSNorm requires 1D or 2D input, 1D weight");
+  EXPECT(message_of([&] { RMSNormOpNode n(x2, w32); }) == "RMSNorm: weight dimension must match input");     // RMSNormOp.cpp:34-36
+  EXPECT(throws([&] { RMSNormOpNode n(x2, w64); }));                                                          // empty buffers
+  Tensor q1{&none, {512}, DataType::Float32, 0};
+  EXPECT(throws([&] { MatMulGgufCarryOpNode n(x2, raw, GgufFormat::Q4_K, 8, NormCarry{}); }));       // batch above 1
+  EXPECT(throws([&] { MatMulGgufCarryOpNode n(q1, raw, GgufFormat::Q4_K, 7, NormCarry{}, DataType::Float32, {}, true); }));   // odd N with row pairs
+  EXPECT(throws([&] { MatMulGgufPairOpNode n(x2, raw, GgufFormat::Q4_K, 8, raw, GgufFormat::Q6_K, 8); }));
+  EXPECT(throws([&] { MatMulGgufArgmaxOpNode n(q1, raw, GgufFormat::Q6_K, 8, NormCarry{}, 2000); }));  // window above 1024
+  {
+    std::vector<uint8_t> rows(8 * 3);
+    for (size_t i = 0; i < rows.size(); ++i) rows[i] = (uint8_t)(i / 3);           // row r holds the byte r
+    const std::vector<uint8_t> gu = interleaveGateUp(rows, 4);                     // gate 0-3 | up 4-7 -> 0 4 1 5 2 6 3 7
+    const uint8_t want_gu[8] = {0, 4, 1, 5, 2, 6, 3, 7};
+    for (int r = 0; r < 8; ++r) EXPECT(gu[3 * r] == want_gu[r] && gu[3 * r + 2] == want_gu[r]);
+    const std::vector<uint8_t> rr = interleaveRopeRows(rows, 8, 4);                // two heads of 4: d = 0 2 1 3 inside each
+    const uint8_t want_rr[8] = {0, 2, 1, 3, 4, 6, 5, 7};
+    for (int r = 0; r < 8; ++r) EXPECT(rr[3 * r] == want_rr[r]);
+    EXPECT(throws([&] { interleaveGateUp(rows, 5); }));
+    EXPECT(throws([&] { interleaveRopeRows(rows, 8, 3); }));
+  }
   SeparatedWeights sw;
   EXPECT(throws([&] { prepareSeparated(sw, raw, GgufFormat::Q6_K, 4, 256); }));
   EXPECT(throws([&] { prepareSeparated(sw, raw, GgufFormat::Q4_0, 3, 64); }));
   EXPECT(throws([&] { prepareSeparated(sw, raw, GgufFormat::Q8_0, 4, 64); }));  // raw too small
-}
-
-template <class F> static std::string message_of(F f) {
-  try {
-    f();
-  } catch (const std::runtime_error &e) {
-    return e.what();
-  }
-  return "";
 }
 
 // Every branch of the 3-input MatMulOpNode constructor (MatMulOp.cpp:283-374): format inference from the shapes, the
@@ -407,12 +432,308 @@ static void test_gpu() {
   }
 }
 
+// Two layers and the output head of a decode step through the nodes of the shim, in the fused form the Python
+// DecodeStep runs (six launches per layer: q | k | v with RoPE and the cache append, attention and its merge, wo +
+// residual, gate + up with SiLU * up, w_down + residual; RMSNorm carried across the matmuls; the arg-max in the
+// epilogue of the head), captured once and replayed for the next position, against the same chain from oracle calls.
+struct ChainConfig {
+  uint32_t hidden = 512, layers = 2, heads = 8, kvHeads = 2, headDim = 64, ffn = 1024, vocab = 2048, maxCtx = 64;
+  float eps = 1e-5f, theta = 500000.0f;
+  uint32_t qDim() const { return heads * headDim; }
+  uint32_t kvDim() const { return kvHeads * headDim; }
+};
+struct LayerHost {
+  std::vector<uint8_t> qk, v, o, gateUp, down;   // GGUF blocks, natural row order
+  std::vector<float> attnNorm, ffnNorm;
+};
+static std::vector<float> round_f16(const std::vector<float> &x) {
+  std::vector<float> r(x.size());
+  for (size_t i = 0; i < x.size(); ++i) r[i] = orc_f16_to_f32(orc_f32_to_f16(x[i]));
+  return r;
+}
+static std::vector<float> cpu_matmul(int fmt, const std::vector<uint8_t> &blocks, const std::vector<float> &a, uint32_t N) {
+  std::vector<double> c(N);
+  EXPECT(orc_matmul_gguf_f64(fmt, blocks.data(), a.data(), 1, (uint32_t)a.size(), N, c.data()) == 0);
+  return std::vector<float>(c.begin(), c.end());
+}
+// activations rounded to fp16 wherever the device chain stores fp16
+static std::vector<float> cpu_chain_step(const ChainConfig &c, const std::vector<LayerHost> &L, const std::vector<float> &outNorm,
+                                         const std::vector<uint8_t> &head, std::vector<float> x, uint32_t pos,
+                                         std::vector<std::vector<uint16_t>> &kc, std::vector<std::vector<uint16_t>> &vc,
+                                         const std::vector<float> &cosT, const std::vector<float> &sinT) {
+  std::vector<float> xn(c.hidden), qRot(c.qDim()), attn(c.qDim()), act(c.ffn);
+  for (uint32_t i = 0; i < c.layers; ++i) {
+    orc_rmsnorm(x.data(), L[i].attnNorm.data(), 1, c.hidden, c.eps, xn.data());
+    xn = round_f16(xn);
+    const std::vector<float> qk = cpu_matmul(CUTHIP_Q4_K, L[i].qk, xn, c.qDim() + c.kvDim());
+    const std::vector<float> v = cpu_matmul(CUTHIP_Q6_K, L[i].v, xn, c.kvDim());
+    orc_rope_kv_write(qk.data(), qk.data() + c.qDim(), v.data(), pos, cosT.data(), sinT.data(), c.qDim(), c.kvDim(), c.headDim,
+                      c.kvDim(), qRot.data(), kc[i].data(), vc[i].data());
+    orc_attention_decode(qRot.data(), kc[i].data(), vc[i].data(), pos + 1, c.heads, c.kvHeads, c.headDim, c.kvDim(),
+                         1.0f / std::sqrt((float)c.headDim), attn.data());
+    const std::vector<float> o = cpu_matmul(CUTHIP_Q4_K, L[i].o, round_f16(attn), c.hidden);
+    for (uint32_t j = 0; j < c.hidden; ++j) x[j] += o[j];
+    orc_rmsnorm(x.data(), L[i].ffnNorm.data(), 1, c.hidden, c.eps, xn.data());
+    const std::vector<float> gu = round_f16(cpu_matmul(CUTHIP_Q4_K, L[i].gateUp, round_f16(xn), 2 * c.ffn));
+    orc_silu_mul(gu.data(), c.ffn, act.data());
+    const std::vector<float> d = cpu_matmul(CUTHIP_Q4_K, L[i].down, round_f16(act), c.hidden);
+    for (uint32_t j = 0; j < c.hidden; ++j) x[j] += d[j];
+  }
+  orc_rmsnorm(x.data(), outNorm.data(), 1, c.hidden, c.eps, xn.data());
+  return cpu_matmul(CUTHIP_Q6_K, head, round_f16(xn), c.vocab);
+}
+
+static void test_gpu_decode_chain() {
+  const ChainConfig c;
+  std::mt19937 rng(11);
+  std::normal_distribution<float> gw(0.0f, 0.05f), ga(0.0f, 1.0f);
+  std::uniform_real_distribution<float> un(0.5f, 1.5f);
+  auto qw = [&](int fmt, uint32_t n, uint32_t k) {
+    std::vector<float> w((size_t)n * k);
+    for (auto &v : w) v = gw(rng);
+    std::vector<uint8_t> b(ggufBytes((GgufFormat)fmt, (uint64_t)n * k));
+    EXPECT(orc_quantize(fmt, w.data(), w.size(), b.data()) == 0);
+    return b;
+  };
+  auto uni = [&](uint32_t n) {
+    std::vector<float> w(n);
+    for (auto &v : w) v = un(rng);
+    return w;
+  };
+  std::vector<LayerHost> L(c.layers);
+  for (auto &l : L) {
+    l.qk = qw(CUTHIP_Q4_K, c.qDim() + c.kvDim(), c.hidden);
+    l.v = qw(CUTHIP_Q6_K, c.kvDim(), c.hidden);
+    l.o = qw(CUTHIP_Q4_K, c.hidden, c.qDim());
+    l.gateUp = qw(CUTHIP_Q4_K, 2 * c.ffn, c.hidden);
+    l.down = qw(CUTHIP_Q4_K, c.hidden, c.ffn);
+    l.attnNorm = uni(c.hidden);
+    l.ffnNorm = uni(c.hidden);
+  }
+  const std::vector<float> outNorm = uni(c.hidden);
+  const std::vector<uint8_t> head = qw(CUTHIP_Q6_K, c.vocab, c.hidden);
+  // RoPE tables [position][headDim / 2]
+  const uint32_t half = c.headDim / 2;
+  std::vector<float> cosT((size_t)c.maxCtx * half), sinT((size_t)c.maxCtx * half);
+  for (uint32_t p = 0; p < c.maxCtx; ++p)
+    for (uint32_t j = 0; j < half; ++j) {
+      const double ang = p / std::pow((double)c.theta, 2.0 * j / c.headDim);
+      cosT[(size_t)p * half + j] = (float)std::cos(ang);
+      sinT[(size_t)p * half + j] = (float)std::sin(ang);
+    }
+  // nine earlier tokens already in the caches, the same bits on both sides
+  uint32_t pos = 9;
+  std::vector<std::vector<uint16_t>> kc(c.layers, std::vector<uint16_t>((size_t)c.maxCtx * c.kvDim(), 0)), vc = kc;
+  for (uint32_t i = 0; i < c.layers; ++i)
+    for (size_t e = 0; e < (size_t)pos * c.kvDim(); ++e) {
+      kc[i][e] = orc_f32_to_f16(0.5f * ga(rng));
+      vc[i][e] = orc_f32_to_f16(ga(rng));
+    }
+
+  // ---- device side: shared tensors, then the nodes of the chain ----
+  struct LayerDev {
+    DeviceBuffer qk, v, o, gateUp, down, attnNorm, ffnNorm, kCache, vCache;
+  };
+  std::vector<LayerDev> D(c.layers);
+  auto bytesTensor = [](DeviceBuffer &b) { return Tensor{&b, {(uint32_t)b.bytes()}, DataType::Float32, 0}; };
+  for (uint32_t i = 0; i < c.layers; ++i) {
+    const std::vector<uint8_t> qkI = interleaveRopeRows(L[i].qk, c.qDim() + c.kvDim(), c.headDim);
+    const std::vector<uint8_t> guI = interleaveGateUp(L[i].gateUp, c.ffn);
+    D[i].qk = DeviceBuffer(qkI.data(), qkI.size());
+    D[i].v = DeviceBuffer(L[i].v.data(), L[i].v.size());
+    D[i].o = DeviceBuffer(L[i].o.data(), L[i].o.size());
+    D[i].gateUp = DeviceBuffer(guI.data(), guI.size());
+    D[i].down = DeviceBuffer(L[i].down.data(), L[i].down.size());
+    D[i].attnNorm = DeviceBuffer(L[i].attnNorm.data(), c.hidden * 4);
+    D[i].ffnNorm = DeviceBuffer(L[i].ffnNorm.data(), c.hidden * 4);
+    D[i].kCache = DeviceBuffer(kc[i].data(), kc[i].size() * 2);
+    D[i].vCache = DeviceBuffer(vc[i].data(), vc[i].size() * 2);
+  }
+  DeviceBuffer outNormDev(outNorm.data(), c.hidden * 4), headDev(head.data(), head.size());
+  DeviceBuffer cosDev(cosT.data(), cosT.size() * 4), sinDev(sinT.data(), sinT.size() * 4);
+  DeviceBuffer xDev((size_t)c.hidden * 4), xnDev((size_t)c.hidden * 2), partsDev((size_t)(c.hidden / 8) * 4);
+  DeviceBuffer qRotDev((size_t)c.qDim() * 4), attnDev((size_t)c.qDim() * 2), actDev((size_t)c.ffn * 2);
+  const Tensor x{&xDev, {c.hidden}, DataType::Float32, 0}, xn{&xnDev, {c.hidden}, DataType::Float16, 0};
+  const Tensor parts{&partsDev, {c.hidden / 8}, DataType::Float32, 0};
+  const Tensor qRot{&qRotDev, {c.qDim()}, DataType::Float32, 0}, attn{&attnDev, {c.qDim()}, DataType::Float16, 0};
+  const Tensor act{&actDev, {c.ffn}, DataType::Float16, 0};
+  const Tensor cosTt{&cosDev, {c.maxCtx, half}, DataType::Float32, 0}, sinTt{&sinDev, {c.maxCtx, half}, DataType::Float32, 0};
+  const Tensor outNormT{&outNormDev, {c.hidden}, DataType::Float32, 0};
+  RuntimeParams params;
+  const NormCarry consume = NormCarry::consumer(parts, c.eps);
+
+  std::vector<Tensor> normA(c.layers), normF(c.layers), kcT(c.layers), vcT(c.layers);
+  for (uint32_t i = 0; i < c.layers; ++i) {
+    normA[i] = Tensor{&D[i].attnNorm, {c.hidden}, DataType::Float32, 0};
+    normF[i] = Tensor{&D[i].ffnNorm, {c.hidden}, DataType::Float32, 0};
+    kcT[i] = Tensor{&D[i].kCache, {c.maxCtx, c.kvDim()}, DataType::Float16, 0};
+    vcT[i] = Tensor{&D[i].vCache, {c.maxCtx, c.kvDim()}, DataType::Float16, 0};
+  }
+  RMSNormOpNode firstNorm(x, normA[0], c.eps, DataType::Float16, xn);
+  std::vector<std::unique_ptr<MatMulGgufPairOpNode>> qkv;
+  std::vector<std::unique_ptr<AttentionOpNode>> att;
+  std::vector<std::unique_ptr<MatMulGgufCarryOpNode>> wo, gateUp, down;
+  for (uint32_t i = 0; i < c.layers; ++i) {
+    // layer 0 reads the output of the RMSNorm node (already scaled); the others the carried form
+    qkv.emplace_back(new MatMulGgufPairOpNode(xn, bytesTensor(D[i].qk), GgufFormat::Q4_K, c.qDim() + c.kvDim(), bytesTensor(D[i].v),
+                                              GgufFormat::Q6_K, c.kvDim(), i > 0 ? consume : NormCarry{}));
+    qkv.back()->setRopeAppend(params, cosTt, sinTt, kcT[i], vcT[i], c.qDim(), c.headDim, qRot);
+    att.emplace_back(new AttentionOpNode(qRot, kcT[i], vcT[i], params, c.heads, c.kvHeads, c.headDim, attn, DataType::Float16));
+    wo.emplace_back(new MatMulGgufCarryOpNode(attn, bytesTensor(D[i].o), GgufFormat::Q4_K, c.hidden,
+                                              NormCarry::producer(normF[i], xn, parts), DataType::Float32, x));
+    wo.back()->setFusion(MatMulFusion::Binary, CUTHIP_BINARY_ADD, x);
+    gateUp.emplace_back(new MatMulGgufCarryOpNode(xn, bytesTensor(D[i].gateUp), GgufFormat::Q4_K, 2 * c.ffn, consume,
+                                                  DataType::Float16, act, true));
+    const Tensor &nextNorm = i + 1 < c.layers ? normA[i + 1] : outNormT;
+    down.emplace_back(new MatMulGgufCarryOpNode(act, bytesTensor(D[i].down), GgufFormat::Q4_K, c.hidden,
+                                                NormCarry::producer(nextNorm, xn, parts), DataType::Float32, x));
+    down.back()->setFusion(MatMulFusion::Binary, CUTHIP_BINARY_ADD, x);
+  }
+  MatMulGgufArgmaxOpNode headNode(xn, bytesTensor(headDev), GgufFormat::Q6_K, c.vocab, consume);
+  EXPECT(qkv[0]->displayName() == "MatMulGgufPairRoPEKVWrite" && wo[0]->displayName() == "MatMulGgufCarry");
+  EXPECT(headNode.output().shape == std::vector<uint32_t>{c.vocab});
+
+  Stream stream;
+  auto encode = [&] {   // what Dispatcher::encode does for the nodes of the step, in graph order
+    firstNorm.dispatch(stream.get());
+    for (uint32_t i = 0; i < c.layers; ++i) {
+      qkv[i]->dispatch(stream.get());
+      att[i]->dispatch(stream.get());
+      wo[i]->dispatch(stream.get());
+      gateUp[i]->dispatch(stream.get());
+      down[i]->dispatch(stream.get());
+    }
+    headNode.dispatch(stream.get());
+  };
+  auto check_step = [&](const std::vector<float> &xHost, const char *what) {
+    const std::vector<float> want = cpu_chain_step(c, L, outNorm, head, xHost, pos, kc, vc, cosT, sinT);
+    std::vector<float> got(c.vocab);
+    headNode.output().buffer->download(got.data(), got.size() * 4);
+    const double err = normwise(got, std::vector<double>(want.begin(), want.end()));
+    if (!(err < 1e-3)) std::printf("decode chain (%s) err %g\n", what, err);
+    EXPECT(err < 1e-3);
+    uint32_t best = 0;
+    for (uint32_t i = 1; i < c.vocab; ++i)
+      if (got[i] > got[best]) best = i;
+    EXPECT(headNode.readToken() == best);
+    // the caches of both sides hold the same row for this position (fp16 bits, up to one unit in the last place)
+    std::vector<uint16_t> row(c.kvDim());
+    for (uint32_t i = 0; i < c.layers; ++i) {
+      std::vector<uint16_t> all((size_t)c.maxCtx * c.kvDim());
+      D[i].vCache.download(all.data(), all.size() * 2);
+      double num = 0, den = 0;
+      for (uint32_t e = 0; e < c.kvDim(); ++e) {
+        const double g = orc_f16_to_f32(all[(size_t)pos * c.kvDim() + e]), w = orc_f16_to_f32(vc[i][(size_t)pos * c.kvDim() + e]);
+        num += (g - w) * (g - w);
+        den += w * w;
+      }
+      EXPECT(std::sqrt(num / den) < 2e-3);
+    }
+    return got;
+  };
+
+  std::vector<float> xHost(c.hidden);
+  for (auto &v : xHost) v = ga(rng);
+  xDev.upload(xHost.data(), xHost.size() * 4);
+  params.set(pos, pos + 1);
+  encode();   // eager
+  stream.sync();
+  const std::vector<float> eager = check_step(xHost, "eager");
+
+  CommandGraph graph;
+  graph.begin(stream);
+  encode();
+  graph.end(stream);
+  // replay on the same input: the eager logits bit for bit (the cache row of the position is rewritten with the same values)
+  xDev.upload(xHost.data(), xHost.size() * 4);
+  graph.replay(stream);
+  stream.sync();
+  {
+    std::vector<float> again(c.vocab);
+    headNode.output().buffer->download(again.data(), again.size() * 4);
+    EXPECT(std::memcmp(again.data(), eager.data(), again.size() * 4) == 0);
+  }
+  // the next two positions through the same graph: only the 8 bytes of the runtime parameters and x change
+  for (int rep = 0; rep < 2; ++rep) {
+    ++pos;
+    for (auto &v : xHost) v = ga(rng);
+    xDev.upload(xHost.data(), xHost.size() * 4);
+    params.set(pos, pos + 1);
+    graph.replay(stream);
+    stream.sync();
+    check_step(xHost, rep ? "replay, position 11" : "replay, position 10");
+  }
+
+  // the unfused operators of the same layer-0 front: RMSNorm, the two projections, FusedRoPEKVWrite, Attention as the
+  // reference's own nodes chain them, against the fused launch (same cache row, same rotated q up to rounding)
+  {
+    const uint32_t p2 = pos + 1;
+    params.set(p2, p2 + 1);
+    for (auto &v : xHost) v = ga(rng);
+    xDev.upload(xHost.data(), xHost.size() * 4);
+    RMSNormOpNode norm(x, normA[0], c.eps, DataType::Float16);
+    DeviceBuffer qkNat(L[0].qk.data(), L[0].qk.size());
+    MatMulGgufPairOpNode proj(norm.output(), bytesTensor(qkNat), GgufFormat::Q4_K, c.qDim() + c.kvDim(), bytesTensor(D[0].v),
+                              GgufFormat::Q6_K, c.kvDim());
+    DeviceBuffer kc2((size_t)c.maxCtx * c.kvDim() * 2), vc2((size_t)c.maxCtx * c.kvDim() * 2);
+    std::vector<uint16_t> kcHost((size_t)c.maxCtx * c.kvDim()), vcHost(kcHost.size());
+    D[0].kCache.download(kcHost.data(), kcHost.size() * 2);
+    D[0].vCache.download(vcHost.data(), vcHost.size() * 2);
+    kc2.upload(kcHost.data(), kcHost.size() * 2);
+    vc2.upload(vcHost.data(), vcHost.size() * 2);
+    const Tensor kc2T{&kc2, {c.maxCtx, c.kvDim()}, DataType::Float16, 0}, vc2T{&vc2, {c.maxCtx, c.kvDim()}, DataType::Float16, 0};
+    // q and k are the two halves of the pair's first output
+    DeviceBuffer qBuf((size_t)c.qDim() * 4), kBuf((size_t)c.kvDim() * 4);
+    const Tensor qT{&qBuf, {c.qDim()}, DataType::Float32, 0}, kT{&kBuf, {c.kvDim()}, DataType::Float32, 0};
+    FusedRoPEKVWriteOpNode rope(qT, kT, proj.outputB(), params, cosTt, sinTt, kc2T, vc2T, c.headDim);
+    AttentionOpNode attention(rope.output(), kc2T, vc2T, params, c.heads, c.kvHeads, c.headDim);
+    norm.dispatch(stream.get());
+    proj.dispatch(stream.get());
+    check(cuthip_memcpy_d2d(qBuf.data(), proj.outputA().data(), (size_t)c.qDim() * 4, stream.get()), "cuthip_memcpy_d2d");
+    check(cuthip_memcpy_d2d(kBuf.data(), static_cast<const uint8_t *>(proj.outputA().data()) + (size_t)c.qDim() * 4,
+                            (size_t)c.kvDim() * 4, stream.get()),
+          "cuthip_memcpy_d2d");
+    rope.dispatch(stream.get());
+    attention.dispatch(stream.get());
+    // the fused form on the same input
+    firstNorm.dispatch(stream.get());
+    qkv[0]->dispatch(stream.get());
+    att[0]->dispatch(stream.get());
+    stream.sync();
+    std::vector<float> unfused(c.qDim());
+    attention.output().buffer->download(unfused.data(), unfused.size() * 4);
+    std::vector<uint16_t> fusedBits(c.qDim());
+    attnDev.download(fusedBits.data(), fusedBits.size() * 2);
+    std::vector<double> fused(c.qDim());
+    for (uint32_t i = 0; i < c.qDim(); ++i) fused[i] = orc_f16_to_f32(fusedBits[i]);
+    const double err = normwise(unfused, fused);
+    if (!(err < 2e-3)) std::printf("unfused against fused attention front err %g\n", err);
+    EXPECT(err < 2e-3);
+    // and against the oracle's operators on the same inputs
+    std::vector<float> xnH(c.hidden), qRotH(c.qDim()), attnH(c.qDim());
+    orc_rmsnorm(xHost.data(), L[0].attnNorm.data(), 1, c.hidden, c.eps, xnH.data());
+    xnH = round_f16(xnH);
+    const std::vector<float> qkH = cpu_matmul(CUTHIP_Q4_K, L[0].qk, xnH, c.qDim() + c.kvDim());
+    const std::vector<float> vH = cpu_matmul(CUTHIP_Q6_K, L[0].v, xnH, c.kvDim());
+    orc_rope_kv_write(qkH.data(), qkH.data() + c.qDim(), vH.data(), p2, cosT.data(), sinT.data(), c.qDim(), c.kvDim(), c.headDim, c.kvDim(),
+                      qRotH.data(), kcHost.data(), vcHost.data());
+    orc_attention_decode(qRotH.data(), kcHost.data(), vcHost.data(), p2 + 1, c.heads, c.kvHeads, c.headDim, c.kvDim(),
+                         1.0f / std::sqrt((float)c.headDim), attnH.data());
+    const double err2 = normwise(unfused, std::vector<double>(attnH.begin(), attnH.end()));
+    if (!(err2 < 1e-3)) std::printf("unfused attention front against the oracle err %g\n", err2);
+    EXPECT(err2 < 1e-3);
+  }
+}
+
 int main(int argc, char **argv) {
   std::string mode = argc > 1 ? argv[1] : "--cpu";
   test_tables();
   test_validation();
   test_matmul_plan();
-  if (mode == "--gpu") test_gpu();
+  if (mode == "--gpu") {
+    test_gpu();
+    test_gpu_decode_chain();
+  }
   std::printf("%s: %d failure(s)\n", mode.c_str(), g_fail);
   return g_fail ? 1 : 0;
 }
