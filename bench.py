@@ -29,7 +29,6 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 N_FF, N_EMBD = 14336, 4096
 COPIES = 6
-kPrimeMinLaunches = 150   # graphs at least this long get an untimed first replay (see timed_graph)
 
 
 def log(*a):
@@ -43,14 +42,15 @@ def make_q_weights(fmt_name, n, k, seed):
     return Q.quantize(fmt_name, w)
 
 
-def timed_graph(torch, fn_step, steps, warmup, launches_per_step=1):
-    """Runs `warmup` eager steps, captures `steps` steps into one HIP graph and times one replay of it.  A graph of
-    kPrimeMinLaunches kernel nodes or more is replayed once untimed before (part of the warm-up): the first replay of
-    a graph also uploads it, 0.5-1 us per node, which is 5-10 % of a long graph of 10-20 us launches and nothing of a
-    graph of a few long ones.  Short graphs are not primed: a second back-to-back replay of 50-200 us bandwidth-bound
-    launches runs 3-10 % slower than the first on this part (it recovers after a 50 ms pause, which in turn costs the
-    short launches 2-4 %: power management in both directions), so every figure here is what a burst of that length
-    reaches from a GPU that has just done the warm-up.  Returns (wall_seconds, event_ms, used_graph)."""
+def timed_graph(torch, fn_step, steps, warmup, prime=False):
+    """Runs `warmup` eager steps, captures `steps` steps into one HIP graph and times one replay of it.  prime: replay
+    it once untimed before (part of the warm-up).  The first replay of a graph also uploads it, 0.5-1 us per kernel
+    node: 3-10 % of a graph of 9-15 us launches (the headline at 20 steps: 9.1 us per launch unprimed, 8.8 primed) and
+    nothing of a graph of a few long ones.  The callers made of short launches (the FFN steps at every batch size, the
+    decode step) prime; the others do not and stay comparable with their earlier figures: a second back-to-back replay
+    of long bandwidth-bound launches runs 3-10 % slower than the first on this part (it recovers after a 50 ms pause,
+    which in turn costs short launches 2-4 %: power management in both directions), so those are burst figures, and a
+    primed run of thousands of short launches is a sustained one.  Returns (wall_seconds, event_ms, used_graph)."""
     for s in range(warmup):
         fn_step(s)
     torch.cuda.synchronize()
@@ -62,7 +62,7 @@ def timed_graph(torch, fn_step, steps, warmup, launches_per_step=1):
                 fn_step(s)
         torch.cuda.synchronize()
         run = g.replay
-        if steps * launches_per_step >= kPrimeMinLaunches:
+        if prime:
             g.replay()
     except Exception as e:  # noqa: BLE001
         log(f"[bench] graph capture failed ({e}); timing eager launches")
@@ -112,13 +112,13 @@ def bench_decode_step(torch, np, ops, dev, x_h, steps=5):
 
     def decode_step(_s):
         dstep.step()           # embedding row of the token the previous step sampled, 32 layers, head, arg-max
-    wall_c, ev_c, _ = timed_graph(torch, decode_step, steps, 1, launches_per_step=6 * 32)
+    wall_c, ev_c, _ = timed_graph(torch, decode_step, steps, 1, prime=True)
     w_bytes_tok = cfg.n_layers * sum(v.numel() for v in base.values()) + head.numel()
     kv_bytes_tok = cfg.n_layers * 2 * cfg.max_ctx * cfg.kv_dim * 2
     # What the launch bound of the attention costs: 256 cached positions, once in the 2048-position cache (the attention
     # launches, and reads, for 2048) and once with a cache and a launch bound of 256 (same weights).
     dstep.set_position(255)
-    _, ev_short, _ = timed_graph(torch, decode_step, steps, 1, launches_per_step=6 * 32)
+    _, ev_short, _ = timed_graph(torch, decode_step, steps, 1, prime=True)
     import dataclasses
     cfg256 = dataclasses.replace(cfg, max_ctx=256)
     dstep256 = DecodeStep(cfg256, layers, ones, head, dev, fuse=int(os.environ.get("CUT_DECODE_FUSE", "4")), embedding=embd)
@@ -126,7 +126,7 @@ def bench_decode_step(torch, np, ops, dev, x_h, steps=5):
         kc.normal_(0.0, 0.5)
         vc.normal_(0.0, 1.0)
     dstep256.set_position(255)
-    _, ev_256, _ = timed_graph(torch, lambda _s: dstep256.step(), steps, 1, launches_per_step=6 * 32)
+    _, ev_256, _ = timed_graph(torch, lambda _s: dstep256.step(), steps, 1, prime=True)
     return {"decode_step_8b_ctx256_in_cache2048_ms_per_token": round(ev_short / steps, 3),
             "decode_step_8b_ctx256_in_cache256_ms_per_token": round(ev_256 / steps, 3),
             "decode_step_8b_ctx2048_ms_per_token": round(ev_c / steps, 3),
@@ -436,18 +436,18 @@ def main():
 
     if args.matmul_batch_only:
         b = args.matmul_batch_only
-        wall_b, ev_b, _ = timed_graph(torch, ffn_step_ws(b), 60, 6, launches_per_step=3)
+        wall_b, ev_b, _ = timed_graph(torch, ffn_step_ws(b), 60, 6, prime=True)
         print(json.dumps({f"q4k_ffn_matmul_batch{b}_GBps": round(ffn_bytes(b) * 60 / wall_b / 1e9, 1),
                           "us_per_matmul": round(ev_b * 1e3 / 180, 2)}))
         return
     if args.gemv_batch_only:
         b = args.gemv_batch_only
-        wall_b, ev_b, _ = timed_graph(torch, ffn_step(b), 120, 12, launches_per_step=3)
+        wall_b, ev_b, _ = timed_graph(torch, ffn_step(b), 120, 12, prime=True)
         print(json.dumps({f"q4k_ffn_gemv_batch{b}_GBps": round(ffn_bytes(b) * 120 / wall_b / 1e9, 1),
                           "us_per_launch": round(ev_b * 1e3 / 360, 2)}))
         return
     # ---- headline: batch 1 --------------------------------------------------
-    wall, ev_ms, used_graph = timed_graph(torch, ffn_step(1), args.steps, args.warmup, launches_per_step=3)
+    wall, ev_ms, used_graph = timed_graph(torch, ffn_step(1), args.steps, args.warmup, prime=True)
     step_bytes = ffn_bytes(1)
     value = step_bytes * args.steps / wall / 1e9
     launches = 3 * args.steps
@@ -482,12 +482,12 @@ def main():
     extras = {}
     if not args.no_extras:
         for b in (2, 4, 8):
-            wall_b, ev_b, _ = timed_graph(torch, ffn_step(b), 120, 12, launches_per_step=3)
+            wall_b, ev_b, _ = timed_graph(torch, ffn_step(b), 120, 12, prime=True)
             extras[f"q4k_ffn_gemv_batch{b}_GBps"] = round(ffn_bytes(b) * 120 / wall_b / 1e9, 1)
         # 16-128 rows (batched decode, short prefill chunks): the same three matmuls through cuthip_matmul_gguf_ws;
         # GB/s over the same bytes
         for b in (16, 32, 64, 128):
-            wall_b, ev_b, _ = timed_graph(torch, ffn_step_ws(b), 60, 6, launches_per_step=3)
+            wall_b, ev_b, _ = timed_graph(torch, ffn_step_ws(b), 60, 6, prime=True)
             extras[f"q4k_ffn_matmul_batch{b}_GBps"] = round(ffn_bytes(b) * 60 / wall_b / 1e9, 1)
             extras[f"q4k_ffn_matmul_batch{b}_us_per_matmul"] = round(wall_b * 1e6 / 180, 1)
         # gate and up as one launch (rows concatenated, the reference's fused w_gate_up: llama.cpp:1288-1330)
