@@ -147,6 +147,16 @@ __global__ void __launch_bounds__(256) read_probe_kernel(const u32x4 *src, size_
   if ((threadIdx.x & 63) == 0) sink[(blockIdx.x * 4 + threadIdx.x / 64) & 0xFFFF] = r;
 }
 
+// Fills the LDS of every CU with a pattern (cuthip_debug_fill_lds): LDS keeps what the last workgroup left in it, so
+// a kernel that reads a location it never wrote gives results that depend on what ran before; the tests run every
+// operator behind different patterns and ask for identical bits.
+__global__ void __launch_bounds__(1024) fill_lds_kernel(uint32_t pattern, uint32_t ndw, uint32_t *sink) {
+  extern __shared__ uint32_t fill_lds[];
+  for (uint32_t i = threadIdx.x; i < ndw; i += 1024) fill_lds[i] = pattern;
+  __syncthreads();
+  if (fill_lds[(threadIdx.x * 37u) % ndw] != pattern && sink) sink[0] = 1;   // never true: keeps the stores
+}
+
 }  // namespace cuthip
 
 namespace cuthip {
@@ -331,6 +341,20 @@ int cuthip_read_probe(const void *src, size_t bytes, uint32_t *sink, void *strea
   hipLaunchKernelGGL(read_probe_kernel, dim3((uint32_t)blocks), dim3(256), 0, (hipStream_t)stream,
                      reinterpret_cast<const u32x4 *>(src), nvec, sink);
   return check_hip(hipGetLastError(), "read probe launch");
+}
+
+int cuthip_debug_fill_lds(uint32_t pattern, void *stream) {
+  constexpr uint32_t kBytes = 160 * 1024;
+  static bool attr = false;   // (single-threaded callers, as everywhere in this library)
+  if (!attr) {
+    if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(fill_lds_kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kBytes), "hipFuncSetAttribute"))
+      return rc;
+    attr = true;
+  }
+  // one workgroup fills the whole LDS of the CU it lands on; four rounds over the 256 CUs
+  hipLaunchKernelGGL(fill_lds_kernel, dim3(1024), dim3(1024), kBytes, (hipStream_t)stream, pattern, kBytes / 4, (uint32_t *)nullptr);
+  return check_hip(hipGetLastError(), "fill lds launch");
 }
 
 // ---- capture and replay of a launch sequence (the reusable command buffer of the reference, CudaCommandBuffer.cpp:261-285)

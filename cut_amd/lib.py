@@ -32,7 +32,7 @@ EXPORTS = [
     "cuthip_malloc", "cuthip_free", "cuthip_memcpy_h2d", "cuthip_memcpy_d2h", "cuthip_memcpy_d2d", "cuthip_memset",
     "cuthip_stream_create", "cuthip_stream_destroy", "cuthip_stream_sync",
     "cuthip_event_create", "cuthip_event_destroy", "cuthip_event_record", "cuthip_event_sync", "cuthip_event_elapsed_ms",
-    "cuthip_read_probe", "cuthip_epilogue_op_supported",
+    "cuthip_read_probe", "cuthip_debug_fill_lds", "cuthip_epilogue_op_supported",
     "cuthip_graph_begin_capture", "cuthip_graph_end_capture", "cuthip_graph_launch", "cuthip_graph_destroy",
     "cuthip_variant_count", "cuthip_variant_default", "cuthip_variant_available", "cuthip_variant_info", "cuthip_variant_lookup",
     "cuthip_dequant", "cuthip_matmul_gguf", "cuthip_matmul_gguf_pro",
@@ -109,6 +109,7 @@ def load() -> C.CDLL:
     lib.cuthip_event_sync.argtypes = [vp]
     lib.cuthip_event_elapsed_ms.argtypes = [vp, vp, C.POINTER(C.c_float)]
     lib.cuthip_read_probe.argtypes = [vp, C.c_size_t, vp, vp]
+    lib.cuthip_debug_fill_lds.argtypes = [C.c_uint32, vp]
     lib.cuthip_epilogue_op_supported.argtypes = [i, i]
     lib.cuthip_graph_begin_capture.argtypes = [vp]
     lib.cuthip_graph_end_capture.argtypes = [vp, C.POINTER(vp)]

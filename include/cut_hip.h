@@ -160,6 +160,10 @@ int cuthip_graph_destroy(void *graph);
  * duration is what a launch of that size can reach on the part when it does nothing but load, the yardstick the
  * streaming kernels are held against (bench.py --calibrate-read). */
 int cuthip_read_probe(const void *src, size_t bytes, uint32_t *sink, void *stream);
+/* Test hook (no counterpart in the reference): fills the LDS of every CU with `pattern`.  LDS keeps what the last
+ * workgroup left there, so an operator that read a location it had not written would return results that depend on
+ * what ran before it; the tests run the operators behind different patterns and ask for identical bits. */
+int cuthip_debug_fill_lds(uint32_t pattern, void *stream);
 
 /* ---- variant tables ---------------------------------------------------- */
 int cuthip_variant_count(int op);

@@ -621,14 +621,18 @@ private:
 class RuntimeParams {
 public:
   RuntimeParams() : buf_(8) { set(0, 1); }
+  // With a stream the copy is ordered on it (the source is a member: it stays valid until the copy has run; do not
+  // call set() again before that).
   void set(uint32_t position, uint32_t seqLen, void *stream = nullptr) {
-    const uint32_t v[2] = {position, seqLen};
-    buf_.upload(v, sizeof(v), stream);
+    host_[0] = position;
+    host_[1] = seqLen;
+    buf_.upload(host_, sizeof(host_), stream);
   }
   const uint32_t *data() const { return static_cast<const uint32_t *>(buf_.data()); }
 
 private:
   DeviceBuffer buf_;
+  uint32_t host_[2] = {0, 1};
 };
 
 // ---- FusedRoPEKVWriteOpNode: operators/impl/attention/AttentionOp.h:156-184, AttentionOp.cpp:553-612 -------

@@ -3,6 +3,7 @@
 // with a CPU reference.  "--cpu": variant tables and constructor validation
 // only (no device call).  "--gpu": known-answer and seeded cases on device 0,
 // checked against the C oracle.
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -593,7 +594,7 @@ static void test_gpu_decode_chain() {
   EXPECT(qkv[0]->displayName() == "MatMulGgufPairRoPEKVWrite" && wo[0]->displayName() == "MatMulGgufCarry");
   EXPECT(headNode.output().shape == std::vector<uint32_t>{c.vocab});
 
-  Stream stream;
+  Stream stream;   // the host's updates of x and of the runtime parameters go through the same stream as the launches
   auto encode = [&] {   // what Dispatcher::encode does for the nodes of the step, in graph order
     firstNorm.dispatch(stream.get());
     for (uint32_t i = 0; i < c.layers; ++i) {
@@ -634,8 +635,8 @@ static void test_gpu_decode_chain() {
 
   std::vector<float> xHost(c.hidden);
   for (auto &v : xHost) v = ga(rng);
-  xDev.upload(xHost.data(), xHost.size() * 4);
-  params.set(pos, pos + 1);
+  xDev.upload(xHost.data(), xHost.size() * 4, stream.get());
+  params.set(pos, pos + 1, stream.get());
   encode();   // eager
   stream.sync();
   const std::vector<float> eager = check_step(xHost, "eager");
@@ -645,20 +646,32 @@ static void test_gpu_decode_chain() {
   encode();
   graph.end(stream);
   // replay on the same input: the eager logits bit for bit (the cache row of the position is rewritten with the same values)
-  xDev.upload(xHost.data(), xHost.size() * 4);
+  xDev.upload(xHost.data(), xHost.size() * 4, stream.get());
   graph.replay(stream);
   stream.sync();
   {
     std::vector<float> again(c.vocab);
     headNode.output().buffer->download(again.data(), again.size() * 4);
+    if (std::memcmp(again.data(), eager.data(), again.size() * 4) != 0) {
+      size_t ndiff = 0, first = 0;
+      double worst = 0;
+      for (size_t i = 0; i < again.size(); ++i)
+        if (again[i] != eager[i]) {
+          if (!ndiff) first = i;
+          ++ndiff;
+          worst = std::max(worst, (double)std::fabs(again[i] - eager[i]));
+        }
+      std::printf("replay differs from the eager pass: %zu of %zu logits, first %zu, largest difference %g\n", ndiff, again.size(),
+                  first, worst);
+    }
     EXPECT(std::memcmp(again.data(), eager.data(), again.size() * 4) == 0);
   }
   // the next two positions through the same graph: only the 8 bytes of the runtime parameters and x change
   for (int rep = 0; rep < 2; ++rep) {
     ++pos;
     for (auto &v : xHost) v = ga(rng);
-    xDev.upload(xHost.data(), xHost.size() * 4);
-    params.set(pos, pos + 1);
+    xDev.upload(xHost.data(), xHost.size() * 4, stream.get());
+    params.set(pos, pos + 1, stream.get());
     graph.replay(stream);
     stream.sync();
     check_step(xHost, rep ? "replay, position 11" : "replay, position 10");
@@ -668,9 +681,9 @@ static void test_gpu_decode_chain() {
   // reference's own nodes chain them, against the fused launch (same cache row, same rotated q up to rounding)
   {
     const uint32_t p2 = pos + 1;
-    params.set(p2, p2 + 1);
+    params.set(p2, p2 + 1, stream.get());
     for (auto &v : xHost) v = ga(rng);
-    xDev.upload(xHost.data(), xHost.size() * 4);
+    xDev.upload(xHost.data(), xHost.size() * 4, stream.get());
     RMSNormOpNode norm(x, normA[0], c.eps, DataType::Float16);
     DeviceBuffer qkNat(L[0].qk.data(), L[0].qk.size());
     MatMulGgufPairOpNode proj(norm.output(), bytesTensor(qkNat), GgufFormat::Q4_K, c.qDim() + c.kvDim(), bytesTensor(D[0].v),
