@@ -6,9 +6,9 @@
 // The library is opened at run time (dlopen), never linked: a process that
 // already holds a copy (PyTorch ships one with the same soname) shares it, and
 // a machine without it simply keeps the hand-written GEMM.
-// It is opt-in: the library's own choice by shape never takes this path unless
-// CUT_HIP_VENDOR_GEMM=1 is set; otherwise only an explicit variant index (5) or a
-// tuning rule that names it does.  The library is opened, and its handle created
+// It is opt-in: the library's own choice by shape never takes this path; only
+// an explicit variant index (5), or a tuning rule that names it, does.  The
+// library is opened, and its handle created
 // for the device current then, by the first cuthip_variant_available(MATMUL_GGUF,
 // 5) or the first use; a caller that captures streams does one of these before it
 // captures.
