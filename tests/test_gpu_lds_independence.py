@@ -120,3 +120,47 @@ def test_decode_step_does_not_read_lds_it_did_not_write(ops):
                 setattr(O, n, saved[n])
         for lg, tok in outs[1:]:
             assert np.array_equal(lg.view(np.uint32), outs[0][0].view(np.uint32)) and tok == outs[0][1]
+
+
+@pytest.mark.parametrize("name", ["Q8_0", "Q4_0", "Q4_K"])
+@pytest.mark.parametrize("M", [1, 4, 40])
+def test_separated_layout_and_preparation_do_not_read_lds_they_did_not_write(ops, name, M):
+    fmt = oracle.FORMATS[name]
+    N, K = 264, 1024
+    w = torch.from_numpy(quantized_weights(fmt, N, K, seed=M + 1)).cuda()
+    a = torch.from_numpy(gauss_acts((M, K), seed=7)).cuda()
+    q4, affine = name != "Q8_0", name == "Q4_K"
+    same_bits_behind_every_fill(lambda: ops.prepare_sep(w, fmt, N, K))
+    b, s = ops.prepare_sep(w, fmt, N, K)
+    out = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    same_bits_behind_every_fill(lambda: (ops.matmul_sep(a, b, s, N, q4=q4, affine=affine, out=out),))
+
+
+@pytest.mark.parametrize("name", list(oracle.FORMATS))
+def test_fused_prologues_do_not_read_lds_they_did_not_write(ops, name):
+    fmt = oracle.FORMATS[name]
+    N, K = 200, 1024
+    w = torch.from_numpy(quantized_weights(fmt, N, K, seed=3)).cuda()
+    x = torch.from_numpy(gauss_acts((K,), seed=8)).cuda()
+    gu = torch.from_numpy(gauss_acts((2 * K,), seed=9, dtype=np.float16)).cuda()
+    nw = torch.from_numpy(np.random.default_rng(2).uniform(0.5, 1.5, K).astype(np.float32)).cuda()
+    out = torch.empty(N, dtype=torch.float32, device="cuda")
+    same_bits_behind_every_fill(lambda: (ops.matmul_gguf_pro(x, w, fmt, N, K, out, "rmsnorm", nw, 1e-5),))
+    same_bits_behind_every_fill(lambda: (ops.matmul_gguf_pro(gu, w, fmt, N, K, out, "swiglu"),))
+
+
+def test_prefill_paths_do_not_read_lds_they_did_not_write(ops):
+    fmt = oracle.Q4_K
+    M, N, K = 300, 520, 1024
+    w = torch.from_numpy(quantized_weights(fmt, N, K, seed=4)).cuda()
+    a = torch.from_numpy(gauss_acts((M, K), seed=10, dtype=np.float16)).cuda()
+    ws = ops.matmul_gguf_workspace(fmt, M, K, N, a.dtype, "cuda")
+    out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    for variant in (2, 4):
+        same_bits_behind_every_fill(lambda: (ops.matmul_gguf(a, w, fmt, N, K, out=out, workspace=ws, variant=variant),))
+    w16 = ops.dequantize(w, fmt, N, K, torch.float16)
+    same_bits_behind_every_fill(lambda: (ops.matmul_dense_f16(a, w16, out=out),))
+    w8 = torch.from_numpy(quantized_weights(oracle.Q8_0, N, K, seed=5)).cuda()
+    same_bits_behind_every_fill(lambda: (ops.matmul_q8_i8(a, w8, N, K, out=out),))
+    x = torch.from_numpy(gauss_acts((64, K), seed=11)).cuda()
+    same_bits_behind_every_fill(lambda: (ops.quantize_rows_q8_0(x),))
