@@ -53,6 +53,7 @@ struct GemvParams {
   // every wave also stores the largest of its 8 outputs (as stored in C) and its row index to argmax_parts[n / 8];
   // a one-workgroup kernel finishes the reduction.
   ArgmaxPart *argmax_parts = nullptr;
+  uint32_t hot = 0;   // 8-row kernel: flag word of its leading kernel arguments (which optional pointers are set)
 };
 
 // ---- per-tile configuration -------------------------------------------------

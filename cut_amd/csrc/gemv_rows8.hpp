@@ -634,12 +634,19 @@ template <int SUBK, int THREADS, int MT, int XR> struct XStageF16 {
   }
 };
 
+// bits of GemvParams::hot, the flag word among the leading kernel arguments of the 8-row kernels (see gemv_rows8_kernel)
+constexpr uint32_t kHotAF16 = 1u, kHotCF16 = 2u, kHotEpiShift = 2, kHotRopeShift = 5, kHotNextNorm = 1u << 7, kHotSumsq = 1u << 8;
+
 // ---- the kernel -----------------------------------------------------------------
 // MT: batch rows held (1, 2 or 4); RWG x KW waves per workgroup; D ring depth.
 // MT == 1 takes the lane-local dot-product path (v_dot2_f32_f16 on the same
 // subnormal operands: a quarter of the issue cycles of the matrix-core path,
 // whose 32 A-rows would be 7/8 padding); MT > 1 goes through the matrix core.
-template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO>
+// PRE: the launch has epilogue operands to request at its start (the D of a binary epilogue, the weight of a carried
+// norm, the tables of the RoPE epilogue).  Without them (PRE = false: plain products, the consumer side of a carried
+// norm, the row-pair and arg-max epilogues) nothing of the argument block beyond the leading kernel arguments is read
+// before the weight ring is requested.
+template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO, bool PRE = true>
 __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t bid) {
   using S = Rows8<FMT>;
   constexpr bool DOT = MT <= rows8_dot_max<FMT>();
@@ -671,24 +678,6 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
   const uint32_t se = (uint32_t)(((uint64_t)p.nsteps * (kw + 1)) / KW);
   const uint32_t cnt = se - sb, last = min(se > sb ? se - 1 : sb, p.nsteps - 1);
 
-  // Batch 1: the epilogue's operands for this thread's output row (D of a binary epilogue, the weight of a carried
-  // norm) are requested now, ahead of everything else, so that the end of the workgroup does not wait for them.
-  // Valid because each output element is read (as D) and written (as C) by the same thread only.
-  float pre_d = 0.0f, pre_g = 0.0f;
-  const uint32_t prow = KW == 1 ? n0 + (uint32_t)r8 : (bid * RWG + (uint32_t)tid / 8) * 8u + ((uint32_t)tid & 7u);
-  const bool pre_ok = MT == 1 && (KW == 1 || tid < RWG * 8) && prow < p.N;
-  if (pre_ok) {
-    if (p.epi.kind == CUTHIP_EPI_BINARY)
-      pre_d = p.c_f16 ? (float)reinterpret_cast<const half_t *>(p.epi.D)[prow] : reinterpret_cast<const float *>(p.epi.D)[prow];
-    if (p.next_norm_w) pre_g = p.next_norm_w[prow];
-  }
-  float pre_cs = 0.0f, pre_sn = 0.0f;
-  const uint32_t rope_pos = p.rope.mode ? p.rope.params[0] : 0u;
-  if (pre_ok && p.rope.mode == 1 && rope_pos < p.rope.max_pos) {
-    const size_t ti = (size_t)rope_pos * (p.rope.head_dim / 2) + ((prow % p.rope.head_dim) >> 1);
-    pre_cs = p.rope.cosT[ti];
-    pre_sn = p.rope.sinT[ti];
-  }
   // activation loads first (they must not queue behind the weight loads), then the weight ring, then the
   // conversion of the activations; batches beyond the first (large M * K only) are staged behind the ring
   // groups of 8 activations per thread and batch row in the first batch: sized so that typical shapes need no
@@ -702,11 +691,31 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
   xst.init();
   if (fastx) xsf.load(p, 0, tid);
   else xst.load(p, 0, tid, gpr);
+  // Batch 1: the epilogue's operands for this thread's output row (D of a binary epilogue, the weight of a carried
+  // norm) are requested now, right behind the activations, so that the end of the workgroup does not wait for them.
+  // Valid because each output element is read (as D) and written (as C) by the same thread only.
+  float pre_d = 0.0f, pre_g = 0.0f, pre_cs = 0.0f, pre_sn = 0.0f;
+  uint32_t rope_pos = 0u;
+  const uint32_t prow = KW == 1 ? n0 + (uint32_t)r8 : (bid * RWG + (uint32_t)tid / 8) * 8u + ((uint32_t)tid & 7u);
+  if constexpr (PRE) {
+    const bool pre_ok = MT == 1 && (KW == 1 || tid < RWG * 8) && prow < p.N;
+    if (pre_ok) {
+      if (p.epi.kind == CUTHIP_EPI_BINARY)
+        pre_d = p.c_f16 ? (float)reinterpret_cast<const half_t *>(p.epi.D)[prow] : reinterpret_cast<const float *>(p.epi.D)[prow];
+      if (p.hot & kHotNextNorm) pre_g = p.next_norm_w[prow];
+    }
+    rope_pos = p.rope.mode ? p.rope.params[0] : 0u;
+    if (pre_ok && p.rope.mode == 1 && rope_pos < p.rope.max_pos) {
+      const size_t ti = (size_t)rope_pos * (p.rope.head_dim / 2) + ((prow % p.rope.head_dim) >> 1);
+      pre_cs = p.rope.cosT[ti];
+      pre_sn = p.rope.sinT[ti];
+    }
+  }
   // carried RMSNorm, consumer side: the K / 8 partial sums of squares travel like the activations: requested ahead of
   // the weight ring, one share per thread, folded per wave and across the waves through LDS at the staging barrier
   // (the order of the additions depends on the launch shape only)
   constexpr int CP = 4;
-  const uint32_t nparts = (MT == 1 && p.sumsq_parts) ? (p.K + 7) / 8 : 0u;   // batch 1 only: the LDS of larger batches has no room for it
+  const uint32_t nparts = (MT == 1 && (p.hot & kHotSumsq)) ? (p.K + 7) / 8 : 0u;   // batch 1 only: the LDS of larger batches has no room for it
   float cpart[CP];
 #pragma unroll
   for (int jj = 0; jj < CP; ++jj) {
@@ -945,9 +954,30 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
   }
 }
 
-template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO>
-__global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_kernel(GemvParams p) {
-  rows8_body<FMT, MT, RWG, KW, D, XWANT, PRO>(p, blockIdx.x);
+// What a wave needs for its first loads travels as leading scalar kernel arguments: with kernel-argument preloading
+// (-mllvm -amdgpu-kernarg-preload-count, gfx940 and later) they arrive in SGPRs with the wave, and the activation loads
+// go out without a scalar-memory round trip in front of them (a cold read of the argument block costs about 0.3 us).
+// The flag word says which of the optional pointers of GemvParams are set, so that a launch without them never reads them.
+inline uint32_t rows8_hot_flags(const GemvParams &p) {
+  return (p.a_f16 ? kHotAF16 : 0u) | (p.c_f16 ? kHotCF16 : 0u) | ((uint32_t)p.epi.kind << kHotEpiShift) |
+         ((uint32_t)p.rope.mode << kHotRopeShift) | (p.next_norm_w ? kHotNextNorm : 0u) | (p.sumsq_parts ? kHotSumsq : 0u);
+}
+// Copies the preloaded arguments over the fields of the by-value block, so that the body reads registers for them.
+__device__ __forceinline__ void rows8_take_hot(GemvParams &p, const void *A, uint32_t K, uint32_t strideA, uint32_t nsteps,
+                                               uint32_t flags) {
+  p.A = A; p.K = K; p.strideA = strideA; p.nsteps = nsteps;
+  p.a_f16 = (int)(flags & kHotAF16); p.c_f16 = (int)((flags & kHotCF16) != 0);
+  p.epi.kind = (int)((flags >> kHotEpiShift) & 7u);
+  p.rope.mode = (int)((flags >> kHotRopeShift) & 3u);
+  p.hot = flags;   // which of the optional pointers are set: tested in place of the pointers, which are then only read where set
+}
+template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO, bool PRE>
+__global__ void __launch_bounds__(64 * RWG * KW, 2)
+gemv_rows8_kernel(const uint8_t *W, const void *A, const float *sumsq_parts, uint32_t M, uint32_t K, uint32_t N, uint32_t strideA,
+                  uint32_t nsteps, uint32_t row_bytes, uint32_t flags, GemvParams p) {
+  p.W = W; p.M = M; p.N = N; p.row_bytes = row_bytes; p.sumsq_parts = sumsq_parts;
+  rows8_take_hot(p, A, K, strideA, nsteps, flags);
+  rows8_body<FMT, MT, RWG, KW, D, XWANT, PRO, PRE>(p, blockIdx.x);
 }
 
 // K split across workgroups for long rows and few of them (the down projection at batch 2-8): workgroup
@@ -976,11 +1006,16 @@ __global__ void __launch_bounds__(64 * 8, 2) gemv_rows8_ksplit_kernel(GemvParams
 // [0, blocks_a) take the rows of the first, the rest the rows of the second.  Saves a launch and a kernel
 // start where a small projection (w_v) sits next to a larger one (w_q | w_k) of another format.
 template <int FA, int FB, int RWG, int KW, int D, int XWANT>
-__global__ void __launch_bounds__(64 * RWG * KW, 2) gemv_rows8_pair_kernel(GemvParams pa, GemvParams pb, uint32_t blocks_a) {
-  if (blockIdx.x < blocks_a)
+__global__ void __launch_bounds__(64 * RWG * KW, 2)
+gemv_rows8_pair_kernel(const void *A, uint32_t K, uint32_t strideA, uint32_t nsteps, uint32_t flags_a, uint32_t flags_b,
+                       uint32_t blocks_a, GemvParams pa, GemvParams pb) {
+  if (blockIdx.x < blocks_a) {
+    rows8_take_hot(pa, A, K, strideA, nsteps, flags_a);
     rows8_body<FA, 1, RWG, KW, D, XWANT, false>(pa, blockIdx.x);
-  else
+  } else {
+    rows8_take_hot(pb, A, K, strideA, nsteps, flags_b);
     rows8_body<FB, 1, RWG, KW, D, XWANT, false>(pb, blockIdx.x - blocks_a);
+  }
 }
 
 inline size_t rows8_lds_bytes_rt(int fmt, uint32_t nsteps, int mt);
@@ -989,15 +1024,18 @@ template <int FMT> static size_t rows8_lds_bytes(const GemvParams &p, int mt) {
   return rows8_lds_bytes_rt(FMT, p.nsteps, mt);
 }
 
-template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO = false>
+template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO = false, bool PRE = false>
 static int launch_rows8(const GemvParams &p, hipStream_t stream) {
   if constexpr (MT == 1 && !PRO) {
-    if (p.pro) return launch_rows8<FMT, MT, RWG, KW, D, XWANT, true>(p, stream);
+    if (p.pro) return launch_rows8<FMT, MT, RWG, KW, D, XWANT, true, true>(p, stream);
+    if constexpr (!PRE) {   // epilogue operands to request at the start: the instance that does
+      if (p.epi.kind == CUTHIP_EPI_BINARY || p.next_norm_w || p.rope.mode) return launch_rows8<FMT, MT, RWG, KW, D, XWANT, false, true>(p, stream);
+    }
   }
   size_t lds = rows8_lds_bytes<FMT>(p, MT);
   size_t red = (size_t)RWG * KW * MT * 8 * 4;
   if (red > lds) lds = red;
-  auto kern = gemv_rows8_kernel<FMT, MT, RWG, KW, D, XWANT, PRO>;
+  auto kern = gemv_rows8_kernel<FMT, MT, RWG, KW, D, XWANT, PRO, PRE>;
   if (lds > 64 * 1024) {
     if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
@@ -1006,7 +1044,7 @@ static int launch_rows8(const GemvParams &p, hipStream_t stream) {
   }
   uint32_t groups = (p.N + 7) / 8;
   dim3 grid((groups + RWG - 1) / RWG), block(64 * RWG * KW);
-  hipLaunchKernelGGL(kern, grid, block, lds, stream, p);
+  hipLaunchKernelGGL(kern, grid, block, lds, stream, p.W, p.A, p.sumsq_parts, p.M, p.K, p.N, p.strideA, p.nsteps, p.row_bytes, rows8_hot_flags(p), p);
   return check_hip(hipGetLastError(), "gemv launch");
 }
 
@@ -1047,7 +1085,9 @@ static int launch_rows8_pair(const GemvParams &pa, const GemvParams &pb, hipStre
       return rc;
   }
   uint32_t blocks_a = ((pa.N + 7) / 8 + RWG - 1) / RWG, blocks_b = ((pb.N + 7) / 8 + RWG - 1) / RWG;
-  hipLaunchKernelGGL(kern, dim3(blocks_a + blocks_b), dim3(64 * RWG * KW), lds, stream, pa, pb, blocks_a);
+  // (both tensors share the activations: A, K, strideA and nsteps are those of the first)
+  hipLaunchKernelGGL(kern, dim3(blocks_a + blocks_b), dim3(64 * RWG * KW), lds, stream, pa.A, pa.K, pa.strideA, pa.nsteps,
+                     rows8_hot_flags(pa), rows8_hot_flags(pb), blocks_a, pa, pb);
   return check_hip(hipGetLastError(), "gemv pair launch");
 }
 
