@@ -166,11 +166,13 @@ constexpr int kAttnRow = kAttnMaxHd + 8;   // LDS row in halfs: +16 bytes keeps 
 
 // partial layout per (query head h, split s): [m, l, o[headDim]] floats at ((h * nsplit + s) * (2 + headDim))
 // HD: the head dimension when it is the common 128 (loops over it unroll and their LDS reads overlap), 0 = any
+// The arguments that the first loads need (up to and including headDimArg: 14 dwords) lead the list: with
+// kernel-argument preloading they arrive in SGPRs with the wave, and the loads of q, K and V wait for no scalar load.
 template <int HD>
-__global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_f16, const half_t *kCache, const half_t *vCache,
-                                                           const uint32_t *params, float *partial, uint32_t nHeads,
-                                                           uint32_t nKvHeads, uint32_t headDimArg, uint32_t alignedKvDim,
-                                                           float scale, uint32_t nsplit, uint32_t maxSeqLen) {
+__global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, const half_t *kCache, const half_t *vCache,
+                                                           const uint32_t *params, uint32_t alignedKvDim, uint32_t maxSeqLen,
+                                                           uint32_t nHeads, uint32_t nKvHeads, int q_f16, uint32_t headDimArg,
+                                                           float *partial, float scale, uint32_t nsplit) {
   const uint32_t headDim = HD ? (uint32_t)HD : headDimArg;
   __shared__ __attribute__((aligned(16))) half_t Ks[kAttnChunk * kAttnRow];
   __shared__ __attribute__((aligned(16))) half_t Vs[kAttnChunk * kAttnRow];
@@ -305,6 +307,164 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, int q_
         dst[2 + 2 * lane + 1] = o1;
       }
     }
+  }
+}
+
+// ---- decode attention with few, wide context splits (head dimension 128) ----
+// One workgroup per (query head, split), at most kAttnWideSplits splits per head, so that a consumer can fold the
+// records of a head while it stages its activations (the output projection, gemv_rows8.hpp) and the merge launch
+// disappears.  Split s takes the 64-position chunks s, s + nsplit, s + 2 * nsplit, ...: one chunk per wave and round,
+// so a short sequence in a large cache still spreads over the splits.  Every wave works alone until the end (its own
+// K chunk in LDS, V straight from memory into registers: a lane's 16-byte piece of V covers 8 dimensions of one
+// position, and the lane multiplies it by that position's weight), then the four waves' (max, sum, o) are folded
+// into the one record [max, sum, o[128]] of the split.  The query heads that share a KV head read the same chunk:
+// the block index puts them on the same XCD (equal index modulo 8 when nKvHeads * nsplit is a multiple of 8), so
+// the chunk crosses the fabric once.
+constexpr int kAttnWideSplits = 8;
+constexpr size_t kAttnWideLds = 4 * (size_t)kAttnChunk * kAttnRow * 2 + 4 * kAttnChunk * 4 + kAttnMaxHd * 4;
+
+__global__ void __launch_bounds__(256) attn_partial_wide_kernel(const void *q, const half_t *kCache, const half_t *vCache,
+                                                                const uint32_t *params, uint32_t alignedKvDim,
+                                                                uint32_t maxSeqLen, uint32_t nHeads, uint32_t nKvHeads,
+                                                                int q_f16, uint32_t nsplit, float *partial, float scale) {
+  constexpr uint32_t HD = 128;
+  extern __shared__ __attribute__((aligned(16))) uint8_t wide_lds[];
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  half_t *Ks = reinterpret_cast<half_t *>(wide_lds) + (size_t)wave * kAttnChunk * kAttnRow;   // this wave's chunk of K
+  float *Pp = reinterpret_cast<float *>(wide_lds + 4 * (size_t)kAttnChunk * kAttnRow * 2) + wave * kAttnChunk;
+  float *Qs = reinterpret_cast<float *>(wide_lds + 4 * (size_t)kAttnChunk * kAttnRow * 2 + 4 * kAttnChunk * 4);
+  const uint32_t nRep = nHeads / nKvHeads, per_rep = nKvHeads * nsplit;
+  const uint32_t rep = blockIdx.x / per_rep, rem = blockIdx.x - rep * per_rep;
+  const uint32_t kvH = rem / nsplit, split = rem - kvH * nsplit, h = kvH * nRep + rep;
+  const uint32_t grp = lane >> 4, c8 = lane & 15;   // V / K piece of a round: position 4 * it + grp, dimensions 8 * c8 ..
+
+  // the query (raw bits) and the first round's chunk of K and V are requested before anything is used; none of these
+  // loads waits for the sequence length (every row below the cache capacity is readable, rows past the sequence are
+  // masked afterwards)
+  uint32_t q_raw = 0u;
+  if (tid < HD) q_raw = q_f16 ? (uint32_t)reinterpret_cast<const uint16_t *>(q)[(size_t)h * HD + tid]
+                              : reinterpret_cast<const uint32_t *>(q)[(size_t)h * HD + tid];
+  float m_run = -INFINITY, l_run = 0.0f, o_run[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o_run[e] = 0.0f;
+  uint32_t seqLen = 0u;
+  for (uint32_t round = 0;; ++round) {
+    const uint32_t t0 = (split + nsplit * (wave + 4u * round)) * (uint32_t)kAttnChunk;
+    // round 0 runs for every wave (its barrier publishes the query); later rounds end at the sequence length
+    if (round > 0 && t0 >= seqLen) break;
+    u32x4 kr[16], vr[16];
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const size_t off = (size_t)min(t0 + 4u * it + grp, maxSeqLen - 1) * alignedKvDim + kvH * HD + c8 * 8;
+      kr[it] = ld_u32x4(reinterpret_cast<const uint8_t *>(kCache + off));
+    }
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const size_t off = (size_t)min(t0 + 4u * it + grp, maxSeqLen - 1) * alignedKvDim + kvH * HD + c8 * 8;
+      vr[it] = ld_u32x4(reinterpret_cast<const uint8_t *>(vCache + off));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (round == 0) {
+      seqLen = min(params[1], maxSeqLen);   // a length beyond the cache capacity attends the capacity only
+      if (tid < HD) Qs[tid] = q_f16 ? (float)__builtin_bit_cast(half_t, (uint16_t)q_raw) : __builtin_bit_cast(float, q_raw);
+    }
+    const uint32_t nvalid = t0 < seqLen ? min((uint32_t)kAttnChunk, seqLen - t0) : 0u;
+#pragma unroll
+    for (int it = 0; it < 16; ++it) *reinterpret_cast<u32x4 *>(Ks + (4 * it + grp) * kAttnRow + c8 * 8) = kr[it];
+    if (round == 0) __syncthreads();   // the query, and this wave's K
+    else {
+      __builtin_amdgcn_wave_barrier();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+    // score of position t0 + lane
+    float sc = 0.0f;
+    const half_t *krow = Ks + lane * kAttnRow;
+    const f32x4 *qv = reinterpret_cast<const f32x4 *>(Qs);
+#pragma unroll
+    for (uint32_t d = 0; d < HD; d += 8) {
+      half8_t k8 = *reinterpret_cast<const half8_t *>(krow + d);
+      f32x4 qa = qv[d / 4], qb = qv[d / 4 + 1];
+      sc = fmaf(qa.x, (float)k8[0], sc); sc = fmaf(qa.y, (float)k8[1], sc);
+      sc = fmaf(qa.z, (float)k8[2], sc); sc = fmaf(qa.w, (float)k8[3], sc);
+      sc = fmaf(qb.x, (float)k8[4], sc); sc = fmaf(qb.y, (float)k8[5], sc);
+      sc = fmaf(qb.z, (float)k8[6], sc); sc = fmaf(qb.w, (float)k8[7], sc);
+    }
+    sc = lane < nvalid ? sc * scale : -INFINITY;
+    const float m_c = wave_max(sc);
+    const float pw = lane < nvalid ? expf(sc - m_c) : 0.0f;
+    const float l_c = wave_sum(pw);
+    // weights to LDS in the order the V pieces want them: group g holds positions g, g + 4, g + 8, ...
+    Pp[(lane & 3) * 16 + (lane >> 2)] = pw;
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    float o_c[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o_c[e] = 0.0f;
+    const f32x4 *pv = reinterpret_cast<const f32x4 *>(Pp + grp * 16);
+    // rows past the sequence carry weight zero, but what the cache holds there is anything: masked to zero (only a
+    // chunk that the sequence ends in pays for the masks)
+    if (nvalid < (uint32_t)kAttnChunk) {
+#pragma unroll
+      for (int it = 0; it < 16; ++it)
+        if (4u * it + grp >= nvalid) vr[it] = u32x4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const f32x4 p4 = pv[i4];
+      const float pj[4] = {p4.x, p4.y, p4.z, p4.w};
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const half8_t v8 = __builtin_bit_cast(half8_t, vr[4 * i4 + u]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o_c[e] = fmaf(pj[u], (float)v8[e], o_c[e]);
+      }
+    }
+    // fold the chunk into the wave's running (max, sum, o)
+    const float m_new = fmaxf(m_run, m_c);
+    const float a = m_run == -INFINITY ? 0.0f : expf(m_run - m_new), b = m_c == -INFINITY ? 0.0f : expf(m_c - m_new);
+    l_run = a * l_run + b * l_c;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o_run[e] = a * o_run[e] + b * o_c[e];
+    m_run = m_new;
+    __builtin_amdgcn_wave_barrier();   // the next round overwrites Ks and Pp
+  }
+  // the four position groups of the wave hold shares of the same dimensions
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    o_run[e] += __shfl_xor(o_run[e], 16);
+    o_run[e] += __shfl_xor(o_run[e], 32);
+  }
+  // fold the waves: their (max, sum, o) go through LDS (each wave's own K region is free now)
+  float *mine = reinterpret_cast<float *>(Ks);
+  if (lane < 16) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mine[2 + 8 * lane + e] = o_run[e];
+  }
+  if (lane == 0) {
+    mine[0] = m_run;
+    mine[1] = l_run;
+  }
+  __syncthreads();
+  if (tid < HD) {
+    const float *w0 = reinterpret_cast<const float *>(wide_lds);
+    constexpr size_t kStride = (size_t)kAttnChunk * kAttnRow * 2 / 4;   // floats between the waves' regions
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) M = fmaxf(M, w0[w * kStride]);
+    float L = 0.0f, o = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float mw = w0[w * kStride];
+      const float f = mw == -INFINITY ? 0.0f : expf(mw - M);
+      L = fmaf(w0[w * kStride + 1], f, L);
+      o = fmaf(w0[w * kStride + 2 + tid], f, o);
+    }
+    float *dst = partial + ((size_t)h * nsplit + split) * (2 + HD);
+    if (tid == 0) {
+      dst[0] = M;
+      dst[1] = L;
+    }
+    dst[2 + tid] = o;
   }
 }
 
@@ -633,9 +793,9 @@ static int attn_launch(const void *q, int q_dtype, const void *k_cache, const vo
                        uint32_t aligned_kv_dim, float scale, uint32_t max_seq_len, void *partial, hipStream_t s) {
   uint32_t nsplit = (max_seq_len + kAttnChunk - 1) / kAttnChunk;
   auto partial_kernel = head_dim == 128 ? attn_partial_kernel<128> : attn_partial_kernel<0>;
-  hipLaunchKernelGGL(partial_kernel, dim3(n_kv_heads, nsplit), dim3(256), 0, s, q, q_dtype == CUTHIP_F16,
-                     (const half_t *)k_cache, (const half_t *)v_cache, runtime_params, (float *)partial, n_heads, n_kv_heads,
-                     head_dim, aligned_kv_dim, scale, nsplit, max_seq_len);
+  hipLaunchKernelGGL(partial_kernel, dim3(n_kv_heads, nsplit), dim3(256), 0, s, q, (const half_t *)k_cache,
+                     (const half_t *)v_cache, runtime_params, aligned_kv_dim, max_seq_len, n_heads, n_kv_heads,
+                     (int)(q_dtype == CUTHIP_F16), head_dim, (float *)partial, scale, nsplit);
   if (int rc = check_hip(hipGetLastError(), "attention launch")) return rc;
   hipLaunchKernelGGL(attn_merge_kernel, dim3(n_heads), dim3(128), 0, s, (const float *)partial, runtime_params, out,
                      out_dtype == CUTHIP_F16, head_dim, nsplit);
@@ -657,6 +817,60 @@ int cuthip_attn_decode(const void *q, int q_dtype, const void *k_cache, const vo
   }
   return attn_launch(q, q_dtype, k_cache, v_cache, runtime_params, out, out_dtype, n_heads, n_kv_heads, head_dim,
                      aligned_kv_dim, scale, max_seq_len, workspace, (hipStream_t)stream);
+}
+
+uint32_t cuthip_attn_partial_splits(uint32_t max_seq_len) {
+  const uint32_t chunks = (max_seq_len + kAttnChunk - 1) / kAttnChunk;
+  return chunks < (uint32_t)kAttnWideSplits ? chunks : (uint32_t)kAttnWideSplits;
+}
+
+size_t cuthip_attn_partial_bytes(uint32_t n_heads, uint32_t head_dim, uint32_t max_seq_len) {
+  return (size_t)n_heads * cuthip_attn_partial_splits(max_seq_len) * (2 + head_dim) * sizeof(float);
+}
+
+int cuthip_attn_decode_partial(const void *q, int q_dtype, const void *k_cache, const void *v_cache,
+                               const uint32_t *runtime_params, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                               uint32_t aligned_kv_dim, float scale, uint32_t max_seq_len, void *records, size_t records_bytes,
+                               void *stream) {
+  // (the records stand in for the output in the shared checks)
+  if (int rc = attn_check_args("cuthip_attn_decode_partial", q, q_dtype, k_cache, v_cache, runtime_params, records, CUTHIP_F32,
+                               n_heads, n_kv_heads, head_dim, aligned_kv_dim, max_seq_len))
+    return rc;
+  if (head_dim != 128) {
+    set_error("cuthip_attn_decode_partial: head_dim %u (the wide-split kernel is built for 128; use cuthip_attn_decode)", head_dim);
+    return CUTHIP_ERR_INVALID;
+  }
+  if ((uintptr_t)records % 8 != 0 || records_bytes < cuthip_attn_partial_bytes(n_heads, head_dim, max_seq_len)) {
+    set_error("cuthip_attn_decode_partial: records of %zu bytes, need %zu, 8-byte aligned", records_bytes,
+              cuthip_attn_partial_bytes(n_heads, head_dim, max_seq_len));
+    return CUTHIP_ERR_INVALID;
+  }
+  const uint32_t nsplit = cuthip_attn_partial_splits(max_seq_len);
+  static std::once_flag lds_once;
+  static int lds_rc = CUTHIP_OK;
+  std::call_once(lds_once, [] {
+    lds_rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(attn_partial_wide_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kAttnWideLds),
+                       "hipFuncSetAttribute(attention LDS)");
+  });
+  if (lds_rc) return lds_rc;
+  hipLaunchKernelGGL(attn_partial_wide_kernel, dim3(n_heads * nsplit), dim3(256), kAttnWideLds, (hipStream_t)stream, q,
+                     (const half_t *)k_cache, (const half_t *)v_cache, runtime_params, aligned_kv_dim, max_seq_len, n_heads,
+                     n_kv_heads, (int)(q_dtype == CUTHIP_F16), nsplit, (float *)records, scale);
+  return check_hip(hipGetLastError(), "attention launch");
+}
+
+int cuthip_attn_merge(const void *records, uint32_t nsplit, uint32_t n_heads, uint32_t head_dim, void *out, int out_dtype,
+                      void *stream) {
+  if (!records || !out || nsplit == 0 || nsplit > (uint32_t)kAttnMaxSplit || n_heads == 0 || head_dim == 0 ||
+      head_dim > (uint32_t)kAttnMaxHd || (uintptr_t)records % 4 != 0 || bad_dtype(out_dtype)) {
+    set_error("cuthip_attn_merge: bad argument (splits %u (<= %d), heads %u, head_dim %u (<= %d))", nsplit, kAttnMaxSplit,
+              n_heads, head_dim, kAttnMaxHd);
+    return CUTHIP_ERR_INVALID;
+  }
+  hipLaunchKernelGGL(attn_merge_kernel, dim3(n_heads), dim3(128), 0, (hipStream_t)stream, (const float *)records,
+                     (const uint32_t *)nullptr, out, out_dtype == CUTHIP_F16, head_dim, nsplit);
+  return check_hip(hipGetLastError(), "attention merge launch");
 }
 
 }  // extern "C"

@@ -429,6 +429,48 @@ int cuthip_matmul_gguf_carry(int fmt, const void *W, const void *A, int a_dtype,
   return rc;
 }
 
+int cuthip_matmul_gguf_attn_merge(int fmt, const void *W, const void *records, uint32_t nsplit, uint32_t n_heads,
+                                  uint32_t head_dim, void *C, int c_dtype, uint32_t N, int epilogue, int epilogue_op,
+                                  const void *D, const cuthip_norm_carry_t *carry, void *stream) {
+  using namespace cuthip;
+  const uint64_t K64 = (uint64_t)n_heads * head_dim;
+  if (fmt < CUTHIP_Q8_0 || fmt > CUTHIP_Q6_K || (c_dtype != CUTHIP_F32 && c_dtype != CUTHIP_F16) || !W || !records || !C ||
+      N == 0 || K64 == 0 || K64 > 0xFFFFFFFFull || K64 % fmt_elems(fmt) != 0 || head_dim % 8 != 0 || nsplit == 0 ||
+      nsplit > (uint32_t)kMergeMax || (uintptr_t)records % 8 != 0 || (uintptr_t)W % 2 != 0 || epilogue < CUTHIP_EPI_NONE ||
+      epilogue > CUTHIP_EPI_BINARY || (epilogue == CUTHIP_EPI_BINARY && !D)) {
+    set_error("cuthip_matmul_gguf_attn_merge: bad argument (format %d, heads %u x %u, splits %u (<= %d), N %u, epilogue %d)", fmt,
+              n_heads, head_dim, nsplit, kMergeMax, N, epilogue);
+    return CUTHIP_ERR_INVALID;
+  }
+  const uint32_t K = (uint32_t)K64;
+  if (int rc = check_epilogue_op("cuthip_matmul_gguf_attn_merge", epilogue, epilogue_op)) return rc;
+  if (epilogue_op_long(epilogue, epilogue_op)) {
+    set_error("cuthip_matmul_gguf_attn_merge: operator %d runs as a launch of its own after a matmul; not offered here", epilogue_op);
+    return CUTHIP_ERR_INVALID;
+  }
+  if (carry && carry->sumsq_parts) {
+    set_error("cuthip_matmul_gguf_attn_merge: the activations are attention records, not a carried RMSNorm (sumsq_parts must be NULL)");
+    return CUTHIP_ERR_INVALID;
+  }
+  GemvParams p = gemv_params(fmt, W, records, CUTHIP_F32, C, c_dtype, 1, K, N, K, N,
+                             Epilogue{epilogue, epilogue_op, epilogue == CUTHIP_EPI_BINARY ? D : nullptr});
+  if (!apply_carry(p, carry, true)) {
+    set_error("cuthip_matmul_gguf_attn_merge: the producer fields (next_norm_weight, next_x16, next_sumsq_parts) come together, "
+              "next_x16 2-byte aligned");
+    return CUTHIP_ERR_INVALID;
+  }
+  p.pro = CUTHIP_PRO_ATTN_MERGE;
+  p.mrg_nsplit = nsplit;
+  p.mrg_head_dim = head_dim;
+  bool taken = false;
+  int rc = launch_rows8_any(fmt, p, reinterpret_cast<hipStream_t>(stream), &taken);
+  if (!taken) {
+    set_error("cuthip_matmul_gguf_attn_merge: K = %u does not fit the LDS budget of the 8-row GEMV", K);
+    return CUTHIP_ERR_INVALID;
+  }
+  return rc;
+}
+
 }  // extern "C"
 
 namespace cuthip {

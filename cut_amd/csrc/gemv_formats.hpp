@@ -19,6 +19,9 @@ struct RopeAppend {
   half_t *k_cache = nullptr, *v_cache = nullptr;
   uint32_t q_dim = 0, head_dim = 0, kv_stride = 0;
   uint32_t max_pos = 0;   // rows of the caches and tables; a position at or beyond it writes nothing
+  // set by a kernel that has read params[0] itself, ahead of everything else (the host leaves them 0)
+  uint32_t pos = 0;
+  int pos_read = 0;
 };
 
 struct ArgmaxPart {
@@ -53,6 +56,7 @@ struct GemvParams {
   // every wave also stores the largest of its 8 outputs (as stored in C) and its row index to argmax_parts[n / 8];
   // a one-workgroup kernel finishes the reduction.
   ArgmaxPart *argmax_parts = nullptr;
+  uint32_t mrg_nsplit = 0, mrg_head_dim = 0;   // CUTHIP_PRO_ATTN_MERGE: records per head in A, and the head dimension
   uint32_t hot = 0;   // 8-row kernel: flag word of its leading kernel arguments (which optional pointers are set)
 };
 

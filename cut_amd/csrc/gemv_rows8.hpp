@@ -502,6 +502,28 @@ template <> struct Rows8<CUTHIP_Q4_0> {
 // leaves the weight loads in flight.
 // PRO: the kernel instance also implements the activation prologues (RMSNorm, SiLU(gate) * up): extra
 // registers for the norm weights and the sum of squares, so only batch-1 decode kernels are built with it.
+// One group of 8 converted activations into LDS (group gi of batch row m) and, from the first lane of a sub-block, the
+// sub-block's sum.  Every lane of the wave calls it (the sums meet through lane shuffles); ok = the group lies inside K,
+// active = inside the padded row.
+template <int SUBK>
+__device__ __forceinline__ void stage_put(half_t (&h)[8], bool ok, bool active, uint32_t m, uint32_t gi, half_t *xs, float *sxs,
+                                          int xrow, int sxrow) {
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    h[i] = ok ? h[i] : (half_t)0.0f;
+    s += (float)h[i];
+  }
+  s += __shfl_xor(s, 1);
+  if (SUBK == 32) s += __shfl_xor(s, 2);
+  if (active) {
+    half8_t o{h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
+    *reinterpret_cast<half8_t *>(xs + m * xrow + (gi >> 3) * kXGroup + (gi & 7) * 8) = o;
+    constexpr uint32_t per = SUBK / 8;
+    if ((gi & (per - 1)) == 0) sxs[m * sxrow + gi / per] = s;
+  }
+}
+
 template <int SUBK, int THREADS, int MT, int XR, bool PRO> struct XStage {
   u32x4 ra[MT * XR], rb[MT * XR];
   u32x4 wa[PRO ? MT * XR : 1], wb[PRO ? MT * XR : 1];   // norm weights of the group (fp32 x 8)
@@ -571,20 +593,7 @@ template <int SUBK, int THREADS, int MT, int XR, bool PRO> struct XStage {
 #pragma unroll
         for (int i = 0; i < 8; ++i) h[i] = (half_t)x[i];
       }
-      float s = 0.0f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        h[i] = ok ? h[i] : (half_t)0.0f;
-        s += (float)h[i];
-      }
-      s += __shfl_xor(s, 1);
-      if (SUBK == 32) s += __shfl_xor(s, 2);
-      if (active) {
-        half8_t o{h[0], h[2], h[1], h[3], h[4], h[6], h[5], h[7]};
-        *reinterpret_cast<half8_t *>(xs + m * xrow + (gi >> 3) * kXGroup + (gi & 7) * 8) = o;
-        constexpr uint32_t per = SUBK / 8;
-        if ((gi & (per - 1)) == 0) sxs[m * sxrow + gi / per] = s;
-      }
+      stage_put<SUBK>(h, ok, active, m, gi, xs, sxs, xrow, sxrow);
     }
   }
 };
@@ -634,6 +643,62 @@ template <int SUBK, int THREADS, int MT, int XR> struct XStageF16 {
   }
 };
 
+// Activations = the output of a split-context decode attention that has not been merged yet (CUTHIP_PRO_ATTN_MERGE):
+// A holds, per query head, mrg_nsplit records [max, sum, o[mrg_head_dim]] (fp32, o un-normalised), K = heads x
+// mrg_head_dim.  A thread folds the records of its group of 8 dimensions: weights exp(max_s - max), the sum of the
+// weighted sums as the divisor.  All loads of a group are requested together (one memory round trip); every workgroup
+// reads all records, which pays while the records are few (at most kMergeMax per head).
+constexpr int kMergeMax = 8;
+typedef uint32_t u32x4_a8 __attribute__((ext_vector_type(4), aligned(8)));
+typedef float f32x2_a8 __attribute__((ext_vector_type(2), aligned(8)));
+template <int SUBK, int THREADS> struct XStageMerge {
+  u32x4 oa[kMergeMax], ob[kMergeMax];
+  f32x2_a8 ml[kMergeMax];
+  __device__ void load(const GemvParams &p, uint32_t gi) {
+    const uint32_t k = gi * 8;
+    if (k >= p.K) return;
+    const uint32_t hd = p.mrg_head_dim, head = k / hd, d0 = k - head * hd, rec = 2 + hd;
+    const float *base = reinterpret_cast<const float *>(p.A) + (size_t)head * p.mrg_nsplit * rec;
+#pragma unroll
+    for (int s = 0; s < kMergeMax; ++s) {
+      if ((uint32_t)s < p.mrg_nsplit) {
+        const float *r = base + (size_t)s * rec;
+        ml[s] = *reinterpret_cast<const f32x2_a8 *>(r);
+        oa[s] = *reinterpret_cast<const u32x4_a8 *>(r + 2 + d0);
+        ob[s] = *reinterpret_cast<const u32x4_a8 *>(r + 2 + d0 + 4);
+      }
+    }
+  }
+  __device__ void store(const GemvParams &p, uint32_t gi, uint32_t gpr, half_t *xs, float *sxs, int xrow, int sxrow) {
+    const bool active = gi < gpr, ok = active && gi * 8 < p.K;
+    float x[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    if (ok) {
+      float M = -INFINITY;
+#pragma unroll
+      for (int s = 0; s < kMergeMax; ++s)
+        if ((uint32_t)s < p.mrg_nsplit) M = fmaxf(M, ml[s].x);
+      float L = 0.0f;
+#pragma unroll
+      for (int s = 0; s < kMergeMax; ++s) {
+        if ((uint32_t)s < p.mrg_nsplit) {
+          const float w = ml[s].x == -INFINITY ? 0.0f : __expf(ml[s].x - M);   // an empty split weighs nothing
+          L = fmaf(ml[s].y, w, L);
+          const f32x4 a = __builtin_bit_cast(f32x4, oa[s]), b = __builtin_bit_cast(f32x4, ob[s]);
+          x[0] = fmaf(a.x, w, x[0]); x[1] = fmaf(a.y, w, x[1]); x[2] = fmaf(a.z, w, x[2]); x[3] = fmaf(a.w, w, x[3]);
+          x[4] = fmaf(b.x, w, x[4]); x[5] = fmaf(b.y, w, x[5]); x[6] = fmaf(b.z, w, x[6]); x[7] = fmaf(b.w, w, x[7]);
+        }
+      }
+      const float inv = L > 0.0f ? 1.0f / L : 0.0f;   // an empty sequence gives zeros
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] *= inv;
+    }
+    half_t h[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h[i] = (half_t)x[i];
+    stage_put<SUBK>(h, ok, active, 0u, gi, xs, sxs, xrow, sxrow);
+  }
+};
+
 // bits of GemvParams::hot, the flag word among the leading kernel arguments of the 8-row kernels (see gemv_rows8_kernel)
 constexpr uint32_t kHotAF16 = 1u, kHotCF16 = 2u, kHotEpiShift = 2, kHotRopeShift = 5, kHotNextNorm = 1u << 7, kHotSumsq = 1u << 8;
 
@@ -646,7 +711,8 @@ constexpr uint32_t kHotAF16 = 1u, kHotCF16 = 2u, kHotEpiShift = 2, kHotRopeShift
 // norm, the tables of the RoPE epilogue).  Without them (PRE = false: plain products, the consumer side of a carried
 // norm, the row-pair and arg-max epilogues) nothing of the argument block beyond the leading kernel arguments is read
 // before the weight ring is requested.
-template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO, bool PRE = true>
+// PRO: 0 = activations as they are; 1 = the RMSNorm / SiLU(gate) * up prologues; 2 = the attention-merge prologue
+template <int FMT, int MT, int RWG, int KW, int D, int XWANT, int PRO, bool PRE = true>
 __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t bid) {
   using S = Rows8<FMT>;
   constexpr bool DOT = MT <= rows8_dot_max<FMT>();
@@ -686,10 +752,12 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
   const uint32_t gpr = kpad / 8;   // 8-element groups per padded row
   // fp16 activations and no prologue: the short staging; otherwise the general one
   const bool fastx = !PRO && p.a_f16;
-  XStage<S::SUBK, THREADS, MT, XR, PRO> xst;
+  XStage<S::SUBK, THREADS, MT, XR, PRO == 1> xst;
   XStageF16<S::SUBK, THREADS, MT, XR> xsf;
+  XStageMerge<S::SUBK, THREADS> xsm;
   xst.init();
-  if (fastx) xsf.load(p, 0, tid);
+  if constexpr (PRO == 2) xsm.load(p, (uint32_t)tid);
+  else if (fastx) xsf.load(p, 0, tid);
   else xst.load(p, 0, tid, gpr);
   // Batch 1: the epilogue's operands for this thread's output row (D of a binary epilogue, the weight of a carried
   // norm) are requested now, right behind the activations, so that the end of the workgroup does not wait for them.
@@ -704,7 +772,7 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
         pre_d = p.c_f16 ? (float)reinterpret_cast<const half_t *>(p.epi.D)[prow] : reinterpret_cast<const float *>(p.epi.D)[prow];
       if (p.hot & kHotNextNorm) pre_g = p.next_norm_w[prow];
     }
-    rope_pos = p.rope.mode ? p.rope.params[0] : 0u;
+    rope_pos = p.rope.mode ? (p.rope.pos_read ? p.rope.pos : p.rope.params[0]) : 0u;
     if (pre_ok && p.rope.mode == 1 && rope_pos < p.rope.max_pos) {
       const size_t ti = (size_t)rope_pos * (p.rope.head_dim / 2) + ((prow % p.rope.head_dim) >> 1);
       pre_cs = p.rope.cosT[ti];
@@ -728,7 +796,13 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
     S::load(buf[i], row, min(sb + i, last), c, p.K);
     __builtin_amdgcn_sched_barrier(0);   // keep issue order = ring order, so that step i waits for its own loads only
   }
-  if (fastx) {
+  if constexpr (PRO == 2) {
+    xsm.store(p, (uint32_t)tid, gpr, xs, sxs, xrow, sxrow);
+    for (uint32_t base = THREADS; base < gpr; base += THREADS) {
+      xsm.load(p, base + (uint32_t)tid);
+      xsm.store(p, base + (uint32_t)tid, gpr, xs, sxs, xrow, sxrow);
+    }
+  } else if (fastx) {
     xsf.store(p, 0, tid, gpr, xs, sxs, xrow, sxrow);
     for (uint32_t base = THREADS * XR; base < gpr; base += THREADS * XR) {
       xsf.load(p, base, tid);
@@ -747,7 +821,7 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
     t = wave_sum_all(t);
     if (lane == 0) nrm[wave] = t;
   }
-  if (PRO && p.pro == CUTHIP_PRO_RMSNORM) {
+  if (PRO == 1 && p.pro == CUTHIP_PRO_RMSNORM) {
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
       const float t = wave_sum_all(xst.ssq[m]);
@@ -760,7 +834,7 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
     xscale[m] = 1.0f;
-    if (PRO && p.pro == CUTHIP_PRO_RMSNORM) {
+    if (PRO == 1 && p.pro == CUTHIP_PRO_RMSNORM) {
       float t = 0.0f;
       for (int w = 0; w < WAVES; ++w) t += nrm[m * WAVES + w];
       xscale[m] = 1.0f / sqrtf(t / (float)p.K + p.eps);
@@ -830,7 +904,7 @@ __device__ __forceinline__ void rows8_body(const GemvParams &p, const uint32_t b
     for (int q = 0; q < RQ; ++q) {
       float v = S::finish_dot(acc[q], cacc[q]);
       v = add_xor32(add_xor2(add_xor1(v)));
-      out[q] = (PRO ? v * xscale[q] : v) * carry_scale;   // linear in the partial sums: applied before the K ranges are folded
+      out[q] = (PRO == 1 ? v * xscale[q] : v) * carry_scale;   // linear in the partial sums: applied before the K ranges are folded
     }
     writer = c.g == 0 && c.kg == 0;
   } else {
@@ -971,11 +1045,12 @@ __device__ __forceinline__ void rows8_take_hot(GemvParams &p, const void *A, uin
   p.rope.mode = (int)((flags >> kHotRopeShift) & 3u);
   p.hot = flags;   // which of the optional pointers are set: tested in place of the pointers, which are then only read where set
 }
-template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO, bool PRE>
+template <int FMT, int MT, int RWG, int KW, int D, int XWANT, int PRO, bool PRE>
 __global__ void __launch_bounds__(64 * RWG * KW, 2)
 gemv_rows8_kernel(const uint8_t *W, const void *A, const float *sumsq_parts, uint32_t M, uint32_t K, uint32_t N, uint32_t strideA,
                   uint32_t nsteps, uint32_t row_bytes, uint32_t flags, GemvParams p) {
   p.W = W; p.M = M; p.N = N; p.row_bytes = row_bytes; p.sumsq_parts = sumsq_parts;
+  p.rope.pos_read = 0;
   rows8_take_hot(p, A, K, strideA, nsteps, flags);
   rows8_body<FMT, MT, RWG, KW, D, XWANT, PRO, PRE>(p, blockIdx.x);
 }
@@ -1007,8 +1082,15 @@ __global__ void __launch_bounds__(64 * 8, 2) gemv_rows8_ksplit_kernel(GemvParams
 // start where a small projection (w_v) sits next to a larger one (w_q | w_k) of another format.
 template <int FA, int FB, int RWG, int KW, int D, int XWANT>
 __global__ void __launch_bounds__(64 * RWG * KW, 2)
-gemv_rows8_pair_kernel(const void *A, uint32_t K, uint32_t strideA, uint32_t nsteps, uint32_t flags_a, uint32_t flags_b,
-                       uint32_t blocks_a, GemvParams pa, GemvParams pb) {
+gemv_rows8_pair_kernel(const void *A, const uint32_t *rope_params, uint32_t K, uint32_t strideA, uint32_t nsteps, uint32_t flags_a,
+                       uint32_t flags_b, uint32_t blocks_a, GemvParams pa, GemvParams pb) {
+  // The position of the RoPE epilogue is requested first of all (its pointer is among the preloaded arguments): the
+  // table loads of the prologue depend on it, and the weight ring is requested behind them.  Without RoPE the host
+  // passes the (aligned) start of the activations instead, so that the load needs no branch.
+  const uint32_t pos = rope_params[0];
+  pa.M = pb.M = 1u;   // the pair launch is a batch-1 launch
+  pa.rope.pos = pb.rope.pos = pos;
+  pa.rope.pos_read = pb.rope.pos_read = 1;
   if (blockIdx.x < blocks_a) {
     rows8_take_hot(pa, A, K, strideA, nsteps, flags_a);
     rows8_body<FA, 1, RWG, KW, D, XWANT, false>(pa, blockIdx.x);
@@ -1024,12 +1106,13 @@ template <int FMT> static size_t rows8_lds_bytes(const GemvParams &p, int mt) {
   return rows8_lds_bytes_rt(FMT, p.nsteps, mt);
 }
 
-template <int FMT, int MT, int RWG, int KW, int D, int XWANT, bool PRO = false, bool PRE = false>
+template <int FMT, int MT, int RWG, int KW, int D, int XWANT, int PRO = 0, bool PRE = false>
 static int launch_rows8(const GemvParams &p, hipStream_t stream) {
-  if constexpr (MT == 1 && !PRO) {
-    if (p.pro) return launch_rows8<FMT, MT, RWG, KW, D, XWANT, true, true>(p, stream);
+  if constexpr (MT == 1 && PRO == 0) {
+    if (p.pro == CUTHIP_PRO_ATTN_MERGE) return launch_rows8<FMT, MT, RWG, KW, D, XWANT, 2, true>(p, stream);
+    if (p.pro) return launch_rows8<FMT, MT, RWG, KW, D, XWANT, 1, true>(p, stream);
     if constexpr (!PRE) {   // epilogue operands to request at the start: the instance that does
-      if (p.epi.kind == CUTHIP_EPI_BINARY || p.next_norm_w || p.rope.mode) return launch_rows8<FMT, MT, RWG, KW, D, XWANT, false, true>(p, stream);
+      if (p.epi.kind == CUTHIP_EPI_BINARY || p.next_norm_w || p.rope.mode) return launch_rows8<FMT, MT, RWG, KW, D, XWANT, 0, true>(p, stream);
     }
   }
   size_t lds = rows8_lds_bytes<FMT>(p, MT);
@@ -1086,8 +1169,9 @@ static int launch_rows8_pair(const GemvParams &pa, const GemvParams &pb, hipStre
   }
   uint32_t blocks_a = ((pa.N + 7) / 8 + RWG - 1) / RWG, blocks_b = ((pb.N + 7) / 8 + RWG - 1) / RWG;
   // (both tensors share the activations: A, K, strideA and nsteps are those of the first)
-  hipLaunchKernelGGL(kern, dim3(blocks_a + blocks_b), dim3(64 * RWG * KW), lds, stream, pa.A, pa.K, pa.strideA, pa.nsteps,
-                     rows8_hot_flags(pa), rows8_hot_flags(pb), blocks_a, pa, pb);
+  const uint32_t *pos_ptr = (pa.rope.mode || pb.rope.mode) ? pa.rope.params : reinterpret_cast<const uint32_t *>((uintptr_t)pa.A & ~(uintptr_t)3);
+  hipLaunchKernelGGL(kern, dim3(blocks_a + blocks_b), dim3(64 * RWG * KW), lds, stream, pa.A, pos_ptr, pa.K, pa.strideA,
+                     pa.nsteps, rows8_hot_flags(pa), rows8_hot_flags(pb), blocks_a, pa, pb);
   return check_hip(hipGetLastError(), "gemv pair launch");
 }
 

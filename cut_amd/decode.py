@@ -78,7 +78,9 @@ class DecodeStep:
         shapes where launches dominate."""
         if fuse >= 3:
             layers = [dict(L, gate_up=interleave_gate_up(L["gate_up"], cfg.ffn)) for L in layers]
-        if fuse == 4:   # rows of q | k interleaved inside every head for the RoPE epilogue
+        if fuse == 5 and cfg.head_dim != 128:
+            raise ValueError("fuse = 5 needs head_dim 128 (the wide-split attention kernel)")
+        if fuse >= 4:   # rows of q | k interleaved inside every head for the RoPE epilogue
             layers = [dict(L, qk=ops.interleave_rope_rows(L["qk"], cfg.q_dim + cfg.kv_dim, cfg.head_dim)) for L in layers]
         self.cfg, self.layers, self.out_norm, self.head, self.fuse = cfg, layers, out_norm, head, fuse
         dev = torch.device(device)
@@ -104,6 +106,7 @@ class DecodeStep:
         self.cos_t = torch.cos(ang).to(f32).to(dev).contiguous()
         self.sin_t = torch.sin(ang).to(f32).to(dev).contiguous()
         self.ws = ops.attn_decode_workspace(c.n_heads, c.head_dim, c.max_ctx, dev)
+        self.records = ops.attn_partial_records(c.n_heads, c.head_dim, c.max_ctx, dev) if fuse == 5 else None
         self.scale = 1.0 / math.sqrt(c.head_dim)
         self.embedding = embedding
         self.head_ws = ops.lm_head_workspace(c.vocab, dev)
@@ -141,7 +144,7 @@ class DecodeStep:
             ops.embedding_rows(self.embedding, c.fmt_embd, self.token, c.vocab, c.hidden, self.x.view(1, -1))
         if self.fuse == 2:
             return self._step_fused()
-        if self.fuse == 4:
+        if self.fuse >= 4:
             return self._step_carry()
         for i, L in enumerate(self.layers):
             ops.rmsnorm(self.x, L["attn_norm"], c.eps, out=self.xn.view(1, -1))
@@ -191,11 +194,19 @@ class DecodeStep:
                                  c.hidden, carry=consume if i > 0 else None,
                                  rope=ops.rope_append(self.params, self.cos_t, self.sin_t, self.q_rot, self.k_cache[i],
                                                       self.v_cache[i], c.q_dim, c.head_dim))
-            ops.attn_decode(self.q_rot, self.k_cache[i], self.v_cache[i], self.params, c.n_heads, c.n_kv_heads, c.head_dim,
-                            self.scale, self.ws, self.attn)
-            ops.matmul_gguf_carry(self.attn, L["o"], c.fmt_attn, c.hidden, c.q_dim, self.x, binary="add", d=self.x,
-                                  carry=ops.norm_carry(next_norm_weight=L["ffn_norm"], next_x16=self.xn,
-                                                       next_sumsq_parts=self.sumsq_parts))
+            produce = ops.norm_carry(next_norm_weight=L["ffn_norm"], next_x16=self.xn, next_sumsq_parts=self.sumsq_parts)
+            if self.fuse == 5:
+                # five launches per layer: the attention leaves at most 8 records per head, wo folds them while it
+                # stages its activations
+                ops.attn_decode_partial(self.q_rot, self.k_cache[i], self.v_cache[i], self.params, c.n_heads, c.n_kv_heads,
+                                        c.head_dim, self.scale, self.records)
+                ops.matmul_gguf_attn_merge(self.records, L["o"], c.fmt_attn, c.hidden, self.x, carry=produce, binary="add",
+                                           d=self.x)
+            else:
+                ops.attn_decode(self.q_rot, self.k_cache[i], self.v_cache[i], self.params, c.n_heads, c.n_kv_heads,
+                                c.head_dim, self.scale, self.ws, self.attn)
+                ops.matmul_gguf_carry(self.attn, L["o"], c.fmt_attn, c.hidden, c.q_dim, self.x, binary="add", d=self.x,
+                                      carry=produce)
             ops.matmul_gguf_carry(self.xn, L["gate_up"], c.fmt_ffn, 2 * c.ffn, c.hidden, self.act, swiglu_pairs=True, carry=consume)
             nxt = self.layers[i + 1]["attn_norm"] if i + 1 < n_layers else self.out_norm
             ops.matmul_gguf_carry(self.act, L["down"], c.fmt_ffn, c.hidden, c.ffn, self.x, binary="add", d=self.x,

@@ -39,6 +39,8 @@ EXPORTS = [
     "cuthip_matmul_gguf_workspace_bytes", "cuthip_matmul_gguf_ws", "cuthip_matmul_gguf_pair", "cuthip_matmul_gguf_carry",
     "cuthip_rmsnorm", "cuthip_rope_kv_write", "cuthip_attn_decode_workspace_bytes", "cuthip_attn_decode",
     "cuthip_attn_decode_static_max_bytes", "cuthip_attn_decode_static",
+    "cuthip_attn_partial_splits", "cuthip_attn_partial_bytes", "cuthip_attn_decode_partial", "cuthip_attn_merge",
+    "cuthip_matmul_gguf_attn_merge",
     "cuthip_silu_mul", "cuthip_argmax", "cuthip_repetition_penalty", "cuthip_argmax_penalized",
     "cuthip_matmul_gguf_argmax_workspace_bytes", "cuthip_matmul_gguf_argmax", "cuthip_embedding_rows", "cuthip_embedding_col",
     "cuthip_matmul_sep_workspace_bytes", "cuthip_matmul_sep_workspace_bytes_for", "cuthip_matmul_q8_sep", "cuthip_matmul_q4_sep",
@@ -134,6 +136,11 @@ def load() -> C.CDLL:
     lib.cuthip_attn_decode_workspace_bytes.argtypes = [u32, u32, u32]
     lib.cuthip_attn_decode.argtypes = [vp, i, vp, vp, vp, vp, i, u32, u32, u32, u32, f32, u32, vp, C.c_size_t, vp]
     lib.cuthip_attn_decode_static_max_bytes.argtypes = []
+    lib.cuthip_attn_partial_splits.argtypes = [u32]
+    lib.cuthip_attn_partial_bytes.argtypes = [u32, u32, u32]
+    lib.cuthip_attn_decode_partial.argtypes = [vp, i, vp, vp, vp, u32, u32, u32, u32, f32, u32, vp, C.c_size_t, vp]
+    lib.cuthip_attn_merge.argtypes = [vp, u32, u32, u32, vp, i, vp]
+    lib.cuthip_matmul_gguf_attn_merge.argtypes = [i, vp, vp, u32, u32, u32, vp, i, u32, i, i, vp, C.POINTER(NormCarry), vp]
     lib.cuthip_attn_decode_static.argtypes = [vp, i, vp, vp, vp, vp, i, u32, u32, u32, u32, f32, u32, vp]
     lib.cuthip_silu_mul.argtypes = [vp, i, vp, i, u32, vp]
     lib.cuthip_argmax.argtypes = [vp, i, u32, vp, vp]
@@ -158,12 +165,13 @@ def load() -> C.CDLL:
     sized = ("cuthip_attn_decode_workspace_bytes", "cuthip_matmul_sep_workspace_bytes", "cuthip_matmul_sep_workspace_bytes_for",
              "cuthip_matmul_gguf_workspace_bytes", "cuthip_matmul_q8_i8_workspace_bytes",
              "cuthip_matmul_dense_f16_workspace_bytes", "cuthip_attn_decode_static_max_bytes",
-             "cuthip_matmul_gguf_argmax_workspace_bytes")
+             "cuthip_matmul_gguf_argmax_workspace_bytes", "cuthip_attn_partial_bytes")
     for n in EXPORTS:
         if n != "cuthip_last_error" and n not in sized:
             getattr(lib, n).restype = i
     for n in sized:
         getattr(lib, n).restype = C.c_size_t
+    lib.cuthip_attn_partial_splits.restype = u32
     _lib = lib
     return lib
 

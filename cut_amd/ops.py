@@ -273,6 +273,58 @@ def attn_decode_static(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Te
     return out
 
 
+def attn_partial_records(n_heads: int, head_dim: int, max_seq_len: int, device) -> torch.Tensor:
+    """Records of attn_decode_partial: [n_heads, splits, 2 + head_dim] fp32 (max, sum, un-normalised output)."""
+    splits = _l.load().cuthip_attn_partial_splits(max_seq_len)
+    return torch.empty((n_heads, splits, 2 + head_dim), dtype=torch.float32, device=device)
+
+
+def attn_decode_partial(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, runtime_params: torch.Tensor, n_heads: int,
+                        n_kv_heads: int, head_dim: int, scale: float, records: torch.Tensor,
+                        max_seq_len: int | None = None) -> torch.Tensor:
+    """The attention up to the per-split records (cuthip_attn_decode_partial); attn_merge or matmul_gguf_attn_merge
+    folds them.  records: attn_partial_records() for the same max_seq_len."""
+    _l.check(_l.load().cuthip_attn_decode_partial(q.data_ptr(), _dt(q), k_cache.data_ptr(), v_cache.data_ptr(),
+                                                  runtime_params.data_ptr(), n_heads, n_kv_heads, head_dim, k_cache.stride(0),
+                                                  scale, max_seq_len or k_cache.shape[0], records.data_ptr(),
+                                                  records.numel() * records.element_size(), _stream_ptr()))
+    return records
+
+
+def attn_merge(records: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[h, :] from records [n_heads, splits, 2 + head_dim] (cuthip_attn_merge)."""
+    if records.dtype != torch.float32 or records.dim() != 3 or not records.is_contiguous() or not out.is_contiguous():
+        raise _l.CutHipError("attn_merge: records must be a contiguous float32 [heads, splits, 2 + head_dim] tensor")
+    n_heads, splits, rec = records.shape
+    if out.numel() != n_heads * (rec - 2):
+        raise _l.CutHipError("attn_merge: out must hold heads x head_dim elements")
+    _l.check(_l.load().cuthip_attn_merge(records.data_ptr(), splits, n_heads, rec - 2, out.data_ptr(), _dt(out), _stream_ptr()))
+    return out
+
+
+def matmul_gguf_attn_merge(records: torch.Tensor, w_blocks: torch.Tensor, fmt, N: int, out: torch.Tensor, carry=None,
+                           binary: str | None = None, d: torch.Tensor | None = None) -> torch.Tensor:
+    """out [N] = merge(records) . dequant(W)^T with K = heads x head_dim (cuthip_matmul_gguf_attn_merge): the merge of the
+    attention splits rides in the staging of the matmul's activations."""
+    f = _fmt(fmt)
+    if records.dtype != torch.float32 or records.dim() != 3 or not records.is_contiguous() or not out.is_contiguous():
+        raise _l.CutHipError("matmul_gguf_attn_merge: records must be a contiguous float32 [heads, splits, 2 + head_dim] tensor")
+    n_heads, splits, rec = records.shape
+    K = n_heads * (rec - 2)
+    if w_blocks.numel() < n_bytes(f, N, K) or out.numel() != N:
+        raise _l.CutHipError("matmul_gguf_attn_merge: weight tensor too small or output of the wrong size")
+    epi, op, dptr = _l.EPI_NONE, 0, None
+    if binary is not None:
+        if d is None or d.numel() != N or d.dtype != out.dtype:
+            raise _l.CutHipError("matmul_gguf_attn_merge: binary epilogue needs D with the size and dtype of C")
+        epi, op, dptr = _l.EPI_BINARY, _l.BINARY[binary], d.data_ptr()
+    import ctypes
+    _l.check(_l.load().cuthip_matmul_gguf_attn_merge(f, w_blocks.data_ptr(), records.data_ptr(), splits, n_heads, rec - 2,
+                                                     out.data_ptr(), _dt(out), N, epi, op, dptr,
+                                                     ctypes.byref(carry) if carry is not None else None, _stream_ptr()))
+    return out
+
+
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     _l.check(_l.load().cuthip_silu_mul(gate_up.data_ptr(), _dt(gate_up), out.data_ptr(), _dt(out), out.numel(), _stream_ptr()))
     return out

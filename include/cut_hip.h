@@ -77,7 +77,8 @@ typedef enum {
 int cuthip_epilogue_op_supported(int epilogue, int op);
 
 /* Prologues on the activations of cuthip_matmul_gguf_pro. */
-typedef enum { CUTHIP_PRO_NONE = 0, CUTHIP_PRO_RMSNORM = 1, CUTHIP_PRO_SWIGLU = 2 } cuthip_prologue;
+/* (CUTHIP_PRO_ATTN_MERGE is the prologue of cuthip_matmul_gguf_attn_merge; cuthip_matmul_gguf_pro refuses it.) */
+typedef enum { CUTHIP_PRO_NONE = 0, CUTHIP_PRO_RMSNORM = 1, CUTHIP_PRO_SWIGLU = 2, CUTHIP_PRO_ATTN_MERGE = 3 } cuthip_prologue;
 
 typedef struct {
   char name[64];
@@ -494,6 +495,29 @@ int cuthip_attn_decode(const void *q, int q_dtype, const void *k_cache, const vo
                        void *out, int out_dtype, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
                        uint32_t aligned_kv_dim, float scale, uint32_t max_seq_len, void *workspace, size_t workspace_bytes,
                        void *stream);
+
+/* The same attention in two halves, so that the second half can ride in the matmul that consumes the attention output
+ * (the attention output projection `wo` of interface/runner/llama/llama.cpp:1790-1795) and a decode step has one launch
+ * per layer fewer.  cuthip_attn_decode_partial leaves, per query head, cuthip_attn_partial_splits(max_seq_len) <= 8
+ * records [max, sum, o[head_dim]] (fp32; o un-normalised: softmax numerators times V over the positions of the split)
+ * in `records` (cuthip_attn_partial_bytes() bytes, 8-byte aligned); head_dim must be 128 (CUTHIP_ERR_INVALID
+ * otherwise: use cuthip_attn_decode).  cuthip_attn_merge folds such records into out[h,:] (what cuthip_attn_decode
+ * does with its own, narrower records); cuthip_matmul_gguf_attn_merge does the same fold while it stages its
+ * activations: C = merge(records) . dequant(W)^T with K = n_heads * head_dim, the merged activations rounded to fp16
+ * as the attention output of the unfused chain is.  M = 1, the 8-row GEMV only; epilogue, D and the producer fields
+ * of `carry` as in cuthip_matmul_gguf_carry (its consumer field sumsq_parts must be NULL: the activations are not a
+ * carried norm).  Other arguments as cuthip_attn_decode / cuthip_matmul_gguf. */
+uint32_t cuthip_attn_partial_splits(uint32_t max_seq_len);
+size_t cuthip_attn_partial_bytes(uint32_t n_heads, uint32_t head_dim, uint32_t max_seq_len);
+int cuthip_attn_decode_partial(const void *q, int q_dtype, const void *k_cache, const void *v_cache,
+                               const uint32_t *runtime_params, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                               uint32_t aligned_kv_dim, float scale, uint32_t max_seq_len, void *records, size_t records_bytes,
+                               void *stream);
+int cuthip_attn_merge(const void *records, uint32_t nsplit, uint32_t n_heads, uint32_t head_dim, void *out, int out_dtype,
+                      void *stream);
+int cuthip_matmul_gguf_attn_merge(int fmt, const void *W, const void *records, uint32_t nsplit, uint32_t n_heads,
+                                  uint32_t head_dim, void *C, int c_dtype, uint32_t N, int epilogue, int epilogue_op,
+                                  const void *D, const cuthip_norm_carry_t *carry, void *stream);
 
 /* cuthip_attn_decode without a caller workspace.  It has no counterpart in the reference; it exists for callers that
  * cannot allocate device memory or carry a workspace around (code under HIP graph capture, tight serving loops,

@@ -443,10 +443,10 @@ def test_matmul_with_fused_prologues(ops, name, N, K):
     assert normwise_rel_err(out.cpu().numpy() - res, want) < 4e-4
 
 
-@pytest.mark.parametrize("fuse", [0, 1, 2, 3, 4])
-def test_small_decode_step_against_oracle_chain(ops, fuse):
+@pytest.mark.parametrize("fuse,hd", [(0, 64), (1, 64), (2, 64), (3, 64), (4, 64), (4, 128), (5, 128)])
+def test_small_decode_step_against_oracle_chain(ops, fuse, hd):
     from cut_amd.decode import DecodeConfig, DecodeStep
-    cfg = DecodeConfig(hidden=512, n_layers=2, n_heads=8, n_kv_heads=2, head_dim=64, ffn=1024, vocab=2048, max_ctx=64)
+    cfg = DecodeConfig(hidden=512, n_layers=2, n_heads=512 // hd, n_kv_heads=2, head_dim=hd, ffn=1024, vocab=2048, max_ctx=64)
     rng = np.random.default_rng(11)
 
     def qw(fmt, n, k):
@@ -595,7 +595,7 @@ def test_full_size_layer_and_head_against_oracle_chain(ops):
                                        rng.choice(cfg.vocab, 480, replace=False)]))
     head_rows = head.reshape(cfg.vocab, rb)[sample].reshape(-1)
 
-    for fuse in (4, 0):
+    for fuse in (4, 5, 0):
         step = DecodeStep(cfg, [{k: dev(v) for k, v in L.items()}], dev(out_norm), dev(head), fuse=fuse)
         step.k_cache[0].copy_(dev(kc.view(np.float16)))
         step.v_cache[0].copy_(dev(vc.view(np.float16)))

@@ -68,12 +68,13 @@ def test_wider_matmuls_do_not_read_lds_they_did_not_write(ops, name, M):
     same_bits_behind_every_fill(lambda: (ops.matmul_gguf(a, w, fmt, N, K, out=out),))
 
 
-def test_decode_step_does_not_read_lds_it_did_not_write(ops):
+@pytest.mark.parametrize("hd,fuses", [(64, (4, 0)), (128, (5,))])
+def test_decode_step_does_not_read_lds_it_did_not_write(ops, hd, fuses):
     """Every kernel of the fused decode step, one fill in front of each launch (the step's own kernels would otherwise
     leave each other the same LDS every time)."""
     from cut_amd.decode import DecodeConfig, DecodeStep
     from cut_amd import ops as O
-    cfg = DecodeConfig(hidden=512, n_layers=2, n_heads=8, n_kv_heads=2, head_dim=64, ffn=1024, vocab=2048, max_ctx=64)
+    cfg = DecodeConfig(hidden=512, n_layers=2, n_heads=512 // hd, n_kv_heads=2, head_dim=hd, ffn=1024, vocab=2048, max_ctx=64)
     rng = np.random.default_rng(11)
 
     def qw(fmt, n, k):
@@ -88,7 +89,7 @@ def test_decode_step_does_not_read_lds_it_did_not_write(ops):
     x = torch.from_numpy(rng.standard_normal(cfg.hidden).astype(np.float32)).cuda()
     kc = torch.from_numpy((rng.standard_normal((9, cfg.kv_dim)) * 0.5).astype(np.float16)).cuda()
     vc = torch.from_numpy(rng.standard_normal((9, cfg.kv_dim)).astype(np.float16)).cuda()
-    for fuse in (4, 0):
+    for fuse in fuses:
         step = DecodeStep(cfg, layers, vec(cfg.hidden), qw(oracle.Q6_K, cfg.vocab, cfg.hidden), fuse=fuse)
         for i in range(cfg.n_layers):
             step.k_cache[i][:9].copy_(kc)
@@ -96,7 +97,8 @@ def test_decode_step_does_not_read_lds_it_did_not_write(ops):
         step.set_position(9)
         # a fill in front of every launch of the step: wrap the entry points the step calls
         names = [n for n in ("rmsnorm", "matmul_gguf", "matmul_gguf_pair", "matmul_gguf_carry", "matmul_gguf_argmax", "attn_decode",
-                             "rope_kv_write", "silu_mul", "argmax", "argmax_penalized")]
+                             "attn_decode_partial", "matmul_gguf_attn_merge", "rope_kv_write", "silu_mul", "argmax",
+                             "argmax_penalized")]
         saved = {n: getattr(O, n) for n in names}
         pattern = [0]
 
