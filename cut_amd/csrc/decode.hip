@@ -313,7 +313,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const void *q, const 
 // ---- decode attention with few, wide context splits (head dimension 128) ----
 // One workgroup per (query head, split), at most kAttnWideSplits splits per head, so that a consumer can fold the
 // records of a head while it stages its activations (the output projection, gemv_rows8.hpp) and the merge launch
-// disappears.  Split s takes the 64-position chunks s, s + nsplit, s + 2 * nsplit, ...: one chunk per wave and round,
+// disappears.  Split s takes the 64-position chunks s, s + nsplit, s + 2 * nsplit, ...: one chunk per wave and pass,
 // so a short sequence in a large cache still spreads over the splits.  Every wave works alone until the end (its own
 // K chunk in LDS, V straight from memory into registers: a lane's 16-byte piece of V covers 8 dimensions of one
 // position, and the lane multiplies it by that position's weight), then the four waves' (max, sum, o) are folded
@@ -336,9 +336,9 @@ __global__ void __launch_bounds__(256) attn_partial_wide_kernel(const void *q, c
   const uint32_t nRep = nHeads / nKvHeads, per_rep = nKvHeads * nsplit;
   const uint32_t rep = blockIdx.x / per_rep, rem = blockIdx.x - rep * per_rep;
   const uint32_t kvH = rem / nsplit, split = rem - kvH * nsplit, h = kvH * nRep + rep;
-  const uint32_t grp = lane >> 4, c8 = lane & 15;   // V / K piece of a round: position 4 * it + grp, dimensions 8 * c8 ..
+  const uint32_t grp = lane >> 4, c8 = lane & 15;   // V / K piece of a pass: position 4 * it + grp, dimensions 8 * c8 ..
 
-  // the query (raw bits) and the first round's chunk of K and V are requested before anything is used; none of these
+  // the query (raw bits) and the first pass's chunk of K and V are requested before anything is used; none of these
   // loads waits for the sequence length (every row below the cache capacity is readable, rows past the sequence are
   // masked afterwards)
   uint32_t q_raw = 0u;
@@ -348,10 +348,10 @@ __global__ void __launch_bounds__(256) attn_partial_wide_kernel(const void *q, c
 #pragma unroll
   for (int e = 0; e < 8; ++e) o_run[e] = 0.0f;
   uint32_t seqLen = 0u;
-  for (uint32_t round = 0;; ++round) {
-    const uint32_t t0 = (split + nsplit * (wave + 4u * round)) * (uint32_t)kAttnChunk;
-    // round 0 runs for every wave (its barrier publishes the query); later rounds end at the sequence length
-    if (round > 0 && t0 >= seqLen) break;
+  for (uint32_t pass = 0;; ++pass) {
+    const uint32_t t0 = (split + nsplit * (wave + 4u * pass)) * (uint32_t)kAttnChunk;
+    // pass 0 runs for every wave (its barrier publishes the query); later passes end at the sequence length
+    if (pass > 0 && t0 >= seqLen) break;
     u32x4 kr[16], vr[16];
 #pragma unroll
     for (int it = 0; it < 16; ++it) {
@@ -364,14 +364,14 @@ __global__ void __launch_bounds__(256) attn_partial_wide_kernel(const void *q, c
       vr[it] = ld_u32x4(reinterpret_cast<const uint8_t *>(vCache + off));
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (round == 0) {
+    if (pass == 0) {
       seqLen = min(params[1], maxSeqLen);   // a length beyond the cache capacity attends the capacity only
       if (tid < HD) Qs[tid] = q_f16 ? (float)__builtin_bit_cast(half_t, (uint16_t)q_raw) : __builtin_bit_cast(float, q_raw);
     }
     const uint32_t nvalid = t0 < seqLen ? min((uint32_t)kAttnChunk, seqLen - t0) : 0u;
 #pragma unroll
     for (int it = 0; it < 16; ++it) *reinterpret_cast<u32x4 *>(Ks + (4 * it + grp) * kAttnRow + c8 * 8) = kr[it];
-    if (round == 0) __syncthreads();   // the query, and this wave's K
+    if (pass == 0) __syncthreads();   // the query, and this wave's K
     else {
       __builtin_amdgcn_wave_barrier();
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -426,7 +426,7 @@ __global__ void __launch_bounds__(256) attn_partial_wide_kernel(const void *q, c
 #pragma unroll
     for (int e = 0; e < 8; ++e) o_run[e] = a * o_run[e] + b * o_c[e];
     m_run = m_new;
-    __builtin_amdgcn_wave_barrier();   // the next round overwrites Ks and Pp
+    __builtin_amdgcn_wave_barrier();   // the next pass overwrites Ks and Pp
   }
   // the four position groups of the wave hold shares of the same dimensions
 #pragma unroll

@@ -38,7 +38,7 @@ def merge_records(rec: np.ndarray) -> np.ndarray:
 @pytest.mark.parametrize("q_dtype", [np.float32, np.float16])
 @pytest.mark.parametrize("n_heads,n_kv,seq,max_ctx", [
     (32, 8, 2048, 2048), (32, 8, 1, 2048), (32, 8, 5, 2048), (32, 8, 257, 2048), (32, 8, 1999, 2048),
-    (16, 4, 4100, 8192),    # four rounds per wave
+    (16, 4, 4100, 8192),    # four passes per wave
     (6, 1, 130, 256),       # six query heads on one KV head, four splits
     (4, 4, 64, 64),         # one split, three waves without a chunk
     (8, 2, 100, 100),       # a capacity that is no multiple of the chunk
@@ -120,7 +120,7 @@ def synthetic_records(rng, n_heads, splits, hd, empty_heads=(), empty_splits=())
     ("Q4_K", 32, 128, 8, 4096),    # the output projection of the 8B shape
     ("Q4_K", 32, 128, 3, 4096),
     ("Q6_K", 4, 128, 1, 40),
-    ("Q4_K", 64, 128, 8, 200),     # K = 8192: two rounds of groups per thread
+    ("Q4_K", 64, 128, 8, 200),     # K = 8192: two passes of groups per thread
     ("Q8_0", 8, 64, 5, 72),        # another head dimension
     ("Q4_K", 16, 80, 8, 9),        # a head dimension that is no power of two
     ("Q4_0", 2, 16, 2, 24)])
