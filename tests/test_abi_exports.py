@@ -155,6 +155,29 @@ def test_argument_validation_without_a_device():
     assert lib.cuthip_dequant(L.Q4_K, one, one, L.F32, 0, 256, 256, None) == 0
 
 
+def test_attention_halves_validate_without_a_device():
+    lib = L.load()
+    one = C.c_void_p(16)
+    assert lib.cuthip_attn_partial_splits(2048) == 8 and lib.cuthip_attn_partial_splits(65) == 2
+    assert lib.cuthip_attn_partial_splits(64) == 1 and lib.cuthip_attn_partial_splits(1 << 16) == 8
+    assert lib.cuthip_attn_partial_bytes(32, 128, 2048) == 32 * 8 * 130 * 4
+    part = lib.cuthip_attn_decode_partial
+    # a head dimension the wide-split kernel is not built for; records too small; heads that do not divide
+    assert part(one, L.F32, one, one, one, 8, 2, 64, 128, 0.125, 64, one, 1 << 20, None) == -1
+    assert b"head_dim" in lib.cuthip_last_error()
+    assert part(one, L.F32, one, one, one, 8, 2, 128, 256, 0.1, 2048, one, 100, None) == -1
+    assert b"records" in lib.cuthip_last_error()
+    assert part(one, L.F32, one, one, one, 8, 3, 128, 384, 0.1, 2048, one, 1 << 20, None) == -1
+    assert lib.cuthip_attn_merge(one, 0, 8, 128, one, L.F32, None) == -1
+    assert lib.cuthip_attn_merge(one, 8, 8, 136, one, L.F32, None) == -1
+    mm = lib.cuthip_matmul_gguf_attn_merge
+    assert mm(L.Q4_K, one, one, 9, 8, 128, one, L.F32, 64, 0, 0, None, None, None) == -1    # more than 8 records per head
+    assert b"splits" in lib.cuthip_last_error()
+    assert mm(L.Q4_K, one, one, 8, 3, 100, one, L.F32, 64, 0, 0, None, None, None) == -1    # K = 300 is no multiple of 256
+    assert mm(L.Q4_K, one, one, 8, 8, 128, one, L.F32, 64, L.EPI_BINARY, 0, None, None, None) == -1   # binary epilogue without D
+    assert mm(L.Q4_K, one, C.c_void_p(12), 8, 8, 128, one, L.F32, 64, 0, 0, None, None, None) == -1   # records not 8-byte aligned
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(L, "_lib", None)
     monkeypatch.setattr(L, "LIB_PATH", "/nonexistent/libcut_hip.so")
