@@ -42,12 +42,16 @@ def make_q_weights(fmt_name, n, k, seed):
     return Q.quantize(fmt_name, w)
 
 
-PRIME_SECONDS = 0.05   # untimed graph replays in front of a timed one last at least this long (timed_graph, prime=True)
+# untimed graph replays in front of a timed one (timed_graph, prime=True) last at least this long; 0 = one replay.
+# (--prime-seconds: 50 ms of them bring the clocks of an idle GPU up and shorten the launches of a 20-step graph by 2 %
+# by events, but the host thread that slept through them then takes 50 us longer over the timed launch, which costs the
+# wall-clock figure of such a run 6 %; one replay, the default, only takes the upload of the graph out of the timing)
+PRIME_SECONDS = 0.0
 
 
 def timed_graph(torch, fn_step, steps, warmup, prime=False):
     """Runs `warmup` eager steps, captures `steps` steps into one HIP graph and times one replay of it.  prime: replay
-    it untimed before, for 50 ms (part of the warm-up).  The first replay of a graph also uploads it, 0.5-1 us per kernel
+    it once untimed before (part of the warm-up; longer with --prime-seconds).  The first replay of a graph also uploads it, 0.5-1 us per kernel
     node: 3-10 % of a graph of 9-15 us launches (the headline at 20 steps: 9.1 us per launch unprimed, 8.8 primed) and
     nothing of a graph of a few long ones.  The callers made of short launches (the FFN steps at every batch size, the
     decode step) prime; the others do not and stay comparable with their earlier figures: a second back-to-back replay
@@ -66,9 +70,7 @@ def timed_graph(torch, fn_step, steps, warmup, prime=False):
         torch.cuda.synchronize()
         run = g.replay
         if prime:
-            # untimed replays until PRIME_SECONDS of work have passed: the first one uploads the graph, the rest bring the
-            # clocks to where a long run has them (a 20-step graph measures 8.65-8.75 us per launch behind one
-            # untimed replay and 8.30-8.35 behind 50 ms of them, which is what the 2000-step graph measures by itself)
+            # the first untimed replay uploads the graph; further ones until PRIME_SECONDS of work have passed
             t_p = time.perf_counter()
             g.replay()
             torch.cuda.synchronize()
@@ -316,11 +318,14 @@ def main():
                     help="only run the FFN step at B rows (9..256) through the workspace entry point, for profiling")
     ap.add_argument("--gemv-batch-only", type=int, default=0, metavar="B",
                     help="only run the FFN GEMV step at batch B (2..8), for profiling")
+    ap.add_argument("--prime-seconds", type=float, default=PRIME_SECONDS,
+                    help="untimed replays of a graph of short launches in front of its timed replay last this long (0 = one replay)")
     ap.add_argument("--decode-only", action="store_true",
                     help="only run the 8B-shape decode step (target of rocprofv3 runs)")
     ap.add_argument("--head-only", action="store_true",
                     help="only run the batch-1 GEMV at the output-head shape (128256 x 4096) on Q6_K and on Q4_K, for profiling")
     args = ap.parse_args()
+    globals()["PRIME_SECONDS"] = max(args.prime_seconds, 0.0)
     if args.gpus != 1:
         log("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it")
         sys.exit(2)
@@ -482,7 +487,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "BASELINE configs[2]: Q4_K GEMV, FFN shapes 14336x4096 (gate, up) + 4096x14336 (down), "
                                "batch 1, fp16 in/out, fp32 accumulate; one step = the three GEMVs of one FFN block",
-                   "weight_copies_rotated": COPIES, "hip_graph": used_graph, "untimed_graph_replays_before_the_timed_one_s": PRIME_SECONDS, "pct_of_hbm_peak": round(value / HBM_PEAK_GBS * 100, 1)},
+                   "weight_copies_rotated": COPIES, "hip_graph": used_graph, "pct_of_hbm_peak": round(value / HBM_PEAK_GBS * 100, 1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
                      "kernel": "cuthip::gemv_rows8_kernel<Q4_K, MT=1>", "algorithmic_bytes_per_launch": int(launch_bytes),
